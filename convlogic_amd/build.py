@@ -1,0 +1,41 @@
+"""Compiles the HIP sources of this package into convlogic_amd/libconvlogic_amd.so for gfx950.
+
+hipcc cross-compiles without a GPU, so this runs in the build container; the built library
+travels with the tree.  Usage:  python -m convlogic_amd.build
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+SOURCES = ["clg_api.hip", "logic_fc.hip", "packbits.hip", "conv_generic.hip", "conv_block.hip"]
+LIB = os.path.join(PKG, "libconvlogic_amd.so")
+
+
+def hipcc_path():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build(verbose=False):
+    srcs = [os.path.join(PKG, "csrc", s) for s in SOURCES]
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(PKG, "csrc")] + srcs + ["-o", LIB]
+    if verbose:
+        print(" ".join(cmd))
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass does not know the -packed-fp32-ops target feature and says so; that is harmless
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,216 @@
+"""ConvLogicLayer, its autograd functions and PoolLogicLayer.
+Interface of the reference's src/convlogic/convlogic_layer.py, on HIP kernels for gfx950."""
+import torch
+from torch import nn
+from torch.autograd import Function
+
+from ..difflogic.functional import GradFactor, bin_op_s
+from ..difflogic.packbitstensor import PackBitsTensor
+from ..hip import convlogic_hip
+from .treelogic_layer import gate_probabilities
+
+
+class ConvLogicFunction(Function):
+    """Split layer: 4 leaf gates per kernel, [N,C,Ho,Wo,4] (src/convlogic/convlogic_layer.py:16-33)."""
+
+    @staticmethod
+    def forward(ctx, x, w_prob, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+        x, w_prob, selection = x.contiguous(), w_prob.contiguous(), selection.contiguous()
+        y = convlogic_hip.convlogic_forward(x, w_prob, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+        ctx.save_for_backward(x, w_prob, selection)
+        ctx.geometry = (stride_h, stride_w, pad_h, pad_w)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        grad_y = grad_y.contiguous()
+        x, w_prob, selection = ctx.saved_tensors
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_x = convlogic_hip.convlogic_backward_x(grad_y, x, w_prob, selection, *ctx.geometry)
+        if ctx.needs_input_grad[1]:
+            grad_w = convlogic_hip.convlogic_backward_weight(grad_y, x, selection, *ctx.geometry)
+        return grad_x, grad_w, None, None, None, None, None, None, None
+
+
+class FullConvLogicFunction(Function):
+    """Fused block: taps -> 4 leaf gates -> 2 gates -> root gate -> 2x2/2 max pool
+    (src/convlogic/convlogic_layer.py:36-82).  Only the pooled output and one byte per pooled value
+    (which window position won) are kept for backward; the leaf and middle planes are produced on
+    request (return_intermediate) by a separate kernel."""
+
+    @staticmethod
+    def forward(ctx, x, w_prob, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w,
+                return_intermediate=False, return_indices=False):
+        x1, w_prob, selection = x.contiguous(), w_prob.contiguous(), selection.contiguous()
+        geo = (stride_h, stride_w, pad_h, pad_w)
+        y, argmax = convlogic_hip.full_convlogic_forward(x1, w_prob, selection, *geo, kernel_h, kernel_w)
+        ctx.save_for_backward(x1, w_prob, selection, argmax)
+        ctx.geometry = geo
+        extra = []
+        if return_intermediate:
+            extra += list(convlogic_hip.full_convlogic_intermediates(x1, w_prob, selection, *geo, kernel_h, kernel_w))
+        if return_indices:
+            extra.append(convlogic_hip.argmax_to_indices(argmax, 2 * argmax.shape[3]))
+        if not extra:
+            return y
+        ctx.mark_non_differentiable(*extra)
+        return (y, *extra)
+
+    @staticmethod
+    def backward(ctx, grad_y, *_unused):
+        grad_y = grad_y.contiguous()
+        x1, w_prob, selection, argmax = ctx.saved_tensors
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
+        if ctx.needs_input_grad[1]:
+            grad_w = convlogic_hip.full_convlogic_backward_weight(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
+        return grad_x, grad_w, None, None, None, None, None, None, None, None, None
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+class ConvLogicLayer(nn.Module):
+    """Logic-gate convolution: every output channel reads 8 taps (from at most two input channels of
+    its group) inside its receptive field and combines them with 4 gates, or with the complete
+    4 -> 2 -> 1 tree followed by 2x2 OR(max)-pooling when complete=True
+    (src/convlogic/convlogic_layer.py:85-160)."""
+
+    def __init__(self, in_channels: int, out_channels: int, stride=1, padding=1, kernel=3, groups: int = 1,
+                 selection=None, residual_init: bool = False, implementation: str = "cuda", grad_factor: float = 1.0,
+                 complete: bool = False, return_intermediate: bool = False, return_indices: bool = False):
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.stride, self.padding, self.kernel = _pair(stride), _pair(padding), _pair(kernel)
+        self.groups, self.grad_factor, self.complete = groups, grad_factor, complete
+        self.return_intermediate, self.return_indices = return_intermediate, return_indices
+        self.input_bits = 8
+        self.implementation = implementation
+        if implementation == "cuda" and not torch.cuda.is_available():
+            raise RuntimeError("CUDA implementation requested, but CUDA is not available.")
+
+        gates = 7 if complete else 4
+        if residual_init:
+            logits = torch.zeros(out_channels, gates, 16)
+            logits[..., 3] = 5.0
+        else:
+            logits = torch.randn(out_channels, gates, 16)
+        self.weights = nn.Parameter(logits)
+
+        if selection is None:
+            selection = self.generate_selection()
+        self.register_buffer("selection", selection)
+        assert selection.shape == (out_channels, 8)
+        assert self.weights.shape[-1] == 16, f"Expected 16 logic functions, got {self.weights.shape[-1]}"
+
+    def forward(self, x):
+        x = x.contiguous()
+        if self.grad_factor != 1.0 and not isinstance(x, PackBitsTensor):
+            x = GradFactor.apply(x, self.grad_factor)
+        if self.implementation == "cuda":
+            return self.forward_cuda(x)
+        if self.implementation == "python":
+            return self.forward_python_full(x) if self.complete else self.forward_python(x)
+        raise ValueError(f"Unknown implementation {self.implementation!r}")
+
+    def unpack_selection(self, selection: torch.Tensor):
+        return (selection >> 16) & 0xFFFF, (selection >> 8) & 0xFF, selection & 0xFF
+
+    def _tap_values(self, x):
+        """[N,C,Ho,Wo,8] tap values, zero outside the image: tap t of kernel c at (oy,ox) reads
+        x[n, ch, oy*sh + ry - ph, ox*sw + rx - pw] (src/convlogic/convlogic_layer.py:262-282)."""
+        (sh, sw), (ph, pw), (kh, kw) = self.stride, self.padding, self.kernel
+        h, w = x.shape[2], x.shape[3]
+        ho, wo = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
+        ch, ry, rx = (t.long() for t in self.unpack_selection(self.selection))
+        xp = torch.nn.functional.pad(x, (pw, pw, ph, ph))
+        rows = (torch.arange(ho, device=x.device) * sh).view(1, ho, 1, 1) + ry.view(-1, 1, 1, 8)
+        cols = (torch.arange(wo, device=x.device) * sw).view(1, 1, wo, 1) + rx.view(-1, 1, 1, 8)
+        shape = (self.out_channels, ho, wo, 8)
+        return xp[:, ch.view(-1, 1, 1, 8).expand(shape), rows.expand(shape), cols.expand(shape)]
+
+    def forward_python(self, x):
+        """Torch-op implementation of the 4-leaf layer -> [N,C,Ho,Wo,4]."""
+        taps = self._tap_values(x)
+        w_prob = gate_probabilities(self.weights[:, 0:4], self.training, self.weights.dtype)
+        return bin_op_s(taps[..., 0::2], taps[..., 1::2], w_prob.view(1, self.out_channels, 1, 1, 4, 16))
+
+    def forward_python_full(self, x):
+        """Torch-op implementation of the complete block: gates 0:4 on the tap pairs, gates 4:6 on the
+        leaf pairs, gate 6 on top, then 2x2 max pooling (src/convlogic/convlogic_layer.py:231-316)."""
+        c = self.out_channels
+        level = self._tap_values(x.contiguous())
+        for lo, hi in ((0, 4), (4, 6), (6, 7)):
+            w_prob = gate_probabilities(self.weights[:, lo:hi], self.training, x.dtype).view(1, c, 1, 1, hi - lo, 16)
+            level = bin_op_s(level[..., 0::2], level[..., 1::2], w_prob)
+        return PoolLogicLayer()(level)
+
+    def forward_cuda(self, x):
+        x = x.contiguous()
+        w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
+        sel = self.selection.contiguous()
+        geo = (*self.stride, *self.padding, *self.kernel)
+        if self.complete:
+            return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)
+        return ConvLogicFunction.apply(x, w_prob, sel, *geo)
+
+    def extra_repr(self):
+        return f"in_channels={self.in_channels}, out_channels={self.out_channels}, groups={self.groups}"
+
+    def generate_selection(self) -> torch.Tensor:
+        """Random taps, int32 [out_channels, 8] packed ch << 16 | row << 8 | col.  Draws from the global
+        torch generator in the order of src/convlogic/convlogic_layer.py:377-452 (two channels per
+        kernel inside its group, a channel pick per tap, rows, columns, then re-draws of the second tap
+        of a pair that landed on the first), so equal seeds give equal selections."""
+        dev = self.weights.device
+        taps, (kh, kw) = self.input_bits, self.kernel
+        c_out, c_in, groups = self.out_channels, self.in_channels, self.groups
+
+        # input channels are split into `groups` nearly equal runs; output channels likewise
+        sizes = [c_in // groups + (1 if gi < c_in % groups else 0) for gi in range(groups)]
+        first = [sum(sizes[:gi]) for gi in range(groups)]
+        group_of = torch.clamp(torch.arange(c_out, device=dev) // (c_out // groups), 0, groups - 1)
+        pair = torch.empty((c_out, 2), dtype=torch.int32, device=dev)
+        for gi in range(groups):
+            members = (group_of == gi).nonzero(as_tuple=True)[0]
+            if members.numel() > 0:
+                for slot in range(2):
+                    pick = torch.randint(0, sizes[gi], (members.numel(),), device=dev)
+                    pair[members, slot] = (pick + first[gi]).to(torch.int32)
+
+        which = torch.randint(0, 2, (c_out, taps), device=dev, dtype=torch.int32)
+        ch = torch.where(which == 0, pair[:, 0:1], pair[:, 1:2]).expand(c_out, taps).contiguous()
+        rows = torch.randint(0, kh, (c_out, taps), device=dev, dtype=torch.int32)
+        cols = torch.randint(0, kw, (c_out, taps), device=dev, dtype=torch.int32)
+
+        # the two taps of a gate must not be the same element (same position on different channels is fine)
+        for t in range(0, taps, 2):
+            same = (ch[:, t] == ch[:, t + 1]) & (rows[:, t] == rows[:, t + 1]) & (cols[:, t] == cols[:, t + 1])
+            for c in same.nonzero(as_tuple=True)[0].tolist():
+                while True:
+                    r = torch.randint(0, kh, (1,), device=dev, dtype=torch.int32)
+                    q = torch.randint(0, kw, (1,), device=dev, dtype=torch.int32)
+                    if (r.item(), q.item()) != (rows[c, t].item(), cols[c, t].item()):
+                        rows[c, t + 1], cols[c, t + 1] = r, q
+                        break
+        return (ch << 16) | (rows << 8) | cols
+
+
+class PoolLogicLayer(nn.Module):
+    """Max pooling, the OR of a logic network (src/convlogic/convlogic_layer.py:455-480)."""
+
+    def __init__(self, kernel=2, stride=2, return_indices=False):
+        super().__init__()
+        self.kernel, self.stride, self.return_indices = _pair(kernel), _pair(stride), return_indices
+
+    def forward(self, x):
+        if x.ndim == 5:
+            if x.size(4) != 1:
+                raise ValueError(f"Expected last dim=1, got {x.size(4)}")
+            x = x.view(x.shape[:4])
+        elif x.ndim != 4:
+            raise ValueError("Input must be 4D or 5D")
+        return nn.functional.max_pool2d(x, self.kernel, self.stride, return_indices=self.return_indices)

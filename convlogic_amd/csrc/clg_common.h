@@ -1,0 +1,128 @@
+// Shared host/device helpers of the gfx950 logic-layer kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "convlogic_amd.h"
+
+// ---- host side: error reporting ------------------------------------------------------------
+void clg_set_error(const char *fmt, ...);
+
+#define CLG_REQUIRE(cond, ...)       \
+    do {                             \
+        if (!(cond)) {               \
+            clg_set_error(__VA_ARGS__); \
+            return CLG_EINVAL;       \
+        }                            \
+    } while (0)
+
+// Checks the launch that was just enqueued (launch-configuration errors only; no sync).
+#define CLG_CHECK_LAUNCH(name)                                                      \
+    do {                                                                            \
+        hipError_t e_ = hipGetLastError();                                          \
+        if (e_ != hipSuccess) {                                                     \
+            clg_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));    \
+            return CLG_ELAUNCH;                                                     \
+        }                                                                           \
+    } while (0)
+
+static inline int64_t clg_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline hipStream_t clg_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+constexpr int kWave = 64;  // CDNA wavefront
+
+// ---- device side ---------------------------------------------------------------------------
+#if defined(__HIPCC__)
+
+template <typename T>
+struct Coef {  // y = ab*a*b + a_*a + b_*b + one
+    T ab, a, b, one;
+};
+
+// Folds 16 gate probabilities into the 4 coefficients of the multilinear form.  Gate i has the
+// truth table bits i = f00*8 + f01*4 + f10*2 + f11 and op_i(a,b) = f00 + (f10-f00) a + (f01-f00) b
+// + (f00-f01-f10+f11) ab; the sums below are those columns written out (fixed order, so forward
+// and backward kernels see bit-identical coefficients).
+template <typename T>
+__device__ __forceinline__ Coef<T> fold16(const T *__restrict__ w)
+{
+    Coef<T> c;
+    c.ab = ((w[1] - w[2]) - w[4]) - T(2) * w[6] - w[7] + w[8] + T(2) * w[9] + w[11] + w[13] - w[14];
+    c.a = (w[2] + w[3]) + (w[6] + w[7]) - (w[8] + w[9]) - (w[12] + w[13]);
+    c.b = (w[4] + w[5]) + (w[6] + w[7]) - (w[8] + w[9]) - (w[10] + w[11]);
+    c.one = ((w[8] + w[9]) + (w[10] + w[11])) + ((w[12] + w[13]) + (w[14] + w[15]));
+    return c;
+}
+
+template <typename T>
+__device__ __forceinline__ T fma_t(T a, T b, T c);
+template <>
+__device__ __forceinline__ float fma_t<float>(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+template <>
+__device__ __forceinline__ double fma_t<double>(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// Gate value in the folded form.  Always this instruction sequence, so equal inputs give equal
+// bits wherever it is evaluated (the pool argmax depends on that).
+template <typename T>
+__device__ __forceinline__ T gate(const Coef<T> &c, T a, T b)
+{
+    return fma_t(c.ab, a * b, fma_t(c.a, a, fma_t(c.b, b, c.one)));
+}
+template <typename T>
+__device__ __forceinline__ T gate_da(const Coef<T> &c, T b) { return fma_t(c.ab, b, c.a); }
+template <typename T>
+__device__ __forceinline__ T gate_db(const Coef<T> &c, T a) { return fma_t(c.ab, a, c.b); }
+
+// grad_w[i] = sum_k COEF[k][i] * s[k] for the partial sums s = (sum g*ab, sum g*a, sum g*b, sum g).
+template <typename T>
+__device__ __forceinline__ T coef_transpose_row(int i, T sab, T sa, T sb, T s1)
+{
+    const int f00 = (i >> 3) & 1, f01 = (i >> 2) & 1, f10 = (i >> 1) & 1, f11 = i & 1;
+    return T(f00 - f01 - f10 + f11) * sab + T(f10 - f00) * sa + T(f01 - f00) * sb + T(f00) * s1;
+}
+
+// ---- wave64 reductions with DPP (no LDS) ---------------------------------------------------
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_zero(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_zero(double v)
+{
+    const uint64_t u = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, CTRL, ROW_MASK, 0xF, false);
+    const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), CTRL, ROW_MASK, 0xF, false);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
+// Sum over the 64 lanes in a fixed tree; the total is valid in lane 63 (returned broadcast).
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v)
+{
+    v += dpp_zero<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v += dpp_zero<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v += dpp_zero<0x141, 0xF>(v);  // row_half_mirror
+    v += dpp_zero<0x140, 0xF>(v);  // row_mirror
+    v += dpp_zero<0x142, 0xA>(v);  // row_bcast15 into rows 1,3
+    v += dpp_zero<0x143, 0xC>(v);  // row_bcast31 into rows 2,3
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)u, 63);
+        const uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(u >> 32), 63);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// selection tap: ch << 16 | row << 8 | col
+struct Tap {
+    int ch, ry, rx;
+};
+__device__ __forceinline__ Tap unpack_tap(int32_t s) { return Tap{(s >> 16) & 0xFFFF, (s >> 8) & 0xFF, s & 0xFF}; }
+
+#endif  // __HIPCC__

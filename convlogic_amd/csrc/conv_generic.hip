@@ -1,0 +1,546 @@
+// Conv-logic kernels that accept any geometry (stride, padding, kernel size, image size, any tap
+// selection).  They read taps straight from global memory with bounds checks.  The split layers
+// (4 leaf gates per kernel, one tree level) always run here; the fused block uses these kernels
+// when its LDS-tiled kernels (conv_block.hip) cannot take the shape.
+//
+// Launch shape: blockIdx.y is the logic kernel (output channel), so the channel is uniform per
+// workgroup and its taps and folded coefficients live in scalar registers; threads run along
+// output positions.  Gradients are deterministic: weight gradients are block-reduced in a fixed
+// order into per-block partials that a second kernel sums in order; input gradients are gathered
+// per input pixel (one writer per element, no atomics).
+#include "conv_common.h"
+
+namespace {
+
+constexpr int kBlk = 256;
+
+template <typename T>
+struct alignas(sizeof(T) * 4) Quad {
+    T v[4];
+};
+template <typename T>
+struct alignas(sizeof(T) * 2) Pair {
+    T v[2];
+};
+
+// ---------------------------------------------------------------------------------------------
+// split layer: 4 leaf gates
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlk) void conv4_forward_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                           const int32_t *__restrict__ sel, T *__restrict__ y, Geom g,
+                                                           int pos_blocks)
+{
+    const int c = blockIdx.y, n = blockIdx.x / pos_blocks;
+    const int pos = (blockIdx.x % pos_blocks) * kBlk + threadIdx.x;
+    const int P = g.ho * g.wo;
+    if (pos >= P) return;
+    const int oy = pos / g.wo, ox = pos % g.wo;
+    const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    Quad<T> out;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
+        const T a = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p]), oy, ox);
+        const T b = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p + 1]), oy, ox);
+        out.v[p] = gate(cf, a, b);
+    }
+    reinterpret_cast<Quad<T> *>(y)[((int64_t)n * g.c + c) * P + pos] = out;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlk) void conv4_backward_w_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                              const int32_t *__restrict__ sel, T *__restrict__ partial,
+                                                              Geom g)
+{
+    const int c = blockIdx.y, nb = gridDim.x;
+    const int P = g.ho * g.wo;
+    const int64_t items = (int64_t)g.n * P;
+    Tap tap[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    T acc[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc[k] = 0;
+    for (int64_t it = (int64_t)blockIdx.x * kBlk + threadIdx.x; it < items; it += (int64_t)nb * kBlk) {
+        const int n = (int)(it / P), pos = (int)(it % P);
+        const int oy = pos / g.wo, ox = pos % g.wo;
+        const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+        const Quad<T> q = reinterpret_cast<const Quad<T> *>(gy)[((int64_t)n * g.c + c) * P + pos];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const T a = read_tap(xn, g, tap[2 * p], oy, ox), b = read_tap(xn, g, tap[2 * p + 1], oy, ox);
+            acc[4 * p + 0] = fma_t(q.v[p], a * b, acc[4 * p + 0]);
+            acc[4 * p + 1] = fma_t(q.v[p], a, acc[4 * p + 1]);
+            acc[4 * p + 2] = fma_t(q.v[p], b, acc[4 * p + 2]);
+            acc[4 * p + 3] += q.v[p];
+        }
+    }
+    block_sum_store<T, 16, kBlk>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 16);
+}
+
+// out[row*G + q][i] = sum_k COEF[k][i] * (sum_blk partial[row][blk][q*4 + k])
+template <typename T>
+__global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t rows, int nb, int G)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= rows * G * 16) return;
+    const int i = (int)(e % 16);
+    const int q = (int)((e / 16) % G);
+    const int64_t row = e / (16 * G);
+    T s[4] = {0, 0, 0, 0};
+    for (int blk = 0; blk < nb; ++blk) {
+        const T *p = partial + ((row * nb + blk) * G + q) * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s[k] += p[k];
+    }
+    out[e] = coef_transpose_row<T>(i, s[0], s[1], s[2], s[3]);
+}
+
+// One thread per input element; every (kernel, tap) that reads the element's channel is visited in
+// a fixed order, so the sum is reproducible.  BLOCK = false: gradient of the 4-leaf layer
+// (grad arrives per leaf gate and conv position).  BLOCK = true: gradient of the fused block
+// (grad arrives per pooled cell and flows to the stored argmax position through the tree).
+template <typename T, bool BLOCK>
+__global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                                    const T *__restrict__ w,
+                                                                    const int32_t *__restrict__ sel,
+                                                                    const uint8_t *__restrict__ argmax,
+                                                                    T *__restrict__ gx, Geom g)
+{
+    const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
+    const int64_t e = (int64_t)blockIdx.x * kBlk + threadIdx.x;
+    if (e >= total) return;
+    const int ix = (int)(e % g.w), iy = (int)((e / g.w) % g.h);
+    const int ch = (int)((e / ((int64_t)g.w * g.h)) % g.cin), n = (int)(e / ((int64_t)g.w * g.h * g.cin));
+    const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    const int P = g.ho * g.wo, wp = g.wo / 2, I = (g.ho / 2) * wp;
+    T acc = 0;
+    for (int c = 0; c < g.c; ++c) {
+        for (int t = 0; t < 8; ++t) {
+            const Tap tp = unpack_tap(sel[c * 8 + t]);
+            if (tp.ch != ch) continue;
+            const int ny = iy + g.ph - tp.ry, nx = ix + g.pw - tp.rx;
+            if (ny < 0 || nx < 0 || ny % g.sh != 0 || nx % g.sw != 0) continue;
+            const int oy = ny / g.sh, ox = nx / g.sw;
+            if (oy >= g.ho || ox >= g.wo) continue;
+            const int p = t >> 1;
+            if constexpr (!BLOCK) {
+                const T gl = gy[(((int64_t)n * g.c + c) * P + oy * g.wo + ox) * 4 + p];
+                const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
+                const T other = read_tap(xn, g, unpack_tap(sel[c * 8 + (t ^ 1)]), oy, ox);
+                acc += gl * ((t & 1) ? gate_db(cf, other) : gate_da(cf, other));
+            } else {
+                const int64_t cell = ((int64_t)n * g.c + c) * I + (oy >> 1) * wp + (ox >> 1);
+                if (argmax[cell] != ((oy & 1) * 2 + (ox & 1))) continue;
+                const Tree<T> tr = load_tree(w + c * 7 * 16);
+                T tap[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) tap[k] = read_tap(xn, g, unpack_tap(sel[c * 8 + k]), oy, ox);
+                const TreeVals<T> v = eval_tree(tr, tap);
+                const T g_root = gy[cell];
+                const int m = p >> 1;  // middle gate above leaf p
+                const T g_mid = g_root * (m ? gate_db(tr.g[6], v.mid[0]) : gate_da(tr.g[6], v.mid[1]));
+                const T g_leaf = g_mid * ((p & 1) ? gate_db(tr.g[4 + m], v.leaf[p ^ 1]) : gate_da(tr.g[4 + m], v.leaf[p ^ 1]));
+                acc += g_leaf * ((t & 1) ? gate_db(tr.g[p], tap[t ^ 1]) : gate_da(tr.g[p], tap[t ^ 1]));
+            }
+        }
+    }
+    gx[e] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// one tree level
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxTreeOut = 1024;
+
+template <typename T, bool BACKWARD>
+__global__ __launch_bounds__(kBlk) void tree_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                  const T *__restrict__ w, T *__restrict__ out, int C, int64_t positions,
+                                                  int xo, int64_t blocks_per_nc)
+{
+    __shared__ Coef<T> cf[kMaxTreeOut];
+    const int c = blockIdx.y;
+    for (int p = threadIdx.x; p < xo; p += kBlk) cf[p] = fold16(w + ((int64_t)c * xo + p) * 16);
+    __syncthreads();
+    const int64_t n = blockIdx.x / blocks_per_nc;
+    const int64_t e = (blockIdx.x % blocks_per_nc) * kBlk + threadIdx.x;  // over positions * xo
+    if (e >= positions * xo) return;
+    const int p = (int)(e % xo);
+    const int64_t base = (n * C + c) * positions * xo + e;
+    const Pair<T> in = reinterpret_cast<const Pair<T> *>(x)[base];
+    if constexpr (!BACKWARD) {
+        out[base] = gate(cf[p], in.v[0], in.v[1]);
+    } else {
+        const T gv = gy[base];
+        Pair<T> r;
+        r.v[0] = gv * gate_da(cf[p], in.v[1]);
+        r.v[1] = gv * gate_db(cf[p], in.v[0]);
+        reinterpret_cast<Pair<T> *>(out)[base] = r;
+    }
+}
+
+// grid.y = c * xo + p; partial [c*xo+p][blk][4]
+template <typename T>
+__global__ __launch_bounds__(kBlk) void tree_backward_w_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                             T *__restrict__ partial, int64_t N, int C, int64_t positions,
+                                                             int xo)
+{
+    const int c = blockIdx.y / xo, p = blockIdx.y % xo, nb = gridDim.x;
+    const int64_t items = N * positions;
+    T acc[4] = {0, 0, 0, 0};
+    for (int64_t it = (int64_t)blockIdx.x * kBlk + threadIdx.x; it < items; it += (int64_t)nb * kBlk) {
+        const int64_t n = it / positions, pos = it % positions;
+        const int64_t base = ((n * C + c) * positions + pos) * xo + p;
+        const Pair<T> in = reinterpret_cast<const Pair<T> *>(x)[base];
+        const T gv = gy[base];
+        acc[0] = fma_t(gv, in.v[0] * in.v[1], acc[0]);
+        acc[1] = fma_t(gv, in.v[0], acc[1]);
+        acc[2] = fma_t(gv, in.v[1], acc[2]);
+        acc[3] += gv;
+    }
+    block_sum_store<T, 4, kBlk>(acc, partial + ((int64_t)blockIdx.y * nb + blockIdx.x) * 4);
+}
+
+// ---------------------------------------------------------------------------------------------
+// fused block, any geometry
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlk) void convblock_forward_generic_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                                       const int32_t *__restrict__ sel, T *__restrict__ y,
+                                                                       uint8_t *__restrict__ argmax, Geom g, int cell_blocks)
+{
+    const int c = blockIdx.y, n = blockIdx.x / cell_blocks;
+    const int cell = (blockIdx.x % cell_blocks) * kBlk + threadIdx.x;
+    const int wp = g.wo / 2, I = (g.ho / 2) * wp;
+    if (cell >= I) return;
+    const int py = cell / wp, px = cell % wp;
+    const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    const Tree<T> tr = load_tree(w + c * 7 * 16);
+    Tap tap[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    T best = -INFINITY;
+    int code = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int oy = 2 * py + (q >> 1), ox = 2 * px + (q & 1);
+        T v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, tap[t], oy, ox);
+        const T r = eval_tree(tr, v).root;
+        if (r > best) {
+            best = r;
+            code = q;
+        }
+    }
+    const int64_t o = ((int64_t)n * g.c + c) * I + cell;
+    y[o] = best;
+    argmax[o] = (uint8_t)code;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlk) void convblock_intermediates_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                                     const int32_t *__restrict__ sel, T *__restrict__ x2,
+                                                                     T *__restrict__ x3, Geom g, int pos_blocks)
+{
+    const int c = blockIdx.y, n = blockIdx.x / pos_blocks;
+    const int pos = (blockIdx.x % pos_blocks) * kBlk + threadIdx.x;
+    const int P = g.ho * g.wo;
+    if (pos >= P) return;
+    const int oy = pos / g.wo, ox = pos % g.wo;
+    const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    const Tree<T> tr = load_tree(w + c * 7 * 16);
+    T v[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t]), oy, ox);
+    const TreeVals<T> tv = eval_tree(tr, v);
+    const int64_t o = ((int64_t)n * g.c + c) * P + pos;
+    if (x2) {
+        Quad<T> q;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) q.v[p] = tv.leaf[p];
+        reinterpret_cast<Quad<T> *>(x2)[o] = q;
+    }
+    if (x3) {
+        Pair<T> pr;
+        pr.v[0] = tv.mid[0];
+        pr.v[1] = tv.mid[1];
+        reinterpret_cast<Pair<T> *>(x3)[o] = pr;
+    }
+}
+
+// 28 partial sums (7 gates x (ab, a, b, 1)) per kernel over all samples and pooled cells.
+template <typename T>
+__global__ __launch_bounds__(kBlk) void convblock_backward_w_generic_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                                          const T *__restrict__ w,
+                                                                          const int32_t *__restrict__ sel,
+                                                                          const uint8_t *__restrict__ argmax,
+                                                                          T *__restrict__ partial, Geom g)
+{
+    const int c = blockIdx.y, nb = gridDim.x;
+    const int wp = g.wo / 2, I = (g.ho / 2) * wp;
+    const int64_t items = (int64_t)g.n * I;
+    const Tree<T> tr = load_tree(w + c * 7 * 16);
+    Tap tap[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    T acc[28];
+#pragma unroll
+    for (int k = 0; k < 28; ++k) acc[k] = 0;
+    for (int64_t it = (int64_t)blockIdx.x * kBlk + threadIdx.x; it < items; it += (int64_t)nb * kBlk) {
+        const int n = (int)(it / I), cell = (int)(it % I);
+        const int64_t o = ((int64_t)n * g.c + c) * I + cell;
+        const int code = argmax[o];
+        const int oy = 2 * (cell / wp) + (code >> 1), ox = 2 * (cell % wp) + (code & 1);
+        const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+        T v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, tap[t], oy, ox);
+        const TreeVals<T> tv = eval_tree(tr, v);
+        T gate_in[7][2], gate_g[7];
+        gate_g[6] = gy[o];
+        gate_in[6][0] = tv.mid[0];
+        gate_in[6][1] = tv.mid[1];
+        gate_g[4] = gate_g[6] * gate_da(tr.g[6], tv.mid[1]);
+        gate_g[5] = gate_g[6] * gate_db(tr.g[6], tv.mid[0]);
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            gate_in[4 + m][0] = tv.leaf[2 * m];
+            gate_in[4 + m][1] = tv.leaf[2 * m + 1];
+            gate_g[2 * m] = gate_g[4 + m] * gate_da(tr.g[4 + m], tv.leaf[2 * m + 1]);
+            gate_g[2 * m + 1] = gate_g[4 + m] * gate_db(tr.g[4 + m], tv.leaf[2 * m]);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            gate_in[p][0] = v[2 * p];
+            gate_in[p][1] = v[2 * p + 1];
+        }
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            acc[4 * k + 0] = fma_t(gate_g[k], gate_in[k][0] * gate_in[k][1], acc[4 * k + 0]);
+            acc[4 * k + 1] = fma_t(gate_g[k], gate_in[k][0], acc[4 * k + 1]);
+            acc[4 * k + 2] = fma_t(gate_g[k], gate_in[k][1], acc[4 * k + 2]);
+            acc[4 * k + 3] += gate_g[k];
+        }
+    }
+    block_sum_store<T, 28, kBlk>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 28);
+}
+
+int partial_blocks(int64_t items)
+{
+    const int64_t nb = clg_ceil_div(items, (int64_t)kBlk * 8);
+    return (int)(nb < 1 ? 1 : (nb > 64 ? 64 : nb));
+}
+
+int check_dtype(int dtype, const char *name)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
+    return CLG_OK;
+}
+
+template <typename T>
+int launch_reduce(const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name)
+{
+    const int64_t total = rows * G * 16;
+    hipLaunchKernelGGL(reduce_coef_partials_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st,
+                       (const T *)partial, (T *)out, rows, nb, G);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
+}
+
+}  // namespace
+
+#define CLG_DISPATCH(dtype, ...)            \
+    do {                                    \
+        if ((dtype) == CLG_F32) {           \
+            using T = float;                \
+            __VA_ARGS__;                    \
+        } else {                            \
+            using T = double;               \
+            __VA_ARGS__;                    \
+        }                                   \
+    } while (0)
+
+static int check_grid(const Geom &g, int64_t per_sample_blocks, const char *name)
+{
+    CLG_REQUIRE(g.c <= 65535, "%s: more than 65535 logic kernels are not supported", name);
+    CLG_REQUIRE((int64_t)g.n * per_sample_blocks < (1ll << 31), "%s: batch too large for one launch", name);
+    return CLG_OK;
+}
+
+extern "C" int clg_conv4_forward(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                 void *y, void *stream)
+{
+    Geom g;
+    if (int e = clg_make_geom(gg, &g, "clg_conv4_forward")) return e;
+    if (int e = check_dtype(dtype, "clg_conv4_forward")) return e;
+    CLG_REQUIRE(x && w && selection && y, "clg_conv4_forward: null pointer argument");
+    const int pos_blocks = (int)clg_ceil_div((int64_t)g.ho * g.wo, kBlk);
+    if (int e = check_grid(g, pos_blocks, "clg_conv4_forward")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(conv4_forward_kernel<T>, dim3((unsigned)(g.n * pos_blocks), g.c), dim3(kBlk), 0,
+                                           clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)y, g, pos_blocks));
+    CLG_CHECK_LAUNCH("clg_conv4_forward");
+    return CLG_OK;
+}
+
+extern "C" int clg_conv4_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                    const int32_t *selection, void *grad_x, void *stream)
+{
+    Geom g;
+    if (int e = clg_make_geom(gg, &g, "clg_conv4_backward_x")) return e;
+    if (int e = check_dtype(dtype, "clg_conv4_backward_x")) return e;
+    CLG_REQUIRE(grad_y && x && w && selection && grad_x, "clg_conv4_backward_x: null pointer argument");
+    const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
+    CLG_REQUIRE(clg_ceil_div(total, kBlk) < (1ll << 31), "clg_conv4_backward_x: input too large for one launch");
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL((conv_backward_x_gather_kernel<T, false>), dim3((unsigned)clg_ceil_div(total, kBlk)),
+                                           dim3(kBlk), 0, clg_stream(stream), (const T *)grad_y, (const T *)x, (const T *)w,
+                                           selection, (const uint8_t *)nullptr, (T *)grad_x, g));
+    CLG_CHECK_LAUNCH("clg_conv4_backward_x");
+    return CLG_OK;
+}
+
+extern "C" int64_t clg_conv4_backward_w_scratch_bytes(int dtype, const clg_conv_geom *gg)
+{
+    Geom g;
+    if (clg_make_geom(gg, &g, "clg_conv4_backward_w_scratch_bytes")) return -1;
+    const int nb = partial_blocks((int64_t)g.n * g.ho * g.wo);
+    return (int64_t)g.c * nb * 16 * (dtype == CLG_F64 ? 8 : 4);
+}
+
+extern "C" int clg_conv4_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x,
+                                    const int32_t *selection, void *grad_w, void *scratch, void *stream)
+{
+    Geom g;
+    if (int e = clg_make_geom(gg, &g, "clg_conv4_backward_w")) return e;
+    if (int e = check_dtype(dtype, "clg_conv4_backward_w")) return e;
+    CLG_REQUIRE(grad_y && x && selection && grad_w && scratch, "clg_conv4_backward_w: null pointer argument");
+    CLG_REQUIRE(g.c <= 65535, "clg_conv4_backward_w: more than 65535 logic kernels are not supported");
+    const int nb = partial_blocks((int64_t)g.n * g.ho * g.wo);
+    hipStream_t st = clg_stream(stream);
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(conv4_backward_w_kernel<T>, dim3(nb, g.c), dim3(kBlk), 0, st, (const T *)grad_y,
+                                           (const T *)x, selection, (T *)scratch, g));
+    CLG_CHECK_LAUNCH("clg_conv4_backward_w");
+    CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, g.c, nb, 4, st, "clg_conv4_backward_w(reduce)"));
+}
+
+static int check_tree(int dtype, int64_t n, int64_t c, int64_t positions, int64_t xo, const char *name)
+{
+    if (int e = check_dtype(dtype, name)) return e;
+    CLG_REQUIRE(n > 0 && c > 0 && positions > 0 && xo > 0, "%s: n, c, positions and xo must be positive", name);
+    CLG_REQUIRE(xo <= kMaxTreeOut, "%s: at most %d gates per channel are supported, got %lld", name, kMaxTreeOut, (long long)xo);
+    CLG_REQUIRE(c * xo <= 65535, "%s: channels * gates above 65535 is not supported", name);
+    CLG_REQUIRE(n * clg_ceil_div(positions * xo, kBlk) < (1ll << 31), "%s: tensor too large for one launch", name);
+    return CLG_OK;
+}
+
+extern "C" int clg_tree_forward(int dtype, const void *x, const void *w, void *y, int64_t n, int64_t c, int64_t positions,
+                                int64_t xo, void *stream)
+{
+    if (int e = check_tree(dtype, n, c, positions, xo, "clg_tree_forward")) return e;
+    CLG_REQUIRE(x && w && y, "clg_tree_forward: null pointer argument");
+    const int64_t bpn = clg_ceil_div(positions * xo, kBlk);
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL((tree_kernel<T, false>), dim3((unsigned)(n * bpn), (unsigned)c), dim3(kBlk), 0,
+                                           clg_stream(stream), (const T *)nullptr, (const T *)x, (const T *)w, (T *)y, (int)c,
+                                           positions, (int)xo, bpn));
+    CLG_CHECK_LAUNCH("clg_tree_forward");
+    return CLG_OK;
+}
+
+extern "C" int clg_tree_backward_x(int dtype, const void *grad_y, const void *x, const void *w, void *grad_x, int64_t n,
+                                   int64_t c, int64_t positions, int64_t xo, void *stream)
+{
+    if (int e = check_tree(dtype, n, c, positions, xo, "clg_tree_backward_x")) return e;
+    CLG_REQUIRE(grad_y && x && w && grad_x, "clg_tree_backward_x: null pointer argument");
+    const int64_t bpn = clg_ceil_div(positions * xo, kBlk);
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL((tree_kernel<T, true>), dim3((unsigned)(n * bpn), (unsigned)c), dim3(kBlk), 0,
+                                           clg_stream(stream), (const T *)grad_y, (const T *)x, (const T *)w, (T *)grad_x,
+                                           (int)c, positions, (int)xo, bpn));
+    CLG_CHECK_LAUNCH("clg_tree_backward_x");
+    return CLG_OK;
+}
+
+extern "C" int64_t clg_tree_backward_w_scratch_bytes(int dtype, int64_t n, int64_t c, int64_t positions, int64_t xo)
+{
+    if (n <= 0 || c <= 0 || positions <= 0 || xo <= 0) return -1;
+    return c * xo * partial_blocks(n * positions) * 4 * (dtype == CLG_F64 ? 8 : 4);
+}
+
+extern "C" int clg_tree_backward_w(int dtype, const void *grad_y, const void *x, void *grad_w, void *scratch, int64_t n,
+                                   int64_t c, int64_t positions, int64_t xo, void *stream)
+{
+    if (int e = check_tree(dtype, n, c, positions, xo, "clg_tree_backward_w")) return e;
+    CLG_REQUIRE(grad_y && x && grad_w && scratch, "clg_tree_backward_w: null pointer argument");
+    const int nb = partial_blocks(n * positions);
+    hipStream_t st = clg_stream(stream);
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(tree_backward_w_kernel<T>, dim3(nb, (unsigned)(c * xo)), dim3(kBlk), 0, st,
+                                           (const T *)grad_y, (const T *)x, (T *)scratch, n, (int)c, positions, (int)xo));
+    CLG_CHECK_LAUNCH("clg_tree_backward_w");
+    CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, c * xo, nb, 1, st, "clg_tree_backward_w(reduce)"));
+}
+
+// ---- fused block, generic entry points (called from conv_block.hip when no tiled kernel applies) ----
+int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name)
+{
+    if (int e = clg_make_geom(gg, g, name)) return e;
+    if (int e = check_dtype(dtype, name)) return e;
+    CLG_REQUIRE(g->ho % 2 == 0 && g->wo % 2 == 0,
+                "%s: Output height and width after convolution must be divisible by 2 for 2x2 max pooling, but got H_out=%d, "
+                "W_out=%d",
+                name, g->ho, g->wo);
+    return CLG_OK;
+}
+
+int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
+                                  uint8_t *argmax, hipStream_t st)
+{
+    const int cell_blocks = (int)clg_ceil_div((int64_t)(g.ho / 2) * (g.wo / 2), kBlk);
+    if (int e = check_grid(g, cell_blocks, "clg_convblock_forward")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_forward_generic_kernel<T>, dim3((unsigned)(g.n * cell_blocks), g.c),
+                                           dim3(kBlk), 0, st, (const T *)x, (const T *)w, selection, (T *)y, argmax, g,
+                                           cell_blocks));
+    CLG_CHECK_LAUNCH("clg_convblock_forward(generic)");
+    return CLG_OK;
+}
+
+int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
+                                     const int32_t *selection, const uint8_t *argmax, void *grad_x, hipStream_t st)
+{
+    const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
+    CLG_REQUIRE(clg_ceil_div(total, kBlk) < (1ll << 31), "clg_convblock_backward_x: input too large for one launch");
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL((conv_backward_x_gather_kernel<T, true>), dim3((unsigned)clg_ceil_div(total, kBlk)),
+                                           dim3(kBlk), 0, st, (const T *)grad_y, (const T *)x, (const T *)w, selection, argmax,
+                                           (T *)grad_x, g));
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(generic)");
+    return CLG_OK;
+}
+
+int clg_convblock_partial_blocks(const Geom &g) { return partial_blocks((int64_t)g.n * (g.ho / 2) * (g.wo / 2)); }
+
+int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
+                                     const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
+                                     hipStream_t st)
+{
+    CLG_REQUIRE(g.c <= 65535, "clg_convblock_backward_w: more than 65535 logic kernels are not supported");
+    const int nb = clg_convblock_partial_blocks(g);
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_backward_w_generic_kernel<T>, dim3(nb, g.c), dim3(kBlk), 0, st,
+                                           (const T *)grad_y, (const T *)x, (const T *)w, selection, argmax, (T *)scratch, g));
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(generic)");
+    CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, g.c, nb, 7, st, "clg_convblock_backward_w(reduce)"));
+}
+
+extern "C" int clg_convblock_intermediates(int dtype, const clg_conv_geom *gg, const void *x, const void *w,
+                                           const int32_t *selection, void *x2, void *x3, void *stream)
+{
+    Geom g;
+    if (int e = clg_make_geom(gg, &g, "clg_convblock_intermediates")) return e;
+    if (int e = check_dtype(dtype, "clg_convblock_intermediates")) return e;
+    CLG_REQUIRE(x && w && selection, "clg_convblock_intermediates: null pointer argument");
+    const int pos_blocks = (int)clg_ceil_div((int64_t)g.ho * g.wo, kBlk);
+    if (int e = check_grid(g, pos_blocks, "clg_convblock_intermediates")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_intermediates_kernel<T>, dim3((unsigned)(g.n * pos_blocks), g.c), dim3(kBlk),
+                                           0, clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)x2, (T *)x3, g,
+                                           pos_blocks));
+    CLG_CHECK_LAUNCH("clg_convblock_intermediates");
+    return CLG_OK;
+}

@@ -1,0 +1,276 @@
+// Fully connected logic layer, feature-major: x [in_dim, batch], y [out_dim, batch].
+//
+// One wavefront owns one neuron (forward, weight gradient) or one input feature (input
+// gradient) and streams its rows with 64 lanes x VEC samples, so every global access is a
+// contiguous row segment.  The neuron index is wave-uniform: wiring indices and the 16 gate
+// probabilities come through the scalar cache and are folded to 4 coefficients in SGPR-uniform
+// registers; the per-sample work is one multiply and three FMAs.
+#include "clg_common.h"
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWavesPerBlock * kWave;
+
+template <typename T, int VEC>
+struct VecT;
+template <>
+struct VecT<float, 4> { using type = float4; };
+template <>
+struct VecT<float, 1> { using type = float; };
+template <>
+struct VecT<double, 2> { using type = double2; };
+template <>
+struct VecT<double, 1> { using type = double; };
+
+template <typename T, int VEC>
+struct Pack {
+    T v[VEC];
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> load_vec(const T *p)
+{
+    using V = typename VecT<T, VEC>::type;
+    const V r = *reinterpret_cast<const V *>(p);
+    return __builtin_bit_cast(Pack<T, VEC>, r);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(T *p, const Pack<T, VEC> &v)
+{
+    using V = typename VecT<T, VEC>::type;
+    *reinterpret_cast<V *>(p) = __builtin_bit_cast(V, v);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                          const int64_t *__restrict__ b, const T *__restrict__ w,
+                                                          T *__restrict__ y, int out_dim, int64_t batch)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    for (int j = blockIdx.x * kWavesPerBlock + wave; j < out_dim; j += gridDim.x * kWavesPerBlock) {
+        const T *xa = x + a[j] * batch;
+        const T *xb = x + b[j] * batch;
+        T *yj = y + (int64_t)j * batch;
+        const Coef<T> c = fold16(w + (int64_t)j * 16);
+        for (int64_t s = (int64_t)lane * VEC; s < batch; s += kWave * VEC) {
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = gate(c, va.v[k], vb.v[k]);
+            store_vec<T, VEC>(yj + s, r);
+        }
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                             const int64_t *__restrict__ b,
+                                                             const T *__restrict__ gy, T *__restrict__ gw, int out_dim,
+                                                             int64_t batch)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    for (int j = blockIdx.x * kWavesPerBlock + wave; j < out_dim; j += gridDim.x * kWavesPerBlock) {
+        const T *xa = x + a[j] * batch;
+        const T *xb = x + b[j] * batch;
+        const T *gj = gy + (int64_t)j * batch;
+        T sab = 0, sa = 0, sb = 0, s1 = 0;
+        for (int64_t s = (int64_t)lane * VEC; s < batch; s += kWave * VEC) {
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s),
+                               vg = load_vec<T, VEC>(gj + s);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                sab = fma_t(vg.v[k], va.v[k] * vb.v[k], sab);
+                sa = fma_t(vg.v[k], va.v[k], sa);
+                sb = fma_t(vg.v[k], vb.v[k], sb);
+                s1 += vg.v[k];
+            }
+        }
+        sab = wave_sum(sab);
+        sa = wave_sum(sa);
+        sb = wave_sum(sb);
+        s1 = wave_sum(s1);
+        if (lane < 16) gw[(int64_t)j * 16 + lane] = coef_transpose_row<T>(lane, sab, sa, sb, s1);
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                             const int64_t *__restrict__ b, const T *__restrict__ w,
+                                                             const T *__restrict__ gy,
+                                                             const int64_t *__restrict__ csr_start,
+                                                             const int64_t *__restrict__ csr_list,
+                                                             T *__restrict__ gx, int in_dim, int64_t batch,
+                                                             int batch_chunks)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    const int64_t items = (int64_t)in_dim * batch_chunks;
+    for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < items; it += (int64_t)gridDim.x * kWavesPerBlock) {
+        const int i = (int)(it / batch_chunks);
+        const int64_t s = ((it % batch_chunks) * kWave + lane) * VEC;
+        const bool live = s < batch;
+        const int64_t beg = csr_start[i], end = csr_start[i + 1];
+        Pack<T, VEC> acc;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc.v[k] = 0;
+        for (int64_t cur = beg; cur < end; ++cur) {
+            const int64_t j = csr_list[cur];
+            const int64_t ia = a[j], ib = b[j];
+            const Coef<T> c = fold16(w + j * 16);
+            // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
+            // feature twice appears twice in the list and takes the B derivative the second time.
+            bool as_a = ia == i;
+            if (as_a && ib == i && cur > beg && csr_list[cur - 1] == j) as_a = false;
+            const T *other = x + (as_a ? ib : ia) * batch;
+            const T c_lin = as_a ? c.a : c.b;
+            if (live) {
+                const Pack<T, VEC> vo = load_vec<T, VEC>(other + s), vg = load_vec<T, VEC>(gy + j * batch + s);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc.v[k] = fma_t(fma_t(c.ab, vo.v[k], c_lin), vg.v[k], acc.v[k]);
+            }
+        }
+        if (live) store_vec<T, VEC>(gx + (int64_t)i * batch + s, acc);
+    }
+}
+
+// ---- 2-D transpose through a padded LDS tile -------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t rows,
+                                                      int64_t cols)
+{
+    __shared__ T tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        const int64_t r = r0 + ty + 4 * k, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + 4 * k][tx] = src[r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        const int64_t c = c0 + ty + 4 * k, r = r0 + tx;
+        if (r < rows && c < cols) dst[c * rows + r] = tile[tx][ty + 4 * k];
+    }
+}
+
+int grid_for(int64_t items)
+{
+    const int64_t blocks = clg_ceil_div(items, kWavesPerBlock);
+    return (int)(blocks < 1 ? 1 : (blocks > (1 << 20) ? (1 << 20) : blocks));
+}
+
+template <typename T>
+constexpr int vec_width() { return 16 / sizeof(T); }
+
+int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const char *name)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && batch > 0, "%s: in_dim, out_dim and batch must be positive (%lld, %lld, %lld)",
+                name, (long long)in_dim, (long long)out_dim, (long long)batch);
+    CLG_REQUIRE(in_dim < (1ll << 31) && out_dim < (1ll << 31), "%s: in_dim/out_dim above 2^31-1 are not supported", name);
+    return CLG_OK;
+}
+
+}  // namespace
+
+extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
+                              int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward")) return e;
+    CLG_REQUIRE(x && a && b && w && y, "clg_fc_forward: null pointer argument");
+    const dim3 grid(grid_for(out_dim)), block(kBlock);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0)
+            hipLaunchKernelGGL((fc_forward_kernel<float, 4>), grid, block, 0, st, (const float *)x, a, b, (const float *)w,
+                               (float *)y, (int)out_dim, batch);
+        else
+            hipLaunchKernelGGL((fc_forward_kernel<float, 1>), grid, block, 0, st, (const float *)x, a, b, (const float *)w,
+                               (float *)y, (int)out_dim, batch);
+    } else {
+        if (batch % 2 == 0)
+            hipLaunchKernelGGL((fc_forward_kernel<double, 2>), grid, block, 0, st, (const double *)x, a, b,
+                               (const double *)w, (double *)y, (int)out_dim, batch);
+        else
+            hipLaunchKernelGGL((fc_forward_kernel<double, 1>), grid, block, 0, st, (const double *)x, a, b,
+                               (const double *)w, (double *)y, (int)out_dim, batch);
+    }
+    CLG_CHECK_LAUNCH("clg_fc_forward");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_w(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                                 void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_w")) return e;
+    CLG_REQUIRE(x && a && b && grad_y && grad_w, "clg_fc_backward_w: null pointer argument");
+    const dim3 grid(grid_for(out_dim)), block(kBlock);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0)
+            hipLaunchKernelGGL((fc_backward_w_kernel<float, 4>), grid, block, 0, st, (const float *)x, a, b,
+                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch);
+        else
+            hipLaunchKernelGGL((fc_backward_w_kernel<float, 1>), grid, block, 0, st, (const float *)x, a, b,
+                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch);
+    } else {
+        if (batch % 2 == 0)
+            hipLaunchKernelGGL((fc_backward_w_kernel<double, 2>), grid, block, 0, st, (const double *)x, a, b,
+                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch);
+        else
+            hipLaunchKernelGGL((fc_backward_w_kernel<double, 1>), grid, block, 0, st, (const double *)x, a, b,
+                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch);
+    }
+    CLG_CHECK_LAUNCH("clg_fc_backward_w");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w,
+                                 const void *grad_y, const int64_t *csr_start, const int64_t *csr_list, void *grad_x,
+                                 int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_x")) return e;
+    CLG_REQUIRE(x && a && b && w && grad_y && csr_start && csr_list && grad_x, "clg_fc_backward_x: null pointer argument");
+    hipStream_t st = clg_stream(stream);
+    const dim3 block(kBlock);
+#define CLG_LAUNCH_BX(T, VEC)                                                                                          \
+    do {                                                                                                               \
+        const int chunks = (int)clg_ceil_div(batch, (int64_t)kWave * VEC);                                             \
+        hipLaunchKernelGGL((fc_backward_x_kernel<T, VEC>), dim3(grid_for(in_dim * chunks)), block, 0, st, (const T *)x, \
+                           a, b, (const T *)w, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (int)in_dim, batch,  \
+                           chunks);                                                                                    \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_BX(float, 4);
+        else CLG_LAUNCH_BX(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_BX(double, 2);
+        else CLG_LAUNCH_BX(double, 1);
+    }
+#undef CLG_LAUNCH_BX
+    CLG_CHECK_LAUNCH("clg_fc_backward_x");
+    return CLG_OK;
+}
+
+extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64_t rows, int64_t cols, void *stream)
+{
+    CLG_REQUIRE(src && dst, "clg_transpose_2d: null pointer argument");
+    CLG_REQUIRE(rows > 0 && cols > 0, "clg_transpose_2d: rows and cols must be positive");
+    const int64_t gx = clg_ceil_div(cols, 64), gy = clg_ceil_div(rows, 64);
+    CLG_REQUIRE(gy <= 65535, "clg_transpose_2d: more than 65535*64 rows are not supported");
+    const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+    hipStream_t st = clg_stream(stream);
+    switch (elem_size) {
+    case 1: hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, block, 0, st, (const uint8_t *)src, (uint8_t *)dst, rows, cols); break;
+    case 2: hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, block, 0, st, (const uint16_t *)src, (uint16_t *)dst, rows, cols); break;
+    case 4: hipLaunchKernelGGL(transpose_kernel<uint32_t>, grid, block, 0, st, (const uint32_t *)src, (uint32_t *)dst, rows, cols); break;
+    case 8: hipLaunchKernelGGL(transpose_kernel<uint64_t>, grid, block, 0, st, (const uint64_t *)src, (uint64_t *)dst, rows, cols); break;
+    default: CLG_REQUIRE(false, "clg_transpose_2d: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
+    }
+    CLG_CHECK_LAUNCH("clg_transpose_2d");
+    return CLG_OK;
+}

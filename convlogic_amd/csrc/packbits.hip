@@ -1,0 +1,317 @@
+// Packed-bit inference: pack bool -> words, bitwise gate evaluation, per-class popcount.
+//
+// A word holds `bits` samples of one feature (sample s = bit s % bits of word s / bits, LSB first).
+// Every gate is bitwise, so the evaluation kernel treats a row as a run of bytes and moves it with
+// 16-byte vectors whatever the word type is; one wavefront evaluates one neuron (gate id, wiring
+// and truth-table masks are wave-uniform) over a column chunk of its two input rows.
+#include "clg_common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// evaluation
+// ---------------------------------------------------------------------------------------------
+struct Masks {
+    uint32_t f00, f01, f10, f11;  // all-ones / all-zeros per truth-table entry
+};
+__device__ __forceinline__ Masks gate_masks(int id)
+{
+    return Masks{0u - ((id >> 3) & 1u), 0u - ((id >> 2) & 1u), 0u - ((id >> 1) & 1u), 0u - (id & 1u)};
+}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// 2:1 multiplexers on bits: b selects inside each half, a selects the half.  V is uint32_t or a
+// vector of them (the masks are splat).
+template <typename V>
+__device__ __forceinline__ V gate_vec(const Masks &m, V a, V b)
+{
+    const V t1 = (b & (V)m.f11) | (~b & (V)m.f10);
+    const V t0 = (b & (V)m.f01) | (~b & (V)m.f00);
+    return (a & t1) | (~a & t0);
+}
+__device__ __forceinline__ uint32_t gate_bits(const Masks &m, uint32_t a, uint32_t b) { return gate_vec<uint32_t>(m, a, b); }
+
+constexpr int kEvalBlock = 256;
+constexpr int kEvalWaves = kEvalBlock / kWave;
+
+// Rows are `row_vecs` vectors of type V.  blockIdx.x enumerates (column chunk, neuron group) with
+// the chunk as the slow index, so that all neurons of one column chunk run back to back and the
+// second read of an input row segment finds it in the last-level cache.
+template <typename V, int UNROLL>
+__global__ __launch_bounds__(kEvalBlock) void eval_packed_kernel(const V *__restrict__ x, const int64_t *__restrict__ a,
+                                                               const int64_t *__restrict__ b,
+                                                               const uint8_t *__restrict__ gate, V *__restrict__ y,
+                                                               int out_dim, int64_t row_vecs, int chunk_vecs,
+                                                               int groups_per_chunk, int neurons_per_wave)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    const int chunk = blockIdx.x / groups_per_chunk;
+    const int group = blockIdx.x % groups_per_chunk;
+    const int64_t v0 = (int64_t)chunk * chunk_vecs;
+    const int64_t v1 = (v0 + chunk_vecs < row_vecs) ? v0 + chunk_vecs : row_vecs;
+    const int j0 = (group * kEvalWaves + wave) * neurons_per_wave;
+    for (int jj = 0; jj < neurons_per_wave; ++jj) {
+        const int j = j0 + jj;
+        if (j >= out_dim) break;
+        const V *xa = x + a[j] * row_vecs;
+        const V *xb = x + b[j] * row_vecs;
+        V *yj = y + (int64_t)j * row_vecs;
+        const Masks m = gate_masks(gate[j]);
+        for (int64_t v = v0 + lane; v < v1; v += (int64_t)kWave * UNROLL) {
+            V ra[UNROLL], rb[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int64_t vv = v + (int64_t)u * kWave;
+                if (vv < v1) {
+                    ra[u] = xa[vv];
+                    rb[u] = xb[vv];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int64_t vv = v + (int64_t)u * kWave;
+                if (vv < v1) __builtin_nontemporal_store(gate_vec(m, ra[u], rb[u]), yj + vv);
+            }
+        }
+    }
+}
+
+// bytewise tail / odd row sizes: one thread per byte of the output
+__global__ void eval_packed_bytes_kernel(const uint8_t *__restrict__ x, const int64_t *__restrict__ a,
+                                         const int64_t *__restrict__ b, const uint8_t *__restrict__ gate,
+                                         uint8_t *__restrict__ y, int64_t out_dim, int64_t row_bytes)
+{
+    const int64_t total = out_dim * row_bytes;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t j = i / row_bytes, c = i % row_bytes;
+        const Masks m = gate_masks(gate[j]);
+        y[i] = (uint8_t)gate_bits(m, x[a[j] * row_bytes + c], x[b[j] * row_bytes + c]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// packing
+// ---------------------------------------------------------------------------------------------
+// 8 bool bytes (any non-zero value counts as true) -> 8 bits, byte k -> bit k.
+__device__ __forceinline__ uint32_t squeeze8(uint64_t v)
+{
+    v |= v >> 4;
+    v |= v >> 2;
+    v |= v >> 1;
+    v &= 0x0101010101010101ull;
+    return (uint32_t)((v * 0x0102040810204080ull) >> 56);
+}
+
+// feature-major input t [F, B]: one thread per output byte (8 samples); the word type only fixes the
+// padded row length, because words are little endian and samples fill them LSB first.
+__global__ void pack_bits_kernel(const uint8_t *__restrict__ t, uint8_t *__restrict__ out, int64_t features, int64_t batch,
+                                 int64_t row_bytes, bool aligned8)
+{
+    const int64_t total = features * row_bytes;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t f = i / row_bytes, c = i % row_bytes;
+        const int64_t s0 = c * 8;
+        const uint8_t *p = t + f * batch + s0;
+        uint32_t bits = 0;
+        if (aligned8 && s0 + 8 <= batch) {
+            bits = squeeze8(*reinterpret_cast<const uint64_t *>(p));
+        } else {
+            for (int k = 0; k < 8; ++k)
+                if (s0 + k < batch && p[k]) bits |= 1u << k;
+        }
+        out[i] = (uint8_t)bits;
+    }
+}
+
+// sample-major input t [B, F]: lanes run along features (contiguous reads), each thread keeps the
+// 64 samples of one feature in a 64-bit register and then stores 8 bytes of that feature's row.
+// Consecutive 64-sample groups of the same features are handled by the same thread one after the
+// other so that its partial-line stores merge in L2.
+constexpr int kPackGroups = 16;  // 64-sample groups per thread
+__global__ __launch_bounds__(256) void pack_bits_sm_kernel(const uint8_t *__restrict__ t, uint8_t *__restrict__ out,
+                                                         int64_t features, int64_t batch, int64_t row_bytes)
+{
+    const int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (f >= features) return;
+    const int64_t g0 = (int64_t)blockIdx.y * kPackGroups;
+    for (int g = 0; g < kPackGroups; ++g) {
+        const int64_t s0 = (g0 + g) * 64;
+        if (s0 >= batch) break;
+        uint64_t word = 0;
+        const int64_t n = batch - s0 < 64 ? batch - s0 : 64;
+        if (n == 64) {
+#pragma unroll 16
+            for (int k = 0; k < 64; ++k) word |= (uint64_t)(t[(s0 + k) * features + f] != 0) << k;
+        } else {
+            for (int k = 0; k < n; ++k) word |= (uint64_t)(t[(s0 + k) * features + f] != 0) << k;
+        }
+        uint8_t *dst = out + f * row_bytes + s0 / 8;
+        const int64_t nbytes = row_bytes - s0 / 8 < 8 ? row_bytes - s0 / 8 : 8;
+        if (nbytes == 8 && (row_bytes & 7) == 0) {
+            *reinterpret_cast<uint64_t *>(dst) = word;
+        } else {
+            for (int k = 0; k < nbytes; ++k) dst[k] = (uint8_t)(word >> (8 * k));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-class bit counts
+// ---------------------------------------------------------------------------------------------
+// One wave per (class, 8-byte column): the 64 lanes are the 64 sample bits of that column; rows of
+// the class are split over `slices` waves whose partial counts meet in integer atomics (exact, so the
+// result does not depend on their order).
+__global__ __launch_bounds__(256) void group_bit_sum_kernel(const uint8_t *__restrict__ x, int32_t *__restrict__ out,
+                                                          int64_t class_rows, int64_t row_bytes, int64_t samples, int k,
+                                                          int cols8, int slices)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t total = (int64_t)k * cols8 * slices;
+    if (item >= total) return;
+    const int slice = (int)(item % slices);
+    const int col = (int)((item / slices) % cols8);
+    const int g = (int)(item / ((int64_t)slices * cols8));
+    const int64_t r0 = class_rows * slice / slices, r1 = class_rows * (slice + 1) / slices;
+    const int64_t byte0 = (int64_t)col * 8;
+    const int nbytes = row_bytes - byte0 < 8 ? (int)(row_bytes - byte0) : 8;
+    const uint8_t *base = x + (int64_t)g * class_rows * row_bytes + byte0;
+    int32_t acc = 0;
+    if (nbytes == 8 && (row_bytes & 7) == 0) {
+        for (int64_t r = r0; r < r1; ++r) {
+            const uint64_t wv = *reinterpret_cast<const uint64_t *>(base + r * row_bytes);
+            acc += (int32_t)((wv >> lane) & 1);
+        }
+    } else {
+        for (int64_t r = r0; r < r1; ++r) {
+            uint64_t wv = 0;
+            for (int b = 0; b < nbytes; ++b) wv |= (uint64_t)base[r * row_bytes + b] << (8 * b);
+            acc += (int32_t)((wv >> lane) & 1);
+        }
+    }
+    const int64_t s = byte0 * 8 + lane;
+    if (s < samples) {
+        if (slices == 1) out[s * k + g] = acc;
+        else atomicAdd(out + s * k + g, acc);
+    }
+}
+
+__global__ void fill_zero_i32_kernel(int32_t *p, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+int small_grid(int64_t items, int block)
+{
+    const int64_t g = clg_ceil_div(items, block);
+    return (int)(g < 1 ? 1 : (g > 65536 * 16 ? 65536 * 16 : g));
+}
+
+template <typename V>
+void launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate, void *y, int64_t out_dim,
+                 int64_t row_bytes, hipStream_t st)
+{
+    const int64_t row_vecs = row_bytes / (int64_t)sizeof(V);
+    // column chunks of at most 2 KiB per row: with both uses of a row segment inside one chunk pass,
+    // the working set of a pass (in_dim x 2 KiB) stays cache resident for layers up to ~100k features.
+    const int max_chunk_vecs = 2048 / (int)sizeof(V);
+    const int chunk_vecs = row_vecs < max_chunk_vecs ? (int)row_vecs : max_chunk_vecs;
+    const int chunks = (int)clg_ceil_div(row_vecs, chunk_vecs);
+    const int neurons_per_wave = 4;
+    const int groups = (int)clg_ceil_div(out_dim, (int64_t)kEvalWaves * neurons_per_wave);
+    hipLaunchKernelGGL((eval_packed_kernel<V, 2>), dim3((unsigned)(chunks * groups)), dim3(kEvalBlock), 0, st, (const V *)x, a,
+                       b, gate, (V *)y, (int)out_dim, row_vecs, chunk_vecs, groups, neurons_per_wave);
+}
+
+bool valid_elem(int e) { return e == 1 || e == 2 || e == 4 || e == 8; }
+
+}  // namespace
+
+extern "C" int clg_fc_eval_packed(int elem_size, const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate,
+                                  void *y, int64_t in_dim, int64_t out_dim, int64_t words, void *stream)
+{
+    CLG_REQUIRE(valid_elem(elem_size), "clg_fc_eval_packed: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
+    CLG_REQUIRE(x && a && b && gate && y, "clg_fc_eval_packed: null pointer argument");
+    CLG_REQUIRE(x != y, "clg_fc_eval_packed: x and y must not overlap");
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && words > 0, "clg_fc_eval_packed: in_dim, out_dim and words must be positive");
+    CLG_REQUIRE(out_dim < (1ll << 31), "clg_fc_eval_packed: out_dim above 2^31-1 is not supported");
+    const int64_t row_bytes = words * elem_size;
+    const uintptr_t align = (uintptr_t)x | (uintptr_t)y | (uintptr_t)row_bytes;
+    hipStream_t st = clg_stream(stream);
+    const int64_t blocks_needed = clg_ceil_div(row_bytes, 2048) * clg_ceil_div(out_dim, 16);
+    if (blocks_needed >= (1ll << 31)) {
+        CLG_REQUIRE(false, "clg_fc_eval_packed: problem too large for one launch (%lld blocks)", (long long)blocks_needed);
+    }
+    if ((align & 15) == 0) launch_eval<u32x4>(x, a, b, gate, y, out_dim, row_bytes, st);
+    else if ((align & 7) == 0) launch_eval<u32x2>(x, a, b, gate, y, out_dim, row_bytes, st);
+    else if ((align & 3) == 0) launch_eval<uint32_t>(x, a, b, gate, y, out_dim, row_bytes, st);
+    else
+        hipLaunchKernelGGL(eval_packed_bytes_kernel, dim3(small_grid(out_dim * row_bytes, 256)), dim3(256), 0, st,
+                           (const uint8_t *)x, a, b, gate, (uint8_t *)y, out_dim, row_bytes);
+    CLG_CHECK_LAUNCH("clg_fc_eval_packed");
+    return CLG_OK;
+}
+
+static int check_pack(const void *t, void *words, int64_t features, int64_t batch, int bit_count, const char *name)
+{
+    CLG_REQUIRE(t && words, "%s: null pointer argument", name);
+    CLG_REQUIRE(bit_count == 8 || bit_count == 16 || bit_count == 32 || bit_count == 64,
+                "%s: `bit_count` has to be in { 8, 16, 32, 64 }, got %d", name, bit_count);
+    CLG_REQUIRE(features > 0 && batch > 0, "%s: features and batch must be positive", name);
+    return CLG_OK;
+}
+
+extern "C" int clg_pack_bits(const uint8_t *t, void *words, int64_t features, int64_t batch, int bit_count, void *stream)
+{
+    if (int e = check_pack(t, words, features, batch, bit_count, "clg_pack_bits")) return e;
+    const int64_t row_bytes = clg_ceil_div(batch, bit_count) * (bit_count / 8);
+    const bool aligned8 = (batch % 8 == 0) && (((uintptr_t)t & 7) == 0);
+    hipLaunchKernelGGL(pack_bits_kernel, dim3(small_grid(features * row_bytes, 256)), dim3(256), 0, clg_stream(stream), t,
+                       (uint8_t *)words, features, batch, row_bytes, aligned8);
+    CLG_CHECK_LAUNCH("clg_pack_bits");
+    return CLG_OK;
+}
+
+extern "C" int clg_pack_bits_sample_major(const uint8_t *t, void *words, int64_t features, int64_t batch, int bit_count,
+                                          void *stream)
+{
+    if (int e = check_pack(t, words, features, batch, bit_count, "clg_pack_bits_sample_major")) return e;
+    const int64_t row_bytes = clg_ceil_div(batch, bit_count) * (bit_count / 8);
+    const int64_t groups = clg_ceil_div(batch, 64);
+    const int64_t gy = clg_ceil_div(groups, kPackGroups);
+    CLG_REQUIRE(gy <= 65535, "clg_pack_bits_sample_major: batch above %lld samples is not supported", 65535ll * kPackGroups * 64);
+    hipLaunchKernelGGL(pack_bits_sm_kernel, dim3((unsigned)clg_ceil_div(features, 256), (unsigned)gy), dim3(256), 0,
+                       clg_stream(stream), t, (uint8_t *)words, features, batch, row_bytes);
+    CLG_CHECK_LAUNCH("clg_pack_bits_sample_major");
+    return CLG_OK;
+}
+
+extern "C" int clg_group_bit_sum(int elem_size, const void *x, int32_t *out, int64_t features, int64_t words, int64_t pad_len,
+                                 int64_t k, void *stream)
+{
+    CLG_REQUIRE(valid_elem(elem_size), "clg_group_bit_sum: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
+    CLG_REQUIRE(x && out, "clg_group_bit_sum: null pointer argument");
+    CLG_REQUIRE(features > 0 && words > 0 && k > 0, "clg_group_bit_sum: features, words and k must be positive");
+    CLG_REQUIRE(features % k == 0, "in_dim (%lld) has to be divisible by k (%lld) but it is not", (long long)features, (long long)k);
+    const int64_t row_bytes = words * elem_size, samples = row_bytes * 8 - pad_len;
+    CLG_REQUIRE(pad_len >= 0 && samples > 0, "clg_group_bit_sum: pad_len %lld leaves no samples", (long long)pad_len);
+    CLG_REQUIRE(k < (1 << 20), "clg_group_bit_sum: k too large");
+    const int cols8 = (int)clg_ceil_div(row_bytes, 8);
+    const int64_t class_rows = features / k;
+    // enough waves to fill the GPU, at least 64 rows per slice
+    int64_t slices = clg_ceil_div(16384, (int64_t)k * cols8);
+    if (slices > class_rows / 64) slices = class_rows / 64;
+    if (slices < 1) slices = 1;
+    hipStream_t st = clg_stream(stream);
+    if (slices > 1)
+        hipLaunchKernelGGL(fill_zero_i32_kernel, dim3(small_grid(samples * k, 256)), dim3(256), 0, st, out, samples * k);
+    const int64_t items = k * cols8 * slices;
+    CLG_REQUIRE(clg_ceil_div(items, 4) < (1ll << 31), "clg_group_bit_sum: problem too large for one launch");
+    hipLaunchKernelGGL(group_bit_sum_kernel, dim3((unsigned)clg_ceil_div(items, 4)), dim3(256), 0, st, (const uint8_t *)x, out,
+                       class_rows, row_bytes, samples, (int)k, cols8, (int)slices);
+    CLG_CHECK_LAUNCH("clg_group_bit_sum");
+    return CLG_OK;
+}

@@ -1,0 +1,197 @@
+"""LogicLayer / GroupSum with the constructor arguments, parameter and buffer names of the
+reference's src/difflogic/difflogic.py, on HIP kernels for gfx950.
+
+implementation="cuda" runs the HIP kernels (on ROCm builds of torch the device type is still
+"cuda") and raises if the GPU or the compiled library is missing.  implementation="python" is the
+reference's second, explicitly selected backend: plain torch ops on whatever device the tensors
+live on.
+"""
+import numpy as np
+import torch
+
+from ..hip import difflogic_hip
+from .functional import GradFactor, bin_op_s, get_unique_connections
+from .packbitstensor import PackBitsTensor
+
+
+def _reverse_wiring(idx0, idx1, in_dim):
+    """CSR map input -> neurons reading it; neuron y is listed under idx0[y] before idx1[y] and
+    neurons appear in increasing order inside every list (same layout as the python loop of
+    src/difflogic/difflogic.py:71-87)."""
+    out_dim = len(idx0)
+    target = np.stack([idx0, idx1], axis=1).reshape(-1)                 # [y0.a, y0.b, y1.a, ...]
+    neuron = np.repeat(np.arange(out_dim, dtype=np.int64), 2)
+    order = np.argsort(target, kind="stable")
+    start = np.zeros(in_dim + 1, dtype=np.int64)
+    np.cumsum(np.bincount(target, minlength=in_dim), out=start[1:])
+    return torch.from_numpy(start), torch.from_numpy(neuron[order].copy())
+
+
+class LogicLayer(torch.nn.Module):
+    """out_dim two-input logic gate neurons over in_dim features (src/difflogic/difflogic.py:14-90)."""
+
+    def __init__(self, in_dim: int, out_dim: int, grad_factor: float = 1.0, implementation: str = None,
+                 connections: str = "random", residual_init: bool = False):
+        super().__init__()
+        if residual_init:                       # gate 3 ("A") gets logit 5 -> p = 0.908
+            logits = torch.zeros(out_dim, 16)
+            logits[:, 3] = 5.0
+        else:
+            logits = torch.randn(out_dim, 16)
+        self.weights = torch.nn.Parameter(logits)
+        self.in_dim, self.out_dim, self.grad_factor = in_dim, out_dim, grad_factor
+
+        if implementation is None:
+            implementation = "cuda" if torch.cuda.is_available() else "python"
+        assert implementation in ["cuda", "python"], f"Invalid implementation: {implementation}"
+        self.implementation = implementation
+
+        self.connections = connections
+        assert self.connections in ["random", "unique"], self.connections
+        a, b = self.get_connections(self.connections)
+        self.register_buffer("indices_0", a.to(torch.int64))
+        self.register_buffer("indices_1", b.to(torch.int64))
+
+        if self.implementation == "cuda":
+            start, flat = _reverse_wiring(self.indices_0.cpu().numpy(), self.indices_1.cpu().numpy(), in_dim)
+            self.register_buffer("given_x_indices_of_y_start", start)
+            self.register_buffer("given_x_indices_of_y", flat)
+
+        self.num_neurons = out_dim
+        self.num_weights = out_dim
+
+    def forward(self, x):
+        if isinstance(x, PackBitsTensor):
+            assert not self.training, "PackBitsTensor is not supported for the differentiable training mode."
+            assert x.is_cuda, (f"PackBitsTensor is only supported for CUDA, but got device {x.device}. "
+                               "If you want fast inference on CPU, please use CompiledDiffLogicModel.")
+        elif self.grad_factor != 1.0:
+            x = GradFactor.apply(x, self.grad_factor)
+
+        if self.implementation == "cuda":
+            if isinstance(x, PackBitsTensor):
+                return self.forward_cuda_eval(x)
+            return self.forward_cuda(x)
+        if self.implementation == "python":
+            return self.forward_python(x)
+        raise ValueError(f"Unsupported implementation: {self.implementation}")
+
+    def _gate_weights(self, dtype):
+        if self.training:
+            return torch.nn.functional.softmax(self.weights, dim=-1).to(dtype)
+        return torch.nn.functional.one_hot(self.weights.argmax(-1), 16).to(dtype)
+
+    def forward_python(self, x):
+        assert x.shape[-1] == self.in_dim, (x.shape[-1], self.in_dim)
+        a, b = x[..., self.indices_0], x[..., self.indices_1]
+        w = self._gate_weights(torch.float32 if not self.training else self.weights.dtype)
+        return bin_op_s(a, b, w)
+
+    def forward_cuda(self, x):
+        if self.training:
+            assert x.is_cuda, f"x must be a CUDA tensor, got device: {x.device}"
+        assert x.ndim == 2, x.ndim
+        assert x.shape[1] == self.in_dim, (tuple(x.shape[::-1]), self.in_dim)
+        xt = _feature_major(x)
+        w = self._gate_weights(xt.dtype)
+        args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
+        if self.training:
+            return LogicLayerCudaFunction.apply(*args).transpose(0, 1)
+        with torch.no_grad():
+            return LogicLayerCudaFunction.apply(*args).transpose(0, 1)
+
+    def forward_cuda_eval(self, x: PackBitsTensor):
+        """Replaces x.t by the layer output (src/difflogic/difflogic.py:149-164)."""
+        assert not self.training
+        assert isinstance(x, PackBitsTensor)
+        assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
+        gate = self.weights.argmax(-1).to(torch.uint8)
+        x.t = difflogic_hip.eval(x.t, self.indices_0, self.indices_1, gate)
+        return x
+
+    def extra_repr(self):
+        return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")
+
+    def get_connections(self, connections):
+        assert self.out_dim * 2 >= self.in_dim, (
+            f"The number of neurons ({self.out_dim}) must not be smaller than half of the "
+            f"number of inputs ({self.in_dim}) because otherwise not all inputs could be "
+            "used or considered.")
+        if connections == "random":
+            # every input is used floor/ceil(2*out/in) times (src/difflogic/difflogic.py:175-181)
+            slots = torch.randperm(2 * self.out_dim) % self.in_dim
+            slots = torch.randperm(self.in_dim)[slots].reshape(2, self.out_dim)
+            return slots[0].to(torch.int64), slots[1].to(torch.int64)
+        if connections == "unique":
+            return get_unique_connections(self.in_dim, self.out_dim)
+        raise ValueError(connections)
+
+
+class _FeatureMajor(torch.autograd.Function):
+    """[batch, features] -> contiguous [features, batch] through the tiled HIP transpose; the gradient
+    is handed back as a transposed view."""
+
+    @staticmethod
+    def forward(ctx, x):
+        return difflogic_hip.transpose(x)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return grad.transpose(0, 1)
+
+
+def _feature_major(x):
+    """[batch, features] -> contiguous [features, batch].  A transposed view of a feature-major
+    tensor (what the previous LogicLayer returned) is used as is, without a copy."""
+    xt = x.transpose(0, 1)
+    if xt.is_contiguous():
+        return xt
+    if x.is_cuda and x.is_contiguous() and x.element_size() in (1, 2, 4, 8):
+        return _FeatureMajor.apply(x)
+    return xt.contiguous()
+
+
+class GroupSum(torch.nn.Module):
+    """Sums k groups of outputs and divides by tau; packed inputs give raw integer counts
+    (src/difflogic/difflogic.py:188-211)."""
+
+    def __init__(self, k: int, tau: float = 1.0):
+        super().__init__()
+        self.k, self.tau = k, tau
+
+    def forward(self, x):
+        if isinstance(x, PackBitsTensor):
+            return x.group_sum(self.k)
+        assert x.shape[-1] % self.k == 0, (x.shape, self.k)
+        return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
+
+    def extra_repr(self):
+        return f"k={self.k}, tau={self.tau}"
+
+
+class LogicLayerCudaFunction(torch.autograd.Function):
+    """y[out,B] = layer(x[in,B]); gradients w.r.t. x and the gate probabilities w
+    (src/difflogic/difflogic.py:214-230)."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y):
+        ctx.save_for_backward(x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y)
+        return difflogic_hip.forward(x, a, b, w)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a, b, w, start, flat = ctx.saved_tensors
+        grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_x = difflogic_hip.backward_x(x, a, b, w, grad_y, start, flat)
+        if ctx.needs_input_grad[3]:
+            grad_w = difflogic_hip.backward_w(x, a, b, grad_y)
+        return grad_x, None, None, grad_w, None, None, None
+
+
+def _contiguous_2d(t):
+    tt = t.transpose(0, 1)
+    if t.is_cuda and t.dim() == 2 and tt.is_contiguous():
+        return difflogic_hip.transpose(tt)      # t is a transposed view: one tiled transpose
+    return t.contiguous()

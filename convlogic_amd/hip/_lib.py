@@ -1,0 +1,99 @@
+"""ctypes binding of libconvlogic_amd.so (the C ABI declared in include/convlogic_amd.h).
+
+The library is loaded on first use.  If it has not been built this raises: there is no
+fallback implementation behind the "cuda" code paths.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG, "libconvlogic_amd.so")
+
+CLG_F32, CLG_F64 = 0, 1
+_DTYPES = {torch.float32: CLG_F32, torch.float64: CLG_F64}
+
+_p, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+
+
+class ConvGeom(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in
+                ("n", "c_in", "h", "w", "c_out", "stride_h", "stride_w", "pad_h", "pad_w", "kernel_h", "kernel_w")]
+
+
+_GP = ctypes.POINTER(ConvGeom)
+
+# name -> (restype, argtypes); every symbol include/convlogic_amd.h declares
+SIGNATURES = {
+    "clg_last_error": (ctypes.c_char_p, []),
+    "clg_abi_version": (_i, []),
+    "clg_fc_forward": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_fc_backward_w": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_fc_backward_x": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_transpose_2d": (_i, [_i, _p, _p, _i64, _i64, _p]),
+    "clg_pack_bits": (_i, [_p, _p, _i64, _i64, _i, _p]),
+    "clg_pack_bits_sample_major": (_i, [_p, _p, _i64, _i64, _i, _p]),
+    "clg_fc_eval_packed": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_group_bit_sum": (_i, [_i, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "clg_conv4_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p]),
+    "clg_conv4_backward_x": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
+    "clg_conv4_backward_w": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
+    "clg_conv4_backward_w_scratch_bytes": (_i64, [_i, _GP]),
+    "clg_tree_forward": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "clg_tree_backward_x": (_i, [_i, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "clg_tree_backward_w": (_i, [_i, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "clg_tree_backward_w_scratch_bytes": (_i64, [_i, _i64, _i64, _i64, _i64]),
+    "clg_convblock_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_intermediates": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_backward_x": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_backward_w": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_backward_w_scratch_bytes": (_i64, [_i, _GP]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads the shared library and declares all signatures (no GPU needed for this)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"convlogic_amd: {LIB_PATH} is missing. Build it with `python -m convlogic_amd.build` "
+                "(needs hipcc); there is no fallback for the 'cuda' implementation.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def available():
+    return os.path.exists(LIB_PATH)
+
+
+def check(rc):
+    if rc != 0:
+        raise RuntimeError(load().clg_last_error().decode())
+
+
+def dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"convlogic_amd kernels support float32 and float64, got {t.dtype}") from None
+
+
+def stream_ptr(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def check_input(t, name):
+    """Same contract as the reference's CHECK_INPUT (src/common/cuda_utils.cuh:9-13)."""
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    return t

@@ -1,0 +1,186 @@
+"""Function set of the reference's `convlogic_cuda` module (src/convlogic/cuda/convlogic.cpp:29-44)
+on top of the HIP C ABI."""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import ConvGeom, check, check_input, dtype_code, stream_ptr
+
+
+def _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    n, c_in, h, w = x.shape
+    return ConvGeom(n, c_in, h, w, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+
+
+def _geom_from_out(x, c_out, ho, wo, stride_h, stride_w, pad_h, pad_w):
+    """The backward bindings of the reference do not receive the kernel size; any kernel size that
+    reproduces the conv output size describes the same index arithmetic."""
+    _, _, h, w = x.shape
+    return _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, h + 2 * pad_h - (ho - 1) * stride_h, w + 2 * pad_w - (wo - 1) * stride_w)
+
+
+def _out_size(g):
+    return (g.h + 2 * g.pad_h - g.kernel_h) // g.stride_h + 1, (g.w + 2 * g.pad_w - g.kernel_w) // g.stride_w + 1
+
+
+def _scratch(nbytes, device):
+    if nbytes < 0:
+        raise RuntimeError(_lib.load().clg_last_error().decode())
+    return torch.empty((max(int(nbytes), 8),), dtype=torch.uint8, device=device)
+
+
+# ---- split layer ------------------------------------------------------------------------------
+def convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """[N,C,Ho,Wo,4]; src/convlogic/cuda/convlogic_kernel.cu:67-106."""
+    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    y = torch.empty((g.n, g.c_out, max(ho, 0), max(wo, 0), 4), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_conv4_forward(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(), selection.data_ptr(),
+                                        y.data_ptr(), stream_ptr(x)))
+    return y
+
+
+def convlogic_backward_x(grad_y, x, weight, selection, stride_h, stride_w, pad_h, pad_w):
+    """src/convlogic/cuda/convlogic_kernel.cu:321-359 (deterministic here)."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], grad_y.shape[2], grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    gx = torch.empty_like(x)
+    check(_lib.load().clg_conv4_backward_x(dtype_code(x), ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                           selection.data_ptr(), gx.data_ptr(), stream_ptr(x)))
+    return gx
+
+
+def convlogic_backward_weight(grad_y, x, selection, stride_h, stride_w, pad_h, pad_w):
+    """[C,4,16]; src/convlogic/cuda/convlogic_kernel.cu:197-248."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], grad_y.shape[2], grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_conv4_backward_w_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gw = torch.empty((g.c_out, 4, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_conv4_backward_w(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), selection.data_ptr(), gw.data_ptr(),
+                                   scratch.data_ptr(), stream_ptr(x)))
+    return gw
+
+
+# ---- tree level -------------------------------------------------------------------------------
+def _tree_dims(x, xo):
+    if x.dim() != 5:
+        raise RuntimeError(f"Expected input tensor x to be 5D (N, C, H, W, 2*Xout), but got {x.dim()}")
+    n, c, h, w, xin = x.shape
+    if xin != 2 * xo:
+        raise RuntimeError(f"Expected input x.size(4) (Xin) to equal 2*Xout ({2 * xo}), but got {xin}")
+    return n, c, h * w
+
+
+def treelogic_forward(x, weights):
+    """[N,C,H,W,Xout]; src/convlogic/cuda/treelogic_kernel.cu:46-85."""
+    check_input(x, "x")
+    check_input(weights, "weights")
+    xo = weights.shape[1]
+    n, c, pos = _tree_dims(x, xo)
+    y = torch.empty(x.shape[:4] + (xo,), dtype=x.dtype, device=x.device)
+    if y.numel():
+        check(_lib.load().clg_tree_forward(dtype_code(x), x.data_ptr(), weights.data_ptr(), y.data_ptr(), n, c, pos, xo,
+                                           stream_ptr(x)))
+    return y
+
+
+def treelogic_backward_x(grad_y, x, weights):
+    """src/convlogic/cuda/treelogic_kernel.cu:252-285."""
+    for t, n_ in ((grad_y, "grad_y"), (x, "x"), (weights, "weights")):
+        check_input(t, n_)
+    xo = weights.shape[1]
+    n, c, pos = _tree_dims(x, xo)
+    gx = torch.empty_like(x)
+    if gx.numel():
+        check(_lib.load().clg_tree_backward_x(dtype_code(x), grad_y.data_ptr(), x.data_ptr(), weights.data_ptr(), gx.data_ptr(),
+                                              n, c, pos, xo, stream_ptr(x)))
+    return gx
+
+
+def treelogic_backward_weight(grad_y, x):
+    """[C,Xout,16]; src/convlogic/cuda/treelogic_kernel.cu:160-206."""
+    check_input(grad_y, "grad_y")
+    check_input(x, "x")
+    xo = grad_y.shape[4]
+    n, c, pos = _tree_dims(x, xo)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_tree_backward_w_scratch_bytes(dt, n, c, pos, xo), x.device)
+    gw = torch.empty((c, xo, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_tree_backward_w(dt, grad_y.data_ptr(), x.data_ptr(), gw.data_ptr(), scratch.data_ptr(), n, c, pos, xo,
+                                  stream_ptr(x)))
+    return gw
+
+
+# ---- fused block ------------------------------------------------------------------------------
+def full_convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """-> (y [N,C,Ho/2,Wo/2], argmax uint8 [N,C,Ho/2,Wo/2] = dy*2+dx of the pooled maximum).
+    src/convlogic/cuda/full_convlogic_kernel.cu:147-231; the leaf / middle gate planes the reference
+    also returns are not materialised (see full_convlogic_intermediates)."""
+    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
+    y = torch.empty(shape, dtype=x.dtype, device=x.device)
+    argmax = torch.empty(shape, dtype=torch.uint8, device=x.device)
+    check(_lib.load().clg_convblock_forward(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(),
+                                            selection.data_ptr(), y.data_ptr(), argmax.data_ptr(), stream_ptr(x)))
+    return y, argmax
+
+
+def full_convlogic_intermediates(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """-> (x2 [N,C,Ho,Wo,4], x3 [N,C,Ho,Wo,2]), the second and third result of the reference's
+    full_convlogic_forward (full_convlogic_kernel.cu:172,194)."""
+    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    x2 = torch.empty((g.n, g.c_out, ho, wo, 4), dtype=x.dtype, device=x.device)
+    x3 = torch.empty((g.n, g.c_out, ho, wo, 2), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_convblock_intermediates(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(),
+                                                  selection.data_ptr(), x2.data_ptr(), x3.data_ptr(), stream_ptr(x)))
+    return x2, x3
+
+
+def argmax_to_indices(argmax, wo):
+    """uint8 window codes -> the reference's int32 indices in_y*Wo + in_x, [N,C,I]
+    (full_convlogic_kernel.cu:138,144)."""
+    n, c, hp, wp = argmax.shape
+    code = argmax.to(torch.int32)
+    py = torch.arange(hp, device=argmax.device, dtype=torch.int32).view(1, 1, hp, 1)
+    px = torch.arange(wp, device=argmax.device, dtype=torch.int32).view(1, 1, 1, wp)
+    idx = (2 * py + (code >> 1)) * wo + 2 * px + (code & 1)
+    return idx.reshape(n, c, hp * wp)
+
+
+def full_convlogic_backward_x(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
+    """src/convlogic/cuda/full_convlogic_kernel.cu:365-461 (deterministic here)."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    gx = torch.empty_like(x)
+    check(_lib.load().clg_convblock_backward_x(dtype_code(x), ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                               selection.data_ptr(), argmax.data_ptr(), gx.data_ptr(), stream_ptr(x)))
+    return gx
+
+
+def full_convlogic_backward_weight(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
+    """[C,7,16]; src/convlogic/cuda/full_convlogic_kernel.cu:616-701."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_convblock_backward_w_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gw = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_convblock_backward_w(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                       selection.data_ptr(), argmax.data_ptr(), gw.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
+    return gw

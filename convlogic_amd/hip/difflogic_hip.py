@@ -1,0 +1,116 @@
+"""Function set of the reference's `difflogic_cuda` module (src/difflogic/cuda/difflogic.cpp:15-34)
+on top of the HIP C ABI.  Tensors are feature-major ([features, batch]) as in the reference."""
+import torch
+
+from . import _lib
+from ._lib import check, check_input, dtype_code, stream_ptr
+
+_WORD_DTYPE = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
+
+
+def forward(x, a, b, w):
+    """y[out, B]; difflogic_cuda.forward (src/difflogic/cuda/difflogic_kernel.cu:89-126)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = w.shape[0]
+    y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
+    if y.numel():
+        check(_lib.load().clg_fc_forward(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(), y.data_ptr(),
+                                         in_dim, out_dim, batch, stream_ptr(x)))
+    return y
+
+
+def backward_w(x, a, b, grad_y):
+    """grad_w[out, 16]; difflogic_cuda.backward_w (difflogic_kernel.cu:128-173)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = grad_y.shape[0]
+    gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_backward_w(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), grad_y.data_ptr(),
+                                        gw.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return gw
+
+
+def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
+    """grad_x[in, B]; difflogic_cuda.backward_x (difflogic_kernel.cu:232-269)."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y"),
+                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = w.shape[0]
+    gx = torch.empty_like(x)
+    check(_lib.load().clg_fc_backward_x(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
+                                        grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
+                                        given_x_indices_of_y.data_ptr(), gx.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return gx
+
+
+def transpose(x):
+    """Contiguous transposed copy of a 2-D tensor through the tiled HIP transpose."""
+    check_input(x, "x")
+    rows, cols = x.shape
+    out = torch.empty((cols, rows), dtype=x.dtype, device=x.device)
+    if out.numel():
+        check(_lib.load().clg_transpose_2d(x.element_size(), x.data_ptr(), out.data_ptr(), rows, cols, stream_ptr(x)))
+    return out
+
+
+def eval(x, a, b, w):  # noqa: A001 - name of the reference binding
+    """Packed-bit layer evaluation; difflogic_cuda.eval (difflogic_kernel.cu:295-330).
+    x: integer words [in, W]; w: uint8 gate ids [out]."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
+        check_input(t, n)
+    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8:
+        raise RuntimeError("eval expects int8/16/32/64 words and uint8 gate ids")
+    in_dim, words = x.shape
+    out_dim = w.shape[0]
+    y = torch.empty((out_dim, words), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_eval_packed(x.element_size(), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
+                                         y.data_ptr(), in_dim, out_dim, words, stream_ptr(x)))
+    return y
+
+
+def _alloc_words(features, batch, bit_count, device):
+    if bit_count not in _WORD_DTYPE:
+        raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")
+    words = -(-batch // bit_count)
+    pad_len = (bit_count - batch % bit_count) % bit_count
+    return torch.empty((features, words), dtype=_WORD_DTYPE[bit_count], device=device), pad_len
+
+
+def tensor_packbits_cuda(t, bit_count):
+    """bool [F, B] -> (words [F, ceil(B/bits)], pad_len); difflogic_kernel.cu:368-413."""
+    check_input(t, "t")
+    if t.dtype != torch.bool:
+        raise RuntimeError("tensor_packbits_cuda expects a bool tensor")
+    features, batch = t.shape
+    out, pad_len = _alloc_words(features, batch, bit_count, t.device)
+    check(_lib.load().clg_pack_bits(t.data_ptr(), out.data_ptr(), features, batch, bit_count, stream_ptr(t)))
+    return out, pad_len
+
+
+def tensor_packbits_sample_major(t, bit_count):
+    """bool [B, F] (sample-major, as PackBitsTensor receives it) -> (words [F, ceil(B/bits)], pad_len),
+    without the transposed bool copy."""
+    check_input(t, "t")
+    if t.dtype != torch.bool:
+        raise RuntimeError("tensor_packbits_sample_major expects a bool tensor")
+    batch, features = t.shape
+    out, pad_len = _alloc_words(features, batch, bit_count, t.device)
+    check(_lib.load().clg_pack_bits_sample_major(t.data_ptr(), out.data_ptr(), features, batch, bit_count, stream_ptr(t)))
+    return out, pad_len
+
+
+def groupbitsum(b, pad_len, k):
+    """int32 [samples, k]; difflogic_cuda.groupbitsum (difflogic.cpp:22-33, difflogic_kernel.cu:450-482)."""
+    check_input(b, "b")
+    features, words = b.shape
+    if features % k != 0:
+        raise ValueError(f"in_dim ({features}) has to be divisible by k ({k}) but it is not")
+    samples = words * 8 * b.element_size() - pad_len
+    out = torch.empty((samples, k), dtype=torch.int32, device=b.device)
+    check(_lib.load().clg_group_bit_sum(b.element_size(), b.data_ptr(), out.data_ptr(), features, words, pad_len, k,
+                                        stream_ptr(b)))
+    return out

@@ -1,0 +1,197 @@
+/* convlogic_amd -- C ABI of the MI355X (gfx950) logic-layer kernels.
+ *
+ * Every entry point is a plain `extern "C"` function taking raw DEVICE pointers,
+ * sizes and a HIP stream (passed as void*, may be NULL for the default stream).
+ * Nothing here allocates, frees or synchronises: outputs and scratch buffers are
+ * provided by the caller, kernels are enqueued on `stream` and the call returns.
+ *
+ * Return value: 0 on success, a negative CLG_E* code on a rejected argument or a
+ * failed launch; clg_last_error() then returns a human readable message for the
+ * calling thread.  Bad arguments are rejected on the host before any launch.
+ *
+ * Each declaration cites the function of the reference's native extension modules
+ * (`difflogic_cuda`, `convlogic_cuda`; paths relative to the reference checkout) that
+ * it stands in for.
+ *
+ * Conventions
+ *   dtype           CLG_F32 or CLG_F64 (all float tensors of a call share it)
+ *   gate weights w  [..., 16] probabilities per gate (softmax or one-hot), gate ids
+ *                   as in src/difflogic/functional.py:7-24
+ *   selection       int32 [C, 8], tap = ch << 16 | row << 8 | col
+ *                   (src/convlogic/convlogic_layer.py:450-452)
+ *   all tensors are dense, row-major, in the shapes written beside each pointer.
+ */
+#ifndef CONVLOGIC_AMD_H
+#define CONVLOGIC_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CLG_F32 0
+#define CLG_F64 1
+
+#define CLG_OK 0
+#define CLG_EINVAL (-1)  /* rejected argument (shape, dtype, null pointer, limit) */
+#define CLG_ELAUNCH (-2) /* hipLaunch / HIP runtime error */
+
+/* Message describing the last error on the calling thread ("" if none). */
+const char *clg_last_error(void);
+/* ABI version of this library (bumped on incompatible changes). */
+int clg_abi_version(void);
+
+/* Geometry of a logic convolution (src/convlogic/convlogic_layer.py:94-109,192-193). */
+typedef struct clg_conv_geom {
+    int32_t n, c_in, h, w;   /* input  [n, c_in, h, w]            */
+    int32_t c_out;           /* logic kernels (output channels)   */
+    int32_t stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w;
+} clg_conv_geom;
+
+/* ---------------------------------------------------------------------------------
+ * fully connected LogicLayer, feature-major like the reference extension
+ * ------------------------------------------------------------------------------- */
+
+/* y[j][s] = sum_i w[j][i] * op_i(x[a[j]][s], x[b[j]][s]).
+ * Replaces difflogic_cuda.forward -- src/difflogic/cuda/difflogic.cpp:17,
+ * logic_layer_cuda_forward src/difflogic/cuda/difflogic_kernel.cu:89-126. */
+int clg_fc_forward(int dtype, const void *x /*[in_dim,batch]*/, const int64_t *a /*[out_dim]*/,
+                   const int64_t *b /*[out_dim]*/, const void *w /*[out_dim,16]*/, void *y /*[out_dim,batch]*/,
+                   int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
+
+/* grad_w[j][i] = sum_s grad_y[j][s] * op_i(x[a[j]][s], x[b[j]][s]) (column 0 is exactly 0).
+ * Replaces difflogic_cuda.backward_w -- src/difflogic/cuda/difflogic.cpp:18,
+ * logic_layer_cuda_backward_w src/difflogic/cuda/difflogic_kernel.cu:128-173. */
+int clg_fc_backward_w(int dtype, const void *x /*[in_dim,batch]*/, const int64_t *a, const int64_t *b,
+                      const void *grad_y /*[out_dim,batch]*/, void *grad_w /*[out_dim,16]*/, int64_t in_dim,
+                      int64_t out_dim, int64_t batch, void *stream);
+
+/* grad_x[i][s] = sum over neurons reading input i of grad_y * d y / d x_i, gathered through the
+ * reverse map (csr_start [in_dim+1], csr_list [2*out_dim]) built as in
+ * src/difflogic/difflogic.py:71-87.  No atomics: the result is bitwise reproducible.
+ * A neuron whose two inputs are the same feature contributes d/da + d/db (the derivative of the
+ * reference's python path).
+ * Replaces difflogic_cuda.backward_x -- src/difflogic/cuda/difflogic.cpp:19,
+ * logic_layer_cuda_backward_x src/difflogic/cuda/difflogic_kernel.cu:232-269. */
+int clg_fc_backward_x(int dtype, const void *x /*[in_dim,batch]*/, const int64_t *a, const int64_t *b,
+                      const void *w /*[out_dim,16]*/, const void *grad_y /*[out_dim,batch]*/,
+                      const int64_t *csr_start /*[in_dim+1]*/, const int64_t *csr_list /*[2*out_dim]*/,
+                      void *grad_x /*[in_dim,batch]*/, int64_t in_dim, int64_t out_dim, int64_t batch,
+                      void *stream);
+
+/* dst[c][r] = src[r][c] for elements of elem_size 1, 2, 4 or 8 bytes (layout change between the
+ * module's [batch, features] tensors and the feature-major kernels; the reference does this with
+ * x.transpose(0,1).contiguous(), src/difflogic/difflogic.py:130-131). */
+int clg_transpose_2d(int elem_size, const void *src /*[rows,cols]*/, void *dst /*[cols,rows]*/, int64_t rows,
+                     int64_t cols, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * packed-bit inference (PackBitsTensor)
+ * ------------------------------------------------------------------------------- */
+
+/* words[f][c] bit i = t[f][bit_count*c + i] (LSB first, zero padded); bit_count in {8,16,32,64};
+ * words holds ceil(batch/bit_count) integers of bit_count bits per feature.
+ * Replaces difflogic_cuda.tensor_packbits_cuda -- src/difflogic/cuda/difflogic.cpp:21,
+ * src/difflogic/cuda/difflogic_kernel.cu:368-413. */
+int clg_pack_bits(const uint8_t *t /*bool [features,batch]*/, void *words /*[features,ceil(batch/bit_count)]*/,
+                  int64_t features, int64_t batch, int bit_count, void *stream);
+
+/* Same result from the sample-major tensor t [batch, features] (what PackBitsTensor receives),
+ * without materialising the transposed copy of src/difflogic/packbitstensor.py:18. */
+int clg_pack_bits_sample_major(const uint8_t *t /*bool [batch,features]*/, void *words, int64_t features,
+                               int64_t batch, int bit_count, void *stream);
+
+/* y[j] = g_j(x[a[j]], x[b[j]]) bitwise on rows of `words` integers of elem_size bytes;
+ * gate[j] in 0..15.  x and y must not overlap.
+ * Replaces difflogic_cuda.eval -- src/difflogic/cuda/difflogic.cpp:20,
+ * logic_layer_cuda_eval src/difflogic/cuda/difflogic_kernel.cu:295-330 (gate switch
+ * src/common/cuda_utils.cuh:162-199). */
+int clg_fc_eval_packed(int elem_size, const void *x /*[in_dim,words]*/, const int64_t *a, const int64_t *b,
+                       const uint8_t *gate /*[out_dim]*/, void *y /*[out_dim,words]*/, int64_t in_dim,
+                       int64_t out_dim, int64_t words, void *stream);
+
+/* out[s][g] = number of features of class g (features/k consecutive rows) whose sample-s bit is set,
+ * for s < words*8*elem_size - pad_len.  features must be divisible by k.
+ * Replaces difflogic_cuda.groupbitsum -- src/difflogic/cuda/difflogic.cpp:22-33,
+ * src/difflogic/cuda/difflogic_kernel.cu:450-482 (which returns the same [samples,k] layout). */
+int clg_group_bit_sum(int elem_size, const void *x /*[features,words]*/, int32_t *out /*[samples,k]*/,
+                      int64_t features, int64_t words, int64_t pad_len, int64_t k, void *stream);
+
+/* ---------------------------------------------------------------------------------
+ * split conv-logic layers (ConvLogicLayer(complete=False), TreeLogicLayer)
+ * ------------------------------------------------------------------------------- */
+
+/* y[n][c][oy][ox][p] = gate(w[c][p], tap 2p, tap 2p+1), taps outside the image read 0.
+ * Replaces convlogic_cuda.convlogic_forward -- src/convlogic/cuda/convlogic.cpp:31,
+ * src/convlogic/cuda/convlogic_kernel.cu:67-106. */
+int clg_conv4_forward(int dtype, const clg_conv_geom *g, const void *x, const void *w /*[c_out,4,16]*/,
+                      const int32_t *selection, void *y /*[n,c_out,ho,wo,4]*/, void *stream);
+
+/* Deterministic (no float atomics) input gradient; grad_x is fully written.
+ * Replaces convlogic_cuda.convlogic_backward_x -- src/convlogic/cuda/convlogic.cpp:32,
+ * src/convlogic/cuda/convlogic_kernel.cu:321-359. */
+int clg_conv4_backward_x(int dtype, const clg_conv_geom *g, const void *grad_y /*[n,c_out,ho,wo,4]*/,
+                         const void *x, const void *w, const int32_t *selection, void *grad_x, void *stream);
+
+/* grad_w [c_out,4,16] w.r.t. the gate probabilities.  scratch: clg_conv4_backward_w_scratch_bytes().
+ * Replaces convlogic_cuda.convlogic_backward_weight -- src/convlogic/cuda/convlogic.cpp:33,
+ * src/convlogic/cuda/convlogic_kernel.cu:197-248. */
+int clg_conv4_backward_w(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x,
+                         const int32_t *selection, void *grad_w, void *scratch, void *stream);
+int64_t clg_conv4_backward_w_scratch_bytes(int dtype, const clg_conv_geom *g);
+
+/* One pairwise tree level: y[r][c][..][p] = gate(w[c][p], x[..][2p], x[..][2p+1]);
+ * x [n,c,h,w,2*xo] -> y [n,c,h,w,xo].  `positions` = h*w.
+ * Replaces convlogic_cuda.treelogic_forward -- src/convlogic/cuda/convlogic.cpp:35,
+ * src/convlogic/cuda/treelogic_kernel.cu:46-85. */
+int clg_tree_forward(int dtype, const void *x, const void *w /*[c,xo,16]*/, void *y, int64_t n, int64_t c,
+                     int64_t positions, int64_t xo, void *stream);
+/* Replaces convlogic_cuda.treelogic_backward_x -- src/convlogic/cuda/convlogic.cpp:36,
+ * src/convlogic/cuda/treelogic_kernel.cu:252-285. */
+int clg_tree_backward_x(int dtype, const void *grad_y, const void *x, const void *w, void *grad_x, int64_t n,
+                        int64_t c, int64_t positions, int64_t xo, void *stream);
+/* grad_w [c,xo,16].  scratch: clg_tree_backward_w_scratch_bytes().
+ * Replaces convlogic_cuda.treelogic_backward_weight -- src/convlogic/cuda/convlogic.cpp:37,
+ * src/convlogic/cuda/treelogic_kernel.cu:160-206 (without its xo <= 4 limit). */
+int clg_tree_backward_w(int dtype, const void *grad_y, const void *x, void *grad_w, void *scratch, int64_t n,
+                        int64_t c, int64_t positions, int64_t xo, void *stream);
+int64_t clg_tree_backward_w_scratch_bytes(int dtype, int64_t n, int64_t c, int64_t positions, int64_t xo);
+
+/* ---------------------------------------------------------------------------------
+ * fused block: tap gather -> 4 leaf gates -> 2 gates -> root gate -> 2x2/2 max pool
+ * (ConvLogicLayer(complete=True)); conv output height and width must be even.
+ * ------------------------------------------------------------------------------- */
+
+/* y [n,c_out,ho/2,wo/2]; argmax [n,c_out,ho/2,wo/2] holds dy*2+dx of the first maximum in window
+ * order (0,0),(0,1),(1,0),(1,1) -- the position the reference stores as in_y*wo+in_x.
+ * Nothing but y and one byte per pooled output is written.
+ * Replaces convlogic_cuda.full_convlogic_forward -- src/convlogic/cuda/convlogic.cpp:39,
+ * src/convlogic/cuda/full_convlogic_kernel.cu:147-231. */
+int clg_convblock_forward(int dtype, const clg_conv_geom *g, const void *x, const void *w /*[c_out,7,16]*/,
+                          const int32_t *selection, void *y, uint8_t *argmax, void *stream);
+
+/* Intermediates of the block for the return_intermediate / return_indices debug outputs:
+ * x2 [n,c_out,ho,wo,4] (leaf gates), x3 [n,c_out,ho,wo,2]; either may be NULL.
+ * (second and third result of full_convlogic_forward, full_convlogic_kernel.cu:172,194,230). */
+int clg_convblock_intermediates(int dtype, const clg_conv_geom *g, const void *x, const void *w,
+                                const int32_t *selection, void *x2, void *x3, void *stream);
+
+/* Input gradient through the stored argmax position; deterministic, grad_x fully written.
+ * Replaces convlogic_cuda.full_convlogic_backward_x -- src/convlogic/cuda/convlogic.cpp:40-41,
+ * src/convlogic/cuda/full_convlogic_kernel.cu:365-461. */
+int clg_convblock_backward_x(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                             const int32_t *selection, const uint8_t *argmax, void *grad_x, void *stream);
+
+/* grad_w [c_out,7,16] w.r.t. the gate probabilities.  scratch: clg_convblock_backward_w_scratch_bytes().
+ * Replaces convlogic_cuda.full_convlogic_backward_weight -- src/convlogic/cuda/convlogic.cpp:42-43,
+ * src/convlogic/cuda/full_convlogic_kernel.cu:616-701. */
+int clg_convblock_backward_w(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                             const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
+                             void *stream);
+int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_conv_geom *g);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CONVLOGIC_AMD_H */

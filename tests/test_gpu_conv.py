@@ -1,0 +1,223 @@
+"""GPU parity of the conv-logic layers (split 4-leaf layer, tree level, fused block) against the CPU
+oracle through the C ABI.  Float32 forward within 1e-5, gradients within 1e-4 relative, pool indices
+exact except on near ties (|gap| <= 1e-5) which are counted."""
+import pytest
+import torch
+
+import convlogic_amd as C
+from convlogic_amd.hip import convlogic_hip
+from oracle import convlogic_oracle as O
+from tests.gpu_util import DEV, assert_grad_close, block_oracle, check_pool_route
+
+pytestmark = pytest.mark.gpu
+
+GEOMS = [(1, 1, 3), (2, 2, 4), (1, 0, 3), (1, 2, 5)]
+
+
+def _pair(v):
+    return (v, v)
+
+
+# ---- split layer ------------------------------------------------------------------------------
+@pytest.mark.parametrize("stride,pad,kernel", GEOMS + [((1, 2), (0, 1), (2, 3))])
+def test_conv4_forward_backward(stride, pad, kernel):
+    torch.manual_seed(1)
+    st, pd, kn = (stride if isinstance(stride, tuple) else _pair(stride), pad if isinstance(pad, tuple) else _pair(pad),
+                  kernel if isinstance(kernel, tuple) else _pair(kernel))
+    layer = C.ConvLogicLayer(3, 5, stride=st, padding=pd, kernel=kn, implementation="cuda").to(DEV)
+    x = torch.randn(4, 3, 9, 10, device=DEV, requires_grad=True)
+    y = layer(x)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    xl = x.detach().cpu().requires_grad_(True)
+    ll = layer.weights.detach().cpu().requires_grad_(True)
+    want = O.conv4_forward(xl, torch.softmax(ll, -1), layer.selection.cpu(), st, pd, kn)
+    want.backward(gy.cpu())
+    assert y.shape == want.shape and (y.detach().cpu() - want.detach()).abs().max().item() <= 1e-5
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8, 6])
+def test_tree_forward_backward(bits):
+    torch.manual_seed(2)
+    layer = C.TreeLogicLayer(5, bits, implementation="cuda").to(DEV)
+    x = torch.rand(3, 5, 4, 6, bits, device=DEV, requires_grad=True)
+    y = layer(x)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    xl = x.detach().cpu().requires_grad_(True)
+    ll = layer.weights.detach().cpu().requires_grad_(True)
+    want = O.tree_forward(xl, torch.softmax(ll, -1))
+    want.backward(gy.cpu())
+    assert (y.detach().cpu() - want.detach()).abs().max().item() <= 1e-5
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+
+
+def test_tree_all_logic_gates_exact():
+    # reference KAT tests/convlogic/test_treelogic_forward.py:66-86
+    layer = C.TreeLogicLayer(channels=16, input_bits=8, implementation="cuda").to(DEV)
+    logits = torch.full((16, 4, 16), float("-inf"), device=DEV)
+    for g in range(16):
+        logits[g, :, g] = 0.0
+    with torch.no_grad():
+        layer.weights.copy_(logits)
+    flat = [0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0]
+    x = torch.tensor(flat, device=DEV).reshape(1, 1, 1, 1, 8).expand(-1, 16, -1, -1, -1)
+    a, b = torch.tensor(flat[::2]), torch.tensor(flat[1::2])
+    want = torch.stack([O.bin_op(a, b, g) for g in range(16)]).view(1, 16, 1, 1, 4)
+    assert torch.equal(layer(x).cpu(), want)
+
+
+# ---- fused block --------------------------------------------------------------------------------
+def _run_block(n, cin, cout, h, w, stride, pad, kernel, dtype=torch.float32, binary=False, seed=0, training=True):
+    torch.manual_seed(seed)
+    layer = C.ConvLogicLayer(cin, cout, stride=stride, padding=pad, kernel=kernel, complete=True, implementation="cuda",
+                             return_indices=True).to(DEV).to(dtype)
+    layer.train(training)
+    if binary:
+        x = torch.randint(0, 2, (n, cin, h, w), device=DEV).to(dtype)
+    else:
+        x = torch.randn(n, cin, h, w, device=DEV, dtype=dtype)
+    x.requires_grad_(True)
+    y, idx = layer(x)
+    return layer, x, y, idx
+
+
+@pytest.mark.parametrize("stride,pad,kernel", GEOMS)
+@pytest.mark.parametrize("binary", [False, True])
+def test_block_forward_backward_small(stride, pad, kernel, binary):
+    n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad
+    if ((h + 2 * pad - kernel) // stride + 1) % 2:
+        h += stride
+    if ((w + 2 * pad - kernel) // stride + 1) % 2:
+        w += stride
+    layer, x, y, idx = _run_block(n, cin, cout, h, w, stride, pad, kernel, binary=binary, seed=stride * 10 + pad)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    routed, y_ref, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, _pair(stride), _pair(pad),
+                                                            _pair(kernel), idx)
+    assert y.shape == y_ref.shape and idx.dtype == torch.int32 and idx.shape == idx_ref.shape
+    check_pool_route(idx, idx_ref, x4)
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
+    routed.backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+
+
+def test_block_binary_ties_pick_first_position():
+    # binary inputs in eval mode: outputs are exactly 0/1, ties are the norm, indices must equal max_pool2d's
+    layer, x, y, idx = _run_block(4, 2, 8, 12, 12, 1, 1, 3, binary=True, seed=4, training=False)
+    _, y_ref, idx_ref, *_ = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx, training=False)
+    assert torch.all((y == 0) | (y == 1))
+    assert torch.equal(y.detach().cpu(), y_ref.detach()) and torch.equal(idx.cpu(), idx_ref)
+
+
+def test_block_return_intermediate_matches_split_layers():
+    # mirrors tests/convlogic/test_full_convlogic_forward.py:165-233
+    for stride, pad in [(1, 1), (2, 2)]:
+        torch.manual_seed(0)
+        full = C.ConvLogicLayer(3, 2, stride=stride, padding=pad, kernel=3, implementation="cuda", complete=True,
+                                return_indices=True, return_intermediate=True).to(DEV)
+        conv = C.ConvLogicLayer(3, 2, stride=stride, padding=pad, kernel=3, implementation="cuda").to(DEV)
+        tree1 = C.TreeLogicLayer(2, 4, implementation="cuda").to(DEV)
+        tree2 = C.TreeLogicLayer(2, 2, implementation="cuda").to(DEV)
+        pool = C.PoolLogicLayer(return_indices=True)
+        conv.selection = full.selection
+        conv.weights.data.copy_(full.weights[:, 0:4])
+        tree1.weights.data.copy_(full.weights[:, 4:6])
+        tree2.weights.data.copy_(full.weights[:, 6:7])
+        x = torch.randn(4, 3, 10, 10, device=DEV)
+        with torch.no_grad():
+            y_full, x1_full, x2_full, idx_full = full(x)
+            x1 = conv(x)
+            x2 = tree1(x1)
+            y_split, idx_split = pool(tree2(x2))
+        assert torch.equal(idx_split.flatten(start_dim=2).to(torch.int32), idx_full)
+        assert torch.allclose(x1, x1_full, atol=1e-6) and torch.allclose(x2, x2_full, atol=1e-6)
+        assert torch.allclose(y_split, y_full, atol=1e-6)
+
+
+@pytest.mark.parametrize("batch", [1, 16])
+@pytest.mark.parametrize("c_in,c_out", [(1, 1), (3, 1), (1, 3)])
+@pytest.mark.parametrize("stride,pad,kernel", [(1, 1, 3), (2, 2, 4)])
+def test_block_gradcheck_float64(batch, c_in, c_out, stride, pad, kernel):
+    # mirrors tests/convlogic/test_full_convlogic_autograd.py:36-104 (no nondet_tol needed: deterministic)
+    torch.manual_seed(batch + c_in * 3 + c_out * 5 + stride)
+    layer = C.ConvLogicLayer(c_in, c_out, stride=stride, padding=pad, kernel=kernel, complete=True).double().to(DEV)
+    x = torch.sigmoid(torch.rand(batch, c_in, 6, 6, dtype=torch.double, device=DEV)).requires_grad_(True)
+    w = layer.weights.clone().detach().requires_grad_(True)
+    sel = layer.selection
+
+    def fn(inp, logits):
+        return C.FullConvLogicFunction.apply(inp, torch.softmax(logits, -1), sel, stride, stride, pad, pad, kernel, kernel, False)
+
+    assert torch.autograd.gradcheck(fn, (x, w), eps=1e-6, atol=1e-4)
+
+
+@pytest.mark.parametrize("stride,pad,kernel", [(1, 1, 3), (2, 2, 4)])
+def test_conv4_and_tree_gradcheck_float64(stride, pad, kernel):
+    torch.manual_seed(3)
+    layer = C.ConvLogicLayer(2, 3, stride=stride, padding=pad, kernel=kernel).double().to(DEV)
+    x = torch.rand(4, 2, 6, 6, dtype=torch.double, device=DEV, requires_grad=True)
+    w = layer.weights.clone().detach().requires_grad_(True)
+    assert torch.autograd.gradcheck(
+        lambda a, l: C.ConvLogicFunction.apply(a, torch.softmax(l, -1), layer.selection, stride, stride, pad, pad, kernel, kernel),
+        (x, w), eps=1e-6, atol=1e-4)
+    xt = torch.rand(2, 3, 2, 2, 4, dtype=torch.double, device=DEV, requires_grad=True)
+    wt = torch.randn(3, 2, 16, dtype=torch.double, device=DEV, requires_grad=True)
+    assert torch.autograd.gradcheck(lambda a, l: C.TreeLogicFunction.apply(a, torch.softmax(l, -1)), (xt, wt), eps=1e-6, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape", [(16, 1, 32, 28, 28), (4, 9, 256, 32, 32), (8, 32, 128, 16, 16), (8, 128, 512, 8, 8),
+                                   (16, 512, 1024, 4, 4), (4, 1, 8, 28, 28)])
+def test_block_benchmark_shapes_vs_oracle(shape):
+    # BASELINE configs 3/4 and the blocks of config 5 at reduced batch, binary inputs
+    n, cin, cout, h, w = shape
+    layer, x, y, idx = _run_block(n, cin, cout, h, w, 1, 1, 3, binary=True, seed=cin)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    routed, y_ref, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
+    flips = check_pool_route(idx, idx_ref, x4)
+    assert flips <= 1e-4 * idx.numel(), flips
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
+    routed.backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+
+
+def test_block_config4_full_size_properties():
+    # BASELINE config 4 at full size: determinism (bitwise) and linearity of the backward in grad_y
+    torch.manual_seed(5)
+    layer = C.ConvLogicLayer(9, 256, complete=True, implementation="cuda").to(DEV)
+    v = (torch.randn(256, 3, 32, 32, device=DEV) * 0.25 + 0.5).clamp(0, 1)
+    x = torch.cat([(v > t).float() for t in (0.25, 0.5, 0.75)], dim=1).requires_grad_(True)
+    y = layer(x)
+    y2 = layer(x)
+    assert y.shape == (256, 256, 16, 16) and torch.equal(y, y2)
+    assert float(y.detach().min()) >= 0 and float(y.detach().max()) <= 1
+    g1, g2 = torch.randn_like(y), torch.randn_like(y)
+
+    def grads(g):
+        return torch.autograd.grad(y, (x, layer.weights), g, retain_graph=True)
+
+    a, b, ab, a2 = grads(g1), grads(g2), grads(g1 + g2), grads(g1)
+    assert torch.equal(a[0], a2[0]) and torch.equal(a[1], a2[1])
+    assert_grad_close(ab[0], a[0] + b[0], name="linearity grad_x")
+    assert_grad_close(ab[1], a[1] + b[1], name="linearity grad_w")
+    # eval mode on binary input is exactly binary, and max pooling is an OR of the four root gates
+    layer.eval()
+    with torch.no_grad():
+        ye = layer(x)
+    assert torch.all((ye == 0) | (ye == 1))
+
+
+def test_block_errors():
+    layer = C.ConvLogicLayer(1, 1, kernel=3, padding=0, complete=True).to(DEV)
+    with pytest.raises(RuntimeError, match="divisible by 2"):
+        layer(torch.rand(1, 1, 5, 5, device=DEV))
+    with pytest.raises(RuntimeError):
+        convlogic_hip.full_convlogic_forward(torch.rand(1, 1, 6, 6), layer.weights.detach().softmax(-1), layer.selection, 1, 1, 0, 0, 3, 3)
+    layer = C.ConvLogicLayer(1, 1, kernel=2, padding=0, complete=True).to(DEV).eval()
+    assert layer(torch.randn(1, 1, 3, 3, device=DEV)).shape == (1, 1, 1, 1)

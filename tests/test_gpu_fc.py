@@ -1,0 +1,147 @@
+"""GPU parity of the fully connected LogicLayer (forward, both gradients) against the CPU oracle,
+through the C ABI.  Tolerances: float32 forward 1e-5 absolute, gradients 1e-4 relative."""
+import pytest
+import torch
+
+import convlogic_amd as C
+from convlogic_amd.hip import difflogic_hip
+from oracle import convlogic_oracle as O
+from tests.gpu_util import DEV, assert_grad_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_grads(x, logits, idx0, idx1, gy):
+    xl = x.detach().cpu().clone().requires_grad_(True)
+    ll = logits.detach().cpu().clone().requires_grad_(True)
+    y = O.logic_fc_forward(xl, idx0.cpu(), idx1.cpu(), torch.softmax(ll, -1))
+    y.backward(gy.cpu())
+    return y.detach(), xl.grad, ll.grad
+
+
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(8, 8, 32), (12, 16, 5), (100, 64, 256), (33, 40, 257), (1, 1, 1)])
+def test_fc_module_forward_backward(in_dim, out_dim, batch):
+    torch.manual_seed(in_dim * 1000 + batch)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV)
+    x = torch.rand(batch, in_dim, device=DEV, requires_grad=True)
+    gy = torch.randn(batch, out_dim, device=DEV)
+    y = layer(x)
+    y.backward(gy)
+    y_ref, gx_ref, gl_ref = _oracle_grads(x, layer.weights, layer.indices_0, layer.indices_1, gy)
+    assert y.shape == (batch, out_dim)
+    assert (y.detach().cpu() - y_ref).abs().max().item() <= 1e-5
+    assert_grad_close(x.grad, gx_ref, name="grad_x")
+    assert_grad_close(layer.weights.grad, gl_ref, name="grad_logits")
+
+
+def test_fc_self_paired_neuron_follows_python_derivative():
+    torch.manual_seed(5)
+    layer = C.LogicLayer(6, 8, implementation="cuda")
+    idx0, idx1 = layer.indices_0.clone(), layer.indices_1.clone()
+    idx1[2] = idx0[2]
+    idx1[5] = idx0[5]
+    layer = C.LogicLayer(6, 8, implementation="cuda")
+    layer.indices_0.copy_(idx0)
+    layer.indices_1.copy_(idx1)
+    from convlogic_amd.difflogic.difflogic import _reverse_wiring
+    s, f = _reverse_wiring(idx0.numpy(), idx1.numpy(), 6)
+    layer.given_x_indices_of_y_start.copy_(s)
+    layer.given_x_indices_of_y.copy_(f)
+    layer = layer.to(DEV)
+    x = torch.rand(9, 6, device=DEV, requires_grad=True)
+    gy = torch.randn(9, 8, device=DEV)
+    layer(x).backward(gy)
+    _, gx_ref, gl_ref = _oracle_grads(x, layer.weights, idx0, idx1, gy)
+    assert_grad_close(x.grad, gx_ref, name="grad_x")
+    assert_grad_close(layer.weights.grad, gl_ref, name="grad_logits")
+
+
+def test_fc_all_logic_gates_exact():
+    # reference KAT tests/difflogic/test_difflogic_forward.py:74-100
+    layer = C.LogicLayer(in_dim=8, out_dim=64, implementation="cuda").to(DEV)
+    layer.indices_0.copy_(torch.tensor([0, 2, 4, 6], device=DEV).repeat(16))
+    layer.indices_1.copy_(torch.tensor([1, 3, 5, 7], device=DEV).repeat(16))
+    logits = torch.full((64, 16), float("-inf"), device=DEV)
+    for g in range(16):
+        logits[g * 4: g * 4 + 4, g] = 0.0
+    with torch.no_grad():
+        layer.weights.copy_(logits)
+    flat = [0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0]
+    y = layer(torch.tensor([flat], device=DEV))
+    a, b = torch.tensor(flat[::2]), torch.tensor(flat[1::2])
+    want = torch.stack([O.bin_op(a, b, g) for g in range(16)]).view(1, -1)
+    assert torch.equal(y.cpu(), want)
+
+
+def test_fc_eval_binary_and_deterministic():
+    torch.manual_seed(7)
+    layer = C.LogicLayer(50, 70, implementation="cuda").to(DEV).eval()
+    x = torch.randint(0, 2, (33, 50), device=DEV).float()
+    y1, y2 = layer(x), layer(x)
+    assert torch.equal(y1, y2) and torch.all((y1 == 0) | (y1 == 1))
+    want = O.logic_fc_forward(x.cpu(), layer.indices_0.cpu(), layer.indices_1.cpu(), O.gate_weights(layer.weights.detach().cpu(), False))
+    assert torch.equal(y1.cpu(), want)
+
+
+@pytest.mark.parametrize("in_dim,out_dim", [(8, 8), (12, 16)])
+def test_fc_gradcheck_float64(in_dim, out_dim):
+    # mirrors tests/difflogic/test_difflogic_autograd.py:31-54
+    torch.manual_seed(11)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").double().to(DEV)
+    x = torch.sigmoid(torch.randn(16, in_dim, dtype=torch.double, device=DEV)).requires_grad_(True)
+    w = layer.weights.clone().detach().requires_grad_(True)
+    a, b, gs, gl = layer.indices_0, layer.indices_1, layer.given_x_indices_of_y_start, layer.given_x_indices_of_y
+
+    def fn(inp, logits):
+        return C.LogicLayerCudaFunction.apply(inp.T.contiguous(), a, b, torch.softmax(logits, -1), gs, gl).T
+
+    assert torch.autograd.gradcheck(fn, (x, w), eps=1e-6, atol=1e-4)
+
+
+def test_fc_chained_layers_avoid_copies_and_match():
+    torch.manual_seed(13)
+    l1 = C.LogicLayer(20, 40, implementation="cuda").to(DEV)
+    l2 = C.LogicLayer(40, 30, implementation="cuda").to(DEV)
+    x = torch.rand(64, 20, device=DEV)
+    y = l2(l1(x))
+    h = O.logic_fc_forward(x.cpu(), l1.indices_0.cpu(), l1.indices_1.cpu(), torch.softmax(l1.weights.detach().cpu(), -1))
+    want = O.logic_fc_forward(h, l2.indices_0.cpu(), l2.indices_1.cpu(), torch.softmax(l2.weights.detach().cpu(), -1))
+    assert (y.detach().cpu() - want).abs().max().item() <= 1e-5
+
+
+def test_fc_config1_shape_properties():
+    # BASELINE config 1 at full size: oracle forward (cheap) + determinism and linearity of backward
+    torch.manual_seed(17)
+    layer = C.LogicLayer(8000, 8000, implementation="cuda").to(DEV)
+    x = torch.rand(256, 8000, device=DEV, requires_grad=True)
+    y = layer(x)
+    want = O.logic_fc_forward(x.detach().cpu(), layer.indices_0.cpu(), layer.indices_1.cpu(),
+                              torch.softmax(layer.weights.detach().cpu(), -1))
+    assert (y.detach().cpu() - want).abs().max().item() <= 1e-5
+    g1, g2 = torch.randn_like(y), torch.randn_like(y)
+
+    def grads(g):
+        gx, gw = torch.autograd.grad(y, (x, layer.weights), g, retain_graph=True)
+        return gx, gw
+
+    a, b, ab, a_again = grads(g1), grads(g2), grads(g1 + g2), grads(g1)
+    assert torch.equal(a[0], a_again[0]) and torch.equal(a[1], a_again[1])          # bitwise reproducible
+    assert_grad_close(ab[0], a[0] + b[0], rel=1e-4, name="linearity grad_x")
+    assert_grad_close(ab[1], a[1] + b[1], rel=1e-4, name="linearity grad_w")
+
+
+def test_transpose_kernel():
+    for shape, dt in (((7, 130), torch.float32), ((129, 64), torch.float64), ((3, 5), torch.int16), ((65, 66), torch.uint8)):
+        t = (torch.rand(shape, device=DEV) * 100).to(dt)
+        assert torch.equal(difflogic_hip.transpose(t), t.T.contiguous())
+
+
+def test_fc_rejects_bad_inputs():
+    layer = C.LogicLayer(8, 8, implementation="cuda").to(DEV)
+    with pytest.raises(RuntimeError):
+        difflogic_hip.forward(torch.rand(8, 4), layer.indices_0, layer.indices_1, torch.rand(8, 16, device=DEV))
+    with pytest.raises(RuntimeError):
+        difflogic_hip.forward(torch.rand(8, 4, device=DEV).half(), layer.indices_0, layer.indices_1,
+                              torch.rand(8, 16, device=DEV).half())
+    with pytest.raises(AssertionError):
+        layer(torch.rand(2, 3, 8, device=DEV))

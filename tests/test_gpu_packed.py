@@ -1,0 +1,105 @@
+"""GPU parity of the packed-bit path (pack, bitwise evaluation, per-class counts): bit-exact against
+the numpy oracle; the reference holds no tests for this path, so the oracle itself is pinned by
+closed forms only (tests/test_oracle.py)."""
+import numpy as np
+import pytest
+import torch
+
+import convlogic_amd as C
+from convlogic_amd.hip import difflogic_hip
+from oracle import convlogic_oracle as O
+from tests.gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+TORCH_WORD = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32, 64])
+@pytest.mark.parametrize("batch,features", [(1, 1), (7, 3), (64, 5), (100, 130), (129, 257), (1000, 33), (4096, 16)])
+def test_pack_bits_both_layouts(bits, batch, features):
+    rng = np.random.default_rng(batch * 7 + features)
+    t = rng.integers(0, 2, (batch, features)).astype(bool)
+    want, pad = O.pack_bits(t.T, bits)
+    tt = torch.from_numpy(t).to(DEV)
+    w1, p1 = difflogic_hip.tensor_packbits_cuda(tt.T.contiguous(), bits)
+    w2, p2 = difflogic_hip.tensor_packbits_sample_major(tt, bits)
+    assert p1 == p2 == pad and w1.dtype == TORCH_WORD[bits]
+    assert np.array_equal(w1.cpu().numpy(), want) and np.array_equal(w2.cpu().numpy(), want)
+    p = C.PackBitsTensor(tt, bits)
+    assert p.pad_len == pad and np.array_equal(p.t.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits,batch", [(64, 4096), (64, 100), (32, 1000), (16, 48), (8, 8), (8, 24), (32, 96)])
+def test_eval_packed_bit_exact(bits, batch):
+    rng = np.random.default_rng(bits + batch)
+    torch.manual_seed(bits + batch)
+    in_dim, out_dim = 37, 53
+    t = rng.integers(0, 2, (in_dim, batch)).astype(bool)
+    words, pad = O.pack_bits(t, bits)
+    idx0, idx1 = torch.randint(0, in_dim, (out_dim,)), torch.randint(0, in_dim, (out_dim,))
+    gate = (torch.arange(out_dim) % 16).to(torch.uint8)
+    want = O.eval_packed(words, idx0.numpy(), idx1.numpy(), gate.numpy())
+    got = difflogic_hip.eval(torch.from_numpy(words).to(DEV), idx0.to(DEV), idx1.to(DEV), gate.to(DEV))
+    assert got.dtype == TORCH_WORD[bits] and np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bits,batch,features,k", [(64, 256, 40, 10), (32, 100, 12, 3), (8, 9, 4, 2), (64, 5000, 2000, 10), (16, 33, 6, 6)])
+def test_group_bit_sum(bits, batch, features, k):
+    rng = np.random.default_rng(batch + features)
+    t = rng.integers(0, 2, (features, batch)).astype(bool)
+    words, pad = O.pack_bits(t, bits)
+    got = difflogic_hip.groupbitsum(torch.from_numpy(words).to(DEV), pad, k)
+    want = O.group_bit_sum(words, pad, k)
+    assert got.dtype == torch.int32 and got.shape == (batch, k) and np.array_equal(got.cpu().numpy(), want)
+
+
+def test_packed_stack_equals_float_eval_path():
+    # 3 LogicLayers + GroupSum in eval mode: packed bits vs the float path on the same binary input
+    torch.manual_seed(3)
+    dims = [96, 192, 160, 120]
+    layers = [C.LogicLayer(a, b, implementation="cuda") for a, b in zip(dims[:-1], dims[1:])]
+    model = torch.nn.Sequential(*layers, C.GroupSum(10, tau=6.5)).to(DEV).eval()
+    x = torch.randint(0, 2, (300, dims[0]), device=DEV).bool()
+    with torch.no_grad():
+        y_float = model(x.float())
+        y_bits = model(C.PackBitsTensor(x, 64))
+    assert y_bits.dtype == torch.int32 and y_bits.shape == (300, 10)
+    assert torch.equal(y_bits.float() / 6.5, y_float)
+    # and against the oracle, bit for bit, layer by layer
+    words, pad = O.pack_bits(x.cpu().numpy().T, 64)
+    for layer in layers:
+        words = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(),
+                              layer.weights.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(O.group_bit_sum(words, pad, 10), y_bits.cpu().numpy())
+
+
+def test_eval_packed_config2_row_shape_properties():
+    # BASELINE config 2 row shape (1024 int64 words per feature) with fewer features; bit-exact vs oracle
+    rng = np.random.default_rng(9)
+    torch.manual_seed(9)
+    in_dim = out_dim = 2000
+    words = rng.integers(-2**63, 2**63 - 1, (in_dim, 1024), dtype=np.int64)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV).eval()
+    gate = layer.weights.argmax(-1).to(torch.uint8)
+    got = difflogic_hip.eval(torch.from_numpy(words).to(DEV), layer.indices_0, layer.indices_1, gate)
+    want = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(), gate.cpu().numpy())
+    assert np.array_equal(got.cpu().numpy(), want)
+    # De Morgan: evaluating the complemented gates on complemented inputs complements the output
+    comp = torch.tensor([15 - ((g & 8) >> 3 | (g & 4) >> 1 | (g & 2) << 1 | (g & 1) << 3) for g in range(16)], dtype=torch.uint8, device=DEV)
+    got_c = difflogic_hip.eval(~torch.from_numpy(words).to(DEV), layer.indices_0, layer.indices_1, comp[gate.long()])
+    assert torch.equal(~got_c, got)
+
+
+def test_packed_errors():
+    x = torch.zeros(8, 4, dtype=torch.bool, device=DEV)
+    with pytest.raises(ValueError):
+        difflogic_hip.tensor_packbits_cuda(x, 12)
+    p = C.PackBitsTensor(x.T.contiguous(), 32)
+    with pytest.raises(ValueError):
+        p.group_sum(3)
+    with pytest.raises(NotImplementedError):
+        C.PackBitsTensor(torch.zeros(4, 4, dtype=torch.bool))
+    layer = C.LogicLayer(8, 8, implementation="cuda").to(DEV)
+    with pytest.raises(AssertionError):
+        layer(p)                       # training mode
+    assert p.flatten() is p

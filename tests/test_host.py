@@ -1,0 +1,153 @@
+"""CPU-only tests: the C-ABI library loads and exports every declared symbol, the host-side python
+backend agrees with the oracle, wiring matches the golden vectors, argument validation raises."""
+import os
+import re
+
+import pytest
+import torch
+
+import convlogic_amd as C
+from convlogic_amd.difflogic import functional as Fn
+from convlogic_amd.difflogic.difflogic import _reverse_wiring
+from convlogic_amd.hip import _lib
+from oracle import convlogic_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "convlogic_amd.h")).read()
+    declared = set(re.findall(r"\b(clg_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.clg_abi_version() == 1
+    assert lib.clg_last_error() == b""
+
+
+def test_c_abi_rejects_bad_arguments_without_gpu():
+    lib = _lib.load()
+    assert lib.clg_fc_forward(7, 0, 0, 0, 0, 0, 4, 4, 4, None) == -1
+    assert b"dtype" in lib.clg_last_error()
+    assert lib.clg_group_bit_sum(8, 1, 1, 10, 4, 0, 3, None) == -1
+    assert b"divisible" in lib.clg_last_error()
+    assert lib.clg_pack_bits(1, 1, 4, 4, 12, None) == -1
+    assert b"bit_count" in lib.clg_last_error()
+    g = _lib.ConvGeom(1, 1, 5, 5, 1, 1, 1, 0, 0, 3, 3)    # conv output 3x3: odd
+    import ctypes
+    assert lib.clg_convblock_forward(0, ctypes.byref(g), 1, 1, 1, 1, 1, None) == -1
+    assert b"divisible by 2" in lib.clg_last_error()
+
+
+@pytest.mark.parametrize("i", range(16))
+def test_bin_op_matches_oracle(i):
+    a, b = torch.rand(20, dtype=torch.float64), torch.rand(20, dtype=torch.float64)
+    assert torch.allclose(Fn.bin_op(a, b, i), O.bin_op(a, b, i), atol=1e-14)
+
+
+def test_bin_op_s_matches_oracle():
+    torch.manual_seed(0)
+    a, b = torch.rand(5, 7, dtype=torch.float64), torch.rand(5, 7, dtype=torch.float64)
+    w = torch.softmax(torch.randn(7, 16, dtype=torch.float64), -1)
+    assert torch.allclose(Fn.bin_op_s(a, b, w), O.bin_op_s(a, b, w), atol=1e-14)
+
+
+def test_wiring_golden(golden):
+    for r in golden["logic_layer"]:
+        torch.manual_seed(r["seed"])
+        layer = C.LogicLayer(r["in_dim"], r["out_dim"], implementation="python", connections=r["connections"])
+        assert layer.indices_0.tolist() == r["indices_0"] and layer.indices_1.tolist() == r["indices_1"]
+        assert abs(float(layer.weights.detach().double().sum()) - r["weights_sum"]) < 1e-9
+    for r in golden["conv_layer"]:
+        torch.manual_seed(r["seed"])
+        layer = C.ConvLogicLayer(r["in_channels"], r["out_channels"], kernel=r["kernel"], groups=r["groups"],
+                                 complete=r["complete"], implementation="python")
+        assert layer.selection.tolist() == r["selection"] and layer.selection.dtype == torch.int32
+        assert abs(float(layer.weights.detach().double().sum()) - r["weights_sum"]) < 1e-9
+
+
+def test_reverse_wiring_matches_oracle_loop():
+    torch.manual_seed(1)
+    idx0, idx1 = torch.randint(0, 9, (14,)), torch.randint(0, 9, (14,))
+    idx1[3] = idx0[3]                                  # a self-paired neuron
+    s1, f1 = _reverse_wiring(idx0.numpy(), idx1.numpy(), 9)
+    s2, f2 = O.csr_build(idx0, idx1, 9)
+    assert torch.equal(s1, s2) and torch.equal(f1, f2)
+
+
+def test_logic_layer_python_matches_oracle():
+    torch.manual_seed(2)
+    layer = C.LogicLayer(10, 12, implementation="python")
+    x = torch.rand(4, 10)
+    y = layer(x)
+    want = O.logic_fc_forward(x, layer.indices_0, layer.indices_1, O.gate_weights(layer.weights, True))
+    assert torch.allclose(y, want, atol=1e-6)
+    layer.eval()
+    xb = torch.randint(0, 2, (4, 10)).float()
+    yb = layer(xb)
+    assert torch.all((yb == 0) | (yb == 1))
+    assert torch.equal(yb, O.logic_fc_forward(xb, layer.indices_0, layer.indices_1, O.gate_weights(layer.weights, False)))
+
+
+@pytest.mark.parametrize("stride,pad,kernel", [(1, 1, 3), (2, 2, 4), (1, 0, 3)])
+def test_conv_layer_python_matches_oracle(stride, pad, kernel):
+    torch.manual_seed(3)
+    layer = C.ConvLogicLayer(3, 4, stride=stride, padding=pad, kernel=kernel, implementation="python", complete=True)
+    x = torch.randn(2, 3, 8, 8)
+    y = layer(x)
+    want = O.conv_block_forward(x, O.gate_weights(layer.weights, True), layer.selection, (stride,) * 2, (pad,) * 2, (kernel,) * 2)
+    assert y.shape == want.shape and torch.allclose(y, want, atol=1e-6)
+    split = C.ConvLogicLayer(3, 4, stride=stride, padding=pad, kernel=kernel, implementation="python", selection=layer.selection)
+    y4 = split(x)
+    want4 = O.conv4_forward(x, O.gate_weights(split.weights, True), layer.selection, (stride,) * 2, (pad,) * 2, (kernel,) * 2)
+    assert torch.allclose(y4, want4, atol=1e-6)
+
+
+def test_tree_layer_python_all_gates():
+    layer = C.TreeLogicLayer(channels=16, input_bits=8, implementation="python")
+    logits = torch.full((16, 4, 16), float("-inf"))
+    for g in range(16):
+        logits[g, :, g] = 0.0
+    with torch.no_grad():
+        layer.weights.copy_(logits)
+    flat = [0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0]
+    x = torch.tensor(flat).reshape(1, 1, 1, 1, 8).expand(-1, 16, -1, -1, -1)
+    a, b = torch.tensor(flat[::2]), torch.tensor(flat[1::2])
+    want = torch.stack([O.bin_op(a, b, g) for g in range(16)]).view(1, 16, 1, 1, 4)
+    assert torch.equal(layer(x), want)
+
+
+def test_pool_layer_and_errors():
+    x = torch.randn(2, 3, 8, 8)
+    assert torch.equal(C.PoolLogicLayer()(x), torch.nn.functional.max_pool2d(x, 2, 2))
+    assert torch.equal(C.PoolLogicLayer()(x.unsqueeze(-1)), torch.nn.functional.max_pool2d(x, 2, 2))
+    with pytest.raises(ValueError):
+        C.PoolLogicLayer()(torch.randn(1, 2, 3))
+    with pytest.raises(ValueError):
+        C.PoolLogicLayer()(torch.randn(1, 1, 1, 4, 2))
+
+
+def test_group_sum_and_grad_factor():
+    x = torch.rand(3, 20, requires_grad=True)
+    y = C.GroupSum(5, tau=2.0)(C.GradFactor.apply(x, 3.0))
+    assert torch.allclose(y, O.group_sum(x.detach(), 5, 2.0))
+    y.sum().backward()
+    assert torch.allclose(x.grad, torch.full_like(x, 1.5))
+
+
+def test_constructor_validation():
+    with pytest.raises(AssertionError):
+        C.LogicLayer(10, 4, implementation="python")          # fewer than in_dim/2 neurons
+    with pytest.raises(AssertionError):
+        C.LogicLayer(4, 4, implementation="tpu")
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError):
+            C.ConvLogicLayer(1, 1, implementation="cuda")
+        with pytest.raises(NotImplementedError):
+            C.PackBitsTensor(torch.zeros(4, 4, dtype=torch.bool))
+    layer = C.ConvLogicLayer(2, 3, residual_init=True, complete=True, implementation="python")
+    assert torch.all(layer.weights.argmax(-1) == 3)
+    assert set(layer.state_dict()) == {"weights", "selection"}
+    fc = C.LogicLayer(4, 4, implementation="python")
+    assert set(fc.state_dict()) == {"weights", "indices_0", "indices_1"}
