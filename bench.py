@@ -1,0 +1,350 @@
+#!/usr/bin/env python3
+"""Benchmark of the logic-layer hot path on one MI355X.
+
+Primary line (BASELINE config 2): packed-bit inference through 3 LogicLayers of 64000 neurons on
+65536 samples packed into int64 words -> samples/s, with the HBM roofline of the evaluation kernel
+and the CPU oracle timed on the host cores beside it.  The "also" array carries the float
+workloads (config 1 LogicLayer, configs 3 and 4 ConvLogic block, forward+backward) in
+Ggate-evals/s, each with its own roofline entry.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2|c1|c3|c4] [--no-cpu]
+
+Prints ONE JSON line.  Inputs are synthetic and resident in HBM before the timed region.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+
+
+def _events(n):
+    import torch
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def _avg_ms(pairs):
+    return sum(a.elapsed_time(b) for a, b in pairs) / max(len(pairs), 1)
+
+
+def _timed(step, steps, warmup):
+    """warmup untimed steps, then exactly `steps` steps between two device synchronisations."""
+    import torch
+    for _ in range(warmup):
+        step(None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(k)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+# ------------------------------------------------------------------------------------------------
+# config 2: packed-bit inference
+# ------------------------------------------------------------------------------------------------
+C2 = dict(width=64000, layers=3, samples=65536, bits=64)
+
+
+def bench_c2(steps, warmup, cpu=True):
+    import numpy as np
+    import torch
+
+    import convlogic_amd as C
+    from convlogic_amd.difflogic.packbitstensor import PackBitsTensor
+
+    dev = "cuda:0"
+    width, nl, samples, bits = C2["width"], C2["layers"], C2["samples"], C2["bits"]
+    words = samples // bits
+    torch.manual_seed(0)
+    layers = [C.LogicLayer(width, width, implementation="cuda").to(dev).eval() for _ in range(nl)]
+    # Bernoulli(0.5) bits, generated directly as random words (a bool [65536, 64000] tensor would be 4 GB)
+    x0 = torch.randint(-2**63, 2**63 - 1, (width, words), dtype=torch.int64, device=dev)
+    packed = PackBitsTensor.__new__(PackBitsTensor)
+    packed.bit_count, packed.pad_len = bits, 0
+    pairs = _events(steps * nl)
+
+    def step(k):
+        packed.t = x0
+        p = packed
+        with torch.no_grad():
+            for li, layer in enumerate(layers):
+                if k is not None:
+                    pairs[k * nl + li][0].record()
+                p = layer(p)
+                if k is not None:
+                    pairs[k * nl + li][1].record()
+        return p
+
+    sec = _timed(step, steps, warmup)
+    kernel_ms = _avg_ms(pairs)
+    row_bytes = words * 8
+    # algorithmic bytes of one layer: every input row read once, every output row written once,
+    # wiring (2 x int64) and gate id (uint8) per neuron
+    alg_bytes = width * row_bytes + width * row_bytes + width * 17
+    achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "packed_bit_infer_samples_per_s",
+        "value": samples / sec,
+        "unit": "samples/s",
+        "ms_per_step": sec * 1e3,
+        "dtype": "int64",
+        "config": {"workload": "C2: 3 x LogicLayer 64000->64000 as packed bits, 65536 samples in int64 words "
+                               "(1024 words/feature), argmax gates, random 2-input wiring"},
+        "gate_evals_per_s": samples * width * nl / sec,
+        "roofline": {"bound": "hbm", "kernel": "eval_packed_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "avg_launch_ms": kernel_ms, "launches_timed": len(pairs)},
+    }
+    if cpu:
+        out["cpu_baseline"] = cpu_c2(layers, x0)
+    return out
+
+
+def cpu_c2(layers, x0):
+    """The C restatement of the packed evaluation (oracle/packed_oracle.c, OpenMP) on the full
+    workload, repeated for about 10 s."""
+    import numpy as np
+    path = os.path.join(ROOT, "oracle", "libpacked_oracle.so")
+    if not os.path.exists(path):
+        return {"value": None, "unit": "samples/s", "cores": 0, "kind": "port", "sample": "oracle/libpacked_oracle.so not built"}
+    lib = ctypes.CDLL(path)
+    threads = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    x_host = x0.cpu().numpy()
+    tmp = [np.empty(tuple(x0.shape), dtype=np.int64), np.empty(tuple(x0.shape), dtype=np.int64)]
+    wiring = [(l.indices_0.cpu().numpy(), l.indices_1.cpu().numpy(), l.weights.argmax(-1).cpu().numpy().astype(np.uint8)) for l in layers]
+    width, words = x0.shape
+    vp = ctypes.c_void_p
+
+    def one_pass():
+        src = x_host
+        for li, (a, b, g) in enumerate(wiring):
+            dst = tmp[li % 2]
+            lib.oracle_eval_packed(src.ctypes.data_as(vp), a.ctypes.data_as(vp), b.ctypes.data_as(vp), g.ctypes.data_as(vp),
+                                   dst.ctypes.data_as(vp), ctypes.c_int64(width), ctypes.c_int64(words * 8))
+            src = dst
+        return src
+
+    one_pass()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        one_pass()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > 10.0 or reps >= 2000:
+            break
+    return {"value": words * 64 * reps / el, "unit": "samples/s", "cores": threads, "kind": "port",
+            "sample": f"full C2 workload (3 layers x {width} neurons x {words * 64} samples), {reps} passes in {el:.1f} s, "
+                      f"oracle/packed_oracle.c with OpenMP"}
+
+
+# ------------------------------------------------------------------------------------------------
+# float workloads: forward + backward
+# ------------------------------------------------------------------------------------------------
+def _roof(name, alg_bytes, ms, extra=None):
+    achieved = alg_bytes / (ms * 1e-3) / 1e9
+    r = {"bound": "hbm", "kernel": name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+         "traffic": None, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": ms}
+    if extra:
+        r.update(extra)
+    return r
+
+
+def bench_c1(steps, warmup, cpu=True):
+    import torch
+
+    import convlogic_amd as C
+    from oracle import convlogic_oracle as O
+
+    dev = "cuda:0"
+    in_dim = out_dim = 8000
+    batch = 256
+    torch.manual_seed(1)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(dev)
+    x = torch.rand(batch, in_dim, device=dev, requires_grad=True)
+    gy = torch.randn(batch, out_dim, device=dev)
+    pairs = _events(steps)
+
+    def step(k):
+        x.grad = None
+        layer.weights.grad = None
+        if k is not None:
+            pairs[k][0].record()
+        y = layer(x)
+        y.backward(gy)
+        if k is not None:
+            pairs[k][1].record()
+
+    sec = _timed(step, steps, warmup)
+    gate_evals = batch * out_dim
+    # x, y read/written once forward; gy, x read and gx written backward; logits + wiring both ways
+    alg = (2 * batch * in_dim * 4 + out_dim * 16 + out_dim * 16 * 4) + (3 * batch * in_dim * 4 + out_dim * 16 * 4 + 4 * out_dim * 8 + in_dim * 8)
+    out = {"workload": "C1: LogicLayer 8000->8000, batch 256, float32, fwd+bwd (module API, incl. layout transposes)",
+           "metric": "fc_fwd_bwd_Ggate_evals_per_s", "value": gate_evals / sec / 1e9, "unit": "Ggate-evals/s", "ms_per_step": sec * 1e3,
+           "dtype": "f32", "roofline": _roof("fc fwd+bwd step (all kernels)", alg, _avg_ms(pairs))}
+    if cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        xl = x.detach().cpu().requires_grad_(True)
+        ll = layer.weights.detach().cpu().requires_grad_(True)
+        a, b, g = layer.indices_0.cpu(), layer.indices_1.cpu(), gy.cpu()
+
+        def cpu_step():
+            xl.grad = None
+            ll.grad = None
+            O.logic_fc_forward(xl, a, b, torch.softmax(ll, -1)).backward(g)
+
+        cpu_step()
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 5.0 and reps < 50:
+            cpu_step()
+            reps += 1
+        el = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": gate_evals * reps / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"full C1 workload, {reps} fwd+bwd steps of the torch-CPU oracle in {el:.1f} s"}
+    return out
+
+
+def _conv_inputs(cfg, dev):
+    import torch
+    n, cin, h, w = cfg["shape"]
+    if cfg["name"] == "C3":
+        return torch.randint(0, 2, (n, cin, h, w), device=dev).float()
+    v = (torch.randn(n, cin // 3, h, w, device=dev) * 0.25 + 0.5).clamp(0, 1)
+    return torch.cat([(v > t).float() for t in (0.25, 0.5, 0.75)], dim=1)
+
+
+CONV = {
+    "c3": dict(name="C3", shape=(256, 1, 28, 28), k=32),
+    "c4": dict(name="C4", shape=(256, 9, 32, 32), k=256),
+}
+
+
+def bench_conv(key, steps, warmup, cpu=True):
+    import torch
+
+    import convlogic_amd as C
+    from convlogic_amd.hip import convlogic_hip
+    from oracle import convlogic_oracle as O
+
+    cfg = CONV[key]
+    dev = "cuda:0"
+    n, cin, h, w = cfg["shape"]
+    k = cfg["k"]
+    torch.manual_seed(2)
+    layer = C.ConvLogicLayer(cin, k, kernel=3, padding=1, complete=True, implementation="cuda").to(dev)
+    x = _conv_inputs(cfg, dev).requires_grad_(True)
+    gy = torch.randn(n, k, h // 2, w // 2, device=dev)
+
+    def step(_k):
+        x.grad = None
+        layer.weights.grad = None
+        y = layer(x)
+        y.backward(gy)
+
+    sec = _timed(step, steps, warmup)
+    gate_evals = n * k * h * w * 7
+
+    # kernel-level durations: forward, input-gradient and weight-gradient launches timed one by one
+    wp = torch.softmax(layer.weights.detach(), -1).contiguous()
+    xd, sel = x.detach(), layer.selection
+    geo = (1, 1, 1, 1)
+    y, am = convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
+    reps = max(steps, 5)
+    ev = {name: _events(reps) for name in ("fwd", "bwd_x", "bwd_w")}
+    for r in range(reps):
+        ev["fwd"][r][0].record()
+        convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
+        ev["fwd"][r][1].record()
+        ev["bwd_x"][r][0].record()
+        convlogic_hip.full_convlogic_backward_x(gy, xd, wp, am, sel, *geo)
+        ev["bwd_x"][r][1].record()
+        ev["bwd_w"][r][0].record()
+        convlogic_hip.full_convlogic_backward_weight(gy, xd, wp, am, sel, *geo)
+        ev["bwd_w"][r][1].record()
+    torch.cuda.synchronize()
+    ms = {name: _avg_ms(p) for name, p in ev.items()}
+    xb, yb, pb = n * cin * h * w * 4, n * k * (h // 2) * (w // 2) * 4, k * 7 * 16 * 4 + k * 8 * 4
+    alg_f, alg_b = xb + yb + pb, yb + xb + xb + pb      # forward: x in, y out; backward: gy, x in, gx out
+    total_ms = ms["fwd"] + ms["bwd_x"] + ms["bwd_w"]
+    out = {"workload": f"{cfg['name']}: ConvLogicLayer block [{n},{cin},{h},{w}] -> k={k}, 3x3 pad 1, depth-2 tree, 2x2 OR-pool, float32 fwd+bwd",
+           "metric": "convlogic_fwd_bwd_Ggate_evals_per_s", "value": gate_evals / sec / 1e9, "unit": "Ggate-evals/s",
+           "ms_per_step": sec * 1e3, "dtype": "f32", "kernel_ms": ms, "kernels_only_Ggate_evals_per_s": gate_evals / (total_ms * 1e-3) / 1e9,
+           "roofline": _roof("convblock fwd + bwd_x + bwd_w kernels", alg_f + alg_b, total_ms,
+                             {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
+                              "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked"})}
+    if cpu:
+        nb = 8                                              # bounded sample: 8 samples of the batch
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        xl = x.detach()[:nb].cpu().requires_grad_(True)
+        ll = layer.weights.detach().cpu().requires_grad_(True)
+        selc, g = sel.cpu(), gy[:nb].cpu()
+
+        def cpu_step():
+            xl.grad = None
+            ll.grad = None
+            O.conv_block_forward(xl, torch.softmax(ll, -1), selc, (1, 1), (1, 1), (3, 3)).backward(g)
+
+        cpu_step()
+        reps_c, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 5.0 and reps_c < 20:
+            cpu_step()
+            reps_c += 1
+        el = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": nb * k * h * w * 7 * reps_c / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"{nb} of {n} samples, {reps_c} fwd+bwd steps of the vectorised torch-CPU oracle in {el:.1f} s"}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", default="", help="c1|c2|c3|c4: run just that workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on one GPU; --gpus must be 1 "
+              "(sharding over more GPUs is design-only in this repository)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from convlogic_amd.hip import _lib
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()
+    cpu = not args.no_cpu
+    runners = {"c2": lambda: bench_c2(args.steps, args.warmup, cpu), "c1": lambda: bench_c1(args.steps, args.warmup, cpu),
+               "c3": lambda: bench_conv("c3", args.steps, args.warmup, cpu), "c4": lambda: bench_conv("c4", args.steps, args.warmup, cpu)}
+    if args.only:
+        res = runners[args.only]()
+        primary, also = res, []
+        if args.only != "c2":
+            primary = dict(res)
+            primary["config"] = {"workload": primary.pop("workload")}
+    else:
+        primary = runners["c2"]()
+        also = [runners[k]() for k in ("c4", "c3", "c1")]
+    line = {"metric": primary["metric"], "value": primary["value"], "unit": primary["unit"], "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": primary["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": primary["dtype"], "data": "synthetic", "config": primary["config"],
+            "roofline": primary["roofline"], "cpu_baseline": primary.get("cpu_baseline"),
+            "device": torch.cuda.get_device_name(0), "host_cores": os.cpu_count()}
+    for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s"):
+        if extra in primary:
+            line[extra] = primary[extra]
+    if also:
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

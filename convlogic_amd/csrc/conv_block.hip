@@ -1,4 +1,25 @@
-// Fused conv-logic block: entry points and shape dispatch.
+// Fused conv-logic block (tap gather -> 4 leaf gates -> 2 gates -> root gate -> 2x2/2 max pool):
+// LDS-tiled kernels for gfx950, shape dispatch and the C entry points.
+//
+// LDS image layout.  A workgroup stages the zero-padded input planes of S samples (all input
+// channels) in LDS.  Padding is shared: a row holds pw halo elements and then the w pixels, so the
+// right halo of a row is the left halo of the next row (row stride rs = w + pw), and the bottom halo
+// rows of a plane are the top halo rows of the next plane (plane stride chs = (h + ph) * rs).  A tap
+// (ch, ry, rx) of a kernel is then one scalar offset ch*chs + ry*rs + rx that is added to a per-lane
+// base, with no bounds checks in the inner loops.
+//
+// Forward: a workgroup owns (S samples) x (CT kernels).  Lanes run along conv-output columns, each
+// lane evaluates the tree at conv rows 2r and 2r+1, the horizontal neighbour comes over DPP, and the
+// even lane keeps the first maximum in window order and writes the pooled value and a 1-byte code.
+// The kernel index is uniform per wavefront, so the 28 folded coefficients and 8 tap offsets sit in
+// scalar registers.
+//
+// Input gradient: deterministic without float atomics in global memory.  Every (sample, input
+// channel) plane of the gradient has exactly one owner wavefront, which walks all kernels that read
+// its channel in increasing order, recomputes their tree at the stored argmax position of every
+// pooled cell and accumulates the tap gradients of ITS channel into an LDS plane that only it
+// touches (the plane has the same shared-halo layout as the input image, so out-of-image taps fall
+// into halo elements that are never read back).  The order of additions is program order.
 #include "conv_common.h"
 
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
@@ -11,21 +32,520 @@ int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_
                                      hipStream_t st);
 int clg_convblock_partial_blocks(const Geom &g);
 
+namespace {
+
+constexpr int kLdsLimit = 160 * 1024;
+
+// Division of a 31-bit value by a runtime constant: q = umulhi(x, mul) >> shr (d == 1: q = x).
+struct FastDiv {
+    uint32_t mul, shr, d;
+};
+FastDiv make_fastdiv(uint32_t d)
+{
+    if (d <= 1) return FastDiv{0, 0, 1};
+    uint32_t lg = 0;
+    while ((1ull << lg) < d) ++lg;
+    const uint32_t p = 31 + lg;
+    const uint32_t mul = (uint32_t)(((1ull << p) + d - 1) / d);
+    return FastDiv{mul, p - 32, d};
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv &f) { return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shr); }
+
+struct TilePlan {
+    int S;              // samples per workgroup
+    int G;              // samples sharing one wavefront pass (input gradient; 1 when a sample has >= 64 cells)
+    int CT;             // kernels per workgroup (forward)
+    int NW;             // wavefronts per workgroup
+    int rs, chs;        // row and plane stride of the LDS image (elements)
+    int xe;             // elements of one LDS image region (S samples + tail)
+    int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
+    FastDiv d_hw, d_w, d_slots, d_wo, d_wp;
+    size_t lds_bytes;
+};
+
+template <typename T>
+__device__ __forceinline__ T dpp_xor1(T v)
+{
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, false);
+        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, false);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T to_sgpr(T v)
+{
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)u);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+// Stages the planes of `samples` consecutive samples into the zeroed LDS image.
+template <typename T>
+__device__ __forceinline__ void stage_image(T *__restrict__ xs, const T *__restrict__ src, int samples, const Geom &g,
+                                            const TilePlan &p, int tid, int nthreads)
+{
+    const uint32_t total = (uint32_t)samples * g.cin * g.h * g.w;
+    for (uint32_t e = tid; e < total; e += nthreads) {
+        const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)(g.h * g.w);
+        const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+        xs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw] = src[e];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ sel,
+                                               T *__restrict__ y, uint8_t *__restrict__ argmax, Geom g, TilePlan p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *xs = reinterpret_cast<T *>(smem);
+    T *coef = xs + ((p.xe + 3) & ~3);                                 // [CT][28]
+    int *toff = reinterpret_cast<int *>(coef + p.CT * 28);            // [CT][8]
+    int2 *slot = reinterpret_cast<int2 *>(toff + p.CT * 8);           // [S * slots]
+
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
+    const int n0 = blockIdx.x * p.S, s_cur = min(p.S, g.n - n0);
+    const int c0 = blockIdx.y * p.CT, ct_cur = min(p.CT, g.c - c0);
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+
+    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
+    for (int q = tid; q < ct_cur * 7; q += nthreads) {
+        const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
+        coef[q * 4 + 0] = cf.ab;
+        coef[q * 4 + 1] = cf.a;
+        coef[q * 4 + 2] = cf.b;
+        coef[q * 4 + 3] = cf.one;
+    }
+    for (int q = tid; q < ct_cur * 8; q += nthreads) {
+        const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
+        toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
+    }
+    const int U = s_cur * p.slots;
+    for (int u = tid; u < U; u += nthreads) {
+        const uint32_t s = fdiv(u, p.d_slots), r = u - s * (uint32_t)p.slots;
+        const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
+        slot[u] = make_int2((int)(s * g.cin * p.chs + (2 * rp * g.sh) * p.rs + ox * g.sw), (int)((s * g.c) * I + rp * wp + (ox >> 1)));
+    }
+    __syncthreads();
+    stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
+    __syncthreads();
+
+    const int row_step = g.sh * p.rs;
+    for (int lc = wave; lc < ct_cur; lc += p.NW) {
+        Tree<T> tr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            tr.g[k].ab = to_sgpr(coef[(lc * 7 + k) * 4 + 0]);
+            tr.g[k].a = to_sgpr(coef[(lc * 7 + k) * 4 + 1]);
+            tr.g[k].b = to_sgpr(coef[(lc * 7 + k) * 4 + 2]);
+            tr.g[k].one = to_sgpr(coef[(lc * 7 + k) * 4 + 3]);
+        }
+        int to[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) to[t] = uniform(toff[lc * 8 + t]);
+        const int64_t obase = ((int64_t)n0 * g.c + c0 + lc) * I;
+        T *yb = y + obase;
+        uint8_t *ab = argmax + obase;
+        for (int u0 = 0; u0 < U; u0 += kWave) {
+            const int u = u0 + lane;
+            const bool valid = u < U;
+            const int2 e = slot[valid ? u : 0];
+            T v[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = xs[e.x + to[t]];
+            const T r0 = eval_tree(tr, v).root;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
+            const T r1 = eval_tree(tr, v).root;
+            const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
+            if (valid && !(lane & 1)) {
+                T best = r0;
+                int code = 0;
+                if (r0o > best) { best = r0o; code = 1; }
+                if (r1 > best) { best = r1; code = 2; }
+                if (r1o > best) { best = r1o; code = 3; }
+                // a NaN in the first window position never loses a strict comparison; a first
+                // position below every comparison (NaN elsewhere) behaves as in the generic kernel
+                yb[e.y] = best;
+                ab[e.y] = (uint8_t)code;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// input gradient
+// ---------------------------------------------------------------------------------------------
+// Scratch of the input-gradient kernel, written by one preparation launch:
+//   folded [c][7][4]   coefficients (ab, a, b, one) of every gate
+//   count  [cin]       number of kernels that read input channel ch
+//   hits   [cin][c]    those kernels in increasing order, entry = kernel | tap mask << 16
+// (the reverse map "input channel -> kernels and taps reading it", built in a fixed order).
+struct BwdScratch {
+    size_t folded_bytes, count_off, hits_off, total;
+};
+BwdScratch bwd_scratch_layout(const Geom &g, int elem)
+{
+    BwdScratch b;
+    b.folded_bytes = (size_t)g.c * 28 * elem;
+    b.count_off = (b.folded_bytes + 15) & ~(size_t)15;
+    b.hits_off = (b.count_off + (size_t)g.cin * 4 + 15) & ~(size_t)15;
+    b.total = b.hits_off + (size_t)g.cin * g.c * 4;
+    return b;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
+                                                              T *__restrict__ folded, int32_t *__restrict__ count,
+                                                              int32_t *__restrict__ hits, int C, int cin, int fold_blocks)
+{
+    if ((int)blockIdx.x < fold_blocks) {
+        const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (q < (int64_t)C * 7) {
+            const Coef<T> cf = fold16(w + q * 16);
+            folded[q * 4 + 0] = cf.ab;
+            folded[q * 4 + 1] = cf.a;
+            folded[q * 4 + 2] = cf.b;
+            folded[q * 4 + 3] = cf.one;
+        }
+        return;
+    }
+    // one wavefront per input channel: lanes test 64 kernels at a time, matches are appended in order
+    const int lane = threadIdx.x & (kWave - 1);
+    const int ch = uniform((int)(blockIdx.x - fold_blocks) * 4 + (int)(threadIdx.x >> 6));
+    if (ch >= cin) return;
+    int n = 0;
+    for (int c0 = 0; c0 < C; c0 += kWave) {
+        const int c = c0 + lane;
+        int mask = 0;
+        if (c < C) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) mask |= (((sel[c * 8 + t] >> 16) & 0xFFFF) == ch) << t;
+        }
+        const uint64_t vote = __ballot(mask != 0);
+        if (mask) {
+            const int before = __builtin_amdgcn_mbcnt_hi((uint32_t)(vote >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)vote, 0));
+            hits[(int64_t)ch * C + n + before] = c | (mask << 16);
+        }
+        n += __popcll(vote);
+    }
+    if (lane == 0) count[ch] = n;
+}
+
+constexpr int kChunk = 4;  // cell blocks (of 64 lanes) whose grad_y / argmax loads are in flight together
+
+template <typename T>
+struct CellLoads {
+    T gy[kChunk];
+    int code[kChunk];
+};
+
+template <typename T>
+__global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                  const T *__restrict__ folded, const int32_t *__restrict__ count,
+                                                  const int32_t *__restrict__ hits, const int32_t *__restrict__ sel,
+                                                  const uint8_t *__restrict__ argmax, T *__restrict__ gx, Geom g, TilePlan p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int xe4 = (p.xe + 3) & ~3;
+    T *xs = reinterpret_cast<T *>(smem);
+    T *gs = xs + xe4;                                               // gradient planes, same layout as xs
+    int2 *cellt = reinterpret_cast<int2 *>(gs + xe4);               // [G * slots]
+
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
+    const int n0 = blockIdx.x * p.S, s_cur = min(p.S, g.n - n0);
+    const int wp = g.wo >> 1, I = p.slots;
+
+    for (int i = tid; i < 2 * xe4; i += nthreads) xs[i] = T(0);
+    const int V = p.G * I;                                          // lanes of one pass: G samples x I cells
+    for (int v = tid; v < V; v += nthreads) {
+        const uint32_t s = fdiv(v, p.d_slots), cell = v - s * (uint32_t)I;
+        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+        cellt[v] = make_int2((int)(s * g.cin * p.chs + (2 * py * g.sh) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
+    }
+    __syncthreads();
+    stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
+    __syncthreads();
+
+    // work items: (group of G samples, input channel); a wavefront owns the gradient planes of its item
+    const int groups = (s_cur + p.G - 1) / p.G;
+    const int items = groups * g.cin;
+    const int row_step = g.sh * p.rs;
+    for (int item = wave; item < items; item += p.NW) {
+        const int grp = item / g.cin, ch = item - grp * g.cin;
+        const int s0 = grp * p.G;
+        const int v_here = min(p.G, s_cur - s0) * I;
+        const int chunks = (v_here + kChunk * kWave - 1) / (kChunk * kWave);
+        const int img0 = s0 * g.cin * p.chs;                        // LDS offset of the group's first plane
+        const int64_t gbase = ((int64_t)(n0 + s0) * g.c) * I;       // global offset of the group's first cell row
+        const int nhits = count[ch];
+        const int32_t *hit = hits + (int64_t)ch * g.c;
+        const int steps = nhits * chunks;                           // step = (hit, chunk), hit-major
+
+        auto issue = [&](int step, CellLoads<T> &L) {
+            const int k = step / chunks, chunk = step - k * chunks;
+            const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
+#pragma unroll
+            for (int j = 0; j < kChunk; ++j) {
+                const int v = (chunk * kChunk + j) * kWave + lane;
+                L.gy[j] = T(0);
+                L.code[j] = 0;
+                if (v < v_here) {
+                    const int o = cellt[v].y;
+                    L.code[j] = argmax[crow + o];
+                    L.gy[j] = gy[crow + o];
+                }
+            }
+        };
+
+        CellLoads<T> cur, nxt;
+        if (steps > 0) issue(0, cur);
+        for (int step = 0; step < steps; ++step) {
+            if (step + 1 < steps) issue(step + 1, nxt);
+            const int k = step / chunks, chunk = step - k * chunks;
+            const int ent = hit[k];
+            const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
+            int to[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const Tap tp = unpack_tap(sel[c * 8 + t]);
+                to[t] = tp.ch * p.chs + tp.ry * p.rs + tp.rx;
+            }
+            Tree<T> tr;
+            const T *fc = folded + (int64_t)c * 28;
+#pragma unroll
+            for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+            // phase 1: tree and tap gradients of every cell block of this chunk (registers only)
+            int pos[kChunk];
+            bool live[kChunk];
+            T gt[kChunk][8];
+#pragma unroll
+            for (int j = 0; j < kChunk; ++j) {
+                const int v = (chunk * kChunk + j) * kWave + lane;
+                live[j] = v < v_here;
+                pos[j] = 0;
+                if (live[j]) {
+                    const int code = cur.code[j];
+                    const T gout = cur.gy[j];
+                    pos[j] = img0 + cellt[v].x + (code >> 1) * row_step + (code & 1) * g.sw;
+                    T tv[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) tv[t] = xs[pos[j] + to[t]];
+                    const TreeVals<T> tvv = eval_tree(tr, tv);
+                    const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
+                    const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if ((mask >> (2 * q)) & 3) {                 // wave-uniform: a tap of this leaf is ours
+                            const int m = q >> 1;
+                            const T g_mid = m ? g_m1 : g_m0;
+                            const T g_leaf = g_mid * ((q & 1) ? gate_db(tr.g[4 + m], tvv.leaf[q ^ 1])
+                                                               : gate_da(tr.g[4 + m], tvv.leaf[q ^ 1]));
+                            gt[j][2 * q] = g_leaf * gate_da(tr.g[q], tv[2 * q + 1]);
+                            gt[j][2 * q + 1] = g_leaf * gate_db(tr.g[q], tv[2 * q]);
+                        }
+                    }
+                }
+            }
+            // phase 2: read-add-write per tap.  For one tap the targets of all cells (all lanes, all
+            // blocks) are distinct elements, so the blocks of a chunk go together; taps may collide
+            // with each other and are applied one after the other.  Only this wavefront touches the plane.
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if ((mask >> t) & 1) {                               // wave-uniform
+                    T old[kChunk];
+#pragma unroll
+                    for (int j = 0; j < kChunk; ++j)
+                        if (live[j]) old[j] = gs[pos[j] + to[t]];
+#pragma unroll
+                    for (int j = 0; j < kChunk; ++j)
+                        if (live[j]) gs[pos[j] + to[t]] = old[j] + gt[j][t];
+                }
+            }
+            cur = nxt;
+        }
+    }
+    __syncthreads();
+    // write the gradient planes of the staged samples back (interior elements only)
+    const uint32_t total = (uint32_t)s_cur * g.cin * g.h * g.w;
+    T *dst = gx + (int64_t)n0 * g.cin * g.h * g.w;
+    for (uint32_t e = tid; e < total; e += nthreads) {
+        const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)(g.h * g.w);
+        const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+        dst[e] = gs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// plans
+// ---------------------------------------------------------------------------------------------
+void plan_common(const Geom &g, TilePlan *p)
+{
+    p->rs = g.w + g.pw;
+    p->chs = (g.h + g.ph) * p->rs;
+    p->d_hw = make_fastdiv((uint32_t)(g.h * g.w));
+    p->d_w = make_fastdiv((uint32_t)g.w);
+    p->d_wo = make_fastdiv((uint32_t)g.wo);
+    p->d_wp = make_fastdiv((uint32_t)(g.wo / 2));
+}
+
+int64_t image_elems(const Geom &g, const TilePlan &p, int S) { return (int64_t)S * g.cin * p.chs + g.ph * p.rs + g.pw; }
+
+// The last tap row/column must stay inside the padded image for the shared-halo layout to hold.
+bool taps_inside(const Geom &g) { return (g.ho - 1) * g.sh + g.kh <= g.h + 2 * g.ph && (g.wo - 1) * g.sw + g.kw <= g.w + 2 * g.pw; }
+
+bool plan_forward(const Geom &g, int elem, TilePlan *p)
+{
+    if (!taps_inside(g)) return false;
+    plan_common(g, p);
+    p->slots = (g.ho / 2) * g.wo;
+    p->G = 1;
+    // samples per workgroup: best lane utilisation within a 64 KiB image, smallest S on ties
+    int best_s = 0;
+    double best_util = 0;
+    for (int S = 1; S <= 16 && S <= g.n; ++S) {
+        if (image_elems(g, *p, S) * elem + (int64_t)S * p->slots * 8 > 64 * 1024 && S > 1) break;
+        const int64_t U = (int64_t)S * p->slots;
+        const double util = (double)U / (double)(clg_ceil_div(U, kWave) * kWave);
+        if (util > best_util + 0.02) { best_util = util; best_s = S; }
+    }
+    if (best_s == 0 || best_util < 0.4) return false;
+    p->S = best_s;
+    p->NW = 4;
+    const int64_t groups = clg_ceil_div(g.n, p->S);
+    int64_t ct = (int64_t)g.c * groups / 1024;
+    ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
+    if (ct > g.c) ct = g.c;
+    p->CT = (int)ct;
+    p->xe = (int)image_elems(g, *p, p->S);
+    p->d_slots = make_fastdiv((uint32_t)p->slots);
+    p->lds_bytes = (size_t)((p->xe + 3) & ~3) * elem + (size_t)p->CT * 28 * elem + (size_t)p->CT * 8 * 4 + (size_t)p->S * p->slots * 8;
+    if (p->lds_bytes > (size_t)kLdsLimit) return false;
+    if (clg_ceil_div(g.c, p->CT) > 65535) return false;
+    return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * ((g.ho / 2) * (g.wo / 2)) < (1ll << 31);
+}
+
+bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
+{
+    if (!taps_inside(g)) return false;
+    plan_common(g, p);
+    const int I = (g.ho / 2) * (g.wo / 2);
+    p->slots = I;
+    p->CT = 0;
+    // G samples share a wavefront pass when a sample has fewer than 64 cells
+    int G = I >= kWave ? 1 : kWave / I;
+    if (G > g.n) G = g.n;
+    // shrink G until two image regions fit
+    while (G > 1 && 2 * ((image_elems(g, *p, G) + 3) & ~3) * elem + (int64_t)G * I * 8 > kLdsLimit) G /= 2;
+    p->G = G;
+    p->S = G;
+    p->xe = (int)image_elems(g, *p, p->S);
+    p->lds_bytes = (size_t)2 * ((p->xe + 3) & ~3) * elem + (size_t)G * I * 8;
+    if (p->lds_bytes > (size_t)kLdsLimit) return false;
+    if ((double)(G * I) / (double)(clg_ceil_div(G * I, kWave) * kWave) < 0.2) return false;
+    const int items = g.cin;                                         // one group per workgroup
+    p->NW = items < 16 ? items : 16;
+    p->d_slots = make_fastdiv((uint32_t)I);
+    return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * I < (1ll << 31);
+}
+
+template <typename K>
+int allow_lds(K kernel, size_t bytes, const char *name)
+{
+    if (bytes > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) {
+            clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+            return CLG_ELAUNCH;
+        }
+    }
+    return CLG_OK;
+}
+
+template <typename T>
+int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const void *w, const int32_t *sel, void *y,
+                         uint8_t *argmax, hipStream_t st)
+{
+    if (int e = allow_lds(convblock_forward_tiled_kernel<T>, p.lds_bytes, "clg_convblock_forward")) return e;
+    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
+    hipLaunchKernelGGL(convblock_forward_tiled_kernel<T>, grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x, (const T *)w, sel,
+                       (T *)y, argmax, g, p);
+    CLG_CHECK_LAUNCH("clg_convblock_forward(tiled)");
+    return CLG_OK;
+}
+
+template <typename T>
+int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, const void *x, const void *w, const int32_t *sel,
+                            const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
+{
+    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T));
+    T *folded = reinterpret_cast<T *>(scratch);
+    int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
+    int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
+    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 7, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
+    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
+                       folded, count, hits, g.c, g.cin, fold_blocks);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
+    if (int e = allow_lds(convblock_backward_x_tiled_kernel<T>, p.lds_bytes, "clg_convblock_backward_x")) return e;
+    hipLaunchKernelGGL(convblock_backward_x_tiled_kernel<T>, dim3((unsigned)clg_ceil_div(g.n, p.S)), dim3(p.NW * kWave), p.lds_bytes, st,
+                       (const T *)gy, (const T *)x, (const T *)folded, (const int32_t *)count, (const int32_t *)hits, sel, argmax,
+                       (T *)gx, g, p);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(tiled)");
+    return CLG_OK;
+}
+
+int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
+
+}  // namespace
+
 extern "C" int clg_convblock_forward(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
                                      void *y, uint8_t *argmax, void *stream)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_forward")) return e;
     CLG_REQUIRE(x && w && selection && y && argmax, "clg_convblock_forward: null pointer argument");
+    TilePlan p;
+    if (plan_forward(g, elem_size(dtype), &p)) {
+        if (dtype == CLG_F32) return launch_forward_tiled<float>(g, p, x, w, selection, y, argmax, clg_stream(stream));
+        return launch_forward_tiled<double>(g, p, x, w, selection, y, argmax, clg_stream(stream));
+    }
     return clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, clg_stream(stream));
 }
 
+extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_conv_geom *gg)
+{
+    Geom g;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x_scratch_bytes")) return -1;
+    return (int64_t)bwd_scratch_layout(g, elem_size(dtype)).total;
+}
+
 extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
-                                        const int32_t *selection, const uint8_t *argmax, void *grad_x, void *stream)
+                                        const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch,
+                                        void *stream)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x")) return e;
-    CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_x, "clg_convblock_backward_x: null pointer argument");
+    CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_x && scratch, "clg_convblock_backward_x: null pointer argument");
+    TilePlan p;
+    if (plan_backward_x(g, elem_size(dtype), &p)) {
+        if (dtype == CLG_F32)
+            return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
+        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
+    }
     return clg_convblock_backward_x_generic(dtype, g, grad_y, x, w, selection, argmax, grad_x, clg_stream(stream));
 }
 
@@ -33,7 +553,7 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
 {
     Geom g;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w_scratch_bytes")) return -1;
-    return (int64_t)g.c * clg_convblock_partial_blocks(g) * 28 * (dtype == CLG_F64 ? 8 : 4);
+    return (int64_t)g.c * clg_convblock_partial_blocks(g) * 28 * elem_size(dtype);
 }
 
 extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,

@@ -166,9 +166,12 @@ def full_convlogic_backward_x(grad_y, x, weight, argmax, selection, stride_h, st
     for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
         check_input(t, n)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_convblock_backward_x_scratch_bytes(dt, ctypes.byref(g)), x.device)
     gx = torch.empty_like(x)
-    check(_lib.load().clg_convblock_backward_x(dtype_code(x), ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
-                                               selection.data_ptr(), argmax.data_ptr(), gx.data_ptr(), stream_ptr(x)))
+    check(lib.clg_convblock_backward_x(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                       selection.data_ptr(), argmax.data_ptr(), gx.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
     return gx
 
 

@@ -178,10 +178,13 @@ int clg_convblock_intermediates(int dtype, const clg_conv_geom *g, const void *x
                                 const int32_t *selection, void *x2, void *x3, void *stream);
 
 /* Input gradient through the stored argmax position; deterministic, grad_x fully written.
+ * scratch: clg_convblock_backward_x_scratch_bytes() bytes (folded gate coefficients).
  * Replaces convlogic_cuda.full_convlogic_backward_x -- src/convlogic/cuda/convlogic.cpp:40-41,
  * src/convlogic/cuda/full_convlogic_kernel.cu:365-461. */
 int clg_convblock_backward_x(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
-                             const int32_t *selection, const uint8_t *argmax, void *grad_x, void *stream);
+                             const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch,
+                             void *stream);
+int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_conv_geom *g);
 
 /* grad_w [c_out,7,16] w.r.t. the gate probabilities.  scratch: clg_convblock_backward_w_scratch_bytes().
  * Replaces convlogic_cuda.full_convlogic_backward_weight -- src/convlogic/cuda/convlogic.cpp:42-43,
