@@ -4,6 +4,8 @@
 // Every gate is bitwise, so the evaluation kernel treats a row as a run of bytes and moves it with
 // 16-byte vectors whatever the word type is; one wavefront evaluates one neuron (gate id, wiring
 // and truth-table masks are wave-uniform) over a column chunk of its two input rows.
+#include <stdlib.h>
+
 #include "clg_common.h"
 
 namespace {
@@ -75,6 +77,64 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_kernel(const V *__rest
                 if (vv < v1) __builtin_nontemporal_store(gate_vec(m, ra[u], rb[u]), yj + vv);
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// evaluation along a precomputed walk of the wiring graph
+// ---------------------------------------------------------------------------------------------
+// Input rows are vertices and neurons are edges of a multigraph.  The plan lists the neurons along
+// trails of that graph, so that a neuron shares one input row with its predecessor; the wavefront
+// keeps that row in registers and loads only the other one.  Every row chunk is then read about once
+// (plus one extra row per segment start) instead of twice.
+// plan[k] = neuron | use << 28 | keep << 30
+//   use : 0 nothing carried, 1 carried row is input a, 2 carried row is input b, 3 it is both
+//   keep: row carried to the next step, 0 = input a, 1 = input b
+template <int R>
+__global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x4 *__restrict__ x, const int64_t *__restrict__ a,
+                                                                    const int64_t *__restrict__ b,
+                                                                    const uint8_t *__restrict__ gate,
+                                                                    const int32_t *__restrict__ plan, u32x4 *__restrict__ y,
+                                                                    int steps, int seg_len, int64_t row_vecs)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    const int k0 = (blockIdx.x * kEvalWaves + wave) * seg_len;
+    if (k0 >= steps) return;
+    const int k1 = k0 + seg_len < steps ? k0 + seg_len : steps;
+    const int64_t col0 = (int64_t)blockIdx.y * (kWave * R) + lane;   // this lane's first vector in the row
+    u32x4 ra[R], rb[R], carry[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) carry[r] = (u32x4)0u;
+    for (int k = k0; k < k1; ++k) {
+        const int p = plan[k];
+        const int j = p & 0x0FFFFFFF, keep = (p >> 30) & 1;
+        const int use = k == k0 ? 0 : (p >> 28) & 3;
+        const u32x4 *xa = x + a[j] * row_vecs + col0;
+        const u32x4 *xb = x + b[j] * row_vecs + col0;
+        if (use != 1 && use != 3) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (col0 + r * kWave < row_vecs) ra[r] = xa[r * kWave];
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) ra[r] = carry[r];
+        }
+        if (use < 2) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (col0 + r * kWave < row_vecs) rb[r] = xb[r * kWave];
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) rb[r] = carry[r];
+        }
+        const Masks m = gate_masks(gate[j]);
+        u32x4 *yj = y + (int64_t)j * row_vecs + col0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (col0 + r * kWave < row_vecs) __builtin_nontemporal_store(gate_vec(m, ra[r], rb[r]), yj + r * kWave);
+#pragma unroll
+        for (int r = 0; r < R; ++r) carry[r] = keep ? rb[r] : ra[r];
     }
 }
 
@@ -215,12 +275,14 @@ void launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_
                  int64_t row_bytes, hipStream_t st)
 {
     const int64_t row_vecs = row_bytes / (int64_t)sizeof(V);
-    // column chunks of at most 2 KiB per row: with both uses of a row segment inside one chunk pass,
-    // the working set of a pass (in_dim x 2 KiB) stays cache resident for layers up to ~100k features.
-    const int max_chunk_vecs = 2048 / (int)sizeof(V);
+    // column chunks of at most 4 KiB per row: both uses of a row segment fall inside one chunk pass,
+    // so the working set of a pass (in_dim x 4 KiB) can stay in the last-level cache (measured best on
+    // 64000 x 8 KiB rows among 0.5..8 KiB).  CLG_EVAL_CHUNK_BYTES / CLG_EVAL_NPW override for tuning.
+    const char *e_chunk = getenv("CLG_EVAL_CHUNK_BYTES"), *e_npw = getenv("CLG_EVAL_NPW");
+    const int max_chunk_vecs = (e_chunk ? atoi(e_chunk) : 4096) / (int)sizeof(V);
     const int chunk_vecs = row_vecs < max_chunk_vecs ? (int)row_vecs : max_chunk_vecs;
     const int chunks = (int)clg_ceil_div(row_vecs, chunk_vecs);
-    const int neurons_per_wave = 4;
+    const int neurons_per_wave = e_npw ? atoi(e_npw) : 1;
     const int groups = (int)clg_ceil_div(out_dim, (int64_t)kEvalWaves * neurons_per_wave);
     hipLaunchKernelGGL((eval_packed_kernel<V, 2>), dim3((unsigned)(chunks * groups)), dim3(kEvalBlock), 0, st, (const V *)x, a,
                        b, gate, (V *)y, (int)out_dim, row_vecs, chunk_vecs, groups, neurons_per_wave);
@@ -313,5 +375,99 @@ extern "C" int clg_group_bit_sum(int elem_size, const void *x, int32_t *out, int
     hipLaunchKernelGGL(group_bit_sum_kernel, dim3((unsigned)clg_ceil_div(items, 4)), dim3(256), 0, st, (const uint8_t *)x, out,
                        class_rows, row_bytes, samples, (int)k, cols8, (int)slices);
     CLG_CHECK_LAUNCH("clg_group_bit_sum");
+    return CLG_OK;
+}
+
+// ---- walk plan (host side) --------------------------------------------------------------------
+extern "C" int clg_fc_eval_plan(const int64_t *a, const int64_t *b, int64_t in_dim, int64_t out_dim, int32_t *plan)
+{
+    CLG_REQUIRE(a && b && plan, "clg_fc_eval_plan: null pointer argument");
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && out_dim < (1ll << 28), "clg_fc_eval_plan: out_dim must be in 1..2^28-1");
+    // adjacency: edges (neurons) incident to each vertex (input row); a self-paired neuron is listed twice
+    int64_t *start = (int64_t *)calloc((size_t)in_dim + 1, sizeof(int64_t));
+    int32_t *adj = (int32_t *)malloc((size_t)out_dim * 2 * sizeof(int32_t));
+    int64_t *fill = (int64_t *)malloc((size_t)in_dim * sizeof(int64_t));
+    uint8_t *used = (uint8_t *)calloc((size_t)out_dim, 1);
+    if (!start || !adj || !fill || !used) {
+        free(start); free(adj); free(fill); free(used);
+        clg_set_error("clg_fc_eval_plan: out of host memory");
+        return CLG_EINVAL;
+    }
+    for (int64_t j = 0; j < out_dim; ++j) {
+        if (a[j] < 0 || a[j] >= in_dim || b[j] < 0 || b[j] >= in_dim) {
+            free(start); free(adj); free(fill); free(used);
+            clg_set_error("clg_fc_eval_plan: neuron %lld is wired to a feature outside 0..%lld", (long long)j, (long long)in_dim - 1);
+            return CLG_EINVAL;
+        }
+        ++start[a[j] + 1];
+        ++start[b[j] + 1];
+    }
+    for (int64_t v = 0; v < in_dim; ++v) start[v + 1] += start[v];
+    for (int64_t v = 0; v < in_dim; ++v) fill[v] = start[v];
+    for (int64_t j = 0; j < out_dim; ++j) {
+        adj[fill[a[j]]++] = (int32_t)j;
+        adj[fill[b[j]]++] = (int32_t)j;
+    }
+    for (int64_t v = 0; v < in_dim; ++v) fill[v] = start[v];       // now: scan position per vertex
+    int64_t n = 0;
+    // trails start at odd-degree vertices first (pass 0), then anywhere edges remain (pass 1)
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int64_t v0 = 0; v0 < in_dim; ++v0) {
+            if (pass == 0 && ((start[v0 + 1] - start[v0]) & 1) == 0) continue;
+            int64_t v = v0;
+            bool carried = false;
+            for (;;) {
+                while (fill[v] < start[v + 1] && used[adj[fill[v]]]) ++fill[v];
+                if (fill[v] == start[v + 1]) break;
+                const int32_t e = adj[fill[v]++];
+                used[e] = 1;
+                const int64_t other = a[e] == v ? b[e] : a[e];
+                int use = 0;
+                if (carried) use = (a[e] == v ? 1 : 0) | (b[e] == v ? 2 : 0);
+                const int keep = other == b[e] ? 1 : 0;
+                plan[n++] = e | (use << 28) | (keep << 30);
+                v = other;
+                carried = true;
+            }
+        }
+    }
+    free(start); free(adj); free(fill); free(used);
+    CLG_REQUIRE(n == out_dim, "clg_fc_eval_plan: internal error, %lld of %lld neurons placed", (long long)n, (long long)out_dim);
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate,
+                                          const int32_t *plan, void *y, int64_t in_dim, int64_t out_dim, int64_t words,
+                                          void *stream)
+{
+    CLG_REQUIRE(valid_elem(elem_size), "clg_fc_eval_packed_planned: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
+    CLG_REQUIRE(x && a && b && gate && plan && y, "clg_fc_eval_packed_planned: null pointer argument");
+    CLG_REQUIRE(x != y, "clg_fc_eval_packed_planned: x and y must not overlap");
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && words > 0, "clg_fc_eval_packed_planned: in_dim, out_dim and words must be positive");
+    CLG_REQUIRE(out_dim < (1ll << 28), "clg_fc_eval_packed_planned: out_dim above 2^28-1 is not supported");
+    const int64_t row_bytes = words * elem_size;
+    const uintptr_t align = (uintptr_t)x | (uintptr_t)y | (uintptr_t)row_bytes;
+    // short or unaligned rows gain nothing from carrying a row in registers
+    if ((align & 15) != 0 || row_bytes < 1024) return clg_fc_eval_packed(elem_size, x, a, b, gate, y, in_dim, out_dim, words, stream);
+    const int64_t row_vecs = row_bytes / 16;
+    const char *e_r = getenv("CLG_EVAL_WALK_R"), *e_l = getenv("CLG_EVAL_WALK_SEG");
+    int R = e_r ? atoi(e_r) : 4;
+    while (R > 1 && (int64_t)kWave * (R / 2) >= row_vecs) R /= 2;
+    const int seg = e_l ? atoi(e_l) : 8;
+    const int64_t col_chunks = clg_ceil_div(row_vecs, (int64_t)kWave * R);
+    CLG_REQUIRE(col_chunks <= 65535, "clg_fc_eval_packed_planned: rows above %lld bytes are not supported", 65535ll * kWave * R * 16);
+    const dim3 grid((unsigned)clg_ceil_div(out_dim, (int64_t)kEvalWaves * seg), (unsigned)col_chunks), block(kEvalBlock);
+    hipStream_t st = clg_stream(stream);
+#define CLG_WALK(RR)                                                                                                          \
+    hipLaunchKernelGGL(eval_packed_walk_kernel<RR>, grid, block, 0, st, (const u32x4 *)x, a, b, gate, plan, (u32x4 *)y, (int)out_dim, \
+                       seg, row_vecs)
+    switch (R) {
+    case 1: CLG_WALK(1); break;
+    case 2: CLG_WALK(2); break;
+    case 4: CLG_WALK(4); break;
+    default: CLG_WALK(8); break;
+    }
+#undef CLG_WALK
+    CLG_CHECK_LAUNCH("clg_fc_eval_packed_planned");
     return CLG_OK;
 }

@@ -105,9 +105,27 @@ class LogicLayer(torch.nn.Module):
         assert not self.training
         assert isinstance(x, PackBitsTensor)
         assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
-        gate = self.weights.argmax(-1).to(torch.uint8)
-        x.t = difflogic_hip.eval(x.t, self.indices_0, self.indices_1, gate)
+        x.t = difflogic_hip.eval_planned(x.t, self.indices_0, self.indices_1, self._eval_gates(), self._eval_plan())
         return x
+
+    def _eval_gates(self):
+        """uint8 arg-max gate id per neuron, recomputed only after the logits changed."""
+        key = (self.weights._version, self.weights.data_ptr())
+        cached = getattr(self, "_gate_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8))
+            self._gate_cache = cached
+        return cached[1]
+
+    def _eval_plan(self):
+        """Walk order of the wiring graph for the packed evaluation kernel; rebuilt when the wiring
+        buffers were modified in place or moved to another device."""
+        key = (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+        cached = getattr(self, "_plan_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, difflogic_hip.eval_plan(self.indices_0, self.indices_1, self.in_dim))
+            self._plan_cache = cached
+        return cached[1]
 
     def extra_repr(self):
         return "{}, {}, {}".format(self.in_dim, self.out_dim, "train" if self.training else "eval")

@@ -72,6 +72,33 @@ def eval(x, a, b, w):  # noqa: A001 - name of the reference binding
     return y
 
 
+def eval_plan(a, b, in_dim):
+    """Walk order of the wiring graph for eval_planned (int32 [out], on the device of `a`).  Host
+    computation, done once per wiring."""
+    a_h = a.detach().to("cpu", torch.int64).contiguous()
+    b_h = b.detach().to("cpu", torch.int64).contiguous()
+    plan = torch.empty(a_h.shape[0], dtype=torch.int32)
+    check(_lib.load().clg_fc_eval_plan(a_h.data_ptr(), b_h.data_ptr(), in_dim, a_h.shape[0], plan.data_ptr()))
+    return plan.to(a.device)
+
+
+def eval_planned(x, a, b, w, plan):
+    """eval() in the order of `plan` (from eval_plan for the same a, b): identical result, about half
+    the input traffic."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (plan, "plan")):
+        check_input(t, n)
+    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8 or plan.dtype != torch.int32:
+        raise RuntimeError("eval_planned expects int8/16/32/64 words, uint8 gate ids and an int32 plan")
+    in_dim, words = x.shape
+    out_dim = w.shape[0]
+    if plan.shape[0] != out_dim:
+        raise RuntimeError("plan does not match the number of neurons")
+    y = torch.empty((out_dim, words), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_eval_packed_planned(x.element_size(), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
+                                                 plan.data_ptr(), y.data_ptr(), in_dim, out_dim, words, stream_ptr(x)))
+    return y
+
+
 def _alloc_words(features, batch, bit_count, device):
     if bit_count not in _WORD_DTYPE:
         raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")

@@ -111,6 +111,22 @@ int clg_fc_eval_packed(int elem_size, const void *x /*[in_dim,words]*/, const in
                        const uint8_t *gate /*[out_dim]*/, void *y /*[out_dim,words]*/, int64_t in_dim,
                        int64_t out_dim, int64_t words, void *stream);
 
+/* HOST function (plain host pointers, no GPU work): orders the neurons of a layer along trails of
+ * its wiring graph (input rows = vertices, neurons = edges) so that consecutive neurons share an input
+ * row.  plan [out_dim] is consumed by clg_fc_eval_packed_planned.  Computed once per wiring, like the
+ * reverse map of src/difflogic/difflogic.py:71-87 is for the backward pass; no counterpart in the
+ * reference's eval path. */
+int clg_fc_eval_plan(const int64_t *a_host /*[out_dim]*/, const int64_t *b_host /*[out_dim]*/, int64_t in_dim,
+                     int64_t out_dim, int32_t *plan_host /*[out_dim]*/);
+
+/* Same result as clg_fc_eval_packed, evaluated in plan order: the shared input row of consecutive
+ * neurons stays in registers, so every input row is fetched about once instead of twice.  plan is
+ * the DEVICE copy of clg_fc_eval_plan's output for the same (a, b).
+ * Replaces difflogic_cuda.eval -- src/difflogic/cuda/difflogic_kernel.cu:295-330. */
+int clg_fc_eval_packed_planned(int elem_size, const void *x /*[in_dim,words]*/, const int64_t *a, const int64_t *b,
+                               const uint8_t *gate /*[out_dim]*/, const int32_t *plan /*[out_dim]*/,
+                               void *y /*[out_dim,words]*/, int64_t in_dim, int64_t out_dim, int64_t words, void *stream);
+
 /* out[s][g] = number of features of class g (features/k consecutive rows) whose sample-s bit is set,
  * for s < words*8*elem_size - pad_len.  features must be divisible by k.
  * Replaces difflogic_cuda.groupbitsum -- src/difflogic/cuda/difflogic.cpp:22-33,

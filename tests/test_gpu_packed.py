@@ -103,3 +103,40 @@ def test_packed_errors():
     with pytest.raises(AssertionError):
         layer(p)                       # training mode
     assert p.flatten() is p
+
+
+@pytest.mark.parametrize("in_dim,out_dim,words,bits", [(37, 53, 128, 64), (64, 64, 1024, 64), (500, 300, 200, 64), (20, 100, 130, 64),
+                                                         (16, 16, 512, 32), (9, 30, 64, 64), (300, 150, 256, 64)])
+def test_eval_planned_equals_unplanned(in_dim, out_dim, words, bits):
+    # the walk-ordered kernel must give the bits of the plain kernel and of the oracle for any wiring,
+    # including neurons wired twice to one feature and features used once
+    rng = np.random.default_rng(in_dim + words)
+    torch.manual_seed(in_dim + words)
+    info = np.iinfo(O.NP_WORD[bits])
+    x = rng.integers(info.min, info.max, (in_dim, words), dtype=O.NP_WORD[bits])
+    if out_dim * 2 >= in_dim and in_dim != 20:
+        layer = C.LogicLayer(in_dim, out_dim, implementation="python")
+        idx0, idx1 = layer.indices_0, layer.indices_1
+    else:
+        idx0, idx1 = torch.randint(0, in_dim, (out_dim,)), torch.randint(0, in_dim, (out_dim,))
+        idx1[:7] = idx0[:7]
+    gate = torch.randint(0, 16, (out_dim,), dtype=torch.uint8)
+    xd, a, b, g = torch.from_numpy(x).to(DEV), idx0.to(DEV), idx1.to(DEV), gate.to(DEV)
+    plan = difflogic_hip.eval_plan(a, b, in_dim)
+    assert sorted((plan.cpu() & 0x0FFFFFFF).tolist()) == list(range(out_dim))
+    got = difflogic_hip.eval_planned(xd, a, b, g, plan)
+    assert torch.equal(got, difflogic_hip.eval(xd, a, b, g))
+    assert np.array_equal(got.cpu().numpy(), O.eval_packed(x, idx0.numpy(), idx1.numpy(), gate.numpy()))
+
+
+def test_eval_plan_follows_in_place_rewiring():
+    torch.manual_seed(4)
+    layer = C.LogicLayer(40, 60, implementation="cuda").to(DEV).eval()
+    bits = torch.randint(0, 2, (2048, 40), device=DEV).bool()
+    y1 = layer(C.PackBitsTensor(bits, 64)).t.clone()
+    layer.indices_0.copy_(torch.randint(0, 40, (60,), device=DEV))      # as the reference tests rewire a layer
+    y2 = layer(C.PackBitsTensor(bits, 64)).t
+    words, _ = O.pack_bits(bits.cpu().numpy().T, 64)
+    want = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(),
+                         layer.weights.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(y2.cpu().numpy(), want) and not torch.equal(y1, y2)
