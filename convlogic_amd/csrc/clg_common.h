@@ -62,12 +62,13 @@ __device__ __forceinline__ float fma_t<float>(float a, float b, float c) { retur
 template <>
 __device__ __forceinline__ double fma_t<double>(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
-// Gate value in the folded form.  Always this instruction sequence, so equal inputs give equal
-// bits wherever it is evaluated (the pool argmax depends on that).
+// Gate value in the folded form, as three FMAs: a*(c_a + c_ab*b) + (c_b*b + c_1).  Always this
+// instruction sequence, so equal inputs give equal bits wherever it is evaluated (the pool argmax
+// depends on that).  With one-hot weights and binary inputs every intermediate is a small integer.
 template <typename T>
 __device__ __forceinline__ T gate(const Coef<T> &c, T a, T b)
 {
-    return fma_t(c.ab, a * b, fma_t(c.a, a, fma_t(c.b, b, c.one)));
+    return fma_t(a, fma_t(c.ab, b, c.a), fma_t(c.b, b, c.one));
 }
 template <typename T>
 __device__ __forceinline__ T gate_da(const Coef<T> &c, T b) { return fma_t(c.ab, b, c.a); }

@@ -20,6 +20,10 @@
 // pooled cell and accumulates the tap gradients of ITS channel into an LDS plane that only it
 // touches (the plane has the same shared-halo layout as the input image, so out-of-image taps fall
 // into halo elements that are never read back).  The order of additions is program order.
+#include <stdlib.h>
+
+#include <mutex>
+
 #include "conv_common.h"
 
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
@@ -31,6 +35,7 @@ int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
                                      hipStream_t st);
 int clg_convblock_partial_blocks(const Geom &g);
+int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name);
 
 namespace {
 
@@ -59,6 +64,7 @@ struct TilePlan {
     int rs, chs;        // row and plane stride of the LDS image (elements)
     int xe;             // elements of one LDS image region (S samples + tail)
     int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
+    int band_rows, bands;  // input gradient: image rows per workgroup band, number of bands
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp;
     size_t lds_bytes;
 };
@@ -195,25 +201,34 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
 //   hits   [cin][c]    those kernels in increasing order, entry = kernel | tap mask << 16
 // (the reverse map "input channel -> kernels and taps reading it", built in a fixed order).
 struct BwdScratch {
-    size_t folded_bytes, count_off, hits_off, total;
+    size_t folded_bytes, count_off, hits_off, taps_off, total;
 };
 BwdScratch bwd_scratch_layout(const Geom &g, int elem)
 {
     BwdScratch b;
     b.folded_bytes = (size_t)g.c * 28 * elem;
-    b.count_off = (b.folded_bytes + 15) & ~(size_t)15;
-    b.hits_off = (b.count_off + (size_t)g.cin * 4 + 15) & ~(size_t)15;
-    b.total = b.hits_off + (size_t)g.cin * g.c * 4;
+    b.count_off = (b.folded_bytes + 63) & ~(size_t)63;
+    b.hits_off = (b.count_off + (size_t)g.cin * 4 + 63) & ~(size_t)63;
+    b.taps_off = (b.hits_off + (size_t)g.cin * g.c * 4 + 63) & ~(size_t)63;
+    b.total = b.taps_off + (size_t)g.c * 16 * 4;                   // per kernel: 8 offsets inside the image, 8 inside the plane
     return b;
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
                                                               T *__restrict__ folded, int32_t *__restrict__ count,
-                                                              int32_t *__restrict__ hits, int C, int cin, int fold_blocks)
+                                                              int32_t *__restrict__ hits, int32_t *__restrict__ taps, int C,
+                                                              int cin, int fold_blocks, int rs, int chs)
 {
     if ((int)blockIdx.x < fold_blocks) {
         const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (q < (int64_t)C * 8) {                                   // tap offsets of the LDS window layout
+            const Tap tp = unpack_tap(sel[q]);
+            const int rel = tp.ry * rs + tp.rx;
+            const int64_t c = q >> 3, t = q & 7;
+            taps[c * 16 + t] = tp.ch * chs + rel;
+            taps[c * 16 + 8 + t] = rel;
+        }
         if (q < (int64_t)C * 7) {
             const Coef<T> cf = fold16(w + q * 16);
             folded[q * 4 + 0] = cf.ab;
@@ -253,33 +268,97 @@ struct CellLoads {
     int code[kChunk];
 };
 
-template <typename T>
+// Row band of the input image owned by one workgroup, the pooled cells whose taps can reach it and
+// the padded rows those cells read.  Identical arithmetic on host (LDS sizing) and device.
+struct Band {
+    int r0, r1;      // image rows [r0, r1) whose gradient this workgroup produces
+    int cell_lo, cb; // first pooled cell and number of pooled cells to visit
+    int R0, rows;    // first staged padded row and number of staged rows
+};
+__host__ __device__ inline Band make_band(const Geom &g, int band, int band_rows)
+{
+    Band b;
+    const int wp = g.wo / 2;
+    if (band_rows >= g.h) {                                         // one band: the whole image
+        b.r0 = 0; b.r1 = g.h; b.cell_lo = 0; b.cb = (g.ho / 2) * wp; b.R0 = 0; b.rows = g.h + 2 * g.ph;
+        return b;
+    }
+    b.r0 = band * band_rows;
+    b.r1 = b.r0 + band_rows < g.h ? b.r0 + band_rows : g.h;
+    const int num = b.r0 + g.ph - g.kh + 1;                       // smallest oy*sh that can reach row r0
+    int oy_lo = num <= 0 ? 0 : (num + g.sh - 1) / g.sh;
+    int oy_hi = (b.r1 + g.ph - 1) / g.sh;
+    if (oy_hi > g.ho - 1) oy_hi = g.ho - 1;
+    int R0 = b.r0 + g.ph, R1 = b.r1 + g.ph;                       // the window always holds the owned rows
+    b.cell_lo = 0;
+    b.cb = 0;
+    if (oy_lo <= oy_hi) {
+        const int py_lo = oy_lo / 2, py_hi = oy_hi / 2;
+        b.cell_lo = py_lo * wp;
+        b.cb = (py_hi - py_lo + 1) * wp;
+        const int t0 = 2 * py_lo * g.sh, t1 = (2 * py_hi + 1) * g.sh + g.kh;   // padded rows the cells read
+        if (t0 < R0) R0 = t0;
+        if (t1 > R1) R1 = t1;
+        if (R1 > g.h + 2 * g.ph) R1 = g.h + 2 * g.ph;
+    }
+    b.R0 = R0;
+    b.rows = R1 - R0;
+    return b;
+}
+
+// grid: (sample groups, bands).  LDS: input window xs, gradient window gs (same layout: planes of
+// `wrows` rows x rs elements, left halo shared with the previous row's right halo), cell table.
+template <typename T, bool BANDED>
 __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
                                                   const T *__restrict__ folded, const int32_t *__restrict__ count,
-                                                  const int32_t *__restrict__ hits, const int32_t *__restrict__ sel,
+                                                  const int32_t *__restrict__ hits, const int32_t *__restrict__ taps,
                                                   const uint8_t *__restrict__ argmax, T *__restrict__ gx, Geom g, TilePlan p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const int xe4 = (p.xe + 3) & ~3;
     T *xs = reinterpret_cast<T *>(smem);
-    T *gs = xs + xe4;                                               // gradient planes, same layout as xs
-    int2 *cellt = reinterpret_cast<int2 *>(gs + xe4);               // [G * slots]
+    T *gs = xs + xe4;
+    T *dummy = gs + xe4;                                            // one element per thread: sink of masked updates
+    int2 *cellt = reinterpret_cast<int2 *>(dummy + ((blockDim.x + 3) & ~3u));   // [G * cells of the band]
+    const int gs_off = xe4, dummy_off = 2 * xe4 + (int)threadIdx.x;
 
     const int tid = threadIdx.x, nthreads = blockDim.x;
     const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
     const int n0 = blockIdx.x * p.S, s_cur = min(p.S, g.n - n0);
     const int wp = g.wo >> 1, I = p.slots;
+    const Band bd = make_band(g, blockIdx.y, p.band_rows);
+    const int chs = p.chs;                                          // plane stride of the windows
 
-    for (int i = tid; i < 2 * xe4; i += nthreads) xs[i] = T(0);
-    const int V = p.G * I;                                          // lanes of one pass: G samples x I cells
+    for (int i = tid; i < 2 * xe4 + nthreads; i += nthreads) xs[i] = T(0);
+    const int V = p.G * bd.cb;                                      // lanes of one pass: G samples x band cells
     for (int v = tid; v < V; v += nthreads) {
-        const uint32_t s = fdiv(v, p.d_slots), cell = v - s * (uint32_t)I;
+        uint32_t s = 0, cl = v;
+        if (!BANDED) {
+            s = fdiv(v, p.d_slots);
+            cl = v - s * (uint32_t)I;
+        }
+        const uint32_t cell = bd.cell_lo + cl;
         const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
-        cellt[v] = make_int2((int)(s * g.cin * p.chs + (2 * py * g.sh) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
+        cellt[v] = make_int2((int)(s * g.cin * chs + (2 * py * g.sh - bd.R0) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
     }
     __syncthreads();
-    stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
+    // stage the image rows that fall into the window (padded row = image row + ph)
+    const int ir0 = bd.R0 - g.ph > 0 ? bd.R0 - g.ph : 0;
+    const int ir1 = bd.R0 + bd.rows - g.ph < g.h ? bd.R0 + bd.rows - g.ph : g.h;
+    const int irows = ir1 > ir0 ? ir1 - ir0 : 0;
+    const int planes = s_cur * g.cin;
+    const T *src = x + (int64_t)n0 * g.cin * g.h * g.w;
+    for (int pr = wave; pr < planes * irows; pr += p.NW) {
+        const int plane = uniform(pr / irows), iy = ir0 + (pr - plane * irows);
+        const T *row = src + ((int64_t)plane * g.h + iy) * g.w;
+        T *dst = xs + plane * chs + (iy + g.ph - bd.R0) * p.rs + g.pw;
+        for (int ix = lane; ix < g.w; ix += kWave) dst[ix] = row[ix];
+    }
     __syncthreads();
+
+    // plane-relative range of elements this workgroup owns (rows r0..r1-1 of every plane)
+    const uint32_t own_lo = (uint32_t)((bd.r0 + g.ph - bd.R0) * p.rs);
+    const uint32_t own_len = (uint32_t)((bd.r1 - bd.r0) * p.rs);
 
     // work items: (group of G samples, input channel); a wavefront owns the gradient planes of its item
     const int groups = (s_cur + p.G - 1) / p.G;
@@ -288,16 +367,14 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     for (int item = wave; item < items; item += p.NW) {
         const int grp = item / g.cin, ch = item - grp * g.cin;
         const int s0 = grp * p.G;
-        const int v_here = min(p.G, s_cur - s0) * I;
+        const int v_here = min(p.G, s_cur - s0) * bd.cb;
         const int chunks = (v_here + kChunk * kWave - 1) / (kChunk * kWave);
-        const int img0 = s0 * g.cin * p.chs;                        // LDS offset of the group's first plane
+        const int img0 = s0 * g.cin * chs;                          // LDS offset of the group's first plane
         const int64_t gbase = ((int64_t)(n0 + s0) * g.c) * I;       // global offset of the group's first cell row
-        const int nhits = count[ch];
+        const int nhits = v_here > 0 ? count[ch] : 0;
         const int32_t *hit = hits + (int64_t)ch * g.c;
-        const int steps = nhits * chunks;                           // step = (hit, chunk), hit-major
-
-        auto issue = [&](int step, CellLoads<T> &L) {
-            const int k = step / chunks, chunk = step - k * chunks;
+        // loads of grad_y and the argmax code for (hit k, chunk): issued one step ahead of their use
+        auto issue = [&](int k, int chunk, CellLoads<T> &L) {
             const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
 #pragma unroll
             for (int j = 0; j < kChunk; ++j) {
@@ -313,38 +390,39 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
         };
 
         CellLoads<T> cur, nxt;
-        if (steps > 0) issue(0, cur);
-        for (int step = 0; step < steps; ++step) {
-            if (step + 1 < steps) issue(step + 1, nxt);
-            const int k = step / chunks, chunk = step - k * chunks;
+        if (nhits > 0) issue(0, 0, cur);
+        for (int k = 0; k < nhits; ++k) {
             const int ent = hit[k];
             const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
-            int to[8];
+            int to[8];                                              // tap offsets inside the group's planes
+            int tr_[8];                                             // the same, relative to the tap's own plane
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                const Tap tp = unpack_tap(sel[c * 8 + t]);
-                to[t] = tp.ch * p.chs + tp.ry * p.rs + tp.rx;
+                to[t] = taps[c * 16 + t];
+                tr_[t] = taps[c * 16 + 8 + t];
             }
             Tree<T> tr;
             const T *fc = folded + (int64_t)c * 28;
 #pragma unroll
             for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
-            // phase 1: tree and tap gradients of every cell block of this chunk (registers only)
-            int pos[kChunk];
-            bool live[kChunk];
-            T gt[kChunk][8];
+            for (int chunk = 0; chunk < chunks; ++chunk) {
+                if (chunk + 1 < chunks) issue(k, chunk + 1, nxt);
+                else if (k + 1 < nhits) issue(k + 1, 0, nxt);
+                // phase 1: tree and tap gradients of every cell block of this chunk (registers only).
+                // No per-lane control flow: a lane without a cell recomputes cell 0 with a zero gradient.
+                int pos[kChunk];
+                bool live[kChunk];
+                T gt[kChunk][8];
 #pragma unroll
-            for (int j = 0; j < kChunk; ++j) {
-                const int v = (chunk * kChunk + j) * kWave + lane;
-                live[j] = v < v_here;
-                pos[j] = 0;
-                if (live[j]) {
+                for (int j = 0; j < kChunk; ++j) {
+                    const int v = (chunk * kChunk + j) * kWave + lane;
+                    live[j] = v < v_here;
                     const int code = cur.code[j];
-                    const T gout = cur.gy[j];
-                    pos[j] = img0 + cellt[v].x + (code >> 1) * row_step + (code & 1) * g.sw;
+                    const T gout = cur.gy[j];                       // 0 for lanes without a cell
+                    pos[j] = cellt[live[j] ? v : 0].x + (code >> 1) * row_step + (code & 1) * g.sw;
                     T tv[8];
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) tv[t] = xs[pos[j] + to[t]];
+                    for (int t = 0; t < 8; ++t) tv[t] = xs[img0 + pos[j] + to[t]];
                     const TreeVals<T> tvv = eval_tree(tr, tv);
                     const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
                     const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
@@ -360,33 +438,175 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
                         }
                     }
                 }
-            }
-            // phase 2: read-add-write per tap.  For one tap the targets of all cells (all lanes, all
-            // blocks) are distinct elements, so the blocks of a chunk go together; taps may collide
-            // with each other and are applied one after the other.  Only this wavefront touches the plane.
+                // phase 2: read-add-write per tap.  For one tap the targets of all cells (all lanes,
+                // all blocks) are distinct elements, so the blocks of a chunk go together; taps may
+                // collide with each other and are applied one after the other.  Only this wavefront
+                // touches the plane rows it owns.  Lanes without a cell, and (with bands) targets
+                // outside the owned rows, are redirected to a private dummy element per lane, so the
+                // whole phase is straight-line code with the LDS reads of a tap in flight together.
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                if ((mask >> t) & 1) {                               // wave-uniform
-                    T old[kChunk];
+                for (int t = 0; t < 8; ++t) {
+                    if ((mask >> t) & 1) {                           // wave-uniform
+                        T old[kChunk];
+                        int at[kChunk];
 #pragma unroll
-                    for (int j = 0; j < kChunk; ++j)
-                        if (live[j]) old[j] = gs[pos[j] + to[t]];
+                        for (int j = 0; j < kChunk; ++j) {
+                            bool mine = live[j];
+                            if (BANDED) mine = mine && ((uint32_t)(pos[j] + tr_[t]) - own_lo) < own_len;
+                            at[j] = mine ? gs_off + img0 + pos[j] + to[t] : dummy_off;
+                        }
 #pragma unroll
-                    for (int j = 0; j < kChunk; ++j)
-                        if (live[j]) gs[pos[j] + to[t]] = old[j] + gt[j][t];
+                        for (int j = 0; j < kChunk; ++j) old[j] = xs[at[j]];
+#pragma unroll
+                        for (int j = 0; j < kChunk; ++j) xs[at[j]] = old[j] + gt[j][t];
+                    }
                 }
+                cur = nxt;
             }
-            cur = nxt;
         }
     }
     __syncthreads();
-    // write the gradient planes of the staged samples back (interior elements only)
-    const uint32_t total = (uint32_t)s_cur * g.cin * g.h * g.w;
-    T *dst = gx + (int64_t)n0 * g.cin * g.h * g.w;
-    for (uint32_t e = tid; e < total; e += nthreads) {
-        const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)(g.h * g.w);
-        const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
-        dst[e] = gs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw];
+    // write the owned rows of the gradient planes back
+    const int orows = bd.r1 - bd.r0;
+    T *dstg = gx + (int64_t)n0 * g.cin * g.h * g.w;
+    for (int pr = wave; pr < planes * orows; pr += p.NW) {
+        const int plane = uniform(pr / orows), iy = bd.r0 + (pr - plane * orows);
+        const T *row = gs + plane * chs + (iy + g.ph - bd.R0) * p.rs + g.pw;
+        T *dst = dstg + ((int64_t)plane * g.h + iy) * g.w;
+        for (int ix = lane; ix < g.w; ix += kWave) dst[ix] = row[ix];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// weight gradient
+// ---------------------------------------------------------------------------------------------
+// Workgroup = (column of sample groups, CT kernels); it walks its sample groups (stage S samples in
+// LDS, barrier) and every wavefront keeps the 28 partial sums (7 gates x (ab, a, b, 1)) of its
+// kKPW kernels in registers across ALL of them, so the cross-lane reduction happens once per kernel
+// and workgroup.  partial [c][gridDim.x][28] is summed in a fixed order by reduce_coef_partials.
+constexpr int kKPW = 2;  // kernels per wavefront
+
+template <typename T>
+__global__ void convblock_backward_w_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x, const T *__restrict__ w,
+                                                  const int32_t *__restrict__ sel, const uint8_t *__restrict__ argmax,
+                                                  T *__restrict__ partial, Geom g, TilePlan p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *xs = reinterpret_cast<T *>(smem);
+    T *coef = xs + ((p.xe + 3) & ~3);                                 // [CT][28]
+    int *toff = reinterpret_cast<int *>(coef + p.CT * 28);            // [CT][8]
+    int2 *cellt = reinterpret_cast<int2 *>(toff + p.CT * 8);          // [S * cells]
+
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
+    const int c0 = blockIdx.y * p.CT, ct_cur = min(p.CT, g.c - c0);
+    const int wp = g.wo >> 1, I = p.slots;
+
+    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
+    for (int q = tid; q < ct_cur * 7; q += nthreads) {
+        const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
+        coef[q * 4 + 0] = cf.ab;
+        coef[q * 4 + 1] = cf.a;
+        coef[q * 4 + 2] = cf.b;
+        coef[q * 4 + 3] = cf.one;
+    }
+    for (int q = tid; q < ct_cur * 8; q += nthreads) {
+        const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
+        toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
+    }
+    for (int v = tid; v < p.S * I; v += nthreads) {
+        const uint32_t s = fdiv(v, p.d_slots), cell = v - s * (uint32_t)I;
+        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+        cellt[v] = make_int2((int)(s * g.cin * p.chs + (2 * py * g.sh) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
+    }
+
+    T acc[kKPW][28];
+#pragma unroll
+    for (int kk = 0; kk < kKPW; ++kk)
+#pragma unroll
+        for (int i = 0; i < 28; ++i) acc[kk][i] = T(0);
+
+    const int row_step = g.sh * p.rs;
+    const int ngroups = (g.n + p.S - 1) / p.S;
+    for (int grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+        const int n0 = grp * p.S, s_cur = min(p.S, g.n - n0);
+        __syncthreads();                                             // everyone is done with the previous image
+        stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
+        __syncthreads();
+        const int V = s_cur * I;
+#pragma unroll
+        for (int kk = 0; kk < kKPW; ++kk) {
+            const int lc = wave * kKPW + kk;
+            if (lc >= ct_cur) break;                                 // wave-uniform
+            Tree<T> tr;
+#pragma unroll
+            for (int k = 0; k < 7; ++k) {
+                tr.g[k].ab = to_sgpr(coef[(lc * 7 + k) * 4 + 0]);
+                tr.g[k].a = to_sgpr(coef[(lc * 7 + k) * 4 + 1]);
+                tr.g[k].b = to_sgpr(coef[(lc * 7 + k) * 4 + 2]);
+                tr.g[k].one = to_sgpr(coef[(lc * 7 + k) * 4 + 3]);
+            }
+            int to[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) to[t] = uniform(toff[lc * 8 + t]);
+            const int64_t crow = ((int64_t)n0 * g.c + c0 + lc) * I;
+            const uint8_t *am = argmax + crow;
+            const T *gr = gy + crow;
+            // grad_y / argmax of the next cell block are requested before the current one is used
+            int2 e = cellt[lane < V ? lane : 0];
+            int code = lane < V ? am[e.y] : 0;
+            T gout = lane < V ? gr[e.y] : T(0);
+            for (int v0 = 0; v0 < V; v0 += kWave) {
+                const int vn = v0 + kWave + lane;
+                const int2 en = cellt[vn < V ? vn : 0];
+                const int code_n = vn < V ? am[en.y] : 0;
+                const T gout_n = vn < V ? gr[en.y] : T(0);
+                const int pos = e.x + (code >> 1) * row_step + (code & 1) * g.sw;
+                T tv[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) tv[t] = xs[pos + to[t]];
+                const TreeVals<T> v = eval_tree(tr, tv);
+                T gin[7][2], gg[7];
+                gg[6] = gout;
+                gin[6][0] = v.mid[0];
+                gin[6][1] = v.mid[1];
+                gg[4] = gout * gate_da(tr.g[6], v.mid[1]);
+                gg[5] = gout * gate_db(tr.g[6], v.mid[0]);
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    gin[4 + m][0] = v.leaf[2 * m];
+                    gin[4 + m][1] = v.leaf[2 * m + 1];
+                    gg[2 * m] = gg[4 + m] * gate_da(tr.g[4 + m], v.leaf[2 * m + 1]);
+                    gg[2 * m + 1] = gg[4 + m] * gate_db(tr.g[4 + m], v.leaf[2 * m]);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    gin[q][0] = tv[2 * q];
+                    gin[q][1] = tv[2 * q + 1];
+                }
+#pragma unroll
+                for (int k = 0; k < 7; ++k) {
+                    acc[kk][4 * k + 0] = fma_t(gg[k], gin[k][0] * gin[k][1], acc[kk][4 * k + 0]);
+                    acc[kk][4 * k + 1] = fma_t(gg[k], gin[k][0], acc[kk][4 * k + 1]);
+                    acc[kk][4 * k + 2] = fma_t(gg[k], gin[k][1], acc[kk][4 * k + 2]);
+                    acc[kk][4 * k + 3] += gg[k];
+                }
+                e = en;
+                code = code_n;
+                gout = gout_n;
+            }
+        }
+    }
+#pragma unroll
+    for (int kk = 0; kk < kKPW; ++kk) {
+        const int lc = wave * kKPW + kk;
+        if (lc >= ct_cur) break;
+        T *dst = partial + ((int64_t)(c0 + lc) * gridDim.x + blockIdx.x) * 28;
+#pragma unroll
+        for (int i = 0; i < 28; ++i) {
+            const T sum = wave_sum(acc[kk][i]);
+            if (lane == 0) dst[i] = sum;
+        }
     }
 }
 
@@ -441,39 +661,125 @@ bool plan_forward(const Geom &g, int elem, TilePlan *p)
 
 bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
 {
-    if (!taps_inside(g)) return false;
+    if (!taps_inside(g) || g.c > 65535) return false;
     plan_common(g, p);
     const int I = (g.ho / 2) * (g.wo / 2);
     p->slots = I;
     p->CT = 0;
-    // G samples share a wavefront pass when a sample has fewer than 64 cells
+    p->d_slots = make_fastdiv((uint32_t)I);
+    p->NW = g.cin < 16 ? g.cin : 16;
+    auto size_for = [&](int G, int band_rows, int *rows_max, int *cb_max) {
+        const int bands = (int)clg_ceil_div(g.h, band_rows);
+        *rows_max = 0;
+        *cb_max = 0;
+        for (int b = 0; b < bands; ++b) {
+            const Band bd = make_band(g, b, band_rows);
+            if (bd.rows > *rows_max) *rows_max = bd.rows;
+            if (bd.cb > *cb_max) *cb_max = bd.cb;
+        }
+        const int64_t xe = (int64_t)G * g.cin * *rows_max * p->rs + g.pw;
+        return (int64_t)2 * ((xe + 3) & ~3) * elem + (int64_t)p->NW * kWave * elem + (int64_t)G * *cb_max * 8;
+    };
+    // samples sharing a wavefront pass when a sample has fewer than 64 cells (whole image, one band)
     int G = I >= kWave ? 1 : kWave / I;
     if (G > g.n) G = g.n;
-    // shrink G until two image regions fit
-    while (G > 1 && 2 * ((image_elems(g, *p, G) + 3) & ~3) * elem + (int64_t)G * I * 8 > kLdsLimit) G /= 2;
+    int rows_max, cb_max;
+    while (G > 1 && size_for(G, g.h, &rows_max, &cb_max) > kLdsLimit) G /= 2;
+    int band_rows = g.h;
+    if (G == 1) {
+        // One band (the whole image) unless it does not fit: the time of this kernel is set by the
+        // dependent chain of steps per visited kernel, which every band would repeat (measured: bands
+        // never paid off, not even at 256 wavefronts in flight).  CLG_BWDX_BANDS overrides for tuning.
+        const char *e_b = getenv("CLG_BWDX_BANDS");
+        int64_t want = e_b ? atoi(e_b) : 1;
+        if (want > g.h / 4) want = g.h / 4;
+        if (want < 1) want = 1;
+        band_rows = (int)clg_ceil_div(g.h, want);
+        // whole images that do not fit are split further until a band window fits
+        while (band_rows > 1 && size_for(1, band_rows, &rows_max, &cb_max) > kLdsLimit) band_rows = (band_rows + 1) / 2;
+    }
+    const int64_t bytes = size_for(G, band_rows, &rows_max, &cb_max);
+    if (bytes > kLdsLimit) return false;
     p->G = G;
     p->S = G;
-    p->xe = (int)image_elems(g, *p, p->S);
-    p->lds_bytes = (size_t)2 * ((p->xe + 3) & ~3) * elem + (size_t)G * I * 8;
-    if (p->lds_bytes > (size_t)kLdsLimit) return false;
-    if ((double)(G * I) / (double)(clg_ceil_div(G * I, kWave) * kWave) < 0.2) return false;
-    const int items = g.cin;                                         // one group per workgroup
-    p->NW = items < 16 ? items : 16;
-    p->d_slots = make_fastdiv((uint32_t)I);
+    p->band_rows = band_rows;
+    p->bands = (int)clg_ceil_div(g.h, band_rows);
+    p->chs = rows_max * p->rs;
+    p->xe = (int)((int64_t)G * g.cin * p->chs + g.pw);
+    p->lds_bytes = (size_t)bytes;
+    if (p->bands > 65535) return false;
+    if (G * I < kWave / 5 && p->bands == 1) return false;            // almost empty wavefronts: gather kernel instead
     return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * I < (1ll << 31);
 }
 
+// weight gradient: S samples per staging round, CT = kKPW * NW kernels per workgroup, `cols` columns
+// of sample groups (= partial sums per kernel)
+bool plan_backward_w(const Geom &g, int elem, TilePlan *p, int *cols)
+{
+    if (!taps_inside(g) || g.c > 65535 * 8) return false;
+    plan_common(g, p);
+    const int I = (g.ho / 2) * (g.wo / 2);
+    // below about 8M pooled values the kernel that reads taps from global memory has more wavefronts in
+    // flight and wins (measured 26 vs 41 us at 1.6M, 125 vs 109 us at 16.8M)
+    if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_TILED")) return false;
+    p->slots = I;
+    p->G = 1;
+    p->d_slots = make_fastdiv((uint32_t)I);
+    // samples per round: enough cells for full wavefronts, image region up to 64 KiB
+    int S = 1;
+    while (S < g.n && S * I < 4 * kWave && (image_elems(g, *p, 2 * S) * elem + (int64_t)2 * S * I * 8) <= 64 * 1024) S *= 2;
+    p->S = S;
+    p->xe = (int)image_elems(g, *p, S);
+    const int64_t groups = clg_ceil_div(g.n, S);
+    // wavefronts per workgroup: as many as give every wavefront kernels to work on, up to 8
+    int nw = (int)clg_ceil_div(g.c, kKPW);
+    if (nw > 8) nw = 8;
+    p->NW = nw;
+    p->CT = nw * kKPW;
+    const int64_t tiles = clg_ceil_div(g.c, p->CT);
+    // columns: fill the GPU about twice, at least 4 staging rounds per workgroup where possible
+    const char *e_cols = getenv("CLG_BWDW_COLS");
+    int64_t c_ = e_cols ? atoi(e_cols) : clg_ceil_div(1024, tiles);
+    if (c_ > groups) c_ = groups;
+    if (c_ > 32) c_ = 32;
+    if (c_ < 1) c_ = 1;
+    *cols = (int)c_;
+    p->lds_bytes = (size_t)((p->xe + 3) & ~3) * elem + (size_t)p->CT * 28 * elem + (size_t)p->CT * 8 * 4 + (size_t)S * I * 8;
+    if (p->lds_bytes > (size_t)kLdsLimit || tiles > 65535) return false;
+    if ((double)(S * I) / (double)(clg_ceil_div((int64_t)S * I, kWave) * kWave) < 0.4) return false;
+    return (int64_t)S * g.cin * p->chs < (1ll << 30) && (int64_t)S * g.c * I < (1ll << 31);
+}
+
+// Kernels that want more than 48 KiB of dynamic LDS must be told once; the largest size granted so
+// far is remembered per kernel so that steady-state launches make no runtime call besides the launch.
+int allow_lds_ptr(const void *kernel, size_t bytes, const char *name)
+{
+    static std::mutex mu;
+    static const void *known[32];
+    static size_t granted[32];
+    static int used = 0;
+    if (bytes <= 48 * 1024) return CLG_OK;
+    std::lock_guard<std::mutex> lock(mu);
+    int slot = -1;
+    for (int i = 0; i < used; ++i)
+        if (known[i] == kernel) slot = i;
+    if (slot >= 0 && granted[slot] >= bytes) return CLG_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+        return CLG_ELAUNCH;
+    }
+    if (slot < 0 && used < 32) slot = used++;
+    if (slot >= 0) {
+        known[slot] = kernel;
+        granted[slot] = bytes;
+    }
+    return CLG_OK;
+}
 template <typename K>
 int allow_lds(K kernel, size_t bytes, const char *name)
 {
-    if (bytes > 48 * 1024) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-        if (e != hipSuccess) {
-            clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
-            return CLG_ELAUNCH;
-        }
-    }
-    return CLG_OK;
+    return allow_lds_ptr(reinterpret_cast<const void *>(kernel), bytes, name);
 }
 
 template <typename T>
@@ -496,16 +802,35 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     T *folded = reinterpret_cast<T *>(scratch);
     int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
     int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
-    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 7, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
+    int32_t *taps = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.taps_off);
+    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
     hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
-                       folded, count, hits, g.c, g.cin, fold_blocks);
+                       folded, count, hits, taps, g.c, g.cin, fold_blocks, p.rs, p.chs);
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
-    if (int e = allow_lds(convblock_backward_x_tiled_kernel<T>, p.lds_bytes, "clg_convblock_backward_x")) return e;
-    hipLaunchKernelGGL(convblock_backward_x_tiled_kernel<T>, dim3((unsigned)clg_ceil_div(g.n, p.S)), dim3(p.NW * kWave), p.lds_bytes, st,
-                       (const T *)gy, (const T *)x, (const T *)folded, (const int32_t *)count, (const int32_t *)hits, sel, argmax,
-                       (T *)gx, g, p);
+    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands), block(p.NW * kWave);
+    if (p.bands > 1) {
+        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, true>, p.lds_bytes, "clg_convblock_backward_x")) return e;
+        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, true>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
+                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, (T *)gx, g, p);
+    } else {
+        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, false>, p.lds_bytes, "clg_convblock_backward_x")) return e;
+        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, false>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
+                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, (T *)gx, g, p);
+    }
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(tiled)");
     return CLG_OK;
+}
+
+template <typename T>
+int launch_backward_w_tiled(const Geom &g, const TilePlan &p, int cols, const void *gy, const void *x, const void *w,
+                            const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st)
+{
+    if (int e = allow_lds(convblock_backward_w_tiled_kernel<T>, p.lds_bytes, "clg_convblock_backward_w")) return e;
+    const dim3 grid((unsigned)cols, (unsigned)clg_ceil_div(g.c, p.CT));
+    hipLaunchKernelGGL(convblock_backward_w_tiled_kernel<T>, grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)gy, (const T *)x,
+                       (const T *)w, sel, argmax, (T *)scratch, g, p);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(tiled)");
+    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, scratch, gw, g.c, cols, 7, st, "clg_convblock_backward_w(reduce)");
 }
 
 int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
@@ -553,7 +878,10 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
 {
     Geom g;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w_scratch_bytes")) return -1;
-    return (int64_t)g.c * clg_convblock_partial_blocks(g) * 28 * elem_size(dtype);
+    // enough for either kernel: partial sums [c][blocks][28] with at most 64 blocks per kernel
+    int64_t nb = clg_convblock_partial_blocks(g);
+    if (nb < 64) nb = 64;
+    return (int64_t)g.c * nb * 28 * elem_size(dtype);
 }
 
 extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -563,5 +891,13 @@ extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, cons
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w")) return e;
     CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "clg_convblock_backward_w: null pointer argument");
+    TilePlan p;
+    int cols = 1;
+    const char *e_tiled = getenv("CLG_BWDW_TILED");
+    if ((!e_tiled || atoi(e_tiled) != 0) && plan_backward_w(g, elem_size(dtype), &p, &cols)) {
+        if (dtype == CLG_F32)
+            return launch_backward_w_tiled<float>(g, p, cols, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+        return launch_backward_w_tiled<double>(g, p, cols, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+    }
     return clg_convblock_backward_w_generic(dtype, g, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
 }

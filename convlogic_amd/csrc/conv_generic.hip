@@ -479,6 +479,11 @@ extern "C" int clg_tree_backward_w(int dtype, const void *grad_y, const void *x,
     CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, c * xo, nb, 1, st, "clg_tree_backward_w(reduce)"));
 }
 
+int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name)
+{
+    CLG_DISPATCH(dtype, return launch_reduce<T>(partial, out, rows, nb, G, st, name));
+}
+
 // ---- fused block, generic entry points (called from conv_block.hip when no tiled kernel applies) ----
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name)
 {

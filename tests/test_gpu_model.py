@@ -1,0 +1,120 @@
+"""BASELINE config 5 as a parity case: the conv-logic network topology (4 fused blocks, flatten, 3
+LogicLayers, GroupSum; src/convlogic/model.py:16-58 with k=32, 9 input channels) built from this
+package's layers, one training step and the packed-bit evaluation of the fully connected tail against
+the CPU oracle at a reduced batch."""
+import numpy as np
+import pytest
+import torch
+
+import convlogic_amd as C
+from oracle import convlogic_oracle as O
+from tests.gpu_util import DEV, assert_grad_close
+
+pytestmark = pytest.mark.gpu
+
+
+def build(k=32, cin=9, size=32, tau=6.5):
+    chans = [cin, k, 4 * k, 16 * k, 32 * k]
+    layers = [C.ConvLogicLayer(a, b, padding=1, complete=True, implementation="cuda") for a, b in zip(chans[:-1], chans[1:])]
+    flat = chans[-1] * (size // 16) ** 2
+    dims = [flat, flat * 10, flat * 5, (flat * 10) // 4]
+    layers.append(torch.nn.Flatten())
+    layers += [C.LogicLayer(a, b, implementation="cuda") for a, b in zip(dims[:-1], dims[1:])]
+    layers.append(C.GroupSum(10, tau))
+    return torch.nn.Sequential(*layers)
+
+
+def oracle_forward(model, x, training=True):
+    h = x
+    for m in model:
+        if isinstance(m, C.ConvLogicLayer):
+            h = O.conv_block_forward(h, O.gate_weights(m.weights.detach().cpu() if not training else m._w, training, h.dtype),
+                                     m.selection.cpu(), (1, 1), (1, 1), (3, 3))
+        elif isinstance(m, torch.nn.Flatten):
+            h = h.flatten(1)
+        elif isinstance(m, C.LogicLayer):
+            h = O.logic_fc_forward(h, m.indices_0.cpu(), m.indices_1.cpu(),
+                                   O.gate_weights(m.weights.detach().cpu() if not training else m._w, training, h.dtype))
+        else:
+            h = O.group_sum(h, m.k, m.tau)
+    return h
+
+
+def test_config5_training_step_matches_oracle():
+    # float64 on both sides: through 7 layers of random-init gates the first-layer gradient is ~1e-10 of
+    # the last one, and in float32 a single near-tie in a pooling window decides its leading digits
+    torch.manual_seed(0)
+    model = build().double().to(DEV)
+    n = 4
+    v = (torch.randn(n, 3, 32, 32, dtype=torch.float64) * 0.25 + 0.5).clamp(0, 1)
+    x = torch.cat([(v > t).double() for t in (0.25, 0.5, 0.75)], dim=1)
+    labels = torch.randint(0, 10, (n,))
+    xg = x.to(DEV).requires_grad_(True)
+    logits = model(xg)
+    assert logits.shape == (n, 10)
+    loss = torch.nn.functional.cross_entropy(logits, labels.to(DEV))
+    loss.backward()
+
+    params = [m for m in model if hasattr(m, "weights")]
+    for m in params:
+        m._w = m.weights.detach().cpu().clone().requires_grad_(True)
+    xc = x.clone().requires_grad_(True)
+    ref = oracle_forward(model, xc)
+    ref_loss = torch.nn.functional.cross_entropy(ref, labels)
+    ref_loss.backward()
+    assert (logits.detach().cpu() - ref.detach()).abs().max().item() <= 1e-9
+    assert abs(loss.item() - ref_loss.item()) <= 1e-10
+    for i, m in enumerate(params):
+        assert_grad_close(m.weights.grad, m._w.grad, rel=1e-6, name=f"layer {i} grad_logits")
+    assert_grad_close(xg.grad, xc.grad, rel=1e-6, name="grad_x")
+
+
+def test_config5_training_step_float32_runs_and_is_deterministic():
+    torch.manual_seed(2)
+    model = build().to(DEV)
+    x = torch.randint(0, 2, (8, 9, 32, 32), device=DEV).float()
+    labels = torch.randint(0, 10, (8,), device=DEV)
+
+    def step():
+        for m in model:
+            if hasattr(m, "weights"):
+                m.weights.grad = None
+        loss = torch.nn.functional.cross_entropy(model(x), labels)
+        loss.backward()
+        return loss.detach().clone(), [m.weights.grad.clone() for m in model if hasattr(m, "weights")]
+
+    l1, g1 = step()
+    l2, g2 = step()
+    assert torch.equal(l1, l2) and all(torch.equal(a, b) for a, b in zip(g1, g2))
+    assert all(torch.isfinite(g).all() for g in g1)
+
+
+def test_config5_eval_float_and_packed_tail():
+    torch.manual_seed(1)
+    model = build().to(DEV).eval()
+    n = 96
+    x = torch.randint(0, 2, (n, 9, 32, 32), device=DEV).float()
+    with torch.no_grad():
+        feats = x
+        for m in list(model)[:5]:
+            feats = m(feats)                       # 4 blocks + flatten, float eval path: exactly binary
+        assert torch.all((feats == 0) | (feats == 1))
+        y_float = feats
+        for m in list(model)[5:]:
+            y_float = m(y_float)
+        p = C.PackBitsTensor(feats.bool(), 64)
+        for m in list(model)[5:]:
+            p = m(p)
+    assert p.dtype == torch.int32 and p.shape == (n, 10)
+    assert torch.equal(p.float() / 6.5, y_float)
+    assert torch.equal(p.float(), torch.round(y_float * 6.5))
+    # against the oracle: float eval of the whole network on the CPU
+    ref = oracle_forward(model, x.cpu(), training=False)
+    # identical counts; torch divides by tau with a reciprocal on the GPU (1 ulp from the CPU division)
+    assert torch.equal(torch.round(y_float.cpu() * 6.5), torch.round(ref * 6.5))
+    assert torch.allclose(y_float.cpu(), ref, rtol=3e-7, atol=0)
+    words, pad = O.pack_bits(feats.cpu().numpy().T.astype(bool), 64)
+    for m in list(model)[5:8]:
+        words = O.eval_packed(words, m.indices_0.cpu().numpy(), m.indices_1.cpu().numpy(),
+                              m.weights.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(O.group_bit_sum(words, pad, 10), p.cpu().numpy())
