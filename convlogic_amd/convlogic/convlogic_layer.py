@@ -62,9 +62,11 @@ class FullConvLogicFunction(Function):
         grad_y = grad_y.contiguous()
         x1, w_prob, selection, argmax = ctx.saved_tensors
         grad_x = grad_w = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
+            grad_x, grad_w = convlogic_hip.full_convlogic_backward(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
+        elif ctx.needs_input_grad[0]:
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
-        if ctx.needs_input_grad[1]:
+        elif ctx.needs_input_grad[1]:
             grad_w = convlogic_hip.full_convlogic_backward_weight(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
         return grad_x, grad_w, None, None, None, None, None, None, None, None, None
 

@@ -111,7 +111,9 @@ __device__ __forceinline__ void stage_image(T *__restrict__ xs, const T *__restr
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
-template <typename T>
+// ROWSTEP: elements between conv rows 2r and 2r+1 in the LDS image when known at compile time (the
+// second row's reads then use the immediate offset of the LDS instruction), 0 = read it from the plan.
+template <typename T, int ROWSTEP>
 __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ sel,
                                                T *__restrict__ y, uint8_t *__restrict__ argmax, Geom g, TilePlan p)
 {
@@ -149,7 +151,7 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
     stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
     __syncthreads();
 
-    const int row_step = g.sh * p.rs;
+    const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
     for (int lc = wave; lc < ct_cur; lc += p.NW) {
         Tree<T> tr;
 #pragma unroll
@@ -782,16 +784,32 @@ int allow_lds(K kernel, size_t bytes, const char *name)
     return allow_lds_ptr(reinterpret_cast<const void *>(kernel), bytes, name);
 }
 
+template <typename T, int ROWSTEP>
+int launch_forward_tiled_rs(const Geom &g, const TilePlan &p, const void *x, const void *w, const int32_t *sel, void *y,
+                            uint8_t *argmax, hipStream_t st)
+{
+    if (int e = allow_lds(convblock_forward_tiled_kernel<T, ROWSTEP>, p.lds_bytes, "clg_convblock_forward")) return e;
+    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
+    hipLaunchKernelGGL((convblock_forward_tiled_kernel<T, ROWSTEP>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
+                       (const T *)w, sel, (T *)y, argmax, g, p);
+    CLG_CHECK_LAUNCH("clg_convblock_forward(tiled)");
+    return CLG_OK;
+}
+
+// Row steps of 3x3 / padding 1 / stride 1 blocks on 32, 28, 16, 8 and 4 pixel wide images get their own
+// instantiation; everything else reads the step from the plan.
 template <typename T>
 int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const void *w, const int32_t *sel, void *y,
                          uint8_t *argmax, hipStream_t st)
 {
-    if (int e = allow_lds(convblock_forward_tiled_kernel<T>, p.lds_bytes, "clg_convblock_forward")) return e;
-    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
-    hipLaunchKernelGGL(convblock_forward_tiled_kernel<T>, grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x, (const T *)w, sel,
-                       (T *)y, argmax, g, p);
-    CLG_CHECK_LAUNCH("clg_convblock_forward(tiled)");
-    return CLG_OK;
+    switch (g.sh * p.rs) {
+    case 33: return launch_forward_tiled_rs<T, 33>(g, p, x, w, sel, y, argmax, st);
+    case 29: return launch_forward_tiled_rs<T, 29>(g, p, x, w, sel, y, argmax, st);
+    case 17: return launch_forward_tiled_rs<T, 17>(g, p, x, w, sel, y, argmax, st);
+    case 9: return launch_forward_tiled_rs<T, 9>(g, p, x, w, sel, y, argmax, st);
+    case 5: return launch_forward_tiled_rs<T, 5>(g, p, x, w, sel, y, argmax, st);
+    default: return launch_forward_tiled_rs<T, 0>(g, p, x, w, sel, y, argmax, st);
+    }
 }
 
 template <typename T>
@@ -900,4 +918,23 @@ extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, cons
         return launch_backward_w_tiled<double>(g, p, cols, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
     }
     return clg_convblock_backward_w_generic(dtype, g, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+}
+
+extern "C" int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *gg)
+{
+    const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg), b = clg_convblock_backward_w_scratch_bytes(dtype, gg);
+    if (a < 0 || b < 0) return -1;
+    return ((a + 255) & ~255ll) + b;
+}
+
+extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                      const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w, void *scratch,
+                                      void *stream)
+{
+    CLG_REQUIRE(scratch, "clg_convblock_backward: null pointer argument");
+    const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
+    if (a < 0) return CLG_EINVAL;
+    if (int e = clg_convblock_backward_x(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream)) return e;
+    return clg_convblock_backward_w(dtype, gg, grad_y, x, w, selection, argmax, grad_w,
+                                    reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream);
 }

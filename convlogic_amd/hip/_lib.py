@@ -52,6 +52,8 @@ SIGNATURES = {
     "clg_convblock_backward_x_scratch_bytes": (_i64, [_i, _GP]),
     "clg_convblock_backward_w": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_w_scratch_bytes": (_i64, [_i, _GP]),
+    "clg_convblock_backward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_backward_scratch_bytes": (_i64, [_i, _GP]),
 }
 
 _lib = None

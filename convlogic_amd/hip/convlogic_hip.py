@@ -187,3 +187,19 @@ def full_convlogic_backward_weight(grad_y, x, weight, argmax, selection, stride_
     check(lib.clg_convblock_backward_w(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
                                        selection.data_ptr(), argmax.data_ptr(), gw.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
     return gw
+
+
+def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
+    """-> (grad_x, grad_w [C,7,16]) in one call (the pair of calls of
+    src/convlogic/convlogic_layer.py:76-81, one scratch buffer, one transition into the library)."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_convblock_backward_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gx = torch.empty_like(x)
+    gw = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_convblock_backward(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(), selection.data_ptr(),
+                                     argmax.data_ptr(), gx.data_ptr(), gw.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
+    return gx, gw

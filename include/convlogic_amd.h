@@ -210,6 +210,16 @@ int clg_convblock_backward_w(int dtype, const clg_conv_geom *g, const void *grad
                              void *stream);
 int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_conv_geom *g);
 
+/* Both gradients of the fused block in one call: clg_convblock_backward_x followed by
+ * clg_convblock_backward_w on the same stream, sharing one scratch buffer of
+ * clg_convblock_backward_scratch_bytes() bytes.
+ * Replaces the pair full_convlogic_backward_x + full_convlogic_backward_weight as
+ * FullConvLogicFunction.backward calls them -- src/convlogic/convlogic_layer.py:71-82. */
+int clg_convblock_backward(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                           const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w, void *scratch,
+                           void *stream);
+int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *g);
+
 #ifdef __cplusplus
 }
 #endif
