@@ -65,6 +65,9 @@ struct TilePlan {
     int xe;             // elements of one LDS image region (S samples + tail)
     int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
     int band_rows, bands;  // input gradient: image rows per workgroup band, number of bands
+    int hit_split;         // input gradient: workgroups sharing the kernels of one (sample, band), partial images
+    int dummy_in_halo;     // input gradient: masked updates go to halo elements instead of a region of their own
+    int64_t part_stride;   // input gradient: elements between partial images (0 when hit_split == 1)
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp;
     size_t lds_bytes;
 };
@@ -203,16 +206,18 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
 //   hits   [cin][c]    those kernels in increasing order, entry = kernel | tap mask << 16
 // (the reverse map "input channel -> kernels and taps reading it", built in a fixed order).
 struct BwdScratch {
-    size_t folded_bytes, count_off, hits_off, taps_off, total;
+    size_t folded_bytes, count_off, hits_off, taps_off, part_off, total;
 };
-BwdScratch bwd_scratch_layout(const Geom &g, int elem)
+constexpr int kMaxHitSplit = 16;
+BwdScratch bwd_scratch_layout(const Geom &g, int elem, int hit_split)
 {
     BwdScratch b;
     b.folded_bytes = (size_t)g.c * 28 * elem;
     b.count_off = (b.folded_bytes + 63) & ~(size_t)63;
     b.hits_off = (b.count_off + (size_t)g.cin * 4 + 63) & ~(size_t)63;
     b.taps_off = (b.hits_off + (size_t)g.cin * g.c * 4 + 63) & ~(size_t)63;
-    b.total = b.taps_off + (size_t)g.c * 16 * 4;                   // per kernel: 8 offsets inside the image, 8 inside the plane
+    b.part_off = (b.taps_off + (size_t)g.c * 16 * 4 + 255) & ~(size_t)255;   // taps: 8 offsets in the image, 8 in the plane
+    b.total = b.part_off + (hit_split > 1 ? (size_t)hit_split * g.n * g.cin * g.h * g.w * elem : 0);   // partial images
     return b;
 }
 
@@ -308,8 +313,11 @@ __host__ __device__ inline Band make_band(const Geom &g, int band, int band_rows
     return b;
 }
 
-// grid: (sample groups, bands).  LDS: input window xs, gradient window gs (same layout: planes of
-// `wrows` rows x rs elements, left halo shared with the previous row's right halo), cell table.
+// grid: (sample groups, bands, hit split).  LDS: input window xs, gradient window gs (same layout: planes
+// of `wrows` rows x rs elements, left halo shared with the previous row's right halo) and, unless halo
+// elements can take them, one sink element per thread for masked updates.  With a hit split > 1 the
+// workgroups blockIdx.z = 0..HS-1 of one (sample group, band) take every HS-th kernel of each channel's
+// list and write partial gradient images that sum_partial_images adds in a fixed order.
 template <typename T, bool BANDED>
 __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
                                                   const T *__restrict__ folded, const int32_t *__restrict__ count,
@@ -320,9 +328,9 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     const int xe4 = (p.xe + 3) & ~3;
     T *xs = reinterpret_cast<T *>(smem);
     T *gs = xs + xe4;
-    T *dummy = gs + xe4;                                            // one element per thread: sink of masked updates
-    int2 *cellt = reinterpret_cast<int2 *>(dummy + ((blockDim.x + 3) & ~3u));   // [G * cells of the band]
-    const int gs_off = xe4, dummy_off = 2 * xe4 + (int)threadIdx.x;
+    const int gs_off = xe4;
+    // sink of masked updates: the first (halo) row of the gradient window, or a region after it
+    const int dummy_off = p.dummy_in_halo ? gs_off + (int)(threadIdx.x & 31) : 2 * xe4 + (int)threadIdx.x;
 
     const int tid = threadIdx.x, nthreads = blockDim.x;
     const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
@@ -331,18 +339,8 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     const Band bd = make_band(g, blockIdx.y, p.band_rows);
     const int chs = p.chs;                                          // plane stride of the windows
 
-    for (int i = tid; i < 2 * xe4 + nthreads; i += nthreads) xs[i] = T(0);
-    const int V = p.G * bd.cb;                                      // lanes of one pass: G samples x band cells
-    for (int v = tid; v < V; v += nthreads) {
-        uint32_t s = 0, cl = v;
-        if (!BANDED) {
-            s = fdiv(v, p.d_slots);
-            cl = v - s * (uint32_t)I;
-        }
-        const uint32_t cell = bd.cell_lo + cl;
-        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
-        cellt[v] = make_int2((int)(s * g.cin * chs + (2 * py * g.sh - bd.R0) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
-    }
+    const int zero_n = 2 * xe4 + (p.dummy_in_halo ? 0 : nthreads);
+    for (int i = tid; i < zero_n; i += nthreads) xs[i] = T(0);
     __syncthreads();
     // stage the image rows that fall into the window (padded row = image row + ph)
     const int ir0 = bd.R0 - g.ph > 0 ? bd.R0 - g.ph : 0;
@@ -375,56 +373,71 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
         const int64_t gbase = ((int64_t)(n0 + s0) * g.c) * I;       // global offset of the group's first cell row
         const int nhits = v_here > 0 ? count[ch] : 0;
         const int32_t *hit = hits + (int64_t)ch * g.c;
-        // loads of grad_y and the argmax code for (hit k, chunk): issued one step ahead of their use
-        auto issue = [&](int k, int chunk, CellLoads<T> &L) {
-            const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
+
+        // chunk-major: the cell table entries of a chunk stay in registers while all kernels that read
+        // this channel are applied to it (hits in increasing kernel order inside every chunk)
+        for (int chunk = 0; chunk < chunks; ++chunk) {
+            int cx[kChunk], cy[kChunk];
+            bool live[kChunk];
 #pragma unroll
             for (int j = 0; j < kChunk; ++j) {
                 const int v = (chunk * kChunk + j) * kWave + lane;
-                L.gy[j] = T(0);
-                L.code[j] = 0;
-                if (v < v_here) {
-                    const int o = cellt[v].y;
-                    L.code[j] = argmax[crow + o];
-                    L.gy[j] = gy[crow + o];
+                live[j] = v < v_here;
+                uint32_t sm = 0, cl = live[j] ? v : 0;              // sample inside the group, cell inside the band
+                if (!BANDED) {
+                    sm = fdiv(cl, p.d_slots);
+                    cl -= sm * (uint32_t)I;
                 }
+                const uint32_t cell = bd.cell_lo + cl;
+                const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+                cx[j] = img0 + (int)(sm * g.cin * chs + (2 * py * g.sh - bd.R0) * p.rs + 2 * px * g.sw);
+                cy[j] = (int)((sm * g.c) * I + cell);
             }
-        };
-
-        CellLoads<T> cur, nxt;
-        if (nhits > 0) issue(0, 0, cur);
-        for (int k = 0; k < nhits; ++k) {
-            const int ent = hit[k];
-            const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
-            int to[8];                                              // tap offsets inside the group's planes
-            int tr_[8];                                             // the same, relative to the tap's own plane
+            // grad_y and the argmax code of hit k: requested one hit ahead of their use
+            auto issue = [&](int k, CellLoads<T> &L) {
+                const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
+                const uint8_t *am = argmax + crow;
+                const T *gr = gy + crow;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                to[t] = taps[c * 16 + t];
-                tr_[t] = taps[c * 16 + 8 + t];
-            }
-            Tree<T> tr;
-            const T *fc = folded + (int64_t)c * 28;
+                for (int j = 0; j < kChunk; ++j) {
+                    L.gy[j] = T(0);
+                    L.code[j] = 0;
+                    if (live[j]) {
+                        L.code[j] = am[cy[j]];
+                        L.gy[j] = gr[cy[j]];
+                    }
+                }
+            };
+            CellLoads<T> cur, nxt;
+            const int hs0 = blockIdx.z, hsn = gridDim.z;
+            if (hs0 < nhits) issue(hs0, cur);
+            for (int k = hs0; k < nhits; k += hsn) {
+                if (k + hsn < nhits) issue(k + hsn, nxt);
+                const int ent = hit[k];
+                const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
+                int to[8];                                          // tap offsets inside the group's planes
+                int tr_[8];                                         // the same, relative to the tap's own plane
 #pragma unroll
-            for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
-            for (int chunk = 0; chunk < chunks; ++chunk) {
-                if (chunk + 1 < chunks) issue(k, chunk + 1, nxt);
-                else if (k + 1 < nhits) issue(k + 1, 0, nxt);
+                for (int t = 0; t < 8; ++t) {
+                    to[t] = taps[c * 16 + t];
+                    tr_[t] = BANDED ? taps[c * 16 + 8 + t] : 0;
+                }
+                Tree<T> tr;
+                const T *fc = folded + (int64_t)c * 28;
+#pragma unroll
+                for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
                 // phase 1: tree and tap gradients of every cell block of this chunk (registers only).
                 // No per-lane control flow: a lane without a cell recomputes cell 0 with a zero gradient.
                 int pos[kChunk];
-                bool live[kChunk];
                 T gt[kChunk][8];
 #pragma unroll
                 for (int j = 0; j < kChunk; ++j) {
-                    const int v = (chunk * kChunk + j) * kWave + lane;
-                    live[j] = v < v_here;
                     const int code = cur.code[j];
                     const T gout = cur.gy[j];                       // 0 for lanes without a cell
-                    pos[j] = cellt[live[j] ? v : 0].x + (code >> 1) * row_step + (code & 1) * g.sw;
+                    pos[j] = cx[j] + (code >> 1) * row_step + (code & 1) * g.sw;
                     T tv[8];
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) tv[t] = xs[img0 + pos[j] + to[t]];
+                    for (int t = 0; t < 8; ++t) tv[t] = xs[pos[j] + to[t]];
                     const TreeVals<T> tvv = eval_tree(tr, tv);
                     const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
                     const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
@@ -454,8 +467,8 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
 #pragma unroll
                         for (int j = 0; j < kChunk; ++j) {
                             bool mine = live[j];
-                            if (BANDED) mine = mine && ((uint32_t)(pos[j] + tr_[t]) - own_lo) < own_len;
-                            at[j] = mine ? gs_off + img0 + pos[j] + to[t] : dummy_off;
+                            if (BANDED) mine = mine && ((uint32_t)(pos[j] - img0 + tr_[t]) - own_lo) < own_len;
+                            at[j] = mine ? gs_off + pos[j] + to[t] : dummy_off;
                         }
 #pragma unroll
                         for (int j = 0; j < kChunk; ++j) old[j] = xs[at[j]];
@@ -470,7 +483,7 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     __syncthreads();
     // write the owned rows of the gradient planes back
     const int orows = bd.r1 - bd.r0;
-    T *dstg = gx + (int64_t)n0 * g.cin * g.h * g.w;
+    T *dstg = gx + (int64_t)blockIdx.z * p.part_stride + (int64_t)n0 * g.cin * g.h * g.w;
     for (int pr = wave; pr < planes * orows; pr += p.NW) {
         const int plane = uniform(pr / orows), iy = bd.r0 + (pr - plane * orows);
         const T *row = gs + plane * chs + (iy + g.ph - bd.R0) * p.rs + g.pw;
@@ -479,136 +492,122 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     }
 }
 
+// gx = ((part[0] + part[1]) + part[2]) + ... : partial gradient images of a split hit list, fixed order
+template <typename T>
+__global__ __launch_bounds__(256) void sum_partial_images_kernel(const T *__restrict__ part, T *__restrict__ gx, int64_t total, int hs)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    T acc = part[e];
+    for (int k = 1; k < hs; ++k) acc += part[(int64_t)k * total + e];
+    gx[e] = acc;
+}
+
 // ---------------------------------------------------------------------------------------------
 // weight gradient
 // ---------------------------------------------------------------------------------------------
-// Workgroup = (column of sample groups, CT kernels); it walks its sample groups (stage S samples in
-// LDS, barrier) and every wavefront keeps the 28 partial sums (7 gates x (ab, a, b, 1)) of its
-// kKPW kernels in registers across ALL of them, so the cross-lane reduction happens once per kernel
-// and workgroup.  partial [c][gridDim.x][28] is summed in a fixed order by reduce_coef_partials.
-constexpr int kKPW = 2;  // kernels per wavefront
+// Kernel-major with plenty of small workgroups: blockIdx.y = kernel (coefficients and tap offsets are
+// scalar), threads run over (sample, pooled cell) and keep the 28 sums (7 gates x (ab, a, b, 1)) in
+// registers across all their cells; one block reduction per workgroup, partial [c][blocks][28], summed in
+// order by reduce_coef_partials.  Taps come from a zero-padded copy of x in global memory (written once
+// per call into scratch, same shared-halo layout as the LDS images), so the loop has no bounds checks
+// and 32-bit offsets only.
+template <typename T>
+__global__ __launch_bounds__(256) void pad_image_kernel(const T *__restrict__ x, T *__restrict__ xp, Geom g, TilePlan p,
+                                                      FastDiv d_sample, FastDiv d_rs, int sample_elems, int64_t total)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const uint32_t n = fdiv((uint32_t)e, d_sample), rem = (uint32_t)e - n * (uint32_t)sample_elems;
+    const uint32_t plane = fdiv(rem, p.d_slots), r2 = rem - plane * (uint32_t)p.chs;      // d_slots holds chs here
+    const uint32_t row = fdiv(r2, d_rs), col = r2 - row * (uint32_t)p.rs;
+    T v = T(0);
+    if (plane < (uint32_t)g.cin && row >= (uint32_t)g.ph && col >= (uint32_t)g.pw)
+        v = x[(((int64_t)n * g.cin + plane) * g.h + (row - g.ph)) * g.w + (col - g.pw)];
+    xp[e] = v;
+}
 
 template <typename T>
-__global__ void convblock_backward_w_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x, const T *__restrict__ w,
-                                                  const int32_t *__restrict__ sel, const uint8_t *__restrict__ argmax,
-                                                  T *__restrict__ partial, Geom g, TilePlan p)
+__global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const T *__restrict__ gy, const T *__restrict__ xp,
+                                                                        const T *__restrict__ folded,
+                                                                        const int32_t *__restrict__ taps,
+                                                                        const uint8_t *__restrict__ argmax,
+                                                                        T *__restrict__ partial, Geom g, TilePlan p,
+                                                                        FastDiv d_cells, int sample_elems)
 {
-    extern __shared__ __align__(16) unsigned char smem[];
-    T *xs = reinterpret_cast<T *>(smem);
-    T *coef = xs + ((p.xe + 3) & ~3);                                 // [CT][28]
-    int *toff = reinterpret_cast<int *>(coef + p.CT * 28);            // [CT][8]
-    int2 *cellt = reinterpret_cast<int2 *>(toff + p.CT * 8);          // [S * cells]
-
-    const int tid = threadIdx.x, nthreads = blockDim.x;
-    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
-    const int c0 = blockIdx.y * p.CT, ct_cur = min(p.CT, g.c - c0);
-    const int wp = g.wo >> 1, I = p.slots;
-
-    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
-    for (int q = tid; q < ct_cur * 7; q += nthreads) {
-        const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
-        coef[q * 4 + 0] = cf.ab;
-        coef[q * 4 + 1] = cf.a;
-        coef[q * 4 + 2] = cf.b;
-        coef[q * 4 + 3] = cf.one;
-    }
-    for (int q = tid; q < ct_cur * 8; q += nthreads) {
-        const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
-        toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
-    }
-    for (int v = tid; v < p.S * I; v += nthreads) {
-        const uint32_t s = fdiv(v, p.d_slots), cell = v - s * (uint32_t)I;
-        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
-        cellt[v] = make_int2((int)(s * g.cin * p.chs + (2 * py * g.sh) * p.rs + 2 * px * g.sw), (int)((s * g.c) * I + cell));
-    }
-
-    T acc[kKPW][28];
+    const int c = blockIdx.y, nb = gridDim.x;
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+    const uint32_t items = (uint32_t)g.n * I;
+    Tree<T> tr;
+    const T *fc = folded + (int64_t)c * 28;
 #pragma unroll
-    for (int kk = 0; kk < kKPW; ++kk)
+    for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+    int to[8];
 #pragma unroll
-        for (int i = 0; i < 28; ++i) acc[kk][i] = T(0);
-
+    for (int t = 0; t < 8; ++t) to[t] = taps[c * 8 + t];
     const int row_step = g.sh * p.rs;
-    const int ngroups = (g.n + p.S - 1) / p.S;
-    for (int grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
-        const int n0 = grp * p.S, s_cur = min(p.S, g.n - n0);
-        __syncthreads();                                             // everyone is done with the previous image
-        stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
-        __syncthreads();
-        const int V = s_cur * I;
+    const int64_t kernel_row = (int64_t)c * I;
+    const int64_t sample_cells = (int64_t)g.c * I;
+    T acc[28];
 #pragma unroll
-        for (int kk = 0; kk < kKPW; ++kk) {
-            const int lc = wave * kKPW + kk;
-            if (lc >= ct_cur) break;                                 // wave-uniform
-            Tree<T> tr;
+    for (int k = 0; k < 28; ++k) acc[k] = T(0);
+    for (uint32_t it = blockIdx.x * 256 + threadIdx.x; it < items; it += (uint32_t)nb * 256) {
+        const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
+        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+        const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
+        const int code = argmax[o];
+        const T gout = gy[o];
+        const int pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
+        T tv[8];
 #pragma unroll
-            for (int k = 0; k < 7; ++k) {
-                tr.g[k].ab = to_sgpr(coef[(lc * 7 + k) * 4 + 0]);
-                tr.g[k].a = to_sgpr(coef[(lc * 7 + k) * 4 + 1]);
-                tr.g[k].b = to_sgpr(coef[(lc * 7 + k) * 4 + 2]);
-                tr.g[k].one = to_sgpr(coef[(lc * 7 + k) * 4 + 3]);
-            }
-            int to[8];
+        for (int t = 0; t < 8; ++t) tv[t] = xp[pos + to[t]];
+        const TreeVals<T> v = eval_tree(tr, tv);
+        T gin[7][2], gg[7];
+        gg[6] = gout;
+        gin[6][0] = v.mid[0];
+        gin[6][1] = v.mid[1];
+        gg[4] = gout * gate_da(tr.g[6], v.mid[1]);
+        gg[5] = gout * gate_db(tr.g[6], v.mid[0]);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) to[t] = uniform(toff[lc * 8 + t]);
-            const int64_t crow = ((int64_t)n0 * g.c + c0 + lc) * I;
-            const uint8_t *am = argmax + crow;
-            const T *gr = gy + crow;
-            // grad_y / argmax of the next cell block are requested before the current one is used
-            int2 e = cellt[lane < V ? lane : 0];
-            int code = lane < V ? am[e.y] : 0;
-            T gout = lane < V ? gr[e.y] : T(0);
-            for (int v0 = 0; v0 < V; v0 += kWave) {
-                const int vn = v0 + kWave + lane;
-                const int2 en = cellt[vn < V ? vn : 0];
-                const int code_n = vn < V ? am[en.y] : 0;
-                const T gout_n = vn < V ? gr[en.y] : T(0);
-                const int pos = e.x + (code >> 1) * row_step + (code & 1) * g.sw;
-                T tv[8];
+        for (int m = 0; m < 2; ++m) {
+            gin[4 + m][0] = v.leaf[2 * m];
+            gin[4 + m][1] = v.leaf[2 * m + 1];
+            gg[2 * m] = gg[4 + m] * gate_da(tr.g[4 + m], v.leaf[2 * m + 1]);
+            gg[2 * m + 1] = gg[4 + m] * gate_db(tr.g[4 + m], v.leaf[2 * m]);
+        }
 #pragma unroll
-                for (int t = 0; t < 8; ++t) tv[t] = xs[pos + to[t]];
-                const TreeVals<T> v = eval_tree(tr, tv);
-                T gin[7][2], gg[7];
-                gg[6] = gout;
-                gin[6][0] = v.mid[0];
-                gin[6][1] = v.mid[1];
-                gg[4] = gout * gate_da(tr.g[6], v.mid[1]);
-                gg[5] = gout * gate_db(tr.g[6], v.mid[0]);
+        for (int q = 0; q < 4; ++q) {
+            gin[q][0] = tv[2 * q];
+            gin[q][1] = tv[2 * q + 1];
+        }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    gin[4 + m][0] = v.leaf[2 * m];
-                    gin[4 + m][1] = v.leaf[2 * m + 1];
-                    gg[2 * m] = gg[4 + m] * gate_da(tr.g[4 + m], v.leaf[2 * m + 1]);
-                    gg[2 * m + 1] = gg[4 + m] * gate_db(tr.g[4 + m], v.leaf[2 * m]);
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    gin[q][0] = tv[2 * q];
-                    gin[q][1] = tv[2 * q + 1];
-                }
-#pragma unroll
-                for (int k = 0; k < 7; ++k) {
-                    acc[kk][4 * k + 0] = fma_t(gg[k], gin[k][0] * gin[k][1], acc[kk][4 * k + 0]);
-                    acc[kk][4 * k + 1] = fma_t(gg[k], gin[k][0], acc[kk][4 * k + 1]);
-                    acc[kk][4 * k + 2] = fma_t(gg[k], gin[k][1], acc[kk][4 * k + 2]);
-                    acc[kk][4 * k + 3] += gg[k];
-                }
-                e = en;
-                code = code_n;
-                gout = gout_n;
-            }
+        for (int k = 0; k < 7; ++k) {
+            acc[4 * k + 0] = fma_t(gg[k], gin[k][0] * gin[k][1], acc[4 * k + 0]);
+            acc[4 * k + 1] = fma_t(gg[k], gin[k][0], acc[4 * k + 1]);
+            acc[4 * k + 2] = fma_t(gg[k], gin[k][1], acc[4 * k + 2]);
+            acc[4 * k + 3] += gg[k];
         }
     }
-#pragma unroll
-    for (int kk = 0; kk < kKPW; ++kk) {
-        const int lc = wave * kKPW + kk;
-        if (lc >= ct_cur) break;
-        T *dst = partial + ((int64_t)(c0 + lc) * gridDim.x + blockIdx.x) * 28;
-#pragma unroll
-        for (int i = 0; i < 28; ++i) {
-            const T sum = wave_sum(acc[kk][i]);
-            if (lane == 0) dst[i] = sum;
-        }
+    block_sum_store<T, 28, 256>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 28);
+}
+
+// folded coefficients [c][28] and tap offsets [c][8] in the padded-image layout
+template <typename T>
+__global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
+                                                                T *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
+                                                                int chs)
+{
+    const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q < (int64_t)C * 8) {
+        const Tap tp = unpack_tap(sel[q]);
+        taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
+    }
+    if (q < (int64_t)C * 7) {
+        const Coef<T> cf = fold16(w + q * 16);
+        folded[q * 4 + 0] = cf.ab;
+        folded[q * 4 + 1] = cf.a;
+        folded[q * 4 + 2] = cf.b;
+        folded[q * 4 + 3] = cf.one;
     }
 }
 
@@ -647,10 +646,11 @@ bool plan_forward(const Geom &g, int elem, TilePlan *p)
     }
     if (best_s == 0 || best_util < 0.4) return false;
     p->S = best_s;
-    p->NW = 4;
+    // 16 wavefronts share one staged image: measured 69 us against 109 us with 4 at [256,9,32,32] -> 256
+    p->NW = 16;
     const int64_t groups = clg_ceil_div(g.n, p->S);
     int64_t ct = (int64_t)g.c * groups / 1024;
-    ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
+    ct = ct < 16 ? 16 : (ct > 64 ? 64 : ct);
     if (ct > g.c) ct = g.c;
     p->CT = (int)ct;
     p->xe = (int)image_elems(g, *p, p->S);
@@ -670,6 +670,7 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     p->CT = 0;
     p->d_slots = make_fastdiv((uint32_t)I);
     p->NW = g.cin < 16 ? g.cin : 16;
+    // two windows (input, gradient); a sink region of one element per thread unless halo elements serve
     auto size_for = [&](int G, int band_rows, int *rows_max, int *cb_max) {
         const int bands = (int)clg_ceil_div(g.h, band_rows);
         *rows_max = 0;
@@ -680,7 +681,8 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
             if (bd.cb > *cb_max) *cb_max = bd.cb;
         }
         const int64_t xe = (int64_t)G * g.cin * *rows_max * p->rs + g.pw;
-        return (int64_t)2 * ((xe + 3) & ~3) * elem + (int64_t)p->NW * kWave * elem + (int64_t)G * *cb_max * 8;
+        const bool halo_sink = bands == 1 && g.ph >= 1 && p->rs >= 32;
+        return (int64_t)2 * ((xe + 3) & ~3) * elem + (halo_sink ? 0 : (int64_t)p->NW * kWave * elem);
     };
     // samples sharing a wavefront pass when a sample has fewer than 64 cells (whole image, one band)
     int G = I >= kWave ? 1 : kWave / I;
@@ -709,47 +711,52 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     p->chs = rows_max * p->rs;
     p->xe = (int)((int64_t)G * g.cin * p->chs + g.pw);
     p->lds_bytes = (size_t)bytes;
+    p->dummy_in_halo = (p->bands == 1 && g.ph >= 1 && p->rs >= 32) ? 1 : 0;
     if (p->bands > 65535) return false;
     if (G * I < kWave / 5 && p->bands == 1) return false;            // almost empty wavefronts: gather kernel instead
+    // hit split: when (sample groups x bands) leave room for more resident workgroups, several workgroups
+    // share the kernels of one image; each handles every HS-th kernel and writes a partial image
+    int64_t per_cu = kLdsLimit / (int64_t)(bytes > 1024 ? bytes : 1024);
+    if (per_cu > 20 / p->NW) per_cu = 20 / p->NW;                    // about 80 VGPRs per lane: 5 wavefronts per SIMD
+    if (per_cu < 1) per_cu = 1;
+    const int64_t wgs = clg_ceil_div(g.n, p->S) * p->bands;
+    const char *e_hs = getenv("CLG_BWDX_SPLIT");
+    int64_t hs = e_hs ? atoi(e_hs) : (256 * per_cu) / wgs;
+    if (hs > kMaxHitSplit) hs = kMaxHitSplit;
+    // every split workgroup stages the image and writes a partial image: worth it only with at least
+    // about 4 kernels left per channel list (a kernel reads at most two channels)
+    const int64_t avg_hits = g.cin == 1 ? g.c : (2 * (int64_t)g.c) / g.cin;
+    if (!e_hs && hs > avg_hits / 4) hs = avg_hits / 4;
+    if (hs < 1) hs = 1;
+    p->hit_split = (int)hs;
+    p->part_stride = hs > 1 ? (int64_t)g.n * g.cin * g.h * g.w : 0;
     return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * I < (1ll << 31);
 }
 
-// weight gradient: S samples per staging round, CT = kKPW * NW kernels per workgroup, `cols` columns
-// of sample groups (= partial sums per kernel)
-bool plan_backward_w(const Geom &g, int elem, TilePlan *p, int *cols)
+// weight gradient from the padded copy: scratch = partials | folded | taps | padded x
+struct WScratch {
+    int nb, sample_elems;
+    size_t folded_off, taps_off, xp_off, total;
+};
+bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
 {
-    if (!taps_inside(g) || g.c > 65535 * 8) return false;
+    if (!taps_inside(g) || g.c > 65535) return false;
     plan_common(g, p);
-    const int I = (g.ho / 2) * (g.wo / 2);
-    // below about 8M pooled values the kernel that reads taps from global memory has more wavefronts in
-    // flight and wins (measured 26 vs 41 us at 1.6M, 125 vs 109 us at 16.8M)
-    if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_TILED")) return false;
-    p->slots = I;
-    p->G = 1;
-    p->d_slots = make_fastdiv((uint32_t)I);
-    // samples per round: enough cells for full wavefronts, image region up to 64 KiB
-    int S = 1;
-    while (S < g.n && S * I < 4 * kWave && (image_elems(g, *p, 2 * S) * elem + (int64_t)2 * S * I * 8) <= 64 * 1024) S *= 2;
-    p->S = S;
-    p->xe = (int)image_elems(g, *p, S);
-    const int64_t groups = clg_ceil_div(g.n, S);
-    // wavefronts per workgroup: as many as give every wavefront kernels to work on, up to 8
-    int nw = (int)clg_ceil_div(g.c, kKPW);
-    if (nw > 8) nw = 8;
-    p->NW = nw;
-    p->CT = nw * kKPW;
-    const int64_t tiles = clg_ceil_div(g.c, p->CT);
-    // columns: fill the GPU about twice, at least 4 staging rounds per workgroup where possible
-    const char *e_cols = getenv("CLG_BWDW_COLS");
-    int64_t c_ = e_cols ? atoi(e_cols) : clg_ceil_div(1024, tiles);
-    if (c_ > groups) c_ = groups;
-    if (c_ > 32) c_ = 32;
-    if (c_ < 1) c_ = 1;
-    *cols = (int)c_;
-    p->lds_bytes = (size_t)((p->xe + 3) & ~3) * elem + (size_t)p->CT * 28 * elem + (size_t)p->CT * 8 * 4 + (size_t)S * I * 8;
-    if (p->lds_bytes > (size_t)kLdsLimit || tiles > 65535) return false;
-    if ((double)(S * I) / (double)(clg_ceil_div((int64_t)S * I, kWave) * kWave) < 0.4) return false;
-    return (int64_t)S * g.cin * p->chs < (1ll << 30) && (int64_t)S * g.c * I < (1ll << 31);
+    const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
+    // the padded copy costs two extra launches: it pays from about 8M pooled values (measured 102 vs 124 us
+    // at 16.8M, 30 vs 27 us at 1.6M)
+    if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_PADDED")) return false;
+    const int64_t sample_elems = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
+    if (sample_elems * g.n >= (1ll << 31) || I * g.n >= (1ll << 31)) return false;
+    p->d_slots = make_fastdiv((uint32_t)p->chs);                    // reused as "divide by plane stride"
+    ws->sample_elems = (int)sample_elems;
+    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);                   // about 8 cells per thread
+    ws->nb = (int)(nb < 1 ? 1 : (nb > 64 ? 64 : nb));
+    ws->folded_off = ((size_t)g.c * 64 * 28 * elem + 255) & ~(size_t)255;   // partials sized for 64 blocks
+    ws->taps_off = (ws->folded_off + (size_t)g.c * 28 * elem + 255) & ~(size_t)255;
+    ws->xp_off = (ws->taps_off + (size_t)g.c * 8 * 4 + 255) & ~(size_t)255;
+    ws->total = ws->xp_off + (size_t)sample_elems * g.n * elem;
+    return true;
 }
 
 // Kernels that want more than 48 KiB of dynamic LDS must be told once; the largest size granted so
@@ -816,7 +823,7 @@ template <typename T>
 int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, const void *x, const void *w, const int32_t *sel,
                             const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
 {
-    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T));
+    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
     T *folded = reinterpret_cast<T *>(scratch);
     int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
     int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
@@ -825,30 +832,50 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
                        folded, count, hits, taps, g.c, g.cin, fold_blocks, p.rs, p.chs);
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
-    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands), block(p.NW * kWave);
+    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
+    T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
+    T *out = p.hit_split > 1 ? part : (T *)gx;
     if (p.bands > 1) {
         if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, true>, p.lds_bytes, "clg_convblock_backward_x")) return e;
         hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, true>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
-                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, (T *)gx, g, p);
+                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, out, g, p);
     } else {
         if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, false>, p.lds_bytes, "clg_convblock_backward_x")) return e;
         hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, false>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
-                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, (T *)gx, g, p);
+                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, out, g, p);
     }
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(tiled)");
+    if (p.hit_split > 1) {
+        const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
+        hipLaunchKernelGGL(sum_partial_images_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)part,
+                           (T *)gx, total, p.hit_split);
+        CLG_CHECK_LAUNCH("clg_convblock_backward_x(sum)");
+    }
     return CLG_OK;
 }
 
 template <typename T>
-int launch_backward_w_tiled(const Geom &g, const TilePlan &p, int cols, const void *gy, const void *x, const void *w,
-                            const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st)
+int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &ws, const void *gy, const void *x, const void *w,
+                             const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st)
 {
-    if (int e = allow_lds(convblock_backward_w_tiled_kernel<T>, p.lds_bytes, "clg_convblock_backward_w")) return e;
-    const dim3 grid((unsigned)cols, (unsigned)clg_ceil_div(g.c, p.CT));
-    hipLaunchKernelGGL(convblock_backward_w_tiled_kernel<T>, grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)gy, (const T *)x,
-                       (const T *)w, sel, argmax, (T *)scratch, g, p);
-    CLG_CHECK_LAUNCH("clg_convblock_backward_w(tiled)");
-    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, scratch, gw, g.c, cols, 7, st, "clg_convblock_backward_w(reduce)");
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    T *partial = reinterpret_cast<T *>(base);
+    T *folded = reinterpret_cast<T *>(base + ws.folded_off);
+    int32_t *taps = reinterpret_cast<int32_t *>(base + ws.taps_off);
+    T *xp = reinterpret_cast<T *>(base + ws.xp_off);
+    hipLaunchKernelGGL(convblock_w_prepare_kernel<T>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
+                       (const T *)w, sel, folded, taps, g.c, p.rs, p.chs);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(prepare)");
+    const int64_t total = (int64_t)ws.sample_elems * g.n;
+    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, p,
+                       make_fastdiv((uint32_t)ws.sample_elems), make_fastdiv((uint32_t)p.rs), ws.sample_elems, total);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(pad)");
+    const int I = (g.ho / 2) * (g.wo / 2);
+    hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
+                       (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p, make_fastdiv((uint32_t)I),
+                       ws.sample_elems);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded)");
+    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, ws.nb, 7, st, "clg_convblock_backward_w(reduce)");
 }
 
 int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
@@ -873,7 +900,9 @@ extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_c
 {
     Geom g;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x_scratch_bytes")) return -1;
-    return (int64_t)bwd_scratch_layout(g, elem_size(dtype)).total;
+    TilePlan p;
+    const int hs = plan_backward_x(g, elem_size(dtype), &p) ? p.hit_split : 1;
+    return (int64_t)bwd_scratch_layout(g, elem_size(dtype), hs).total;
 }
 
 extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -896,10 +925,10 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
 {
     Geom g;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w_scratch_bytes")) return -1;
-    // enough for either kernel: partial sums [c][blocks][28] with at most 64 blocks per kernel
-    int64_t nb = clg_convblock_partial_blocks(g);
-    if (nb < 64) nb = 64;
-    return (int64_t)g.c * nb * 28 * elem_size(dtype);
+    TilePlan p;
+    WScratch ws;
+    if (plan_backward_w(g, elem_size(dtype), &p, &ws)) return (int64_t)ws.total;
+    return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the any-shape kernel
 }
 
 extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -910,12 +939,12 @@ extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, cons
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w")) return e;
     CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "clg_convblock_backward_w: null pointer argument");
     TilePlan p;
-    int cols = 1;
-    const char *e_tiled = getenv("CLG_BWDW_TILED");
-    if ((!e_tiled || atoi(e_tiled) != 0) && plan_backward_w(g, elem_size(dtype), &p, &cols)) {
+    WScratch ws;
+    const char *e_pad = getenv("CLG_BWDW_PADDED");
+    if ((!e_pad || atoi(e_pad) != 0) && plan_backward_w(g, elem_size(dtype), &p, &ws)) {
         if (dtype == CLG_F32)
-            return launch_backward_w_tiled<float>(g, p, cols, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
-        return launch_backward_w_tiled<double>(g, p, cols, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+            return launch_backward_w_padded<float>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+        return launch_backward_w_padded<double>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
     }
     return clg_convblock_backward_w_generic(dtype, g, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
 }
