@@ -29,8 +29,9 @@
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
 int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
                                   uint8_t *argmax, hipStream_t st);
-int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
-                                     const int32_t *selection, const uint8_t *argmax, void *grad_x, hipStream_t st);
+int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *folded,
+                                     const int32_t *count, const int32_t *hits, const int32_t *selection, const uint8_t *argmax,
+                                     void *grad_x, hipStream_t st);
 int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
                                      hipStream_t st);
@@ -155,7 +156,14 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
     __syncthreads();
 
     const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
-    for (int lc = wave; lc < ct_cur; lc += p.NW) {
+    // work items = (kernel, block of 64 slots), kernel-major; every wavefront takes a contiguous range, so
+    // the scalar coefficients are reloaded only when its range crosses into the next kernel
+    const int nblk = (U + kWave - 1) / kWave;
+    const int items = ct_cur * nblk;
+    const int per = (items + p.NW - 1) / p.NW;
+    const int first = wave * per, last = min(items, first + per);
+    int lc = first / nblk, blk = first - lc * nblk;
+    for (int item = first; item < last;) {
         Tree<T> tr;
 #pragma unroll
         for (int k = 0; k < 7; ++k) {
@@ -170,8 +178,8 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
         const int64_t obase = ((int64_t)n0 * g.c + c0 + lc) * I;
         T *yb = y + obase;
         uint8_t *ab = argmax + obase;
-        for (int u0 = 0; u0 < U; u0 += kWave) {
-            const int u = u0 + lane;
+        for (; blk < nblk && item < last; ++blk, ++item) {
+            const int u = blk * kWave + lane;
             const bool valid = u < U;
             const int2 e = slot[valid ? u : 0];
             T v[8];
@@ -188,12 +196,12 @@ __global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T 
                 if (r0o > best) { best = r0o; code = 1; }
                 if (r1 > best) { best = r1; code = 2; }
                 if (r1o > best) { best = r1o; code = 3; }
-                // a NaN in the first window position never loses a strict comparison; a first
-                // position below every comparison (NaN elsewhere) behaves as in the generic kernel
                 yb[e.y] = best;
                 ab[e.y] = (uint8_t)code;
             }
         }
+        blk = 0;
+        ++lc;
     }
 }
 
@@ -650,7 +658,7 @@ bool plan_forward(const Geom &g, int elem, TilePlan *p)
     p->NW = 16;
     const int64_t groups = clg_ceil_div(g.n, p->S);
     int64_t ct = (int64_t)g.c * groups / 1024;
-    ct = ct < 16 ? 16 : (ct > 64 ? 64 : ct);
+    ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
     if (ct > g.c) ct = g.c;
     p->CT = (int)ct;
     p->xe = (int)image_elems(g, *p, p->S);
@@ -819,6 +827,21 @@ int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const 
     }
 }
 
+// folded coefficients, per-channel kernel lists and tap offsets (for LDS rows of rs, planes of chs elements)
+template <typename T>
+int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const void *w, const int32_t *sel, void *scratch,
+                   hipStream_t st)
+{
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
+    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
+                       reinterpret_cast<T *>(base), reinterpret_cast<int32_t *>(base + lay.count_off),
+                       reinterpret_cast<int32_t *>(base + lay.hits_off), reinterpret_cast<int32_t *>(base + lay.taps_off), g.c, g.cin,
+                       fold_blocks, rs, chs);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
+    return CLG_OK;
+}
+
 template <typename T>
 int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, const void *x, const void *w, const int32_t *sel,
                             const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
@@ -828,10 +851,7 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
     int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
     int32_t *taps = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.taps_off);
-    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
-    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
-                       folded, count, hits, taps, g.c, g.cin, fold_blocks, p.rs, p.chs);
-    CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
+    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st)) return e;
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
     T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
     T *out = p.hit_split > 1 ? part : (T *)gx;
@@ -918,7 +938,17 @@ extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, cons
             return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
         return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
     }
-    return clg_convblock_backward_x_generic(dtype, g, grad_y, x, w, selection, argmax, grad_x, clg_stream(stream));
+    // any other shape: per-element gather driven by the same per-channel kernel lists
+    const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    if (dtype == CLG_F32) {
+        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, clg_stream(stream))) return e;
+    } else {
+        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, clg_stream(stream))) return e;
+    }
+    return clg_convblock_backward_x_generic(dtype, g, grad_y, x, scratch, reinterpret_cast<const int32_t *>(base + lay.count_off),
+                                            reinterpret_cast<const int32_t *>(base + lay.hits_off), selection, argmax, grad_x,
+                                            clg_stream(stream));
 }
 
 extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_conv_geom *gg)

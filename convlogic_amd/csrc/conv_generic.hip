@@ -28,13 +28,13 @@ struct alignas(sizeof(T) * 2) Pair {
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kBlk) void conv4_forward_kernel(const T *__restrict__ x, const T *__restrict__ w,
-                                                           const int32_t *__restrict__ sel, T *__restrict__ y, Geom g,
-                                                           int pos_blocks)
+                                                           const int32_t *__restrict__ sel, T *__restrict__ y, Geom g)
 {
-    const int c = blockIdx.y, n = blockIdx.x / pos_blocks;
-    const int pos = (blockIdx.x % pos_blocks) * kBlk + threadIdx.x;
+    const int c = blockIdx.y;
     const int P = g.ho * g.wo;
-    if (pos >= P) return;
+    const int64_t item = (int64_t)blockIdx.x * kBlk + threadIdx.x;       // (sample, position)
+    if (item >= (int64_t)g.n * P) return;
+    const int n = (int)(item / P), pos = (int)(item - (int64_t)n * P);
     const int oy = pos / g.wo, ox = pos % g.wo;
     const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
     Quad<T> out;
@@ -149,6 +149,59 @@ __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *_
     gx[e] = acc;
 }
 
+// Input gradient of the fused block for shapes the LDS kernels do not take: one thread per input element
+// walks the list of kernels that read its channel (count / hits, built in increasing kernel order by the
+// preparation kernel) and, where the stored argmax position of the touched pooled cell is the one that
+// reads this element, recomputes that tree and adds the tap gradient.  One writer per element, fixed
+// order: reproducible.
+template <typename T>
+__global__ __launch_bounds__(kBlk) void convblock_backward_x_hits_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+                                                                       const T *__restrict__ folded,
+                                                                       const int32_t *__restrict__ count,
+                                                                       const int32_t *__restrict__ hits,
+                                                                       const int32_t *__restrict__ sel,
+                                                                       const uint8_t *__restrict__ argmax, T *__restrict__ gx,
+                                                                       Geom g)
+{
+    const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
+    const int64_t e = (int64_t)blockIdx.x * kBlk + threadIdx.x;
+    if (e >= total) return;
+    const int ix = (int)(e % g.w), iy = (int)((e / g.w) % g.h);
+    const int ch = (int)((e / ((int64_t)g.w * g.h)) % g.cin), n = (int)(e / ((int64_t)g.w * g.h * g.cin));
+    const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    const int wp = g.wo / 2, I = (g.ho / 2) * wp;
+    const int nhits = count[ch];
+    const int32_t *hit = hits + (int64_t)ch * g.c;
+    T acc = 0;
+    for (int k = 0; k < nhits; ++k) {
+        const int ent = hit[k];
+        const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
+        for (int t = 0; t < 8; ++t) {
+            if (!((mask >> t) & 1)) continue;
+            const Tap tp = unpack_tap(sel[c * 8 + t]);
+            const int ny = iy + g.ph - tp.ry, nx = ix + g.pw - tp.rx;
+            if (ny < 0 || nx < 0 || ny % g.sh != 0 || nx % g.sw != 0) continue;
+            const int oy = ny / g.sh, ox = nx / g.sw;
+            if (oy >= g.ho || ox >= g.wo) continue;
+            const int64_t cell = ((int64_t)n * g.c + c) * I + (oy >> 1) * wp + (ox >> 1);
+            if (argmax[cell] != ((oy & 1) * 2 + (ox & 1))) continue;
+            Tree<T> tr;
+            const T *fc = folded + (int64_t)c * 28;
+#pragma unroll
+            for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+            T tap[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) tap[q] = read_tap(xn, g, unpack_tap(sel[c * 8 + q]), oy, ox);
+            const TreeVals<T> v = eval_tree(tr, tap);
+            const int p = t >> 1, m = p >> 1;
+            const T g_mid = gy[cell] * (m ? gate_db(tr.g[6], v.mid[0]) : gate_da(tr.g[6], v.mid[1]));
+            const T g_leaf = g_mid * ((p & 1) ? gate_db(tr.g[4 + m], v.leaf[p ^ 1]) : gate_da(tr.g[4 + m], v.leaf[p ^ 1]));
+            acc += g_leaf * ((t & 1) ? gate_db(tr.g[p], tap[t ^ 1]) : gate_da(tr.g[p], tap[t ^ 1]));
+        }
+    }
+    gx[e] = acc;
+}
+
 // ---------------------------------------------------------------------------------------------
 // one tree level
 // ---------------------------------------------------------------------------------------------
@@ -208,12 +261,13 @@ __global__ __launch_bounds__(kBlk) void tree_backward_w_kernel(const T *__restri
 template <typename T>
 __global__ __launch_bounds__(kBlk) void convblock_forward_generic_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                                        const int32_t *__restrict__ sel, T *__restrict__ y,
-                                                                       uint8_t *__restrict__ argmax, Geom g, int cell_blocks)
+                                                                       uint8_t *__restrict__ argmax, Geom g)
 {
-    const int c = blockIdx.y, n = blockIdx.x / cell_blocks;
-    const int cell = (blockIdx.x % cell_blocks) * kBlk + threadIdx.x;
+    const int c = blockIdx.y;
     const int wp = g.wo / 2, I = (g.ho / 2) * wp;
-    if (cell >= I) return;
+    const int64_t item = (int64_t)blockIdx.x * kBlk + threadIdx.x;       // (sample, pooled cell)
+    if (item >= (int64_t)g.n * I) return;
+    const int n = (int)(item / I), cell = (int)(item - (int64_t)n * I);
     const int py = cell / wp, px = cell % wp;
     const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
     const Tree<T> tr = load_tree(w + c * 7 * 16);
@@ -242,12 +296,13 @@ __global__ __launch_bounds__(kBlk) void convblock_forward_generic_kernel(const T
 template <typename T>
 __global__ __launch_bounds__(kBlk) void convblock_intermediates_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                                      const int32_t *__restrict__ sel, T *__restrict__ x2,
-                                                                     T *__restrict__ x3, Geom g, int pos_blocks)
+                                                                     T *__restrict__ x3, Geom g)
 {
-    const int c = blockIdx.y, n = blockIdx.x / pos_blocks;
-    const int pos = (blockIdx.x % pos_blocks) * kBlk + threadIdx.x;
+    const int c = blockIdx.y;
     const int P = g.ho * g.wo;
-    if (pos >= P) return;
+    const int64_t item = (int64_t)blockIdx.x * kBlk + threadIdx.x;       // (sample, position)
+    if (item >= (int64_t)g.n * P) return;
+    const int n = (int)(item / P), pos = (int)(item - (int64_t)n * P);
     const int oy = pos / g.wo, ox = pos % g.wo;
     const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
     const Tree<T> tr = load_tree(w + c * 7 * 16);
@@ -362,10 +417,10 @@ int launch_reduce(const void *partial, void *out, int64_t rows, int nb, int G, h
         }                                   \
     } while (0)
 
-static int check_grid(const Geom &g, int64_t per_sample_blocks, const char *name)
+static int check_grid(const Geom &g, int64_t blocks, const char *name)
 {
     CLG_REQUIRE(g.c <= 65535, "%s: more than 65535 logic kernels are not supported", name);
-    CLG_REQUIRE((int64_t)g.n * per_sample_blocks < (1ll << 31), "%s: batch too large for one launch", name);
+    CLG_REQUIRE(blocks < (1ll << 31), "%s: batch too large for one launch", name);
     return CLG_OK;
 }
 
@@ -376,10 +431,10 @@ extern "C" int clg_conv4_forward(int dtype, const clg_conv_geom *gg, const void 
     if (int e = clg_make_geom(gg, &g, "clg_conv4_forward")) return e;
     if (int e = check_dtype(dtype, "clg_conv4_forward")) return e;
     CLG_REQUIRE(x && w && selection && y, "clg_conv4_forward: null pointer argument");
-    const int pos_blocks = (int)clg_ceil_div((int64_t)g.ho * g.wo, kBlk);
-    if (int e = check_grid(g, pos_blocks, "clg_conv4_forward")) return e;
-    CLG_DISPATCH(dtype, hipLaunchKernelGGL(conv4_forward_kernel<T>, dim3((unsigned)(g.n * pos_blocks), g.c), dim3(kBlk), 0,
-                                           clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)y, g, pos_blocks));
+    const int64_t blocks = clg_ceil_div((int64_t)g.n * g.ho * g.wo, kBlk);
+    if (int e = check_grid(g, blocks, "clg_conv4_forward")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(conv4_forward_kernel<T>, dim3((unsigned)blocks, g.c), dim3(kBlk), 0,
+                                           clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)y, g));
     CLG_CHECK_LAUNCH("clg_conv4_forward");
     return CLG_OK;
 }
@@ -499,24 +554,24 @@ int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char 
 int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
                                   uint8_t *argmax, hipStream_t st)
 {
-    const int cell_blocks = (int)clg_ceil_div((int64_t)(g.ho / 2) * (g.wo / 2), kBlk);
-    if (int e = check_grid(g, cell_blocks, "clg_convblock_forward")) return e;
-    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_forward_generic_kernel<T>, dim3((unsigned)(g.n * cell_blocks), g.c),
-                                           dim3(kBlk), 0, st, (const T *)x, (const T *)w, selection, (T *)y, argmax, g,
-                                           cell_blocks));
+    const int64_t blocks = clg_ceil_div((int64_t)g.n * (g.ho / 2) * (g.wo / 2), kBlk);
+    if (int e = check_grid(g, blocks, "clg_convblock_forward")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_forward_generic_kernel<T>, dim3((unsigned)blocks, g.c), dim3(kBlk), 0, st,
+                                           (const T *)x, (const T *)w, selection, (T *)y, argmax, g));
     CLG_CHECK_LAUNCH("clg_convblock_forward(generic)");
     return CLG_OK;
 }
 
-int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
-                                     const int32_t *selection, const uint8_t *argmax, void *grad_x, hipStream_t st)
+int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *folded,
+                                     const int32_t *count, const int32_t *hits, const int32_t *selection, const uint8_t *argmax,
+                                     void *grad_x, hipStream_t st)
 {
     const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
     CLG_REQUIRE(clg_ceil_div(total, kBlk) < (1ll << 31), "clg_convblock_backward_x: input too large for one launch");
-    CLG_DISPATCH(dtype, hipLaunchKernelGGL((conv_backward_x_gather_kernel<T, true>), dim3((unsigned)clg_ceil_div(total, kBlk)),
-                                           dim3(kBlk), 0, st, (const T *)grad_y, (const T *)x, (const T *)w, selection, argmax,
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_backward_x_hits_kernel<T>, dim3((unsigned)clg_ceil_div(total, kBlk)), dim3(kBlk),
+                                           0, st, (const T *)grad_y, (const T *)x, (const T *)folded, count, hits, selection, argmax,
                                            (T *)grad_x, g));
-    CLG_CHECK_LAUNCH("clg_convblock_backward_x(generic)");
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(any shape)");
     return CLG_OK;
 }
 
@@ -541,11 +596,10 @@ extern "C" int clg_convblock_intermediates(int dtype, const clg_conv_geom *gg, c
     if (int e = clg_make_geom(gg, &g, "clg_convblock_intermediates")) return e;
     if (int e = check_dtype(dtype, "clg_convblock_intermediates")) return e;
     CLG_REQUIRE(x && w && selection, "clg_convblock_intermediates: null pointer argument");
-    const int pos_blocks = (int)clg_ceil_div((int64_t)g.ho * g.wo, kBlk);
-    if (int e = check_grid(g, pos_blocks, "clg_convblock_intermediates")) return e;
-    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_intermediates_kernel<T>, dim3((unsigned)(g.n * pos_blocks), g.c), dim3(kBlk),
-                                           0, clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)x2, (T *)x3, g,
-                                           pos_blocks));
+    const int64_t blocks = clg_ceil_div((int64_t)g.n * g.ho * g.wo, kBlk);
+    if (int e = check_grid(g, blocks, "clg_convblock_intermediates")) return e;
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_intermediates_kernel<T>, dim3((unsigned)blocks, g.c), dim3(kBlk), 0,
+                                           clg_stream(stream), (const T *)x, (const T *)w, selection, (T *)x2, (T *)x3, g));
     CLG_CHECK_LAUNCH("clg_convblock_intermediates");
     return CLG_OK;
 }
