@@ -500,6 +500,114 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     }
 }
 
+// Input gradient without an LDS copy of the input: for blocks whose sample images are too large for LDS,
+// or so small that one sample leaves most of a wavefront idle.  A wavefront owns the gradient planes of
+// one input channel for G consecutive samples (lanes = (sample, pooled cell)), keeps only those planes in
+// LDS (same shared-halo layout, private to the wavefront, so the kernel has no barriers) and reads the
+// taps from a zero-padded copy of x in global memory, which the L2 serves.  Same walk as the tiled
+// kernel: kernels that read the channel in increasing order, taps in order, read-add-write per tap.
+template <typename T>
+__global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const T *__restrict__ gy, const T *__restrict__ xp,
+                                                                        const T *__restrict__ folded,
+                                                                        const int32_t *__restrict__ count,
+                                                                        const int32_t *__restrict__ hits,
+                                                                        const int32_t *__restrict__ taps,
+                                                                        const uint8_t *__restrict__ argmax, T *__restrict__ gx,
+                                                                        Geom g, TilePlan p, int sample_elems)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    const int groups = (g.n + p.G - 1) / p.G;
+    const int item = uniform((int)blockIdx.x * p.NW + wave);           // channel fastest: a workgroup shares its samples
+    if (item >= groups * g.cin) return;
+    const int grp = item / g.cin, ch = item - grp * g.cin;
+    const int n0 = grp * p.G, g_here = min(p.G, g.n - n0);
+    const int wp = g.wo >> 1, I = p.slots;
+    T *gs = reinterpret_cast<T *>(smem) + wave * (p.xe + kWave);       // G planes + tail, then one sink element per lane
+    const int dummy = p.xe + lane;
+    for (int i = lane; i < p.xe + kWave; i += kWave) gs[i] = T(0);
+
+    const int v_here = g_here * I;
+    const int nhits = count[ch];
+    const int32_t *hit = hits + (int64_t)ch * g.c;
+    const int64_t gbase = (int64_t)n0 * g.c * I;
+    const int row_step = g.sh * p.rs;
+    for (int blk = 0; blk * kWave < v_here; ++blk) {
+        const int v = blk * kWave + lane;
+        const bool live = v < v_here;
+        uint32_t cl = live ? v : 0;
+        const uint32_t sm = fdiv(cl, p.d_slots);
+        cl -= sm * (uint32_t)I;
+        const uint32_t py = fdiv(cl, p.d_wp), px = cl - py * (uint32_t)wp;
+        const int rel = (int)((2 * py * g.sh) * p.rs + 2 * px * g.sw);
+        const int gp = (int)((n0 + sm) * (uint32_t)sample_elems) + rel;
+        const int lp = (int)(sm * p.chs) + rel;
+        const int cy = (int)((sm * g.c) * I + cl);
+        int code_n = 0;
+        T gy_n = T(0);
+        auto issue = [&](int k) {
+            const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
+            code_n = 0;
+            gy_n = T(0);
+            if (live) {
+                code_n = argmax[crow + cy];
+                gy_n = gy[crow + cy];
+            }
+        };
+        if (nhits > 0) issue(0);
+        for (int k = 0; k < nhits; ++k) {
+            const int code = code_n;
+            const T gout = gy_n;
+            if (k + 1 < nhits) issue(k + 1);
+            const int ent = hit[k];
+            const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
+            int to[8], tr_[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                to[t] = taps[c * 16 + t];
+                tr_[t] = taps[c * 16 + 8 + t];
+            }
+            Tree<T> tr;
+            const T *fc = folded + (int64_t)c * 28;
+#pragma unroll
+            for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+            const int off = (code >> 1) * row_step + (code & 1) * g.sw;
+            T tv[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) tv[t] = xp[gp + off + to[t]];
+            const TreeVals<T> tvv = eval_tree(tr, tv);
+            const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
+            const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
+            T gt[8];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if ((mask >> (2 * q)) & 3) {                         // wave-uniform: a tap of this leaf is ours
+                    const int m = q >> 1;
+                    const T g_mid = m ? g_m1 : g_m0;
+                    const T g_leaf = g_mid * ((q & 1) ? gate_db(tr.g[4 + m], tvv.leaf[q ^ 1]) : gate_da(tr.g[4 + m], tvv.leaf[q ^ 1]));
+                    gt[2 * q] = g_leaf * gate_da(tr.g[q], tv[2 * q + 1]);
+                    gt[2 * q + 1] = g_leaf * gate_db(tr.g[q], tv[2 * q]);
+                }
+            }
+            // for one tap the targets of all lanes are distinct elements; taps are applied one after the other
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if ((mask >> t) & 1) {                               // wave-uniform
+                    const int at = live ? lp + off + tr_[t] : dummy;
+                    gs[at] = gs[at] + gt[t];
+                }
+            }
+        }
+    }
+    // interior of the G planes -> gx
+    const int hw = g.h * g.w;
+    for (int e = lane; e < g_here * hw; e += kWave) {
+        const uint32_t sm = fdiv((uint32_t)e, p.d_hw), rem = (uint32_t)e - sm * (uint32_t)hw;
+        const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+        gx[((int64_t)(n0 + sm) * g.cin + ch) * hw + rem] = gs[sm * p.chs + (iy + g.ph) * p.rs + ix + g.pw];
+    }
+}
+
 // gx = ((part[0] + part[1]) + part[2]) + ... : partial gradient images of a split hit list, fixed order
 template <typename T>
 __global__ __launch_bounds__(256) void sum_partial_images_kernel(const T *__restrict__ part, T *__restrict__ gx, int64_t total, int hs)
@@ -741,6 +849,66 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * I < (1ll << 31);
 }
 
+// Plan of the input-gradient kernel that reads taps from a padded global copy of x.
+bool plan_backward_x_direct(const Geom &g, int elem, TilePlan *p, int *sample_elems)
+{
+    if (!taps_inside(g) || g.c > 65535) return false;
+    plan_common(g, p);
+    const int I = (g.ho / 2) * (g.wo / 2);
+    if (I < 1) return false;
+    p->slots = I;
+    p->CT = 0;
+    p->d_slots = make_fastdiv((uint32_t)I);
+    int G = I >= kWave ? 1 : kWave / I;
+    if (G > g.n) G = g.n;
+    p->G = G;
+    p->S = G;
+    p->bands = 1;
+    p->band_rows = g.h;
+    p->hit_split = 1;
+    p->part_stride = 0;
+    p->dummy_in_halo = 0;
+    p->xe = (int)(((int64_t)G * p->chs + g.ph * p->rs + g.pw + 3) & ~3ll);
+    int nw = 4;
+    while (nw > 1 && (int64_t)nw * (p->xe + kWave) * elem > 64 * 1024) nw /= 2;
+    p->NW = nw;
+    p->lds_bytes = (size_t)nw * (p->xe + kWave) * elem;
+    if (p->lds_bytes > (size_t)kLdsLimit) return false;
+    const int64_t se = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
+    if (se * g.n >= (1ll << 31) || (int64_t)G * g.c * I >= (1ll << 31)) return false;
+    if (clg_ceil_div(clg_ceil_div(g.n, G) * g.cin, nw) >= (1ll << 31)) return false;
+    *sample_elems = (int)se;
+    return true;
+}
+
+enum BwdXMode { kBwdXGather = 0, kBwdXTiled = 1, kBwdXDirect = 2 };
+
+// Tiled (input image in LDS) when a wavefront pass is reasonably full there; the direct kernel when the
+// image does not fit or fills at least twice as many lanes; the per-element gather for everything else.
+BwdXMode choose_backward_x(const Geom &g, int elem, TilePlan *p, int *sample_elems)
+{
+    TilePlan pt, pd;
+    int se = 0;
+    const bool tiled = plan_backward_x(g, elem, &pt);
+    const bool direct = plan_backward_x_direct(g, elem, &pd, &se);
+    const int I = (g.ho / 2) * (g.wo / 2);
+    auto lanes = [&](const TilePlan &q) { return q.G * I < kWave ? q.G * I : kWave; };
+    bool use_direct = direct && (!tiled || lanes(pd) >= 2 * lanes(pt));
+    if (const char *e = getenv("CLG_BWDX_DIRECT")) use_direct = direct && (atoi(e) != 0 || !tiled);
+    if (use_direct) {
+        *p = pd;
+        *sample_elems = se;
+        return kBwdXDirect;
+    }
+    if (tiled) {
+        *p = pt;
+        return kBwdXTiled;
+    }
+    return kBwdXGather;
+}
+
+size_t bwd_x_direct_xp_off(const BwdScratch &lay) { return (lay.total + 255) & ~(size_t)255; }
+
 // weight gradient from the padded copy: scratch = partials | folded | taps | padded x
 struct WScratch {
     int nb, sample_elems;
@@ -875,6 +1043,30 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
 }
 
 template <typename T>
+int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems, const void *gy, const void *x, const void *w,
+                             const int32_t *sel, const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
+{
+    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), 1);
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    T *xp = reinterpret_cast<T *>(base + bwd_x_direct_xp_off(lay));
+    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st)) return e;
+    TilePlan pp = p;
+    pp.d_slots = make_fastdiv((uint32_t)p.chs);                      // the pad kernel divides by the plane stride
+    const int64_t total = (int64_t)sample_elems * g.n;
+    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, pp,
+                       make_fastdiv((uint32_t)sample_elems), make_fastdiv((uint32_t)p.rs), sample_elems, total);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(pad)");
+    if (int e = allow_lds(convblock_backward_x_direct_kernel<T>, p.lds_bytes, "clg_convblock_backward_x")) return e;
+    const int64_t items = clg_ceil_div(g.n, p.G) * g.cin;
+    hipLaunchKernelGGL(convblock_backward_x_direct_kernel<T>, dim3((unsigned)clg_ceil_div(items, p.NW)), dim3(p.NW * kWave),
+                       p.lds_bytes, st, (const T *)gy, (const T *)xp, reinterpret_cast<const T *>(base),
+                       reinterpret_cast<const int32_t *>(base + lay.count_off), reinterpret_cast<const int32_t *>(base + lay.hits_off),
+                       reinterpret_cast<const int32_t *>(base + lay.taps_off), argmax, (T *)gx, g, p, sample_elems);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_x(direct)");
+    return CLG_OK;
+}
+
+template <typename T>
 int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &ws, const void *gy, const void *x, const void *w,
                              const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st)
 {
@@ -921,8 +1113,11 @@ extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_c
     Geom g;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x_scratch_bytes")) return -1;
     TilePlan p;
-    const int hs = plan_backward_x(g, elem_size(dtype), &p) ? p.hit_split : 1;
-    return (int64_t)bwd_scratch_layout(g, elem_size(dtype), hs).total;
+    int se = 0;
+    const BwdXMode mode = choose_backward_x(g, elem_size(dtype), &p, &se);
+    const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), mode == kBwdXTiled ? p.hit_split : 1);
+    if (mode == kBwdXDirect) return (int64_t)(bwd_x_direct_xp_off(lay) + (size_t)se * g.n * elem_size(dtype));
+    return (int64_t)lay.total;
 }
 
 extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -933,22 +1128,27 @@ extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, cons
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x")) return e;
     CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_x && scratch, "clg_convblock_backward_x: null pointer argument");
     TilePlan p;
-    if (plan_backward_x(g, elem_size(dtype), &p)) {
-        if (dtype == CLG_F32)
-            return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
-        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, clg_stream(stream));
+    int se = 0;
+    const BwdXMode mode = choose_backward_x(g, elem_size(dtype), &p, &se);
+    hipStream_t st = clg_stream(stream);
+    if (mode == kBwdXTiled) {
+        if (dtype == CLG_F32) return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st);
+        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st);
+    }
+    if (mode == kBwdXDirect) {
+        if (dtype == CLG_F32) return launch_backward_x_direct<float>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st);
+        return launch_backward_x_direct<double>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st);
     }
     // any other shape: per-element gather driven by the same per-channel kernel lists
     const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     if (dtype == CLG_F32) {
-        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, clg_stream(stream))) return e;
+        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st)) return e;
     } else {
-        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, clg_stream(stream))) return e;
+        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st)) return e;
     }
     return clg_convblock_backward_x_generic(dtype, g, grad_y, x, scratch, reinterpret_cast<const int32_t *>(base + lay.count_off),
-                                            reinterpret_cast<const int32_t *>(base + lay.hits_off), selection, argmax, grad_x,
-                                            clg_stream(stream));
+                                            reinterpret_cast<const int32_t *>(base + lay.hits_off), selection, argmax, grad_x, st);
 }
 
 extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_conv_geom *gg)

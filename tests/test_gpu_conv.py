@@ -87,7 +87,11 @@ def _run_block(n, cin, cout, h, w, stride, pad, kernel, dtype=torch.float32, bin
 
 @pytest.mark.parametrize("stride,pad,kernel", GEOMS)
 @pytest.mark.parametrize("binary", [False, True])
-def test_block_forward_backward_small(stride, pad, kernel, binary):
+@pytest.mark.parametrize("direct", [None, "1"])
+def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monkeypatch):
+    # direct="1" forces the input-gradient kernel that reads taps from a padded global copy of x
+    if direct:
+        monkeypatch.setenv("CLG_BWDX_DIRECT", direct)
     n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad
     if ((h + 2 * pad - kernel) // stride + 1) % 2:
         h += stride
@@ -181,6 +185,23 @@ def test_block_benchmark_shapes_vs_oracle(shape):
     routed, y_ref, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
     flips = check_pool_route(idx, idx_ref, x4)
     assert flips <= 1e-4 * idx.numel(), flips
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
+    routed.backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+
+
+@pytest.mark.parametrize("shape", [(37, 24, 48, 4, 4), (5, 200, 40, 16, 16), (3, 64, 32, 32, 32), (9, 40, 24, 6, 6),
+                                   (70, 6, 12, 2, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_block_deep_and_wide_shapes_vs_oracle(shape, dtype):
+    # few cells per sample (several samples share a wavefront, ragged last group) and images too large for LDS
+    n, cin, cout, h, w = shape
+    layer, x, y, idx = _run_block(n, cin, cout, h, w, 1, 1, 3, dtype=dtype, seed=n)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    routed, y_ref, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
+    check_pool_route(idx, idx_ref, x4)
     assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
     routed.backward(gy.cpu())
     assert_grad_close(x.grad, xl.grad, name="grad_x")
