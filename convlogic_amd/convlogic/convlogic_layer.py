@@ -109,8 +109,10 @@ class ConvLogicLayer(nn.Module):
         assert self.weights.shape[-1] == 16, f"Expected 16 logic functions, got {self.weights.shape[-1]}"
 
     def forward(self, x):
+        if isinstance(x, PackBitsTensor):
+            return self.forward_cuda_eval(x)
         x = x.contiguous()
-        if self.grad_factor != 1.0 and not isinstance(x, PackBitsTensor):
+        if self.grad_factor != 1.0:
             x = GradFactor.apply(x, self.grad_factor)
         if self.implementation == "cuda":
             return self.forward_cuda(x)
@@ -158,6 +160,29 @@ class ConvLogicLayer(nn.Module):
         if self.complete:
             return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)
         return ConvLogicFunction.apply(x, w_prob, sel, *geo)
+
+    def forward_cuda_eval(self, x: PackBitsTensor):
+        """Packed-bit inference of the complete block on a group-major image batch: replaces x.t by the
+        block output, 64 samples per word (the counterpart of LogicLayer.forward_cuda_eval,
+        src/difflogic/difflogic.py:149-164, for the fused block; arg-max gates as in :321-325 of
+        src/convlogic/convlogic_layer.py, max pool of {0,1} values = OR)."""
+        assert not self.training, "packed evaluation needs eval mode"
+        assert self.complete, "packed evaluation is implemented for the complete block only"
+        if self.implementation != "cuda":
+            raise RuntimeError("packed evaluation needs implementation='cuda'")
+        assert x.image and x.t.dim() == 4 and x.t.shape[1] == self.in_channels, (x.image, tuple(x.t.shape), self.in_channels)
+        x.t = convlogic_hip.full_convlogic_eval_packed(x.t.contiguous(), self._eval_gates(), self.selection.contiguous(),
+                                                       *self.stride, *self.padding, *self.kernel)
+        return x
+
+    def _eval_gates(self):
+        """uint8 [C, 7] arg-max gate ids, recomputed only after the logits changed."""
+        key = (self.weights._version, self.weights.data_ptr())
+        cached = getattr(self, "_gate_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8).contiguous())
+            self._gate_cache = cached
+        return cached[1]
 
     def extra_repr(self):
         return f"in_channels={self.in_channels}, out_channels={self.out_channels}, groups={self.groups}"

@@ -126,4 +126,26 @@ struct Tap {
 };
 __device__ __forceinline__ Tap unpack_tap(int32_t s) { return Tap{(s >> 16) & 0xFFFF, (s >> 8) & 0xFF, s & 0xFF}; }
 
+// ---- bitwise gates on packed samples ---------------------------------------------------------
+struct Masks {
+    uint32_t f00, f01, f10, f11;  // all-ones / all-zeros per truth-table entry
+};
+__device__ __forceinline__ Masks gate_masks(int id)
+{
+    return Masks{0u - ((id >> 3) & 1u), 0u - ((id >> 2) & 1u), 0u - ((id >> 1) & 1u), 0u - (id & 1u)};
+}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// 2:1 multiplexers on bits: b selects inside each half, a selects the half.  V is uint32_t or a
+// vector of them (the masks are splat).
+template <typename V>
+__device__ __forceinline__ V gate_vec(const Masks &m, V a, V b)
+{
+    const V t1 = (b & (V)m.f11) | (~b & (V)m.f10);
+    const V t0 = (b & (V)m.f01) | (~b & (V)m.f00);
+    return (a & t1) | (~a & t0);
+}
+__device__ __forceinline__ uint32_t gate_bits(const Masks &m, uint32_t a, uint32_t b) { return gate_vec<uint32_t>(m, a, b); }
+
 #endif  // __HIPCC__

@@ -24,7 +24,7 @@
 
 #include <mutex>
 
-#include "conv_common.h"
+#include "conv_tile.h"
 
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
 int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
@@ -39,171 +39,6 @@ int clg_convblock_partial_blocks(const Geom &g);
 int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name);
 
 namespace {
-
-constexpr int kLdsLimit = 160 * 1024;
-
-// Division of a 31-bit value by a runtime constant: q = umulhi(x, mul) >> shr (d == 1: q = x).
-struct FastDiv {
-    uint32_t mul, shr, d;
-};
-FastDiv make_fastdiv(uint32_t d)
-{
-    if (d <= 1) return FastDiv{0, 0, 1};
-    uint32_t lg = 0;
-    while ((1ull << lg) < d) ++lg;
-    const uint32_t p = 31 + lg;
-    const uint32_t mul = (uint32_t)(((1ull << p) + d - 1) / d);
-    return FastDiv{mul, p - 32, d};
-}
-__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv &f) { return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shr); }
-
-struct TilePlan {
-    int S;              // samples per workgroup
-    int G;              // samples sharing one wavefront pass (input gradient; 1 when a sample has >= 64 cells)
-    int CT;             // kernels per workgroup (forward)
-    int NW;             // wavefronts per workgroup
-    int rs, chs;        // row and plane stride of the LDS image (elements)
-    int xe;             // elements of one LDS image region (S samples + tail)
-    int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
-    int band_rows, bands;  // input gradient: image rows per workgroup band, number of bands
-    int hit_split;         // input gradient: workgroups sharing the kernels of one (sample, band), partial images
-    int dummy_in_halo;     // input gradient: masked updates go to halo elements instead of a region of their own
-    int64_t part_stride;   // input gradient: elements between partial images (0 when hit_split == 1)
-    FastDiv d_hw, d_w, d_slots, d_wo, d_wp;
-    size_t lds_bytes;
-};
-
-template <typename T>
-__device__ __forceinline__ T dpp_xor1(T v)
-{
-    if constexpr (sizeof(T) == 4) {
-        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
-    } else {
-        const uint64_t u = __builtin_bit_cast(uint64_t, v);
-        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, false);
-        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, false);
-        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
-    }
-}
-
-template <typename T>
-__device__ __forceinline__ T to_sgpr(T v)
-{
-    if constexpr (sizeof(T) == 4) {
-        return __builtin_bit_cast(T, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
-    } else {
-        const uint64_t u = __builtin_bit_cast(uint64_t, v);
-        const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)u);
-        const uint32_t hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
-        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
-    }
-}
-
-// Stages the planes of `samples` consecutive samples into the zeroed LDS image.
-template <typename T>
-__device__ __forceinline__ void stage_image(T *__restrict__ xs, const T *__restrict__ src, int samples, const Geom &g,
-                                            const TilePlan &p, int tid, int nthreads)
-{
-    const uint32_t total = (uint32_t)samples * g.cin * g.h * g.w;
-    for (uint32_t e = tid; e < total; e += nthreads) {
-        const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)(g.h * g.w);
-        const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
-        xs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw] = src[e];
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// forward
-// ---------------------------------------------------------------------------------------------
-// ROWSTEP: elements between conv rows 2r and 2r+1 in the LDS image when known at compile time (the
-// second row's reads then use the immediate offset of the LDS instruction), 0 = read it from the plan.
-template <typename T, int ROWSTEP>
-__global__ void convblock_forward_tiled_kernel(const T *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ sel,
-                                               T *__restrict__ y, uint8_t *__restrict__ argmax, Geom g, TilePlan p)
-{
-    extern __shared__ __align__(16) unsigned char smem[];
-    T *xs = reinterpret_cast<T *>(smem);
-    T *coef = xs + ((p.xe + 3) & ~3);                                 // [CT][28]
-    int *toff = reinterpret_cast<int *>(coef + p.CT * 28);            // [CT][8]
-    int2 *slot = reinterpret_cast<int2 *>(toff + p.CT * 8);           // [S * slots]
-
-    const int tid = threadIdx.x, nthreads = blockDim.x;
-    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
-    const int n0 = blockIdx.x * p.S, s_cur = min(p.S, g.n - n0);
-    const int c0 = blockIdx.y * p.CT, ct_cur = min(p.CT, g.c - c0);
-    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
-
-    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
-    for (int q = tid; q < ct_cur * 7; q += nthreads) {
-        const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
-        coef[q * 4 + 0] = cf.ab;
-        coef[q * 4 + 1] = cf.a;
-        coef[q * 4 + 2] = cf.b;
-        coef[q * 4 + 3] = cf.one;
-    }
-    for (int q = tid; q < ct_cur * 8; q += nthreads) {
-        const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
-        toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
-    }
-    const int U = s_cur * p.slots;
-    for (int u = tid; u < U; u += nthreads) {
-        const uint32_t s = fdiv(u, p.d_slots), r = u - s * (uint32_t)p.slots;
-        const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
-        slot[u] = make_int2((int)(s * g.cin * p.chs + (2 * rp * g.sh) * p.rs + ox * g.sw), (int)((s * g.c) * I + rp * wp + (ox >> 1)));
-    }
-    __syncthreads();
-    stage_image(xs, x + (int64_t)n0 * g.cin * g.h * g.w, s_cur, g, p, tid, nthreads);
-    __syncthreads();
-
-    const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
-    // work items = (kernel, block of 64 slots), kernel-major; every wavefront takes a contiguous range, so
-    // the scalar coefficients are reloaded only when its range crosses into the next kernel
-    const int nblk = (U + kWave - 1) / kWave;
-    const int items = ct_cur * nblk;
-    const int per = (items + p.NW - 1) / p.NW;
-    const int first = wave * per, last = min(items, first + per);
-    int lc = first / nblk, blk = first - lc * nblk;
-    for (int item = first; item < last;) {
-        Tree<T> tr;
-#pragma unroll
-        for (int k = 0; k < 7; ++k) {
-            tr.g[k].ab = to_sgpr(coef[(lc * 7 + k) * 4 + 0]);
-            tr.g[k].a = to_sgpr(coef[(lc * 7 + k) * 4 + 1]);
-            tr.g[k].b = to_sgpr(coef[(lc * 7 + k) * 4 + 2]);
-            tr.g[k].one = to_sgpr(coef[(lc * 7 + k) * 4 + 3]);
-        }
-        int to[8];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) to[t] = uniform(toff[lc * 8 + t]);
-        const int64_t obase = ((int64_t)n0 * g.c + c0 + lc) * I;
-        T *yb = y + obase;
-        uint8_t *ab = argmax + obase;
-        for (; blk < nblk && item < last; ++blk, ++item) {
-            const int u = blk * kWave + lane;
-            const bool valid = u < U;
-            const int2 e = slot[valid ? u : 0];
-            T v[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) v[t] = xs[e.x + to[t]];
-            const T r0 = eval_tree(tr, v).root;
-#pragma unroll
-            for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
-            const T r1 = eval_tree(tr, v).root;
-            const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
-            if (valid && !(lane & 1)) {
-                T best = r0;
-                int code = 0;
-                if (r0o > best) { best = r0o; code = 1; }
-                if (r1 > best) { best = r1; code = 2; }
-                if (r1o > best) { best = r1o; code = 3; }
-                yb[e.y] = best;
-                ab[e.y] = (uint8_t)code;
-            }
-        }
-        blk = 0;
-        ++lc;
-    }
-}
 
 // ---------------------------------------------------------------------------------------------
 // input gradient
@@ -730,53 +565,6 @@ __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const T *__res
 // ---------------------------------------------------------------------------------------------
 // plans
 // ---------------------------------------------------------------------------------------------
-void plan_common(const Geom &g, TilePlan *p)
-{
-    p->rs = g.w + g.pw;
-    p->chs = (g.h + g.ph) * p->rs;
-    p->d_hw = make_fastdiv((uint32_t)(g.h * g.w));
-    p->d_w = make_fastdiv((uint32_t)g.w);
-    p->d_wo = make_fastdiv((uint32_t)g.wo);
-    p->d_wp = make_fastdiv((uint32_t)(g.wo / 2));
-}
-
-int64_t image_elems(const Geom &g, const TilePlan &p, int S) { return (int64_t)S * g.cin * p.chs + g.ph * p.rs + g.pw; }
-
-// The last tap row/column must stay inside the padded image for the shared-halo layout to hold.
-bool taps_inside(const Geom &g) { return (g.ho - 1) * g.sh + g.kh <= g.h + 2 * g.ph && (g.wo - 1) * g.sw + g.kw <= g.w + 2 * g.pw; }
-
-bool plan_forward(const Geom &g, int elem, TilePlan *p)
-{
-    if (!taps_inside(g)) return false;
-    plan_common(g, p);
-    p->slots = (g.ho / 2) * g.wo;
-    p->G = 1;
-    // samples per workgroup: best lane utilisation within a 64 KiB image, smallest S on ties
-    int best_s = 0;
-    double best_util = 0;
-    for (int S = 1; S <= 16 && S <= g.n; ++S) {
-        if (image_elems(g, *p, S) * elem + (int64_t)S * p->slots * 8 > 64 * 1024 && S > 1) break;
-        const int64_t U = (int64_t)S * p->slots;
-        const double util = (double)U / (double)(clg_ceil_div(U, kWave) * kWave);
-        if (util > best_util + 0.02) { best_util = util; best_s = S; }
-    }
-    if (best_s == 0 || best_util < 0.4) return false;
-    p->S = best_s;
-    // 16 wavefronts share one staged image: measured 69 us against 109 us with 4 at [256,9,32,32] -> 256
-    p->NW = 16;
-    const int64_t groups = clg_ceil_div(g.n, p->S);
-    int64_t ct = (int64_t)g.c * groups / 1024;
-    ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
-    if (ct > g.c) ct = g.c;
-    p->CT = (int)ct;
-    p->xe = (int)image_elems(g, *p, p->S);
-    p->d_slots = make_fastdiv((uint32_t)p->slots);
-    p->lds_bytes = (size_t)((p->xe + 3) & ~3) * elem + (size_t)p->CT * 28 * elem + (size_t)p->CT * 8 * 4 + (size_t)p->S * p->slots * 8;
-    if (p->lds_bytes > (size_t)kLdsLimit) return false;
-    if (clg_ceil_div(g.c, p->CT) > 65535) return false;
-    return (int64_t)p->S * g.cin * p->chs < (1ll << 30) && (int64_t)p->S * g.c * ((g.ho / 2) * (g.wo / 2)) < (1ll << 31);
-}
-
 bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
 {
     if (!taps_inside(g) || g.c > 65535) return false;
@@ -935,66 +723,6 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     return true;
 }
 
-// Kernels that want more than 48 KiB of dynamic LDS must be told once; the largest size granted so
-// far is remembered per kernel so that steady-state launches make no runtime call besides the launch.
-int allow_lds_ptr(const void *kernel, size_t bytes, const char *name)
-{
-    static std::mutex mu;
-    static const void *known[32];
-    static size_t granted[32];
-    static int used = 0;
-    if (bytes <= 48 * 1024) return CLG_OK;
-    std::lock_guard<std::mutex> lock(mu);
-    int slot = -1;
-    for (int i = 0; i < used; ++i)
-        if (known[i] == kernel) slot = i;
-    if (slot >= 0 && granted[slot] >= bytes) return CLG_OK;
-    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) {
-        clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
-        return CLG_ELAUNCH;
-    }
-    if (slot < 0 && used < 32) slot = used++;
-    if (slot >= 0) {
-        known[slot] = kernel;
-        granted[slot] = bytes;
-    }
-    return CLG_OK;
-}
-template <typename K>
-int allow_lds(K kernel, size_t bytes, const char *name)
-{
-    return allow_lds_ptr(reinterpret_cast<const void *>(kernel), bytes, name);
-}
-
-template <typename T, int ROWSTEP>
-int launch_forward_tiled_rs(const Geom &g, const TilePlan &p, const void *x, const void *w, const int32_t *sel, void *y,
-                            uint8_t *argmax, hipStream_t st)
-{
-    if (int e = allow_lds(convblock_forward_tiled_kernel<T, ROWSTEP>, p.lds_bytes, "clg_convblock_forward")) return e;
-    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
-    hipLaunchKernelGGL((convblock_forward_tiled_kernel<T, ROWSTEP>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
-                       (const T *)w, sel, (T *)y, argmax, g, p);
-    CLG_CHECK_LAUNCH("clg_convblock_forward(tiled)");
-    return CLG_OK;
-}
-
-// Row steps of 3x3 / padding 1 / stride 1 blocks on 32, 28, 16, 8 and 4 pixel wide images get their own
-// instantiation; everything else reads the step from the plan.
-template <typename T>
-int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const void *w, const int32_t *sel, void *y,
-                         uint8_t *argmax, hipStream_t st)
-{
-    switch (g.sh * p.rs) {
-    case 33: return launch_forward_tiled_rs<T, 33>(g, p, x, w, sel, y, argmax, st);
-    case 29: return launch_forward_tiled_rs<T, 29>(g, p, x, w, sel, y, argmax, st);
-    case 17: return launch_forward_tiled_rs<T, 17>(g, p, x, w, sel, y, argmax, st);
-    case 9: return launch_forward_tiled_rs<T, 9>(g, p, x, w, sel, y, argmax, st);
-    case 5: return launch_forward_tiled_rs<T, 5>(g, p, x, w, sel, y, argmax, st);
-    default: return launch_forward_tiled_rs<T, 0>(g, p, x, w, sel, y, argmax, st);
-    }
-}
-
 // folded coefficients, per-channel kernel lists and tap offsets (for LDS rows of rs, planes of chs elements)
 template <typename T>
 int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const void *w, const int32_t *sel, void *scratch,
@@ -1094,18 +822,31 @@ int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
 
 }  // namespace
 
-extern "C" int clg_convblock_forward(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
-                                     void *y, uint8_t *argmax, void *stream)
+// Kernels that want more than 48 KiB of dynamic LDS must be told once; the largest size granted so
+// far is remembered per kernel so that steady-state launches make no runtime call besides the launch.
+int clg_allow_lds(const void *kernel, size_t bytes, const char *name)
 {
-    Geom g;
-    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_forward")) return e;
-    CLG_REQUIRE(x && w && selection && y && argmax, "clg_convblock_forward: null pointer argument");
-    TilePlan p;
-    if (plan_forward(g, elem_size(dtype), &p)) {
-        if (dtype == CLG_F32) return launch_forward_tiled<float>(g, p, x, w, selection, y, argmax, clg_stream(stream));
-        return launch_forward_tiled<double>(g, p, x, w, selection, y, argmax, clg_stream(stream));
+    static std::mutex mu;
+    static const void *known[32];
+    static size_t granted[32];
+    static int used = 0;
+    if (bytes <= 48 * 1024) return CLG_OK;
+    std::lock_guard<std::mutex> lock(mu);
+    int slot = -1;
+    for (int i = 0; i < used; ++i)
+        if (known[i] == kernel) slot = i;
+    if (slot >= 0 && granted[slot] >= bytes) return CLG_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+        return CLG_ELAUNCH;
     }
-    return clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, clg_stream(stream));
+    if (slot < 0 && used < 32) slot = used++;
+    if (slot >= 0) {
+        known[slot] = kernel;
+        granted[slot] = bytes;
+    }
+    return CLG_OK;
 }
 
 extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_conv_geom *gg)

@@ -1,0 +1,418 @@
+// Fused conv-logic block, forward: LDS-tiled kernel for gfx950 in two element flavours.
+//
+//   float / double  relaxed gates in the folded form, 2x2 max pool with a 1-byte arg-max code
+//   uint64_t        64 samples per element (bit s of word group g = sample 64 g + s), gates as bitwise
+//                   multiplexers, 2x2 pool = OR, no arg-max
+//
+// Both read images laid out [n, c_in, h, w] (for packed words n counts 64-sample groups) and write
+// [n, c_out, ho/2, wo/2], so staging, tap addressing and the lane mapping are shared.
+//
+// A workgroup owns (S samples) x (CT kernels) and stages zero-padded input planes in LDS with shared
+// halos (row stride rs = w + pw, plane stride chs = (h + ph) * rs): either all input channels of its
+// samples, or -- for layers with many input channels -- only the (at most two) channels each kernel of
+// its tile reads, two LDS planes per kernel.  A kernel whose taps name more than two channels (possible
+// with a caller-made selection) reads its taps from global memory instead.  Lanes run along conv-output
+// columns, each lane evaluates the tree at conv rows 2r and 2r+1, the horizontal neighbour comes over
+// DPP, and the even lane pools and writes.  The kernel index is uniform per wavefront, so gate
+// parameters and tap offsets sit in scalar registers.
+#include <stdlib.h>
+
+#include "conv_tile.h"
+
+int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
+int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
+                                  uint8_t *argmax, hipStream_t st);
+
+namespace {
+
+// ---- element policies ------------------------------------------------------------------------
+template <typename T>
+struct FloatOps {
+    using Elem = T;
+    static constexpr int kParams = 28;                               // LDS elements per kernel: 7 gates x (ab, a, b, one)
+    struct Params {
+        Tree<T> tr;
+    };
+    // params = gate probabilities [c_out, 7, 16]
+    static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
+                                                        int tid, int nthreads)
+    {
+        const T *w = reinterpret_cast<const T *>(params);
+        for (int q = tid; q < ct_cur * 7; q += nthreads) {
+            const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
+            dst[q * 4 + 0] = cf.ab;
+            dst[q * 4 + 1] = cf.a;
+            dst[q * 4 + 2] = cf.b;
+            dst[q * 4 + 3] = cf.one;
+        }
+    }
+    static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
+    {
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            pr.tr.g[k].ab = to_sgpr(src[(lc * 7 + k) * 4 + 0]);
+            pr.tr.g[k].a = to_sgpr(src[(lc * 7 + k) * 4 + 1]);
+            pr.tr.g[k].b = to_sgpr(src[(lc * 7 + k) * 4 + 2]);
+            pr.tr.g[k].one = to_sgpr(src[(lc * 7 + k) * 4 + 3]);
+        }
+        return pr;
+    }
+    static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8]) { return eval_tree(pr.tr, v).root; }
+    // strict > in window order (0,0),(0,1),(1,0),(1,1): the first maximum wins
+    static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
+                                                      uint8_t *__restrict__ ab, int idx)
+    {
+        Elem best = r0;
+        int code = 0;
+        if (r0o > best) { best = r0o; code = 1; }
+        if (r1 > best) { best = r1; code = 2; }
+        if (r1o > best) { best = r1o; code = 3; }
+        yb[idx] = best;
+        ab[idx] = (uint8_t)code;
+    }
+};
+
+struct BitOps {
+    using Elem = uint64_t;
+    static constexpr int kParams = 1;                                // 7 gate ids, 4 bits each
+    struct Params {
+        Masks m[7];
+    };
+    // params = gate ids uint8 [c_out, 7]
+    static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
+                                                        int tid, int nthreads)
+    {
+        const uint8_t *gid = reinterpret_cast<const uint8_t *>(params);
+        for (int q = tid; q < ct_cur; q += nthreads) {
+            uint64_t pk = 0;
+            for (int k = 0; k < 7; ++k) pk |= (uint64_t)(gid[((int64_t)c0 + q) * 7 + k] & 15) << (4 * k);
+            dst[q] = pk;
+        }
+    }
+    static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
+    {
+        const uint32_t pk = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src[lc]);
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks((pk >> (4 * k)) & 15);
+        return pr;
+    }
+    static __device__ __forceinline__ Elem gate64(const Masks &m, Elem a, Elem b)
+    {
+        const uint32_t lo = gate_bits(m, (uint32_t)a, (uint32_t)b), hi = gate_bits(m, (uint32_t)(a >> 32), (uint32_t)(b >> 32));
+        return ((uint64_t)hi << 32) | lo;
+    }
+    static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8])
+    {
+        Elem leaf[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) leaf[q] = gate64(pr.m[q], v[2 * q], v[2 * q + 1]);
+        return gate64(pr.m[6], gate64(pr.m[4], leaf[0], leaf[1]), gate64(pr.m[5], leaf[2], leaf[3]));
+    }
+    static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
+                                                      uint8_t *__restrict__, int idx)
+    {
+        yb[idx] = (r0 | r0o) | (r1 | r1o);
+    }
+};
+
+// ---- kernel ------------------------------------------------------------------------------------
+// ROWSTEP: elements between conv rows 2r and 2r+1 in the LDS image when known at compile time (the
+// second row's reads then use the immediate offset of the LDS instruction), 0 = read it from the plan.
+// SUBSET: stage two planes per kernel of the tile instead of all input channels.
+template <typename Ops, int ROWSTEP, bool SUBSET>
+__global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
+                                               const int32_t *__restrict__ sel, typename Ops::Elem *__restrict__ y,
+                                               uint8_t *__restrict__ argmax, Geom g, TilePlan p)
+{
+    using T = typename Ops::Elem;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *xs = reinterpret_cast<T *>(smem);
+    T *coef = xs + ((p.xe + 3) & ~3);                                 // [CT][kParams]
+    int *toff = reinterpret_cast<int *>(coef + ((p.CT * Ops::kParams + 1) & ~1));   // [CT][8]
+    int *chan = toff + p.CT * 8;                                      // [2 CT]  channel of every LDS plane (SUBSET)
+    int *wide = chan + 2 * p.CT;                                      // [CT]    kernel reads more than two channels (SUBSET)
+    int2 *slot = reinterpret_cast<int2 *>(wide + ((p.CT + 1) & ~1));  // [S * slots]
+
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
+    const int n0 = blockIdx.x * p.S, s_cur = min(p.S, g.n - n0);
+    const int c0 = blockIdx.y * p.CT, ct_cur = min(p.CT, g.c - c0);
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+    const int hw = g.h * g.w;
+
+    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
+    Ops::stage_params(coef, params, c0, ct_cur, tid, nthreads);
+    if (!SUBSET) {
+        for (int q = tid; q < ct_cur * 8; q += nthreads) {
+            const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
+            toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
+        }
+    } else {
+        for (int q = tid; q < p.CT; q += nthreads) {
+            int ch_a = 0, ch_b = 0, wd = 0;
+            if (q < ct_cur) {
+                const int32_t *sq = sel + ((int64_t)c0 + q) * 8;
+                ch_a = ch_b = unpack_tap(sq[0]).ch;
+                for (int t = 7; t >= 1; --t)
+                    if (unpack_tap(sq[t]).ch != ch_a) ch_b = unpack_tap(sq[t]).ch;   // ends on the first other channel
+                for (int t = 0; t < 8; ++t) {
+                    const Tap tp = unpack_tap(sq[t]);
+                    int pl = 2 * q;
+                    if (tp.ch == ch_b) pl = 2 * q + 1;
+                    if (tp.ch == ch_a) pl = 2 * q;
+                    if (tp.ch != ch_a && tp.ch != ch_b) wd = 1;
+                    toff[q * 8 + t] = pl * p.chs + tp.ry * p.rs + tp.rx;
+                }
+            }
+            chan[2 * q] = ch_a;
+            chan[2 * q + 1] = ch_b;
+            wide[q] = wd;
+        }
+    }
+    const int U = s_cur * p.slots;
+    for (int u = tid; u < U; u += nthreads) {
+        const uint32_t s = fdiv(u, p.d_slots), r = u - s * (uint32_t)p.slots;
+        const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
+        slot[u] = make_int2((int)(s * p.planes * p.chs + (2 * rp * g.sh) * p.rs + ox * g.sw), (int)((s * g.c) * I + rp * wp + (ox >> 1)));
+    }
+    __syncthreads();
+    {
+        // planes of the samples into the zeroed LDS image
+        const T *src = x + (int64_t)n0 * g.cin * hw;
+        const uint32_t total = (uint32_t)(s_cur * p.planes) * (uint32_t)hw;
+        for (uint32_t e = tid; e < total; e += nthreads) {
+            const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)hw;
+            const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+            T v;
+            if (!SUBSET) {
+                v = src[e];
+            } else {
+                const uint32_t s = fdiv(plane, p.d_planes), pl = plane - s * (uint32_t)p.planes;
+                v = src[((int64_t)s * g.cin + chan[pl]) * hw + rem];
+            }
+            xs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw] = v;
+        }
+    }
+    __syncthreads();
+
+    const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
+    // work items = (kernel, block of 64 slots), kernel-major; every wavefront takes a contiguous range, so
+    // the scalar parameters are reloaded only when its range crosses into the next kernel
+    const int nblk = (U + kWave - 1) / kWave;
+    const int items = ct_cur * nblk;
+    const int per = (items + p.NW - 1) / p.NW;
+    const int first = wave * per, last = min(items, first + per);
+    int lc = first / nblk, blk = first - lc * nblk;
+    for (int item = first; item < last;) {
+        const typename Ops::Params pr = Ops::load(coef, lc);
+        int to[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) to[t] = uniform(toff[lc * 8 + t]);
+        const bool from_global = SUBSET && uniform(wide[lc]) != 0;
+        const int64_t obase = ((int64_t)n0 * g.c + c0 + lc) * I;
+        T *yb = y + obase;
+        uint8_t *ab = argmax ? argmax + obase : nullptr;
+        for (; blk < nblk && item < last; ++blk, ++item) {
+            const int u = blk * kWave + lane;
+            const bool valid = u < U;
+            const int2 e = slot[valid ? u : 0];
+            T v[8];
+            T r0, r1;
+            if (!from_global) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = xs[e.x + to[t]];
+                r0 = Ops::root(pr, v);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
+                r1 = Ops::root(pr, v);
+            } else {
+                const uint32_t uu = valid ? u : 0;
+                const uint32_t s = fdiv(uu, p.d_slots), r = uu - s * (uint32_t)p.slots;
+                const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
+                const T *xn = x + (int64_t)(n0 + s) * g.cin * hw;
+                const int32_t *sq = sel + ((int64_t)c0 + lc) * 8;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(2 * rp), (int)ox);
+                r0 = Ops::root(pr, v);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(2 * rp + 1), (int)ox);
+                r1 = Ops::root(pr, v);
+            }
+            const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
+            if (valid && !(lane & 1)) Ops::pool_store(r0, r0o, r1, r1o, yb, ab, e.y);
+        }
+        blk = 0;
+        ++lc;
+    }
+}
+
+// Any shape, packed: one thread per (group, kernel, pooled cell), taps from global memory with bounds checks.
+__global__ __launch_bounds__(256) void convblock_packed_generic_kernel(const uint64_t *__restrict__ x, const uint8_t *__restrict__ gid,
+                                                                     const int32_t *__restrict__ sel, uint64_t *__restrict__ y,
+                                                                     Geom g)
+{
+    const int c = blockIdx.y;
+    const int wp = g.wo / 2, I = (g.ho / 2) * wp;
+    const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (item >= (int64_t)g.n * I) return;
+    const int n = (int)(item / I), cell = (int)(item - (int64_t)n * I);
+    const int py = cell / wp, px = cell - py * wp;
+    BitOps::Params pr;
+#pragma unroll
+    for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks(gid[(int64_t)c * 7 + k] & 15);
+    const uint64_t *xn = x + (int64_t)n * g.cin * g.h * g.w;
+    uint64_t acc = 0;
+    for (int q = 0; q < 4; ++q) {
+        uint64_t v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t]), 2 * py + (q >> 1), 2 * px + (q & 1));
+        acc |= BitOps::root(pr, v);
+    }
+    y[((int64_t)n * g.c + c) * I + cell] = acc;
+}
+
+// ---- plan --------------------------------------------------------------------------------------
+size_t forward_lds_bytes(const TilePlan &p, int elem, int params_per_kernel)
+{
+    return (size_t)((p.xe + 3) & ~3) * elem + (size_t)((p.CT * params_per_kernel + 1) & ~1) * elem + (size_t)p.CT * 8 * 4 +
+           (size_t)p.CT * 2 * 4 + (size_t)((p.CT + 1) & ~1) * 4 + (size_t)p.S * p.slots * 8;
+}
+
+bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
+{
+    if (!taps_inside(g)) return false;
+    plan_common(g, p);
+    p->slots = (g.ho / 2) * g.wo;
+    p->G = 1;
+    // 16 wavefronts share one staged image: measured 69 us against 109 us with 4 at [256,9,32,32] -> 256
+    p->NW = 16;
+    p->d_slots = make_fastdiv((uint32_t)p->slots);
+    const int64_t tail = g.ph * p->rs + g.pw;
+    auto util_of = [&](int S) {
+        const int64_t U = (int64_t)S * p->slots;
+        return (double)U / (double)(clg_ceil_div(U, kWave) * kWave);
+    };
+    // (a) all input channels staged: best lane utilisation within a 64 KiB image, smallest S on ties
+    int sa = 0;
+    double ua = 0;
+    for (int S = 1; S <= 16 && S <= g.n; ++S) {
+        const int64_t bytes = ((int64_t)S * g.cin * p->chs + tail) * elem + (int64_t)S * p->slots * 8;
+        if (S > 1 && bytes > 64 * 1024) break;
+        if (bytes > kLdsLimit - 8 * 1024) break;
+        if (util_of(S) > ua + 0.02) { ua = util_of(S); sa = S; }
+    }
+    // (b) two planes per kernel of a 16-kernel tile: the largest S within 64 KiB among the best utilisations
+    const int ctb = g.c < 16 ? g.c : 16;
+    int sb = 0;
+    double ub = 0;
+    for (int S = 1; S <= 32 && S <= g.n; ++S) {
+        const int64_t bytes = ((int64_t)S * 2 * ctb * p->chs + tail) * elem + (int64_t)S * p->slots * 8;
+        if (S > 1 && bytes > 64 * 1024) break;
+        if (bytes > kLdsLimit - 8 * 1024) break;
+        if (util_of(S) > ub + 0.02 || (util_of(S) > ub - 0.02 && (int64_t)S * p->slots <= 4 * kWave)) {
+            ub = util_of(S) > ub ? util_of(S) : ub;
+            sb = S;
+        }
+    }
+    bool subset = sb > 0 && (sa == 0 || g.cin > 2 * ctb || ub > ua + 0.2);
+    if (const char *e = getenv("CLG_FWD_SUBSET")) subset = sb > 0 && (atoi(e) != 0 || sa == 0);
+    const double util = subset ? ub : ua;
+    if ((subset ? sb : sa) == 0 || util < 0.4) return false;
+    p->subset = subset ? 1 : 0;
+    p->S = subset ? sb : sa;
+    if (subset) {
+        p->CT = ctb;
+    } else {
+        const int64_t groups = clg_ceil_div(g.n, p->S);
+        int64_t ct = (int64_t)g.c * groups / 1024;
+        ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
+        if (ct > g.c) ct = g.c;
+        p->CT = (int)ct;
+    }
+    p->planes = subset ? 2 * p->CT : g.cin;
+    p->d_planes = make_fastdiv((uint32_t)p->planes);
+    p->xe = (int)((int64_t)p->S * p->planes * p->chs + tail);
+    p->lds_bytes = forward_lds_bytes(*p, elem, params_per_kernel);
+    if (p->lds_bytes > (size_t)kLdsLimit) return false;
+    if (clg_ceil_div(g.c, p->CT) > 65535) return false;
+    return (int64_t)p->S * p->planes * p->chs < (1ll << 30) && (int64_t)p->S * g.c * ((g.ho / 2) * (g.wo / 2)) < (1ll << 31) &&
+           (int64_t)p->S * p->planes * g.h * g.w < (1ll << 31);
+}
+
+// ---- launch ------------------------------------------------------------------------------------
+template <typename Ops, int ROWSTEP, bool SUBSET>
+int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
+                       uint8_t *argmax, hipStream_t st, const char *name)
+{
+    using T = typename Ops::Elem;
+    if (int e = allow_lds(convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET>, p.lds_bytes, name)) return e;
+    const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
+    hipLaunchKernelGGL((convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
+                       params, sel, (T *)y, argmax, g, p);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
+}
+
+// Row steps of 3x3 / padding 1 / stride 1 blocks on 32, 28, 16, 8 and 4 pixel wide images get their own
+// instantiation; everything else reads the step from the plan.
+template <typename Ops>
+int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
+                         uint8_t *argmax, hipStream_t st, const char *name)
+{
+#define CLG_FWD_CASE(RS)                                                                                              \
+    case RS:                                                                                                          \
+        return p.subset ? launch_forward_one<Ops, RS, true>(g, p, x, params, sel, y, argmax, st, name)                \
+                        : launch_forward_one<Ops, RS, false>(g, p, x, params, sel, y, argmax, st, name)
+    switch (g.sh * p.rs) {
+        CLG_FWD_CASE(33);
+        CLG_FWD_CASE(29);
+        CLG_FWD_CASE(17);
+        CLG_FWD_CASE(9);
+        CLG_FWD_CASE(5);
+    default:
+        return p.subset ? launch_forward_one<Ops, 0, true>(g, p, x, params, sel, y, argmax, st, name)
+                        : launch_forward_one<Ops, 0, false>(g, p, x, params, sel, y, argmax, st, name);
+    }
+#undef CLG_FWD_CASE
+}
+
+}  // namespace
+
+extern "C" int clg_convblock_forward(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                     void *y, uint8_t *argmax, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_forward")) return e;
+    CLG_REQUIRE(x && w && selection && y && argmax, "clg_convblock_forward: null pointer argument");
+    TilePlan p;
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) {
+        if (plan_forward(g, 4, FloatOps<float>::kParams, &p))
+            return launch_forward_tiled<FloatOps<float>>(g, p, x, w, selection, y, argmax, st, "clg_convblock_forward");
+    } else {
+        if (plan_forward(g, 8, FloatOps<double>::kParams, &p))
+            return launch_forward_tiled<FloatOps<double>>(g, p, x, w, selection, y, argmax, st, "clg_convblock_forward");
+    }
+    return clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, st);
+}
+
+extern "C" int clg_convblock_eval_packed(const clg_conv_geom *gg, const uint64_t *x, const uint8_t *gates, const int32_t *selection,
+                                         uint64_t *y, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed")) return e;
+    CLG_REQUIRE(x && gates && selection && y, "clg_convblock_eval_packed: null pointer argument");
+    CLG_REQUIRE(x != y, "clg_convblock_eval_packed: x and y must not overlap");
+    TilePlan p;
+    hipStream_t st = clg_stream(stream);
+    if (plan_forward(g, 8, BitOps::kParams, &p))
+        return launch_forward_tiled<BitOps>(g, p, x, gates, selection, y, nullptr, st, "clg_convblock_eval_packed");
+    const int64_t blocks = clg_ceil_div((int64_t)g.n * (g.ho / 2) * (g.wo / 2), 256);
+    CLG_REQUIRE(g.c <= 65535 && blocks < (1ll << 31), "clg_convblock_eval_packed: problem too large for one launch");
+    hipLaunchKernelGGL(convblock_packed_generic_kernel, dim3((unsigned)blocks, (unsigned)g.c), dim3(256), 0, st, x, gates, selection, y,
+                       g);
+    CLG_CHECK_LAUNCH("clg_convblock_eval_packed(any shape)");
+    return CLG_OK;
+}

@@ -1,0 +1,90 @@
+// Plans and small device helpers shared by the LDS-tiled conv-logic kernels.
+#pragma once
+
+#include "conv_common.h"
+
+constexpr int kLdsLimit = 160 * 1024;
+
+// Division of a 31-bit value by a runtime constant: q = umulhi(x, mul) >> shr (d == 1: q = x).
+struct FastDiv {
+    uint32_t mul, shr, d;
+};
+static inline FastDiv make_fastdiv(uint32_t d)
+{
+    if (d <= 1) return FastDiv{0, 0, 1};
+    uint32_t lg = 0;
+    while ((1ull << lg) < d) ++lg;
+    const uint32_t p = 31 + lg;
+    const uint32_t mul = (uint32_t)(((1ull << p) + d - 1) / d);
+    return FastDiv{mul, p - 32, d};
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv &f) { return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shr); }
+
+struct TilePlan {
+    int S;              // samples per workgroup
+    int G;              // samples sharing one wavefront pass (input gradient; 1 when a sample has >= 64 cells)
+    int CT;             // kernels per workgroup (forward)
+    int NW;             // wavefronts per workgroup
+    int rs, chs;        // row and plane stride of the LDS image (elements)
+    int xe;             // elements of one LDS image region (S samples + tail)
+    int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
+    int band_rows, bands;  // input gradient: image rows per workgroup band, number of bands
+    int hit_split;         // input gradient: workgroups sharing the kernels of one (sample, band), partial images
+    int dummy_in_halo;     // input gradient: masked updates go to halo elements instead of a region of their own
+    int64_t part_stride;   // input gradient: elements between partial images (0 when hit_split == 1)
+    int planes;            // forward: LDS planes per sample (all input channels, or 2 per kernel of the tile)
+    int subset;            // forward: 1 = only the channels the kernel tile reads are staged
+    FastDiv d_hw, d_w, d_slots, d_wo, d_wp, d_planes;
+    size_t lds_bytes;
+};
+
+template <typename T>
+__device__ __forceinline__ T dpp_xor1(T v)
+{
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, false);
+        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, false);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T to_sgpr(T v)
+{
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)u);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(u >> 32));
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+// ---- plan helpers (host) ---------------------------------------------------------------------
+static inline void plan_common(const Geom &g, TilePlan *p)
+{
+    p->rs = g.w + g.pw;
+    p->chs = (g.h + g.ph) * p->rs;
+    p->d_hw = make_fastdiv((uint32_t)(g.h * g.w));
+    p->d_w = make_fastdiv((uint32_t)g.w);
+    p->d_wo = make_fastdiv((uint32_t)g.wo);
+    p->d_wp = make_fastdiv((uint32_t)(g.wo / 2));
+}
+
+static inline int64_t image_elems(const Geom &g, const TilePlan &p, int S) { return (int64_t)S * g.cin * p.chs + g.ph * p.rs + g.pw; }
+
+// The last tap row/column must stay inside the padded image for the shared-halo layout to hold.
+static inline bool taps_inside(const Geom &g) { return (g.ho - 1) * g.sh + g.kh <= g.h + 2 * g.ph && (g.wo - 1) * g.sw + g.kw <= g.w + 2 * g.pw; }
+
+// Kernels that want more than 48 KiB of dynamic LDS must be told once; the largest size granted so
+// far is remembered per kernel so that steady-state launches make no runtime call besides the launch.
+int clg_allow_lds(const void *kernel, size_t bytes, const char *name);
+template <typename K>
+static inline int allow_lds(K kernel, size_t bytes, const char *name)
+{
+    return clg_allow_lds(reinterpret_cast<const void *>(kernel), bytes, name);
+}

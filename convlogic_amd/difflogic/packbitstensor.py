@@ -9,13 +9,27 @@ from ..hip import difflogic_hip
 class PackBitsTensor:
     """t: bool [batch, features] on the GPU -> self.t integer words [features, ceil(batch/bit_count)]
     (bit i of word c = sample bit_count*c + i), self.pad_len unused high bits of the last word
-    (src/difflogic/packbitstensor.py:11-21)."""
+    (src/difflogic/packbitstensor.py:11-21).
+
+    Beyond the reference: a 4-D bool image batch [batch, C, H, W] (bit_count 64 only) is kept
+    group-major, self.t int64 [ceil(batch/64), C, H, W] with self.image True -- the layout the packed
+    conv-logic block reads and writes; flatten() (what nn.Flatten calls) turns it into the
+    feature-major layout above with features in c*H*W + y*W + x order."""
 
     def __init__(self, t: torch.Tensor, bit_count=32):
-        assert len(t.shape) == 2, t.shape
+        assert len(t.shape) in (2, 4), t.shape
         self.bit_count = bit_count
+        self.image = False
         if not t.is_cuda:
             raise NotImplementedError(f"PackBitsTensor only supports CUDA tensors, but got {t.device}.")
+        if t.dim() == 4:
+            if bit_count != 64:
+                raise ValueError(f"image batches are packed 64 samples per word, got bit_count={bit_count}")
+            n, c, h, w = t.shape
+            words, self.pad_len = difflogic_hip.tensor_packbits_sample_major(t.contiguous().view(n, c * h * w), 64)
+            self.t = difflogic_hip.transpose(words).view(-1, c, h, w)
+            self.image = True
+            return
         # packs straight from the sample-major tensor (no transposed bool copy)
         self.t, self.pad_len = difflogic_hip.tensor_packbits_sample_major(t.contiguous(), self.bit_count)
 
@@ -29,10 +43,17 @@ class PackBitsTensor:
 
     def group_sum(self, k):
         """int32 [batch, k] per-class counts of set bits (src/difflogic/packbitstensor.py:23-24)."""
+        if self.image:
+            self.flatten()
         return difflogic_hip.groupbitsum(self.t, self.pad_len, k)
 
     def flatten(self, start_dim=0, end_dim=-1, **kwargs):
-        """nn.Flatten is a no-op on packed activations (src/difflogic/packbitstensor.py:26-31)."""
+        """nn.Flatten is a no-op on feature-major packed activations (src/difflogic/packbitstensor.py:26-31);
+        a group-major image batch becomes feature-major here (one 8-byte transpose)."""
+        if self.image:
+            groups = self.t.shape[0]
+            self.t = difflogic_hip.transpose(self.t.reshape(groups, -1))
+            self.image = False
         return self
 
     def _row_repr(self, row):
@@ -43,4 +64,5 @@ class PackBitsTensor:
         return " ".join(bits(v) for v in row[:3]) + " ... " + bits(row[-1])
 
     def __repr__(self):
-        return "\n".join(self._row_repr(row) for row in self.t.cpu())
+        rows = self.t.reshape(self.t.shape[0], -1).t() if self.image else self.t
+        return "\n".join(self._row_repr(row) for row in rows.cpu())

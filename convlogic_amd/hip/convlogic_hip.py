@@ -136,6 +136,25 @@ def full_convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_
     return y, argmax
 
 
+def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """Packed-bit inference of the fused block.  x: int64 words [G, C_in, H, W], 64 samples per word
+    (bit s of group g = sample 64 g + s); gates: uint8 [C, 7] arg-max gate ids; -> int64 [G, C, Ho/2, Wo/2].
+    Equals the eval-mode float block on binary inputs (src/convlogic/convlogic_layer.py:231-316,321-325);
+    the reference has no packed conv kernel."""
+    for t, n in ((x, "x"), (gates, "gates"), (selection, "selection")):
+        check_input(t, n)
+    if x.dtype != torch.int64 or gates.dtype != torch.uint8 or x.dim() != 4:
+        raise RuntimeError("full_convlogic_eval_packed expects int64 words [G, C, H, W] and uint8 gate ids [C, 7]")
+    if gates.dim() != 2 or gates.shape[1] != 7:
+        raise RuntimeError(f"full_convlogic_eval_packed expects gate ids of shape [C, 7], got {tuple(gates.shape)}")
+    g = _geom(x, gates.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    y = torch.empty((g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2), dtype=torch.int64, device=x.device)
+    check(_lib.load().clg_convblock_eval_packed(ctypes.byref(g), x.data_ptr(), gates.data_ptr(), selection.data_ptr(),
+                                                y.data_ptr(), stream_ptr(x)))
+    return y
+
+
 def full_convlogic_intermediates(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
     """-> (x2 [N,C,Ho,Wo,4], x3 [N,C,Ho,Wo,2]), the second and third result of the reference's
     full_convlogic_forward (full_convlogic_kernel.cu:172,194)."""

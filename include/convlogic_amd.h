@@ -187,6 +187,16 @@ int64_t clg_tree_backward_w_scratch_bytes(int dtype, int64_t n, int64_t c, int64
 int clg_convblock_forward(int dtype, const clg_conv_geom *g, const void *x, const void *w /*[c_out,7,16]*/,
                           const int32_t *selection, void *y, uint8_t *argmax, void *stream);
 
+/* Packed-bit inference of the block: 64 samples per uint64 word, images word-group major
+ * x [n, c_in, h, w] with n = ceil(samples / 64) groups (bit s of group g = sample 64 g + s),
+ * gates uint8 [c_out, 7] = arg-max gate id of every tree node (0..3 leaves, 4..5 middle, 6 root),
+ * y [n, c_out, ho/2, wo/2]; the 2x2 max pool of {0,1} values is the OR of the four positions.
+ * The reference has no packed conv path (its packed kernels cover LogicLayer only,
+ * src/difflogic/cuda/difflogic_kernel.cu:271-330); the result equals the eval-mode float block
+ * (src/convlogic/convlogic_layer.py:231-316 with one-hot weights, :321-325) on binary inputs. */
+int clg_convblock_eval_packed(const clg_conv_geom *g, const uint64_t *x, const uint8_t *gates,
+                              const int32_t *selection, uint64_t *y, void *stream);
+
 /* Intermediates of the block for the return_intermediate / return_indices debug outputs:
  * x2 [n,c_out,ho,wo,4] (leaf gates), x3 [n,c_out,ho,wo,2]; either may be NULL.
  * (second and third result of full_convlogic_forward, full_convlogic_kernel.cu:172,194,230). */

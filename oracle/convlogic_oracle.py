@@ -412,3 +412,53 @@ def group_bit_sum(words, pad_len, k):
     f, s = bits.shape
     assert f % k == 0
     return bits.reshape(k, f // k, s).sum(1).astype(np.int32).T.copy()
+
+
+def pack_image(t_nchw):
+    """bool [N,C,H,W] -> (int64 words [ceil(N/64), C, H, W], pad_len): bit s of group g is sample
+    64 g + s (the sample-to-bit rule of difflogic_kernel.cu:354-362 with the group index leading)."""
+    t = np.asarray(t_nchw).astype(bool)
+    n, c, h, w = t.shape
+    words, pad_len = pack_bits(t.reshape(n, c * h * w).T, 64)      # [F, G]
+    return np.ascontiguousarray(words.T).reshape(-1, c, h, w), pad_len
+
+
+def unpack_image(words, pad_len=0):
+    """inverse of pack_image -> bool [N,C,H,W]."""
+    words = np.asarray(words)
+    g, c, h, w = words.shape
+    bits = unpack_bits(np.ascontiguousarray(words.reshape(g, c * h * w).T), pad_len)   # [F, N]
+    return np.ascontiguousarray(bits.T).reshape(-1, c, h, w)
+
+
+def conv_block_eval_packed(words, gates, sel, stride, pad, kernel):
+    """Packed-bit inference of the fused block on group-major words [G,Cin,H,W] -> [G,C,Ho/2,Wo/2].
+    No counterpart in the reference (its packed kernels cover LogicLayer only); defined as its
+    eval-mode block (arg-max gates, src/convlogic/convlogic_layer.py:321-325; taps :262-282; tree
+    pairs :289-305; 2x2 max pool :316) on {0,1} inputs: every gate becomes its bitwise twin
+    (src/common/cuda_utils.cuh:162-199) and the max of bits is their OR."""
+    words = np.asarray(words)
+    gates = np.asarray(gates)
+    g, _, h, w = words.shape
+    ho, wo = conv_out_size(h, w, stride, pad, kernel)
+    ch, ry, rx = (np.asarray(v) for v in unpack_selection(torch.as_tensor(np.asarray(sel)).long()))   # [C,8]
+    c = ch.shape[0]
+    xp = np.pad(words, ((0, 0), (0, 0), (pad[0], pad[0]), (pad[1], pad[1])))
+    oy = np.arange(ho).reshape(1, ho, 1) * stride[0]
+    ox = np.arange(wo).reshape(1, 1, wo) * stride[1]
+
+    def tap(t):
+        return xp[:, ch[:, t].reshape(c, 1, 1), oy + ry[:, t].reshape(c, 1, 1), ox + rx[:, t].reshape(c, 1, 1)]   # [G,C,Ho,Wo]
+
+    def level(inputs, first_gate):
+        out = []
+        for q in range(len(inputs) // 2):
+            a, b = inputs[2 * q], inputs[2 * q + 1]
+            r = np.empty_like(a)
+            for k in range(c):
+                r[:, k] = bin_op_eval(a[:, k], b[:, k], int(gates[k, first_gate + q]))
+            out.append(r)
+        return out
+
+    root = level(level(level([tap(t) for t in range(8)], 0), 4), 6)[0]
+    return root[:, :, 0::2, 0::2] | root[:, :, 0::2, 1::2] | root[:, :, 1::2, 0::2] | root[:, :, 1::2, 1::2]

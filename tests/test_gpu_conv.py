@@ -89,9 +89,11 @@ def _run_block(n, cin, cout, h, w, stride, pad, kernel, dtype=torch.float32, bin
 @pytest.mark.parametrize("binary", [False, True])
 @pytest.mark.parametrize("direct", [None, "1"])
 def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monkeypatch):
-    # direct="1" forces the input-gradient kernel that reads taps from a padded global copy of x
+    # direct="1" forces the input-gradient kernel that reads taps from a padded global copy of x and the
+    # forward staging of two LDS planes per kernel
     if direct:
         monkeypatch.setenv("CLG_BWDX_DIRECT", direct)
+        monkeypatch.setenv("CLG_FWD_SUBSET", direct)
     n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad
     if ((h + 2 * pad - kernel) // stride + 1) % 2:
         h += stride

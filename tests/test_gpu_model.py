@@ -118,3 +118,19 @@ def test_config5_eval_float_and_packed_tail():
         words = O.eval_packed(words, m.indices_0.cpu().numpy(), m.indices_1.cpu().numpy(),
                               m.weights.argmax(-1).cpu().numpy().astype(np.uint8))
     assert np.array_equal(O.group_bit_sum(words, pad, 10), p.cpu().numpy())
+
+
+def test_config5_eval_fully_packed_from_the_input():
+    # the whole network on packed bits: group-major image words through the four blocks, nn.Flatten turns
+    # them feature-major, three packed LogicLayers, per-class bit counts == the float eval path's scores
+    torch.manual_seed(4)
+    model = build().to(DEV).eval()
+    n = 200
+    bits = torch.randint(0, 2, (n, 9, 32, 32), device=DEV).bool()
+    with torch.no_grad():
+        y_float = model(bits.float())
+        p = model(C.PackBitsTensor(bits, 64))
+    assert p.dtype == torch.int32 and p.shape == (n, 10)
+    assert torch.equal(p.float(), torch.round(y_float * 6.5))
+    ref = oracle_forward(model, bits[:48].float().cpu(), training=False)
+    assert torch.equal(p[:48].cpu().float(), torch.round(ref * 6.5))

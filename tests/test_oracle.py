@@ -300,3 +300,50 @@ def test_c_oracle_matches_numpy_oracle(bits):
     lib.oracle_group_bit_sum(y.ctypes.data_as(ctypes.c_void_p), gs.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(out),
                              ctypes.c_int64(row_bytes), ctypes.c_int64(pad), ctypes.c_int64(k))
     assert np.array_equal(gs, O.group_bit_sum(y, pad, k))
+
+
+# ---- packed conv block -----------------------------------------------------------------------------
+def test_pack_image_round_trip_and_bit_positions():
+    rng = np.random.default_rng(3)
+    t = rng.integers(0, 2, (130, 2, 3, 5)).astype(bool)
+    words, pad = O.pack_image(t)
+    assert words.shape == (3, 2, 3, 5) and words.dtype == np.int64 and pad == 62
+    assert np.array_equal(O.unpack_image(words, pad), t)
+    # sample 64 g + s sits in bit s of group g, straight from the definition
+    for n, c, y, x in [(0, 0, 0, 0), (63, 1, 2, 4), (64, 0, 1, 1), (129, 1, 0, 3)]:
+        assert ((int(words[n // 64, c, y, x]) >> (n % 64)) & 1) == int(t[n, c, y, x])
+
+
+@pytest.mark.parametrize("stride,pad,kernel", [(1, 1, 3), (2, 2, 4), (1, 0, 3), ((1, 2), (0, 1), (2, 3))])
+def test_conv_block_eval_packed_equals_float_eval_on_bits(stride, pad, kernel):
+    # the packed block is DEFINED as the float eval-mode block on {0,1} inputs: compare against the float
+    # oracle (itself pinned by the brute-force and max_pool2d tests above) sample by sample
+    pr = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+    stride, pad, kernel = pr(stride), pr(pad), pr(kernel)
+    torch.manual_seed(11)
+    n, cin, c, h, w = 70, 3, 5, 9, 11
+    ho, wo = O.conv_out_size(h, w, stride, pad, kernel)
+    h += (ho % 2) * stride[0]
+    w += (wo % 2) * stride[1]
+    sel = O.generate_selection(cin, c, kernel)
+    logits = torch.randn(c, 7, 16)
+    bits = torch.randint(0, 2, (n, cin, h, w)).bool()
+    want = O.conv_block_forward(bits.float(), O.gate_weights(logits, False, torch.float32), sel, stride, pad, kernel)
+    assert torch.all((want == 0) | (want == 1))
+    words, pad_len = O.pack_image(bits.numpy())
+    got = O.conv_block_eval_packed(words, logits.argmax(-1).numpy().astype(np.uint8), sel.numpy(), stride, pad, kernel)
+    assert np.array_equal(O.unpack_image(got, pad_len), want.numpy() > 0.5)
+
+
+def test_conv_block_eval_packed_all_gates_truth_table():
+    # one kernel, 1x1 taps on a 2x2 image of constants: root gate id i over leaves that pass tap 0 / tap 1
+    # through (gate 3 = A) must reproduce bit (3 - 2a - b) of i -- the truth-table rule of the gate ids
+    sel = torch.tensor([[(0 << 16), (1 << 16), (0 << 16), (1 << 16), (1 << 16), (0 << 16), (1 << 16), (0 << 16)]], dtype=torch.int32)
+    for i in range(16):
+        gates = np.array([[3, 3, 3, 3, 3, 3, i]], dtype=np.uint8)      # leaves: taps 0,2,4,6; middles pass leaf 0 / leaf 2
+        for a in (0, 1):
+            for b in (0, 1):
+                img = np.zeros((1, 2, 2, 2), dtype=np.int64)
+                img[:, 0], img[:, 1] = -a, -b                           # all 64 samples set or clear
+                y = O.conv_block_eval_packed(img, gates, sel.numpy(), (1, 1), (0, 0), (1, 1))
+                assert y.shape == (1, 1, 1, 1) and int(y[0, 0, 0, 0]) == -((i >> (3 - 2 * a - b)) & 1), (i, a, b)
