@@ -179,20 +179,31 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     }
     __syncthreads();
     {
-        // planes of the samples into the zeroed LDS image
+        // planes of the samples into the zeroed LDS image, four global loads in flight per thread
         const T *src = x + (int64_t)n0 * g.cin * hw;
         const uint32_t total = (uint32_t)(s_cur * p.planes) * (uint32_t)hw;
-        for (uint32_t e = tid; e < total; e += nthreads) {
-            const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)hw;
-            const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
-            T v;
-            if (!SUBSET) {
-                v = src[e];
-            } else {
-                const uint32_t s = fdiv(plane, p.d_planes), pl = plane - s * (uint32_t)p.planes;
-                v = src[((int64_t)s * g.cin + chan[pl]) * hw + rem];
+        for (uint32_t e0 = tid; e0 < total; e0 += 4 * nthreads) {
+            T v[4];
+            int at[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t e = e0 + k * nthreads;
+                at[k] = -1;
+                if (e < total) {
+                    const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)hw;
+                    const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+                    at[k] = (int)(plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw);
+                    if (!SUBSET) {
+                        v[k] = src[e];
+                    } else {
+                        const uint32_t s = fdiv(plane, p.d_planes), pl = plane - s * (uint32_t)p.planes;
+                        v[k] = src[((int64_t)s * g.cin + chan[pl]) * hw + rem];
+                    }
+                }
             }
-            xs[plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw] = v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (at[k] >= 0) xs[at[k]] = v[k];
         }
     }
     __syncthreads();
@@ -303,8 +314,8 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
         if (bytes > kLdsLimit - 8 * 1024) break;
         if (util_of(S) > ua + 0.02) { ua = util_of(S); sa = S; }
     }
-    // (b) two planes per kernel of a 16-kernel tile: the largest S within 64 KiB among the best utilisations
-    const int ctb = g.c < 16 ? g.c : 16;
+    // (b) two planes per kernel of an 8-kernel tile: the largest S within 64 KiB among the best utilisations
+    const int ctb = g.c < 8 ? g.c : 8;
     int sb = 0;
     double ub = 0;
     for (int S = 1; S <= 32 && S <= g.n; ++S) {
@@ -316,25 +327,39 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
             sb = S;
         }
     }
-    bool subset = sb > 0 && (sa == 0 || g.cin > 2 * ctb || ub > ua + 0.2);
+    // Staging all channels wins whenever it fits with reasonable lane use (measured on 8x8 and 16x16 layers
+    // with 32..128 input channels); the two-planes-per-kernel staging is for what is left.
+    bool subset = sb > 0 && (sa == 0 || ua < 0.4);
     if (const char *e = getenv("CLG_FWD_SUBSET")) subset = sb > 0 && (atoi(e) != 0 || sa == 0);
     const double util = subset ? ub : ua;
     if ((subset ? sb : sa) == 0 || util < 0.4) return false;
     p->subset = subset ? 1 : 0;
     p->S = subset ? sb : sa;
     if (subset) {
-        p->CT = ctb;
+        p->CT = g.c < 8 ? g.c : 8;
+        p->NW = 8;
     } else {
+        // as many kernels per staged image as leave about two workgroups per CU (the prologue -- zero, stage,
+        // two barriers -- is what small layers pay for)
         const int64_t groups = clg_ceil_div(g.n, p->S);
-        int64_t ct = (int64_t)g.c * groups / 1024;
-        ct = ct < 4 ? 4 : (ct > 64 ? 64 : ct);
-        if (ct > g.c) ct = g.c;
+        const int64_t ct_cap = 32768 / ((int64_t)params_per_kernel * elem);   // at most 32 KiB of gate parameters
+        int64_t ct = g.c < ct_cap ? g.c : ct_cap;
+        while (ct > 4 && groups * clg_ceil_div(g.c, ct) < 512) ct = (ct + 1) / 2;
         p->CT = (int)ct;
     }
-    p->planes = subset ? 2 * p->CT : g.cin;
+    // measurement overrides
+    if (const char *e = getenv("CLG_FWD_S")) p->S = atoi(e) < g.n ? atoi(e) : g.n;
+    if (const char *e = getenv("CLG_FWD_CT")) p->CT = atoi(e) < g.c ? atoi(e) : g.c;
+    if (const char *e = getenv("CLG_FWD_NW")) p->NW = atoi(e);
+    if (p->S < 1 || p->CT < 1 || p->NW < 1 || p->NW > 16) return false;
+    for (;;) {
+        p->planes = subset ? 2 * p->CT : g.cin;
+        p->xe = (int)((int64_t)p->S * p->planes * p->chs + tail);
+        p->lds_bytes = forward_lds_bytes(*p, elem, params_per_kernel);
+        if (p->lds_bytes <= (size_t)kLdsLimit || p->CT <= 4) break;
+        p->CT = (p->CT + 1) / 2;                                      // the gate parameters of the tile share LDS with the image
+    }
     p->d_planes = make_fastdiv((uint32_t)p->planes);
-    p->xe = (int)((int64_t)p->S * p->planes * p->chs + tail);
-    p->lds_bytes = forward_lds_bytes(*p, elem, params_per_kernel);
     if (p->lds_bytes > (size_t)kLdsLimit) return false;
     if (clg_ceil_div(g.c, p->CT) > 65535) return false;
     return (int64_t)p->S * p->planes * p->chs < (1ll << 30) && (int64_t)p->S * g.c * ((g.ho / 2) * (g.wo / 2)) < (1ll << 31) &&

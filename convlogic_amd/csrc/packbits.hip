@@ -238,6 +238,110 @@ __global__ __launch_bounds__(256) void group_bit_sum_kernel(const uint8_t *__res
     }
 }
 
+// Many samples: lanes along 8-byte columns, so a wavefront reads 512 contiguous bytes of a row.  A
+// workgroup owns 64 columns of one class (and one row slice); its 8 wavefronts split the rows.  Every
+// thread counts the 64 bit positions of its column with vertical counters (plane p holds bit p of the 64
+// running counts): four words are combined by three carry-save adders and the resulting "fours" word
+// ripples into planes 2 and up.  The wavefronts' planes meet in LDS, are added as binary numbers, and
+// every wavefront expands 8 of the 64 bit positions into counts.
+constexpr int kCountPlanes = 14;                                     // a wavefront counts at most 2^14 - 8 rows
+constexpr int kCountWaves = 8;
+__device__ __forceinline__ void csa(uint64_t &hi, uint64_t &lo, uint64_t a, uint64_t b, uint64_t c)
+{
+    const uint64_t u = a ^ b;
+    hi = (a & b) | (u & c);
+    lo = u ^ c;
+}
+__device__ __forceinline__ void count8(uint64_t (&plane)[kCountPlanes], const uint64_t (&w)[8])
+{
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        uint64_t two_a, two_b, four;
+        csa(two_a, plane[0], plane[0], w[4 * h], w[4 * h + 1]);
+        csa(two_b, plane[0], plane[0], w[4 * h + 2], w[4 * h + 3]);
+        csa(four, plane[1], plane[1], two_a, two_b);
+#pragma unroll
+        for (int q = 2; q < kCountPlanes; ++q) {
+            const uint64_t t = plane[q] & four;
+            plane[q] ^= four;
+            four = t;
+        }
+    }
+}
+__global__ __launch_bounds__(kCountWaves *kWave) void group_bit_sum_columns_kernel(const uint64_t *__restrict__ x,
+                                                                                  int32_t *__restrict__ out, int64_t class_rows,
+                                                                                  int64_t row_words, int64_t samples, int k,
+                                                                                  int slices)
+{
+    __shared__ uint64_t meet[kCountWaves][kCountPlanes][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    const int64_t col = (int64_t)blockIdx.x * kWave + lane;
+    const bool live = col < row_words;
+    const int g = blockIdx.y;
+    const int part = blockIdx.z * kCountWaves + wave, parts = slices * kCountWaves;
+    const int64_t r0 = class_rows * part / parts, r1 = class_rows * (part + 1) / parts;
+    const uint64_t *p = x + ((int64_t)g * class_rows + r0) * row_words + (live ? col : 0);
+    uint64_t plane[kCountPlanes];
+#pragma unroll
+    for (int q = 0; q < kCountPlanes; ++q) plane[q] = 0;
+    int64_t r = r0;
+    if (r + 8 <= r1) {
+        uint64_t cur[8], nxt[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) cur[j] = p[(int64_t)j * row_words];
+        p += 8 * row_words;
+        r += 8;
+        for (; r + 8 <= r1; r += 8) {                                // next 8 rows are in flight while these are counted
+#pragma unroll
+            for (int j = 0; j < 8; ++j) nxt[j] = p[(int64_t)j * row_words];
+            p += 8 * row_words;
+            count8(plane, cur);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cur[j] = nxt[j];
+        }
+        count8(plane, cur);
+    }
+    for (; r < r1; ++r) {
+        uint64_t carry = *p;
+        p += row_words;
+#pragma unroll
+        for (int q = 0; q < kCountPlanes; ++q) {
+            const uint64_t t = plane[q] & carry;
+            plane[q] ^= carry;
+            carry = t;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < kCountPlanes; ++q) meet[wave][q][lane] = plane[q];
+    __syncthreads();
+    // total = sum of the wavefronts' counters, as binary numbers spread over the planes (a total above
+    // 2^14 - 1 cannot occur: the host keeps the rows of a workgroup below that)
+#pragma unroll
+    for (int q = 0; q < kCountPlanes; ++q) plane[q] = meet[0][q][lane];
+    for (int wv = 1; wv < kCountWaves; ++wv) {
+        uint64_t carry = 0;
+#pragma unroll
+        for (int q = 0; q < kCountPlanes; ++q) {
+            const uint64_t b = meet[wv][q][lane], u = plane[q] ^ b;
+            const uint64_t c = (plane[q] & b) | (u & carry);
+            plane[q] = u ^ carry;
+            carry = c;
+        }
+    }
+    if (!live) return;
+    const int64_t s0 = col * 64;
+#pragma unroll
+    for (int bb = 0; bb < 64 / kCountWaves; ++bb) {
+        const int b = wave * (64 / kCountWaves) + bb;
+        if (s0 + b >= samples) break;
+        int32_t cnt = 0;
+#pragma unroll
+        for (int q = 0; q < kCountPlanes; ++q) cnt |= (int32_t)((plane[q] >> b) & 1) << q;
+        if (slices == 1) out[(s0 + b) * k + g] = cnt;
+        else atomicAdd(out + (s0 + b) * k + g, cnt);
+    }
+}
+
 __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
@@ -342,11 +446,30 @@ extern "C" int clg_group_bit_sum(int elem_size, const void *x, int32_t *out, int
     CLG_REQUIRE(k < (1 << 20), "clg_group_bit_sum: k too large");
     const int cols8 = (int)clg_ceil_div(row_bytes, 8);
     const int64_t class_rows = features / k;
+    hipStream_t st = clg_stream(stream);
+    if ((row_bytes & 7) == 0 && ((uintptr_t)x & 7) == 0 && cols8 >= 64 && k <= 65535) {
+        // wide rows: lanes along columns, vertical counters; row slices (combined by integer atomics) until
+        // about two workgroups per CU, at least 64 rows per wavefront, at most 2^14 - 8 rows per workgroup
+        const int64_t row_words = row_bytes / 8;
+        const int64_t col_blocks = clg_ceil_div(row_words, kWave);
+        int64_t slices = clg_ceil_div(512, col_blocks * k);
+        if (slices > class_rows / (64 * kCountWaves)) slices = class_rows / (64 * kCountWaves);
+        const int64_t need = clg_ceil_div(class_rows, (1 << kCountPlanes) - 8);
+        if (slices < need) slices = need;
+        if (slices < 1) slices = 1;
+        CLG_REQUIRE(slices <= 65535 && col_blocks < (1ll << 31), "clg_group_bit_sum: problem too large for one launch");
+        if (slices > 1)
+            hipLaunchKernelGGL(fill_zero_i32_kernel, dim3(small_grid(samples * k, 256)), dim3(256), 0, st, out, samples * k);
+        hipLaunchKernelGGL(group_bit_sum_columns_kernel, dim3((unsigned)col_blocks, (unsigned)k, (unsigned)slices),
+                           dim3(kCountWaves * kWave), 0, st, (const uint64_t *)x, out, class_rows, row_words, samples, (int)k,
+                           (int)slices);
+        CLG_CHECK_LAUNCH("clg_group_bit_sum");
+        return CLG_OK;
+    }
     // enough waves to fill the GPU, at least 64 rows per slice
     int64_t slices = clg_ceil_div(16384, (int64_t)k * cols8);
     if (slices > class_rows / 64) slices = class_rows / 64;
     if (slices < 1) slices = 1;
-    hipStream_t st = clg_stream(stream);
     if (slices > 1)
         hipLaunchKernelGGL(fill_zero_i32_kernel, dim3(small_grid(samples * k, 256)), dim3(256), 0, st, out, samples * k);
     const int64_t items = k * cols8 * slices;

@@ -43,7 +43,9 @@ def test_eval_packed_bit_exact(bits, batch):
     assert got.dtype == TORCH_WORD[bits] and np.array_equal(got.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("bits,batch,features,k", [(64, 256, 40, 10), (32, 100, 12, 3), (8, 9, 4, 2), (64, 5000, 2000, 10), (16, 33, 6, 6)])
+@pytest.mark.parametrize("bits,batch,features,k", [(64, 256, 40, 10), (32, 100, 12, 3), (8, 9, 4, 2), (64, 5000, 2000, 10), (16, 33, 6, 6),
+                                                   (64, 4133, 84, 4), (32, 4200, 30, 3), (8, 600, 9, 1), (64, 8192, 2400, 4),
+                                                   (64, 4096, 7, 7)])
 def test_group_bit_sum(bits, batch, features, k):
     rng = np.random.default_rng(batch + features)
     t = rng.integers(0, 2, (features, batch)).astype(bool)
