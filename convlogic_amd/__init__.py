@@ -2,13 +2,14 @@
 differentiable logic gate networks.
 
   convlogic_amd.difflogic   LogicLayer, GroupSum, PackBitsTensor, ...   (mirror of the `difflogic` package)
-  convlogic_amd.convlogic   ConvLogicLayer, TreeLogicLayer, PoolLogicLayer (mirror of the `convlogic` package)
+  convlogic_amd.convlogic   ConvLogicLayer, TreeLogicLayer, PoolLogicLayer, model topologies (mirror of `convlogic`)
   convlogic_amd.hip         function sets of the native extension modules, on the C ABI of
                             include/convlogic_amd.h (libconvlogic_amd.so)
 """
-from .convlogic import (ConvLogicFunction, ConvLogicLayer, FullConvLogicFunction, PoolLogicLayer, TreeLogicFunction,
+from .convlogic import (ConvLogicCifarModel, ConvLogicFunction, ConvLogicLayer, ConvLogicMnistModel, FullConvLogicFunction, PoolLogicLayer, TreeLogicFunction,
                         TreeLogicLayer)
 from .difflogic import GradFactor, GroupSum, LogicLayer, LogicLayerCudaFunction, PackBitsTensor
 
 __all__ = ["ConvLogicLayer", "ConvLogicFunction", "FullConvLogicFunction", "PoolLogicLayer", "TreeLogicLayer",
-           "TreeLogicFunction", "LogicLayer", "GroupSum", "LogicLayerCudaFunction", "PackBitsTensor", "GradFactor"]
+           "TreeLogicFunction", "LogicLayer", "GroupSum", "LogicLayerCudaFunction", "PackBitsTensor", "GradFactor", "ConvLogicCifarModel",
+           "ConvLogicMnistModel"]

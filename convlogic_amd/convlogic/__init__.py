@@ -1,5 +1,6 @@
 from .convlogic_layer import ConvLogicFunction, ConvLogicLayer, FullConvLogicFunction, PoolLogicLayer
+from .model import ConvLogicCifarModel, ConvLogicMnistModel
 from .treelogic_layer import TreeLogicFunction, TreeLogicLayer
 
 __all__ = ["ConvLogicLayer", "ConvLogicFunction", "FullConvLogicFunction", "PoolLogicLayer", "TreeLogicLayer",
-           "TreeLogicFunction"]
+           "TreeLogicFunction", "ConvLogicCifarModel", "ConvLogicMnistModel"]

@@ -1,0 +1,58 @@
+"""Network topologies of the reference's src/convlogic/model.py as plain nn.Modules: the caller side of
+the logic-layer kernels.  Constructor arguments, layer order and the `network` attribute are the
+reference's, so parameters are drawn in the same RNG order and state_dict keys (`network.<i>.weights`,
+`network.<i>.selection`, `network.<i>.indices_0`, ...) match checkpoints written from there (the
+Lightning wrapper of src/convlogic/model.py:111-200 prefixes them with `model.`)."""
+from torch import nn
+
+from ..difflogic import GroupSum, LogicLayer
+from .convlogic_layer import ConvLogicLayer
+
+
+def _block(c_in, c_out, implementation, **kw):
+    return ConvLogicLayer(in_channels=c_in, out_channels=c_out, residual_init=True, complete=True,
+                          implementation=implementation, **kw)
+
+
+def _head(dims, tau, implementation):
+    fc = [LogicLayer(a, b, grad_factor=1, residual_init=True, implementation=implementation) for a, b in zip(dims, dims[1:])]
+    return [nn.Flatten(), *fc, GroupSum(k=10, tau=tau)]
+
+
+class ConvLogicCifarModel(nn.Module):
+    """Four 3x3 / padding 1 blocks of k, 4k, 16k, 32k kernels (each halves the image), then three
+    LogicLayers of 10, 5 and 2.5 times the flattened width (doubled from k = 1024) and a 10-class
+    GroupSum (src/convlogic/model.py:11-60)."""
+
+    def __init__(self, k_param=32, input_channels=3, input_size=32, tau=20, implementation="cuda"):
+        super().__init__()
+        self.input_size = input_size
+        self.k_param = k_param
+        self.extra_layers = 2 if k_param >= 1024 else 1
+        widths = [input_channels] + [m * k_param for m in (1, 4, 16, 32)]
+        blocks = [_block(a, b, implementation, padding=1, groups=1) for a, b in zip(widths, widths[1:])]
+        side = input_size // 2 ** len(blocks)
+        flat = widths[-1] * side * side
+        m = self.extra_layers
+        dims = [flat, m * flat * 10, m * flat * 5, m * (flat * 10) // 4]
+        self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
+
+    def forward(self, x):
+        return self.network(x)
+
+
+class ConvLogicMnistModel(nn.Module):
+    """A 5x5 / padding 0 block of k kernels (28 -> 24 -> 12), two 3x3 / padding 1 blocks of 3k and 9k
+    kernels (-> 6 -> 3), then LogicLayers 81k -> 1280k -> 640k -> 320k and a 10-class GroupSum
+    (src/convlogic/model.py:63-108)."""
+
+    def __init__(self, input_channels=1, input_size=28, k_param=32, tau=6.5, implementation="cuda"):
+        super().__init__()
+        k = k_param
+        blocks = [_block(input_channels, k, implementation, kernel=5, padding=0),
+                  _block(k, 3 * k, implementation, kernel=3, padding=1),
+                  _block(3 * k, 9 * k, implementation, kernel=3, padding=1)]
+        self.network = nn.Sequential(*blocks, *_head([81 * k, 1280 * k, 640 * k, 320 * k], tau, implementation))
+
+    def forward(self, x):
+        return self.network(x)

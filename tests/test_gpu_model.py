@@ -29,7 +29,7 @@ def oracle_forward(model, x, training=True):
     for m in model:
         if isinstance(m, C.ConvLogicLayer):
             h = O.conv_block_forward(h, O.gate_weights(m.weights.detach().cpu() if not training else m._w, training, h.dtype),
-                                     m.selection.cpu(), (1, 1), (1, 1), (3, 3))
+                                     m.selection.cpu(), tuple(m.stride), tuple(m.padding), tuple(m.kernel))
         elif isinstance(m, torch.nn.Flatten):
             h = h.flatten(1)
         elif isinstance(m, C.LogicLayer):
@@ -134,3 +134,55 @@ def test_config5_eval_fully_packed_from_the_input():
     assert torch.equal(p.float(), torch.round(y_float * 6.5))
     ref = oracle_forward(model, bits[:48].float().cpu(), training=False)
     assert torch.equal(p[:48].cpu().float(), torch.round(ref * 6.5))
+
+
+def test_mnist_topology_training_step_and_packed_eval():
+    # ConvLogicMnistModel (5x5 / padding 0 first block; src/convlogic/model.py:63-108) at k = 4: one float64
+    # training step against the oracle, an optimizer step, then eval: float path == packed path == oracle
+    torch.manual_seed(6)
+    model = C.ConvLogicMnistModel(k_param=4).double().to(DEV)
+    net = model.network
+    with torch.no_grad():
+        for m in net:
+            if hasattr(m, "weights"):
+                m.weights.copy_(torch.randn_like(m.weights))      # off the residual init, so every gate matters
+    n = 6
+    x = torch.randint(0, 2, (n, 1, 28, 28)).double()
+    labels = torch.randint(0, 10, (n,))
+    opt = torch.optim.AdamW(model.parameters(), lr=0.01)
+    logits = model(x.to(DEV))
+    loss = torch.nn.functional.cross_entropy(logits, labels.to(DEV))
+    loss.backward()
+    params = [m for m in net if hasattr(m, "weights")]
+    for m in params:
+        m._w = m.weights.detach().cpu().clone().requires_grad_(True)
+    ref = oracle_forward(net, x.clone())
+    torch.nn.functional.cross_entropy(ref, labels).backward()
+    assert (logits.detach().cpu() - ref.detach()).abs().max().item() <= 1e-9
+    for i, m in enumerate(params):
+        assert_grad_close(m.weights.grad, m._w.grad, rel=1e-6, name=f"layer {i} grad_logits")
+    before = [m.weights.detach().clone() for m in params]
+    opt.step()
+    assert all(not torch.equal(b, m.weights) for b, m in zip(before, params))
+
+    model = model.float().eval()
+    bits = torch.randint(0, 2, (150, 1, 28, 28), device=DEV).bool()
+    with torch.no_grad():
+        y_float = model(bits.float())
+        counts = model(C.PackBitsTensor(bits, 64))
+    assert counts.dtype == torch.int32 and torch.equal(counts.float(), torch.round(y_float * 6.5))
+    ref = oracle_forward(net, bits[:40].float().cpu(), training=False)
+    assert torch.equal(counts[:40].cpu().float(), torch.round(ref * 6.5))
+
+
+def test_cifar_topology_state_dict_round_trip():
+    torch.manual_seed(8)
+    a = C.ConvLogicCifarModel(k_param=4, input_channels=9, tau=6.5).to(DEV).eval()
+    b = C.ConvLogicCifarModel(k_param=4, input_channels=9, tau=6.5).to(DEV).eval()
+    x = torch.randint(0, 2, (70, 9, 32, 32), device=DEV).bool()
+    with torch.no_grad():
+        ya = a(x.float())
+        assert not torch.equal(ya, b(x.float()))                  # different wiring and taps
+        b.load_state_dict(a.state_dict())
+        assert torch.equal(ya, b(x.float()))
+        assert torch.equal(b(C.PackBitsTensor(x, 64)).float(), torch.round(ya * 6.5))

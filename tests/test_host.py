@@ -151,3 +151,39 @@ def test_constructor_validation():
     assert set(layer.state_dict()) == {"weights", "selection"}
     fc = C.LogicLayer(4, 4, implementation="python")
     assert set(fc.state_dict()) == {"weights", "indices_0", "indices_1"}
+
+
+# ---- model topologies -----------------------------------------------------------------------------
+def test_model_topologies_layers_keys_and_shapes():
+    # src/convlogic/model.py:16-58 and :68-106: layer order, widths and state_dict names
+    torch.manual_seed(0)
+    m = C.ConvLogicMnistModel(k_param=2, implementation="python")
+    kinds = [type(l).__name__ for l in m.network]
+    assert kinds == ["ConvLogicLayer"] * 3 + ["Flatten"] + ["LogicLayer"] * 3 + ["GroupSum"]
+    assert [(l.in_channels, l.out_channels, l.kernel, l.padding) for l in m.network[:3]] == \
+        [(1, 2, (5, 5), (0, 0)), (2, 6, (3, 3), (1, 1)), (6, 18, (3, 3), (1, 1))]
+    assert [(l.in_dim, l.out_dim) for l in m.network[4:7]] == [(162, 2560), (2560, 1280), (1280, 640)]
+    assert m.network[7].k == 10 and m.network[7].tau == 6.5
+    keys = list(m.state_dict())
+    assert keys[:2] == ["network.0.weights", "network.0.selection"]
+    assert "network.4.indices_0" in keys and "network.4.indices_1" in keys
+    assert m(torch.rand(3, 1, 28, 28)).shape == (3, 10)
+    # residual init: gate 3 ("A") carries p = e^5 / (e^5 + 15)
+    p = torch.softmax(m.network[0].weights, -1)[0, 0]
+    assert abs(p[3].item() - 0.908208) < 1e-5
+
+    c = C.ConvLogicCifarModel(k_param=2, input_channels=3, implementation="python")
+    assert [(l.in_channels, l.out_channels) for l in c.network[:4]] == [(3, 2), (2, 8), (8, 32), (32, 64)]
+    assert [(l.in_dim, l.out_dim) for l in c.network[5:8]] == [(256, 2560), (2560, 1280), (1280, 640)]
+    assert c.extra_layers == 1 and c.network[8].tau == 20
+    assert c(torch.rand(2, 3, 32, 32)).shape == (2, 10)
+
+
+def test_model_construction_draws_like_the_layers_in_order():
+    # equal seeds give equal parameters whether the layers are built by the model or by hand in its order
+    torch.manual_seed(5)
+    m = C.ConvLogicMnistModel(k_param=1, implementation="python")
+    torch.manual_seed(5)
+    first = C.ConvLogicLayer(1, 1, kernel=5, padding=0, residual_init=True, complete=True, implementation="python")
+    second = C.ConvLogicLayer(1, 3, kernel=3, padding=1, residual_init=True, complete=True, implementation="python")
+    assert torch.equal(m.network[0].selection, first.selection) and torch.equal(m.network[1].selection, second.selection)
