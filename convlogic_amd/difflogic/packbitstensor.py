@@ -33,6 +33,14 @@ class PackBitsTensor:
         # packs straight from the sample-major tensor (no transposed bool copy)
         self.t, self.pad_len = difflogic_hip.tensor_packbits_sample_major(t.contiguous(), self.bit_count)
 
+    @classmethod
+    def from_image_words(cls, words: torch.Tensor, pad_len: int):
+        """Wraps group-major packed image words int64 [groups, C, H, W] (64 samples per word)."""
+        assert words.dim() == 4 and words.dtype == torch.int64, (words.shape, words.dtype)
+        self = cls.__new__(cls)
+        self.t, self.pad_len, self.bit_count, self.image = words, int(pad_len), 64, True
+        return self
+
     @property
     def is_cuda(self):
         return self.t.is_cuda

@@ -47,6 +47,8 @@ SIGNATURES = {
     "clg_tree_backward_w": (_i, [_i, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "clg_tree_backward_w_scratch_bytes": (_i64, [_i, _i64, _i64, _i64, _i64]),
     "clg_convblock_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
+    "clg_threshold_images": (_i, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "clg_threshold_pack_images": (_i, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "clg_convblock_eval_packed": (_i, [_GP, _p, _p, _p, _p, _p]),
     "clg_convblock_intermediates": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_x": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p]),

@@ -222,3 +222,36 @@ def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stri
     check(lib.clg_convblock_backward(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(), selection.data_ptr(),
                                      argmax.data_ptr(), gx.data_ptr(), gw.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
     return gx, gw
+
+
+# ---- input binarisation -------------------------------------------------------------------------
+def _threshold_args(x, thresholds):
+    check_input(x, "x")
+    check_input(thresholds, "thresholds")
+    if x.dtype != torch.float32 or thresholds.dtype != torch.float32 or x.dim() != 4 or thresholds.dim() != 1:
+        raise RuntimeError("expected float32 images [N, C, H, W] and float32 thresholds [L]")
+    n, c0, h, w = x.shape
+    return n, c0, h, w, thresholds.shape[0]
+
+
+def threshold_images(x, thresholds):
+    """float32 [N, C, H, W] -> float32 {0,1} [N, L*C, H, W], channel l*C + c = x[:, c] > thresholds[l]
+    (src/convlogic/data.py:46-50 on a batch)."""
+    n, c0, h, w, levels = _threshold_args(x, thresholds)
+    out = torch.empty((n, levels * c0, h, w), dtype=torch.float32, device=x.device)
+    if out.numel():
+        check(_lib.load().clg_threshold_images(x.data_ptr(), thresholds.data_ptr(), out.data_ptr(), n, c0, h * w, levels,
+                                               stream_ptr(x)))
+    return out
+
+
+def threshold_pack_images(x, thresholds):
+    """float32 [N, C, H, W] -> (int64 words [ceil(N/64), L*C, H, W], pad_len): the thresholded channels
+    packed 64 samples per word, group-major, without materialising them as floats."""
+    n, c0, h, w, levels = _threshold_args(x, thresholds)
+    groups = -(-n // 64)
+    out = torch.empty((groups, levels * c0, h, w), dtype=torch.int64, device=x.device)
+    if out.numel():
+        check(_lib.load().clg_threshold_pack_images(x.data_ptr(), thresholds.data_ptr(), out.data_ptr(), n, c0, h * w, levels,
+                                                    stream_ptr(x)))
+    return out, groups * 64 - n

@@ -230,6 +230,23 @@ int clg_convblock_backward(int dtype, const clg_conv_geom *g, const void *grad_y
                            void *stream);
 int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *g);
 
+/* ---------------------------------------------------------------------------------
+ * input binarisation (the step in front of the first layer)
+ * --------------------------------------------------------------------------------- */
+
+/* out[s, l*c0 + c, p] = x[s, c, p] > thresholds[l] ? 1 : 0 for l < levels: the threshold-major channel
+ * concatenation of the reference's input transform (torch.cat([(x > t).float() for t in thresholds]),
+ * src/convlogic/data.py:46-50), applied to a batch x [n, c0, hw] of float32 images. */
+int clg_threshold_images(const float *x, const float *thresholds, float *out /*[n, levels*c0, hw]*/, int64_t n,
+                         int64_t c0, int64_t hw, int64_t levels, void *stream);
+
+/* The same comparison written straight into packed words for clg_convblock_eval_packed:
+ * words [ceil(n/64), levels*c0, hw], bit s of group g = sample 64 g + s (missing samples of the last
+ * group are 0).  Fuses src/convlogic/data.py:46-50 with the packing of
+ * src/difflogic/packbitstensor.py:12-21; the float {0,1} tensor is never materialised. */
+int clg_threshold_pack_images(const float *x, const float *thresholds, uint64_t *words, int64_t n, int64_t c0,
+                              int64_t hw, int64_t levels, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -462,3 +462,25 @@ def conv_block_eval_packed(words, gates, sel, stride, pad, kernel):
 
     root = level(level(level([tap(t) for t in range(8)], 0), 4), 6)[0]
     return root[:, :, 0::2, 0::2] | root[:, :, 0::2, 1::2] | root[:, :, 1::2, 0::2] | root[:, :, 1::2, 1::2]
+
+
+# ----------------------------------------------------------------------------
+# input binarisation -- src/convlogic/data.py:46-71
+# ----------------------------------------------------------------------------
+def thresholds_uniform(levels):
+    """src/convlogic/data.py:56-59."""
+    return torch.linspace(1, levels, levels, dtype=torch.float32) / (levels + 1)
+
+
+def thresholds_distributive(x_all, levels):
+    """src/convlogic/data.py:62-65."""
+    sorted_x = torch.sort(x_all.reshape(-1))[0]
+    idx = (sorted_x.shape[0] * torch.arange(1, levels + 1) / (levels + 1)).long()
+    return sorted_x[idx]
+
+
+def apply_thresholds(x, thresholds):
+    """One image [C,H,W] -> [L*C,H,W], or a batch [N,C,H,W] -> [N,L*C,H,W]: threshold-major
+    concatenation of (x > t) (src/convlogic/data.py:46-50 concatenates along dim 0 of one image)."""
+    dim = 0 if x.dim() == 3 else 1
+    return torch.cat([(x > t).float() for t in thresholds], dim=dim)

@@ -347,3 +347,24 @@ def test_conv_block_eval_packed_all_gates_truth_table():
                 img[:, 0], img[:, 1] = -a, -b                           # all 64 samples set or clear
                 y = O.conv_block_eval_packed(img, gates, sel.numpy(), (1, 1), (0, 0), (1, 1))
                 assert y.shape == (1, 1, 1, 1) and int(y[0, 0, 0, 0]) == -((i >> (3 - 2 * a - b)) & 1), (i, a, b)
+
+
+# ---- input binarisation --------------------------------------------------------------------------
+def test_thresholds_closed_forms():
+    assert torch.allclose(O.thresholds_uniform(3), torch.tensor([0.25, 0.5, 0.75]))          # BASELINE config 4: linspace(1,3,3)/4
+    assert torch.allclose(O.thresholds_uniform(1), torch.tensor([0.5]))
+    x = torch.arange(100, dtype=torch.float32).flip(0) / 100                                  # sorted: 0.00 .. 0.99
+    assert torch.allclose(O.thresholds_distributive(x, 3), torch.tensor([0.25, 0.50, 0.75]))  # index floor(100 i / 4)
+    assert torch.allclose(O.thresholds_distributive(x, 1), torch.tensor([0.50]))
+
+
+def test_apply_thresholds_is_threshold_major_and_strict():
+    img = torch.tensor([[[0.25, 0.3]], [[0.5, 0.9]]])                                         # [C=2, 1, 2]
+    out = O.apply_thresholds(img, torch.tensor([0.25, 0.5, 0.75]))
+    assert out.shape == (6, 1, 2)
+    # channel l*C + c; the comparison is strict (0.25 > 0.25 is false)
+    assert out[:, 0].tolist() == [[0.0, 1.0], [1.0, 1.0], [0.0, 0.0], [0.0, 1.0], [0.0, 0.0], [0.0, 1.0]]
+    batch = torch.rand(5, 2, 3, 4)
+    got = O.apply_thresholds(batch, torch.tensor([0.3, 0.6]))
+    for n in range(5):
+        assert torch.equal(got[n], O.apply_thresholds(batch[n], torch.tensor([0.3, 0.6])))
