@@ -4,10 +4,11 @@
 Primary line (BASELINE config 2): packed-bit inference through 3 LogicLayers of 64000 neurons on
 65536 samples packed into int64 words -> samples/s, with the HBM roofline of the evaluation kernel
 and the CPU oracle timed on the host cores beside it.  The "also" array carries the float
-workloads (config 1 LogicLayer, configs 3 and 4 ConvLogic block, forward+backward) in
-Ggate-evals/s, each with its own roofline entry.
+workloads (config 1 LogicLayer, configs 3 and 4 ConvLogic block, config 5 whole network,
+forward+backward) in Ggate-evals/s, each with its own roofline entry, the packed inference of the
+whole network and the streaming kernels around the packed path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2|c1|c3|c4] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only c2|c1|c3|c4|c5|stream] [--no-cpu]
 
 Prints ONE JSON line.  Inputs are synthetic and resident in HBM before the timed region.
 """
@@ -371,12 +372,179 @@ def bench_conv(key, steps, warmup, cpu=True):
     return out
 
 
+# ------------------------------------------------------------------------------------------------
+# config 5: whole network, training step and packed inference
+# ------------------------------------------------------------------------------------------------
+def bench_c5(steps, warmup, cpu=True):
+    import torch
+
+    import convlogic_amd as C
+    from convlogic_amd.convlogic import binarize
+
+    dev = "cuda:0"
+    n, k = 256, 32
+    torch.manual_seed(3)
+    model = C.ConvLogicCifarModel(k_param=k, input_channels=9, input_size=32, tau=6.5).to(dev)
+    with torch.no_grad():
+        for m in model.network:
+            if hasattr(m, "weights"):
+                m.weights.copy_(torch.randn_like(m.weights))          # random init, as the config says
+    v = (torch.randn(n, 3, 32, 32, device=dev) * 0.25 + 0.5).clamp(0, 1)
+    thr = binarize.uniform_thresholds(3)
+    x = binarize.apply_thresholds(v, thr)
+    labels = torch.randint(0, 10, (n,), device=dev)
+    params = [p for p in model.parameters()]
+
+    def step(_k):
+        for p in params:
+            p.grad = None
+        torch.nn.functional.cross_entropy(model(x), labels).backward()
+
+    sec = _timed(step, steps, warmup)
+    import copy
+
+    def leaves():
+        m2 = copy.deepcopy(model)
+        return [m2] + [p for p in m2.parameters()]
+
+    def run(lv):
+        torch.nn.functional.cross_entropy(lv[0](x), labels).backward()
+
+    graph_ms = _graph_step_ms(leaves, run, max(steps, 20))
+    # gate evaluations of one forward pass: 7 per kernel and conv position, 1 per neuron and sample
+    ge = 0
+    size = 32
+    for m in model.network:
+        if isinstance(m, C.ConvLogicLayer):
+            ge += n * m.out_channels * size * size * 7
+            size //= 2
+        elif isinstance(m, C.LogicLayer):
+            ge += n * m.out_dim
+    alg = 525e6                                                   # compulsory bytes of one training step (all layers, fwd+bwd)
+    out = {"workload": f"C5: ConvLogicCifarModel k={k}, 9 input channels, batch {n}, float32 training step (fwd + CE loss + bwd)",
+           "metric": "convlogic_fwd_bwd_Ggate_evals_per_s", "value": ge / sec / 1e9, "unit": "Ggate-evals/s", "ms_per_step": sec * 1e3,
+           "dtype": "f32", "ms_per_step_hip_graph": graph_ms, "value_hip_graph": (ge / (graph_ms * 1e-3) / 1e9) if graph_ms else None,
+           "roofline": _roof("whole training step (all kernels)", alg, graph_ms if graph_ms else sec * 1e3)}
+
+    # packed inference of the same network: thresholds + packing fused, 65536 samples
+    model.eval()
+    big = 65536
+    vb = (torch.randn(big, 3, 32, 32, device=dev) * 0.25 + 0.5).clamp(0, 1)
+    ev = _events(max(steps, 5))
+    with torch.no_grad():
+        for _ in range(2):
+            model(binarize.pack_thresholds(vb, thr))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for a_, b_ in ev:
+            p = binarize.pack_thresholds(vb, thr)
+            a_.record()
+            model(p)
+            b_.record()
+        torch.cuda.synchronize()
+        el = (time.perf_counter() - t0) / len(ev)
+    net_ms = _avg_ms(ev)
+    out["packed_inference"] = {"samples": big, "samples_per_s_from_float_images": big / el, "samples_per_s_network_only": big / (net_ms * 1e-3),
+                               "ms_network_only": net_ms, "ms_with_threshold_pack": el * 1e3,
+                               "note": "float32 images [65536,3,32,32] resident in HBM -> thresholds + bit packing -> 4 packed blocks, "
+                                       "flatten, 3 packed LogicLayers, per-class counts"}
+    if cpu:
+        out["cpu_baseline"] = _cpu_c5(model, x, labels, ge // n)
+    return out
+
+
+def _cpu_c5(model, x, labels, gate_evals_per_sample):
+    """Training step of the torch-CPU oracle on a bounded sample of the batch."""
+    import torch
+
+    import convlogic_amd as C
+    from oracle import convlogic_oracle as O
+
+    nb = 4
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    xs, ys = x[:nb].cpu(), labels[:nb].cpu()
+    layers = []
+    for m in model.network:
+        if hasattr(m, "weights"):
+            layers.append((m, m.weights.detach().cpu().requires_grad_(True)))
+        else:
+            layers.append((m, None))
+
+    def cpu_step():
+        h = xs
+        for m, w in layers:
+            if w is not None:
+                w.grad = None
+            if isinstance(m, C.ConvLogicLayer):
+                h = O.conv_block_forward(h, torch.softmax(w, -1), m.selection.cpu(), tuple(m.stride), tuple(m.padding), tuple(m.kernel))
+            elif isinstance(m, C.LogicLayer):
+                h = O.logic_fc_forward(h, m.indices_0.cpu(), m.indices_1.cpu(), torch.softmax(w, -1))
+            elif isinstance(m, torch.nn.Flatten):
+                h = h.flatten(1)
+            else:
+                h = O.group_sum(h, m.k, m.tau)
+        torch.nn.functional.cross_entropy(h, ys).backward()
+
+    cpu_step()
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 5.0 and reps < 20:
+        cpu_step()
+        reps += 1
+    el = time.perf_counter() - t0
+    return {"value": nb * gate_evals_per_sample * reps / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{nb} of {x.shape[0]} samples, {reps} training steps of the vectorised torch-CPU oracle in {el:.1f} s"}
+
+
+# ------------------------------------------------------------------------------------------------
+# streaming kernels around the packed path: pack, per-class counts, thresholds + pack
+# ------------------------------------------------------------------------------------------------
+def bench_stream(steps, warmup, cpu=True):
+    import torch
+
+    from convlogic_amd.hip import convlogic_hip, difflogic_hip
+
+    dev = "cuda:0"
+    reps = max(steps, 5)
+    res = []
+
+    def timed(fn):
+        for _ in range(max(warmup, 2)):
+            fn()
+        ev = _events(reps)
+        for a_, b_ in ev:
+            a_.record()
+            fn()
+            b_.record()
+        torch.cuda.synchronize()
+        return _avg_ms(ev)
+
+    batch, feats = 8192, 64000
+    t = torch.randint(0, 2, (batch, feats), device=dev, dtype=torch.uint8).bool()
+    ms = timed(lambda: difflogic_hip.tensor_packbits_sample_major(t, 64))
+    res.append(dict(_roof("pack_bits_sm_kernel", batch * feats + batch * feats // 8, ms),
+                    workload=f"PackBitsTensor: bool [{batch},{feats}] -> int64 words [{feats},{batch // 64}]"))
+    del t
+    words = torch.randint(-2**63, 2**63 - 1, (feats, 1024), device=dev, dtype=torch.int64)
+    ms = timed(lambda: difflogic_hip.groupbitsum(words, 0, 10))
+    res.append(dict(_roof("group_bit_sum_columns_kernel", feats * 1024 * 8 + 65536 * 10 * 4, ms),
+                    workload=f"group_sum: words [{feats},1024] -> int32 [65536,10]"))
+    del words
+    imgs = torch.rand(65536, 3, 32, 32, device=dev)
+    thr = torch.tensor([0.25, 0.5, 0.75], device=dev)
+    ms = timed(lambda: convlogic_hip.threshold_pack_images(imgs, thr))
+    res.append(dict(_roof("threshold_pack_kernel", imgs.numel() * 4 + imgs.numel() * 3 // 8, ms),
+                    workload="thresholds + packing: float32 [65536,3,32,32], 3 levels -> words [1024,9,32,32]"))
+    return {"workload": "streaming kernels of the packed path (kernel launches timed with events)", "metric": "hbm_GBps",
+            "value": max(r["achieved"] for r in res), "unit": "GB/s", "ms_per_step": sum(r["avg_launch_ms"] for r in res), "dtype": "u8",
+            "roofline": res[0], "kernels": res}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", default="", help="c1|c2|c3|c4: run just that workload")
+    ap.add_argument("--only", default="", help="c1|c2|c3|c4|c5|stream: run just that workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -392,7 +560,8 @@ def main():
     _lib.load()
     cpu = not args.no_cpu
     runners = {"c2": lambda: bench_c2(args.steps, args.warmup, cpu), "c1": lambda: bench_c1(args.steps, args.warmup, cpu),
-               "c3": lambda: bench_conv("c3", args.steps, args.warmup, cpu), "c4": lambda: bench_conv("c4", args.steps, args.warmup, cpu)}
+               "c3": lambda: bench_conv("c3", args.steps, args.warmup, cpu), "c4": lambda: bench_conv("c4", args.steps, args.warmup, cpu),
+               "c5": lambda: bench_c5(args.steps, args.warmup, cpu), "stream": lambda: bench_stream(args.steps, args.warmup, cpu)}
     if args.only:
         res = runners[args.only]()
         primary, also = res, []
@@ -401,13 +570,14 @@ def main():
             primary["config"] = {"workload": primary.pop("workload")}
     else:
         primary = runners["c2"]()
-        also = [runners[k]() for k in ("c4", "c3", "c1")]
+        also = [runners[k]() for k in ("c4", "c3", "c1", "c5", "stream")]
     line = {"metric": primary["metric"], "value": primary["value"], "unit": primary["unit"], "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": primary["ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": primary["dtype"], "data": "synthetic", "config": primary["config"],
             "roofline": primary["roofline"], "cpu_baseline": primary.get("cpu_baseline"),
             "device": torch.cuda.get_device_name(0), "host_cores": os.cpu_count()}
-    for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s"):
+    for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s", "kernels", "packed_inference",
+                  "ms_per_step_hip_graph", "value_hip_graph"):
         if extra in primary:
             line[extra] = primary[extra]
     if also:

@@ -15,7 +15,8 @@ TORCH_WORD = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
 
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
-@pytest.mark.parametrize("batch,features", [(1, 1), (7, 3), (64, 5), (100, 130), (129, 257), (1000, 33), (4096, 16)])
+@pytest.mark.parametrize("batch,features", [(1, 1), (7, 3), (64, 5), (100, 130), (129, 257), (1000, 33), (4096, 16), (70, 48),
+                                            (257, 1024), (64, 4112), (5, 32)])
 def test_pack_bits_both_layouts(bits, batch, features):
     rng = np.random.default_rng(batch * 7 + features)
     t = rng.integers(0, 2, (batch, features)).astype(bool)
@@ -45,7 +46,7 @@ def test_eval_packed_bit_exact(bits, batch):
 
 @pytest.mark.parametrize("bits,batch,features,k", [(64, 256, 40, 10), (32, 100, 12, 3), (8, 9, 4, 2), (64, 5000, 2000, 10), (16, 33, 6, 6),
                                                    (64, 4133, 84, 4), (32, 4200, 30, 3), (8, 600, 9, 1), (64, 8192, 2400, 4),
-                                                   (64, 4096, 7, 7)])
+                                                   (64, 4096, 7, 7), (64, 4096, 40000, 2)])
 def test_group_bit_sum(bits, batch, features, k):
     rng = np.random.default_rng(batch + features)
     t = rng.integers(0, 2, (features, batch)).astype(bool)
