@@ -345,6 +345,7 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
         const int64_t ct_cap = 32768 / ((int64_t)params_per_kernel * elem);   // at most 32 KiB of gate parameters
         int64_t ct = g.c < ct_cap ? g.c : ct_cap;
         while (ct > 4 && groups * clg_ceil_div(g.c, ct) < 512) ct = (ct + 1) / 2;
+        ct = clg_ceil_div(g.c, clg_ceil_div(g.c, ct));               // equal tiles
         p->CT = (int)ct;
     }
     // measurement overrides
