@@ -43,22 +43,35 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 // input gradient
 // ---------------------------------------------------------------------------------------------
-// Scratch of the input-gradient kernel, written by one preparation launch:
+// Scratch of the input-gradient kernels, written by the preparation launches:
 //   folded [c][7][4]   coefficients (ab, a, b, one) of every gate
-//   count  [cin]       number of kernels that read input channel ch
-//   hits   [cin][c]    those kernels in increasing order, entry = kernel | tap mask << 16
-// (the reverse map "input channel -> kernels and taps reading it", built in a fixed order).
+//   count  [cin][2]    (number of kernels that read input channel ch, offset of its list in hits)
+//   hits               those kernels in increasing order, entry = kernel | tap mask << 16
+// (the reverse map "input channel -> kernels and taps reading it", built in a fixed order).  Small maps
+// are dense, hits[cin][c], filled by one wavefront per channel.  Large ones (cin * c above 2^20) are
+// compressed: lists back to back (at most 8 c entries), filled through integer atomics and then sorted per
+// channel, so the order of the lists -- and with it the order of the float additions -- stays fixed.
 struct BwdScratch {
-    size_t folded_bytes, count_off, hits_off, taps_off, part_off, total;
+    size_t folded_bytes, count_off, cursor_off, hits_off, unsorted_off, taps_off, part_off, total;
+    int csr;
 };
 constexpr int kMaxHitSplit = 16;
+bool hits_compressed(const Geom &g)
+{
+    if (const char *e = getenv("CLG_BWDX_CSR")) return atoi(e) != 0;
+    return (int64_t)g.cin * g.c > (1ll << 20);
+}
 BwdScratch bwd_scratch_layout(const Geom &g, int elem, int hit_split)
 {
     BwdScratch b;
+    b.csr = hits_compressed(g) ? 1 : 0;
+    const size_t list_bytes = b.csr ? (size_t)g.c * 8 * 4 : (size_t)g.cin * g.c * 4;
     b.folded_bytes = (size_t)g.c * 28 * elem;
     b.count_off = (b.folded_bytes + 63) & ~(size_t)63;
-    b.hits_off = (b.count_off + (size_t)g.cin * 4 + 63) & ~(size_t)63;
-    b.taps_off = (b.hits_off + (size_t)g.cin * g.c * 4 + 63) & ~(size_t)63;
+    b.cursor_off = (b.count_off + (size_t)g.cin * 8 + 63) & ~(size_t)63;
+    b.hits_off = (b.cursor_off + (b.csr ? (size_t)g.cin * 4 : 0) + 63) & ~(size_t)63;
+    b.unsorted_off = (b.hits_off + list_bytes + 63) & ~(size_t)63;
+    b.taps_off = (b.unsorted_off + (b.csr ? list_bytes : 0) + 63) & ~(size_t)63;
     b.part_off = (b.taps_off + (size_t)g.c * 16 * 4 + 255) & ~(size_t)255;   // taps: 8 offsets in the image, 8 in the plane
     b.total = b.part_off + (hit_split > 1 ? (size_t)hit_split * g.n * g.cin * g.h * g.w * elem : 0);   // partial images
     return b;
@@ -91,7 +104,7 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
     // one wavefront per input channel: lanes test 64 kernels at a time, matches are appended in order
     const int lane = threadIdx.x & (kWave - 1);
     const int ch = uniform((int)(blockIdx.x - fold_blocks) * 4 + (int)(threadIdx.x >> 6));
-    if (ch >= cin) return;
+    if (ch >= cin || hits == nullptr) return;
     int n = 0;
     for (int c0 = 0; c0 < C; c0 += kWave) {
         const int c = c0 + lane;
@@ -107,7 +120,96 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
         }
         n += __popcll(vote);
     }
-    if (lane == 0) count[ch] = n;
+    if (lane == 0) {
+        count[2 * ch] = n;
+        count[2 * ch + 1] = ch * C;
+    }
+}
+
+// ---- compressed lists ------------------------------------------------------------------------
+// tap mask of kernel c for the channel of its tap t, or 0 when an earlier tap names the same channel
+__device__ __forceinline__ int first_use_mask(const int32_t *__restrict__ sq, int t)
+{
+    const int ch = (sq[t] >> 16) & 0xFFFF;
+    int mask = 0;
+    for (int u = 0; u < 8; ++u) {
+        if (((sq[u] >> 16) & 0xFFFF) == ch) {
+            if (u < t) return 0;
+            mask |= 1 << u;
+        }
+    }
+    return mask;
+}
+__global__ __launch_bounds__(256) void hits_zero_kernel(int32_t *__restrict__ count, int32_t *__restrict__ cursor, int cin)
+{
+    const int ch = blockIdx.x * 256 + threadIdx.x;
+    if (ch >= cin) return;
+    count[2 * ch] = 0;
+    count[2 * ch + 1] = 0;
+    cursor[ch] = 0;
+}
+__global__ __launch_bounds__(256) void hits_count_kernel(const int32_t *__restrict__ sel, int32_t *__restrict__ count, int C)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int32_t *sq = sel + (int64_t)c * 8;
+    for (int t = 0; t < 8; ++t)
+        if (first_use_mask(sq, t)) atomicAdd(count + 2 * ((sq[t] >> 16) & 0xFFFF), 1);
+}
+// exclusive prefix sum of the counts into the offsets, one workgroup
+__global__ __launch_bounds__(1024) void hits_scan_kernel(int32_t *__restrict__ count, int cin)
+{
+    __shared__ int part[1024];
+    const int tid = threadIdx.x;
+    const int per = (cin + 1023) / 1024;
+    const int lo = tid * per, hi = min(cin, lo + per);
+    int sum = 0;
+    for (int ch = lo; ch < hi; ++ch) sum += count[2 * ch];
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int v = tid >= d ? part[tid - d] : 0;
+        __syncthreads();
+        part[tid] += v;
+        __syncthreads();
+    }
+    int run = part[tid] - sum;
+    for (int ch = lo; ch < hi; ++ch) {
+        count[2 * ch + 1] = run;
+        run += count[2 * ch];
+    }
+}
+__global__ __launch_bounds__(256) void hits_fill_kernel(const int32_t *__restrict__ sel, const int32_t *__restrict__ count,
+                                                      int32_t *__restrict__ cursor, int32_t *__restrict__ unsorted, int C)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int32_t *sq = sel + (int64_t)c * 8;
+    for (int t = 0; t < 8; ++t) {
+        const int mask = first_use_mask(sq, t);
+        if (mask) {
+            const int ch = (sq[t] >> 16) & 0xFFFF;
+            unsorted[count[2 * ch + 1] + atomicAdd(cursor + ch, 1)] = c | (mask << 16);
+        }
+    }
+}
+// one wavefront per channel: every entry goes to the position given by the number of smaller kernel
+// indices in its list (a kernel occurs once per list)
+__global__ __launch_bounds__(256) void hits_sort_kernel(const int32_t *__restrict__ count, const int32_t *__restrict__ unsorted,
+                                                      int32_t *__restrict__ hits, int cin)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int ch = uniform((int)blockIdx.x * 4 + (int)(threadIdx.x >> 6));
+    if (ch >= cin) return;
+    const int n = count[2 * ch];
+    const int32_t *src = unsorted + count[2 * ch + 1];
+    int32_t *dst = hits + count[2 * ch + 1];
+    for (int i = lane; i < n; i += kWave) {
+        const int e = src[i], key = e & 0xFFFF;
+        int rank = 0;
+        for (int j = 0; j < n; ++j) rank += (src[j] & 0xFFFF) < key;
+        dst[rank] = e;
+    }
 }
 
 constexpr int kChunk = 4;  // cell blocks (of 64 lanes) whose grad_y / argmax loads are in flight together
@@ -214,8 +316,8 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
         const int chunks = (v_here + kChunk * kWave - 1) / (kChunk * kWave);
         const int img0 = s0 * g.cin * chs;                          // LDS offset of the group's first plane
         const int64_t gbase = ((int64_t)(n0 + s0) * g.c) * I;       // global offset of the group's first cell row
-        const int nhits = v_here > 0 ? count[ch] : 0;
-        const int32_t *hit = hits + (int64_t)ch * g.c;
+        const int nhits = v_here > 0 ? count[2 * ch] : 0;
+        const int32_t *hit = hits + count[2 * ch + 1];
 
         // chunk-major: the cell table entries of a chunk stay in registers while all kernels that read
         // this channel are applied to it (hits in increasing kernel order inside every chunk)
@@ -363,8 +465,8 @@ __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const 
     for (int i = lane; i < p.xe + kWave; i += kWave) gs[i] = T(0);
 
     const int v_here = g_here * I;
-    const int nhits = count[ch];
-    const int32_t *hit = hits + (int64_t)ch * g.c;
+    const int nhits = count[2 * ch];
+    const int32_t *hit = hits + count[2 * ch + 1];
     const int64_t gbase = (int64_t)n0 * g.c * I;
     const int row_step = g.sh * p.rs;
     for (int blk = 0; blk * kWave < v_here; ++blk) {
@@ -729,11 +831,21 @@ int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
                    hipStream_t st)
 {
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
-    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), csr_blocks = (int)clg_ceil_div(g.cin, 4);
-    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + csr_blocks)), dim3(256), 0, st, (const T *)w, sel,
-                       reinterpret_cast<T *>(base), reinterpret_cast<int32_t *>(base + lay.count_off),
-                       reinterpret_cast<int32_t *>(base + lay.hits_off), reinterpret_cast<int32_t *>(base + lay.taps_off), g.c, g.cin,
-                       fold_blocks, rs, chs);
+    int32_t *count = reinterpret_cast<int32_t *>(base + lay.count_off), *hits = reinterpret_cast<int32_t *>(base + lay.hits_off);
+    const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), list_blocks = lay.csr ? 0 : (int)clg_ceil_div(g.cin, 4);
+    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + list_blocks)), dim3(256), 0, st, (const T *)w, sel,
+                       reinterpret_cast<T *>(base), count, lay.csr ? nullptr : hits, reinterpret_cast<int32_t *>(base + lay.taps_off),
+                       g.c, g.cin, fold_blocks, rs, chs);
+    if (lay.csr) {
+        int32_t *cursor = reinterpret_cast<int32_t *>(base + lay.cursor_off), *unsorted = reinterpret_cast<int32_t *>(base + lay.unsorted_off);
+        const unsigned cb = (unsigned)clg_ceil_div(g.c, 256);
+        hipLaunchKernelGGL(hits_zero_kernel, dim3((unsigned)clg_ceil_div(g.cin, 256)), dim3(256), 0, st, count, cursor, g.cin);
+        hipLaunchKernelGGL(hits_count_kernel, dim3(cb), dim3(256), 0, st, sel, count, g.c);
+        hipLaunchKernelGGL(hits_scan_kernel, dim3(1), dim3(1024), 0, st, count, g.cin);
+        hipLaunchKernelGGL(hits_fill_kernel, dim3(cb), dim3(256), 0, st, sel, (const int32_t *)count, cursor, unsorted, g.c);
+        hipLaunchKernelGGL(hits_sort_kernel, dim3((unsigned)clg_ceil_div(g.cin, 4)), dim3(256), 0, st, (const int32_t *)count,
+                           (const int32_t *)unsorted, hits, g.cin);
+    }
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(prepare)");
     return CLG_OK;
 }

@@ -170,8 +170,8 @@ __global__ __launch_bounds__(kBlk) void convblock_backward_x_hits_kernel(const T
     const int ch = (int)((e / ((int64_t)g.w * g.h)) % g.cin), n = (int)(e / ((int64_t)g.w * g.h * g.cin));
     const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
     const int wp = g.wo / 2, I = (g.ho / 2) * wp;
-    const int nhits = count[ch];
-    const int32_t *hit = hits + (int64_t)ch * g.c;
+    const int nhits = count[2 * ch];
+    const int32_t *hit = hits + count[2 * ch + 1];
     T acc = 0;
     for (int k = 0; k < nhits; ++k) {
         const int ent = hit[k];

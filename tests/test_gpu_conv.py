@@ -94,6 +94,8 @@ def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monke
     if direct:
         monkeypatch.setenv("CLG_BWDX_DIRECT", direct)
         monkeypatch.setenv("CLG_FWD_SUBSET", direct)
+    if binary:
+        monkeypatch.setenv("CLG_BWDX_CSR", "1")                    # compressed channel -> kernel lists (wide layers)
     n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad
     if ((h + 2 * pad - kernel) // stride + 1) % 2:
         h += stride
@@ -194,7 +196,7 @@ def test_block_benchmark_shapes_vs_oracle(shape):
 
 
 @pytest.mark.parametrize("shape", [(37, 24, 48, 4, 4), (5, 200, 40, 16, 16), (3, 64, 32, 32, 32), (9, 40, 24, 6, 6),
-                                   (70, 6, 12, 2, 2)])
+                                   (70, 6, 12, 2, 2), (4, 1024, 2048, 4, 4)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_block_deep_and_wide_shapes_vs_oracle(shape, dtype):
     # few cells per sample (several samples share a wavefront, ragged last group) and images too large for LDS
