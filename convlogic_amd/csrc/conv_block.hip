@@ -480,41 +480,46 @@ __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const 
         const int gp = (int)((n0 + sm) * (uint32_t)sample_elems) + rel;
         const int lp = (int)(sm * p.chs) + rel;
         const int cy = (int)((sm * g.c) * I + cl);
-        int code_n = 0;
-        T gy_n = T(0);
-        auto issue = [&](int k) {
+        // three hits in flight: grad_y / arg-max of hit k+2 and the taps of hit k+1 (which need the arg-max
+        // loaded one step earlier) are requested before hit k is computed
+        auto load_cell = [&](int k, int &code, T &gout) {
             const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
-            code_n = 0;
-            gy_n = T(0);
+            code = 0;
+            gout = T(0);
             if (live) {
-                code_n = argmax[crow + cy];
-                gy_n = gy[crow + cy];
+                code = argmax[crow + cy];
+                gout = gy[crow + cy];
             }
         };
-        if (nhits > 0) issue(0);
+        auto load_taps = [&](int k, int code, int &off, T (&tv)[8]) {
+            const int c = hit[k] & 0xFFFF;
+            off = (code >> 1) * row_step + (code & 1) * g.sw;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) tv[t] = xp[gp + off + taps[c * 16 + t]];
+        };
+        int code1 = 0, code2 = 0, off0 = 0, off1 = 0;
+        T gy0 = T(0), gy1 = T(0), gy2 = T(0);
+        T tv0[8], tv1[8];
+        if (nhits > 0) {
+            load_cell(0, code1, gy0);
+            load_taps(0, code1, off0, tv0);
+        }
+        if (nhits > 1) load_cell(1, code1, gy1);
         for (int k = 0; k < nhits; ++k) {
-            const int code = code_n;
-            const T gout = gy_n;
-            if (k + 1 < nhits) issue(k + 1);
+            if (k + 2 < nhits) load_cell(k + 2, code2, gy2);
+            if (k + 1 < nhits) load_taps(k + 1, code1, off1, tv1);
             const int ent = hit[k];
             const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
-            int to[8], tr_[8];
+            int tr_[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                to[t] = taps[c * 16 + t];
-                tr_[t] = taps[c * 16 + 8 + t];
-            }
+            for (int t = 0; t < 8; ++t) tr_[t] = taps[c * 16 + 8 + t];
             Tree<T> tr;
             const T *fc = folded + (int64_t)c * 28;
 #pragma unroll
             for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
-            const int off = (code >> 1) * row_step + (code & 1) * g.sw;
-            T tv[8];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) tv[t] = xp[gp + off + to[t]];
-            const TreeVals<T> tvv = eval_tree(tr, tv);
-            const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
-            const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
+            const TreeVals<T> tvv = eval_tree(tr, tv0);
+            const T g_m0 = gy0 * gate_da(tr.g[6], tvv.mid[1]);
+            const T g_m1 = gy0 * gate_db(tr.g[6], tvv.mid[0]);
             T gt[8];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -522,18 +527,24 @@ __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const 
                     const int m = q >> 1;
                     const T g_mid = m ? g_m1 : g_m0;
                     const T g_leaf = g_mid * ((q & 1) ? gate_db(tr.g[4 + m], tvv.leaf[q ^ 1]) : gate_da(tr.g[4 + m], tvv.leaf[q ^ 1]));
-                    gt[2 * q] = g_leaf * gate_da(tr.g[q], tv[2 * q + 1]);
-                    gt[2 * q + 1] = g_leaf * gate_db(tr.g[q], tv[2 * q]);
+                    gt[2 * q] = g_leaf * gate_da(tr.g[q], tv0[2 * q + 1]);
+                    gt[2 * q + 1] = g_leaf * gate_db(tr.g[q], tv0[2 * q]);
                 }
             }
             // for one tap the targets of all lanes are distinct elements; taps are applied one after the other
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 if ((mask >> t) & 1) {                               // wave-uniform
-                    const int at = live ? lp + off + tr_[t] : dummy;
+                    const int at = live ? lp + off0 + tr_[t] : dummy;
                     gs[at] = gs[at] + gt[t];
                 }
             }
+            off0 = off1;
+            gy0 = gy1;
+            gy1 = gy2;
+            code1 = code2;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) tv0[t] = tv1[t];
         }
     }
     // interior of the G planes -> gx
