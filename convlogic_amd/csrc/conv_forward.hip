@@ -58,6 +58,15 @@ struct FloatOps {
         }
         return pr;
     }
+    // folded = [c_out][7][4] coefficients written by convblock_w_prepare_kernel
+    static __device__ __forceinline__ Params load_global(const void *__restrict__ folded, int c)
+    {
+        const T *fc = reinterpret_cast<const T *>(folded) + (int64_t)c * 28;
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) pr.tr.g[k] = Coef<T>{fc[4 * k], fc[4 * k + 1], fc[4 * k + 2], fc[4 * k + 3]};
+        return pr;
+    }
     static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8]) { return eval_tree(pr.tr, v).root; }
     // strict > in window order (0,0),(0,1),(1,0),(1,1): the first maximum wins
     static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
@@ -96,6 +105,14 @@ struct BitOps {
         Params pr;
 #pragma unroll
         for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks((pk >> (4 * k)) & 15);
+        return pr;
+    }
+    static __device__ __forceinline__ Params load_global(const void *__restrict__ gates, int c)
+    {
+        const uint8_t *gid = reinterpret_cast<const uint8_t *>(gates) + (int64_t)c * 7;
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks(gid[k] & 15);
         return pr;
     }
     static __device__ __forceinline__ Elem gate64(const Masks &m, Elem a, Elem b)
@@ -259,6 +276,53 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     }
 }
 
+// Forward without LDS: for layers whose input channels do not fit LDS or whose images leave lanes idle.
+// Taps come from a zero-padded global copy of x (shared-halo layout, served by L1/L2), so there is no
+// staging, no barrier and no bounds check.  A wavefront keeps one set of 64 lane slots (sample, conv row
+// pair, column) and runs the CT kernels of its tile over it; gate parameters and tap offsets are scalar loads.
+template <typename Ops>
+__global__ __launch_bounds__(256) void convblock_forward_direct_kernel(const typename Ops::Elem *__restrict__ xp,
+                                                                     const void *__restrict__ params,
+                                                                     const int32_t *__restrict__ taps,
+                                                                     typename Ops::Elem *__restrict__ y,
+                                                                     uint8_t *__restrict__ argmax, Geom g, TilePlan p,
+                                                                     int sample_elems, int nblk)
+{
+    using T = typename Ops::Elem;
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    const int groups = (g.n + p.G - 1) / p.G;
+    const int set = uniform((int)blockIdx.x * 4 + wave);
+    if (set >= groups * nblk) return;
+    const int grp = set / nblk, blk = set - grp * nblk;
+    const int n0 = grp * p.G, g_here = min(p.G, g.n - n0);
+    const int U = g_here * p.slots;
+    const int u = blk * kWave + lane;
+    const bool valid = u < U;
+    const uint32_t uu = valid ? u : 0;
+    const uint32_t s = fdiv(uu, p.d_slots), r = uu - s * (uint32_t)p.slots;
+    const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+    const int base = (int)((n0 + s) * (uint32_t)sample_elems + (2 * rp * g.sh) * p.rs + ox * g.sw);
+    const int64_t obase = ((int64_t)(n0 + s) * g.c) * I + rp * wp + (ox >> 1);
+    const int row_step = g.sh * p.rs;
+    const int c0 = blockIdx.y * p.CT, c1 = min(g.c, c0 + p.CT);
+    const bool writer = valid && !(lane & 1);
+    for (int c = c0; c < c1; ++c) {
+        const typename Ops::Params pr = Ops::load_global(params, c);
+        int to[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) to[t] = taps[c * 8 + t];
+        T v0[8], v1[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v0[t] = xp[base + to[t]];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v1[t] = xp[base + row_step + to[t]];
+        const T r0 = Ops::root(pr, v0), r1 = Ops::root(pr, v1);
+        const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
+        if (writer) Ops::pool_store(r0, r0o, r1, r1o, y + obase + (int64_t)c * I, argmax ? argmax + obase + (int64_t)c * I : nullptr, 0);
+    }
+}
+
 // Any shape, packed: one thread per (group, kernel, pooled cell), taps from global memory with bounds checks.
 __global__ __launch_bounds__(256) void convblock_packed_generic_kernel(const uint64_t *__restrict__ x, const uint8_t *__restrict__ gid,
                                                                      const int32_t *__restrict__ sel, uint64_t *__restrict__ y,
@@ -367,6 +431,93 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
            (int64_t)p->S * p->planes * g.h * g.w < (1ll << 31);
 }
 
+// ---- direct (padded global copy) plan ----------------------------------------------------------
+struct DirectPlan {
+    TilePlan p;
+    int sample_elems, nblk;
+    size_t folded_off, taps_off, xp_off, total;   // scratch: [folded] | taps | padded x
+};
+bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan *d)
+{
+    if (!taps_inside(g) || g.c > 65535) return false;
+    TilePlan *p = &d->p;
+    plan_common(g, p);
+    p->slots = (g.ho / 2) * g.wo;
+    p->d_slots = make_fastdiv((uint32_t)p->slots);
+    int G = p->slots >= kWave ? 1 : kWave / p->slots;
+    if (G > g.n) G = g.n;
+    p->G = G;
+    p->S = G;
+    p->NW = 4;
+    const int64_t se = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
+    const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
+    if (se * g.n >= (1ll << 31) || (int64_t)g.n * g.c * I >= (1ll << 62)) return false;
+    d->sample_elems = (int)se;
+    d->nblk = (int)clg_ceil_div((int64_t)G * p->slots, kWave);
+    const int64_t sets = clg_ceil_div(g.n, G) * d->nblk, wgs_x = clg_ceil_div(sets, 4);
+    // kernels per wavefront: enough to amortise the lane set-up, few enough for about 16 workgroups per CU
+    int64_t ct = g.c;
+    while (ct > 16 && wgs_x * clg_ceil_div(g.c, ct) < 4096) ct = (ct + 1) / 2;
+    ct = clg_ceil_div(g.c, clg_ceil_div(g.c, ct));
+    if (const char *e = getenv("CLG_FWD_CT")) ct = atoi(e) < g.c ? atoi(e) : g.c;
+    if (ct < 1) ct = 1;
+    p->CT = (int)ct;
+    if (wgs_x >= (1ll << 31) || clg_ceil_div(g.c, ct) > 65535) return false;
+    d->folded_off = 0;
+    d->taps_off = needs_folded ? (((size_t)g.c * 28 * elem + 255) & ~(size_t)255) : 0;
+    d->xp_off = (d->taps_off + (size_t)g.c * 8 * 4 + 255) & ~(size_t)255;
+    d->total = d->xp_off + (size_t)se * g.n * elem;
+    return true;
+}
+
+// Which forward path a shape takes: 0 = tiled (all channels in LDS), 1 = tiled with channel subsets,
+// 2 = direct from a padded copy (needs scratch), 3 = any-shape kernel.
+int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scratch, TilePlan *tp, DirectPlan *dp)
+{
+    const bool tiled = plan_forward(g, elem, params_per_kernel, tp);
+    const bool direct = have_scratch && plan_forward_direct(g, elem, params_per_kernel > 1, dp);
+    // 4-byte elements: direct beats the channel-subset staging (354 -> 163 us at [256,256,16,16] -> 1024); 8-byte
+    // elements load twice the bytes per tap and stay on the staged kernels (200 vs 329 us at [256,4096,4,4] -> 8192)
+    // (4x4 images: the padded copy is 1.6x the image and both paths tie, 30 vs 35 us at [256,512,4,4] -> 1024).
+    bool use_direct = direct && (!tiled || (tp->subset && elem == 4 && g.h * g.w >= 64));
+    if (const char *e = getenv("CLG_FWD_DIRECT")) use_direct = direct && (atoi(e) != 0 || !tiled);
+    if (use_direct) return 2;
+    if (tiled) return tp->subset ? 1 : 0;
+    return 3;
+}
+
+template <typename Ops, typename P>
+int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, const void *params, const int32_t *sel, void *y,
+                          uint8_t *argmax, void *scratch, hipStream_t st, const char *name)
+{
+    using T = typename Ops::Elem;
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    int32_t *taps = reinterpret_cast<int32_t *>(base + d.taps_off);
+    T *xp = reinterpret_cast<T *>(base + d.xp_off);
+    const void *kernel_params = params;
+    if (Ops::kParams > 1) {                                           // float: fold the probabilities once
+        hipLaunchKernelGGL(convblock_w_prepare_kernel<P>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
+                           (const P *)params, sel, reinterpret_cast<P *>(base), taps, g.c, d.p.rs, d.p.chs);
+        kernel_params = base;
+    } else {
+        hipLaunchKernelGGL(convblock_w_prepare_kernel<P>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
+                           (const P *)nullptr, sel, (P *)nullptr, taps, g.c, d.p.rs, d.p.chs);
+    }
+    CLG_CHECK_LAUNCH(name);
+    TilePlan pp = d.p;
+    pp.d_slots = make_fastdiv((uint32_t)d.p.chs);                     // the pad kernel divides by the plane stride
+    const int64_t total = (int64_t)d.sample_elems * g.n;
+    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, pp,
+                       make_fastdiv((uint32_t)d.sample_elems), make_fastdiv((uint32_t)d.p.rs), d.sample_elems, total);
+    CLG_CHECK_LAUNCH(name);
+    const int64_t sets = clg_ceil_div(g.n, d.p.G) * d.nblk;
+    hipLaunchKernelGGL(convblock_forward_direct_kernel<Ops>, dim3((unsigned)clg_ceil_div(sets, 4), (unsigned)clg_ceil_div(g.c, d.p.CT)),
+                       dim3(256), 0, st, (const T *)xp, kernel_params, (const int32_t *)taps, (T *)y, argmax, g, d.p, d.sample_elems,
+                       d.nblk);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
+}
+
 // ---- launch ------------------------------------------------------------------------------------
 template <typename Ops, int ROWSTEP, bool SUBSET>
 int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
@@ -441,4 +592,53 @@ extern "C" int clg_convblock_eval_packed(const clg_conv_geom *gg, const uint64_t
                        g);
     CLG_CHECK_LAUNCH("clg_convblock_eval_packed(any shape)");
     return CLG_OK;
+}
+
+extern "C" int64_t clg_convblock_forward_scratch_bytes(int dtype, const clg_conv_geom *gg)
+{
+    Geom g;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_forward_scratch_bytes")) return -1;
+    TilePlan tp;
+    DirectPlan dp;
+    const int elem = dtype == CLG_F64 ? 8 : 4;
+    return choose_forward(g, elem, 28, true, &tp, &dp) == 2 ? (int64_t)dp.total : 0;
+}
+
+extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                        void *y, uint8_t *argmax, void *scratch, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_forward_ws")) return e;
+    CLG_REQUIRE(x && w && selection && y && argmax, "clg_convblock_forward_ws: null pointer argument");
+    TilePlan tp;
+    DirectPlan dp;
+    const int elem = dtype == CLG_F64 ? 8 : 4;
+    if (choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp) != 2) return clg_convblock_forward(dtype, gg, x, w, selection, y, argmax, stream);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32)
+        return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
+    return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
+}
+
+extern "C" int64_t clg_convblock_eval_packed_scratch_bytes(const clg_conv_geom *gg)
+{
+    Geom g;
+    if (clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed_scratch_bytes")) return -1;
+    TilePlan tp;
+    DirectPlan dp;
+    return choose_forward(g, 8, 1, true, &tp, &dp) == 2 ? (int64_t)dp.total : 0;
+}
+
+extern "C" int clg_convblock_eval_packed_ws(const clg_conv_geom *gg, const uint64_t *x, const uint8_t *gates, const int32_t *selection,
+                                            uint64_t *y, void *scratch, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed_ws")) return e;
+    CLG_REQUIRE(x && gates && selection && y, "clg_convblock_eval_packed_ws: null pointer argument");
+    CLG_REQUIRE(x != y, "clg_convblock_eval_packed_ws: x and y must not overlap");
+    TilePlan tp;
+    DirectPlan dp;
+    if (choose_forward(g, 8, 1, scratch != nullptr, &tp, &dp) != 2) return clg_convblock_eval_packed(gg, x, gates, selection, y, stream);
+    return launch_forward_direct<BitOps, float>(g, dp, x, gates, selection, y, nullptr, scratch, clg_stream(stream),
+                                                "clg_convblock_eval_packed_ws");
 }

@@ -88,3 +88,43 @@ static inline int allow_lds(K kernel, size_t bytes, const char *name)
 {
     return clg_allow_lds(reinterpret_cast<const void *>(kernel), bytes, name);
 }
+
+// ---- kernels shared by the paths that read taps from a padded global copy of x ------------------
+#if defined(__HIPCC__)
+// xp = zero-padded copy of x in the shared-halo layout: sample n at n * sample_elems, plane stride chs, row
+// stride rs, pixel (iy, ix) at (iy + ph) * rs + ix + pw.  p.d_slots must hold the divisor chs.
+template <typename T>
+__global__ __launch_bounds__(256) void pad_image_kernel(const T *__restrict__ x, T *__restrict__ xp, Geom g, TilePlan p,
+                                                      FastDiv d_sample, FastDiv d_rs, int sample_elems, int64_t total)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const uint32_t n = fdiv((uint32_t)e, d_sample), rem = (uint32_t)e - n * (uint32_t)sample_elems;
+    const uint32_t plane = fdiv(rem, p.d_slots), r2 = rem - plane * (uint32_t)p.chs;      // d_slots holds chs here
+    const uint32_t row = fdiv(r2, d_rs), col = r2 - row * (uint32_t)p.rs;
+    T v = T(0);
+    if (plane < (uint32_t)g.cin && row >= (uint32_t)g.ph && col >= (uint32_t)g.pw)
+        v = x[(((int64_t)n * g.cin + plane) * g.h + (row - g.ph)) * g.w + (col - g.pw)];
+    xp[e] = v;
+}
+
+// folded coefficients [c][28] (skipped when folded is null) and tap offsets [c][8] in the padded-image layout
+template <typename T>
+__global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
+                                                                T *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
+                                                                int chs)
+{
+    const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q < (int64_t)C * 8) {
+        const Tap tp = unpack_tap(sel[q]);
+        taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
+    }
+    if (folded != nullptr && q < (int64_t)C * 7) {
+        const Coef<T> cf = fold16(w + q * 16);
+        folded[q * 4 + 0] = cf.ab;
+        folded[q * 4 + 1] = cf.a;
+        folded[q * 4 + 2] = cf.b;
+        folded[q * 4 + 3] = cf.one;
+    }
+}
+#endif

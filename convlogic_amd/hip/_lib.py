@@ -50,6 +50,10 @@ SIGNATURES = {
     "clg_threshold_images": (_i, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "clg_threshold_pack_images": (_i, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "clg_convblock_eval_packed": (_i, [_GP, _p, _p, _p, _p, _p]),
+    "clg_convblock_eval_packed_ws": (_i, [_GP, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_eval_packed_scratch_bytes": (_i64, [_GP]),
+    "clg_convblock_forward_ws": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_forward_scratch_bytes": (_i64, [_i, _GP]),
     "clg_convblock_intermediates": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_x": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_x_scratch_bytes": (_i64, [_i, _GP]),

@@ -131,8 +131,11 @@ def full_convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_
     shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
     y = torch.empty(shape, dtype=x.dtype, device=x.device)
     argmax = torch.empty(shape, dtype=torch.uint8, device=x.device)
-    check(_lib.load().clg_convblock_forward(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(),
-                                            selection.data_ptr(), y.data_ptr(), argmax.data_ptr(), stream_ptr(x)))
+    lib = _lib.load()
+    scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
+    check(lib.clg_convblock_forward_ws(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(), selection.data_ptr(),
+                                       y.data_ptr(), argmax.data_ptr(), scratch.data_ptr() if scratch is not None else None,
+                                       stream_ptr(x)))
     return y, argmax
 
 
@@ -150,8 +153,10 @@ def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, p
     g = _geom(x, gates.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     y = torch.empty((g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2), dtype=torch.int64, device=x.device)
-    check(_lib.load().clg_convblock_eval_packed(ctypes.byref(g), x.data_ptr(), gates.data_ptr(), selection.data_ptr(),
-                                                y.data_ptr(), stream_ptr(x)))
+    lib = _lib.load()
+    scratch = _scratch(lib.clg_convblock_eval_packed_scratch_bytes(ctypes.byref(g)), x.device)
+    check(lib.clg_convblock_eval_packed_ws(ctypes.byref(g), x.data_ptr(), gates.data_ptr(), selection.data_ptr(), y.data_ptr(),
+                                           scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))
     return y
 
 

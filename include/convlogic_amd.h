@@ -187,6 +187,15 @@ int64_t clg_tree_backward_w_scratch_bytes(int dtype, int64_t n, int64_t c, int64
 int clg_convblock_forward(int dtype, const clg_conv_geom *g, const void *x, const void *w /*[c_out,7,16]*/,
                           const int32_t *selection, void *y, uint8_t *argmax, void *stream);
 
+/* clg_convblock_forward with a caller-provided workspace of clg_convblock_forward_scratch_bytes() bytes
+ * (0 for shapes that do not use one; scratch may then be NULL).  With a workspace, layers whose input
+ * channels do not fit LDS read their taps from a zero-padded copy of x made in it instead of staging
+ * channel subsets.  Same results as clg_convblock_forward; no counterpart in the reference (its forward,
+ * src/convlogic/cuda/full_convlogic_kernel.cu:147-231, allocates its intermediates itself). */
+int64_t clg_convblock_forward_scratch_bytes(int dtype, const clg_conv_geom *g);
+int clg_convblock_forward_ws(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection,
+                             void *y, uint8_t *argmax, void *scratch, void *stream);
+
 /* Packed-bit inference of the block: 64 samples per uint64 word, images word-group major
  * x [n, c_in, h, w] with n = ceil(samples / 64) groups (bit s of group g = sample 64 g + s),
  * gates uint8 [c_out, 7] = arg-max gate id of every tree node (0..3 leaves, 4..5 middle, 6 root),
@@ -196,6 +205,11 @@ int clg_convblock_forward(int dtype, const clg_conv_geom *g, const void *x, cons
  * (src/convlogic/convlogic_layer.py:231-316 with one-hot weights, :321-325) on binary inputs. */
 int clg_convblock_eval_packed(const clg_conv_geom *g, const uint64_t *x, const uint8_t *gates,
                               const int32_t *selection, uint64_t *y, void *stream);
+
+/* clg_convblock_eval_packed with a workspace, as clg_convblock_forward_ws. */
+int64_t clg_convblock_eval_packed_scratch_bytes(const clg_conv_geom *g);
+int clg_convblock_eval_packed_ws(const clg_conv_geom *g, const uint64_t *x, const uint8_t *gates,
+                                 const int32_t *selection, uint64_t *y, void *scratch, void *stream);
 
 /* Intermediates of the block for the return_intermediate / return_indices debug outputs:
  * x2 [n,c_out,ho,wo,4] (leaf gates), x3 [n,c_out,ho,wo,2]; either may be NULL.

@@ -87,13 +87,16 @@ def _run_block(n, cin, cout, h, w, stride, pad, kernel, dtype=torch.float32, bin
 
 @pytest.mark.parametrize("stride,pad,kernel", GEOMS)
 @pytest.mark.parametrize("binary", [False, True])
-@pytest.mark.parametrize("direct", [None, "1"])
+@pytest.mark.parametrize("direct", [None, "1", "subset"])
 def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monkeypatch):
-    # direct="1" forces the input-gradient kernel that reads taps from a padded global copy of x and the
-    # forward staging of two LDS planes per kernel
-    if direct:
-        monkeypatch.setenv("CLG_BWDX_DIRECT", direct)
-        monkeypatch.setenv("CLG_FWD_SUBSET", direct)
+    # "1" forces the kernels that read taps from a padded global copy of x (forward and input gradient);
+    # "subset" forces the forward staging of two LDS planes per kernel
+    if direct == "1":
+        monkeypatch.setenv("CLG_BWDX_DIRECT", "1")
+        monkeypatch.setenv("CLG_FWD_DIRECT", "1")
+    if direct == "subset":
+        monkeypatch.setenv("CLG_FWD_SUBSET", "1")
+        monkeypatch.setenv("CLG_FWD_DIRECT", "0")
     if binary:
         monkeypatch.setenv("CLG_BWDX_CSR", "1")                    # compressed channel -> kernel lists (wide layers)
     n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad

@@ -34,10 +34,13 @@ def _fit_even(h, w, stride, pad, kernel):
 
 @pytest.mark.parametrize("stride,pad,kernel", GEOMS)
 @pytest.mark.parametrize("n", [1, 64, 130])
-@pytest.mark.parametrize("subset", [None, "1"])
+@pytest.mark.parametrize("subset", [None, "1", "direct"])
 def test_packed_block_small_vs_oracle(stride, pad, kernel, n, subset, monkeypatch):
-    if subset:
-        monkeypatch.setenv("CLG_FWD_SUBSET", subset)       # two LDS planes per kernel instead of all channels
+    if subset == "1":
+        monkeypatch.setenv("CLG_FWD_SUBSET", "1")          # two LDS planes per kernel instead of all channels
+        monkeypatch.setenv("CLG_FWD_DIRECT", "0")
+    if subset == "direct":
+        monkeypatch.setenv("CLG_FWD_DIRECT", "1")          # taps from a padded global copy, no LDS
     cin, cout = 3, 6
     h, w = _fit_even(8 + pad, 10 + pad, stride, pad, kernel)
     layer = _layer(cin, cout, stride, pad, kernel, seed=n + stride)
@@ -74,6 +77,7 @@ def test_packed_block_equals_float_eval_path(shape):
 
 @pytest.mark.parametrize("subset", ["0", "1"])
 def test_selection_with_more_than_two_channels_per_kernel(subset, monkeypatch):
+    monkeypatch.setenv("CLG_FWD_DIRECT", "0")
     # a caller-made selection may name up to 8 channels per kernel; the two-planes-per-kernel staging then
     # reads those kernels' taps from global memory (float and packed)
     monkeypatch.setenv("CLG_FWD_SUBSET", subset)
