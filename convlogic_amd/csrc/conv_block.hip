@@ -759,7 +759,11 @@ BwdXMode choose_backward_x(const Geom &g, int elem, TilePlan *p, int *sample_ele
     const bool direct = plan_backward_x_direct(g, elem, &pd, &se);
     const int I = (g.ho / 2) * (g.wo / 2);
     auto lanes = [&](const TilePlan &q) { return q.G * I < kWave ? q.G * I : kWave; };
-    bool use_direct = direct && (!tiled || lanes(pd) >= 2 * lanes(pt));
+    // The direct kernel has one independent wavefront per (sample group, channel) and no barriers: it also wins
+    // when there are thousands of such owners with short kernel lists (48 vs 88 us at [256,32,16,16] -> 128,
+    // 74 vs 164 us at [256,64,16,16] -> 256; few channels with long lists stay tiled: 141 vs 248 us at C4).
+    const int64_t owners = clg_ceil_div(g.n, pd.G) * g.cin, avg_hits = (2 * (int64_t)g.c) / g.cin;
+    bool use_direct = direct && (!tiled || lanes(pd) >= 2 * lanes(pt) || (owners >= 4096 && avg_hits <= 16));
     if (const char *e = getenv("CLG_BWDX_DIRECT")) use_direct = direct && (atoi(e) != 0 || !tiled);
     if (use_direct) {
         *p = pd;
