@@ -186,3 +186,28 @@ def test_cifar_topology_state_dict_round_trip():
         b.load_state_dict(a.state_dict())
         assert torch.equal(ya, b(x.float()))
         assert torch.equal(b(C.PackBitsTensor(x, 64)).float(), torch.round(ya * 6.5))
+
+
+def test_compiled_netlist_runs_the_packed_kernels(tmp_path):
+    # CompiledLogicNet(device="cuda"): the frozen netlist (conv blocks + LogicLayers) evaluated by the packed
+    # kernels equals the module path, before and after a trip through the .npz file
+    from convlogic_amd.difflogic import CompiledLogicNet
+    torch.manual_seed(10)
+    model = C.ConvLogicMnistModel(k_param=4).to(DEV).eval()
+    with torch.no_grad():
+        for m in model.network:
+            if hasattr(m, "weights"):
+                m.weights.copy_(torch.randn_like(m.weights))
+    bits = torch.randint(0, 2, (130, 1, 28, 28), device=DEV).bool()
+    with torch.no_grad():
+        want = model(C.PackBitsTensor(bits, 64))
+    net = CompiledLogicNet(model, device="cuda")
+    assert torch.equal(net(bits), want)
+    net.save(str(tmp_path / "mnist.npz"))
+    back = CompiledLogicNet.load_netlist(str(tmp_path / "mnist.npz"))
+    assert torch.equal(back(bits.cpu()), want) and torch.equal(back(C.PackBitsTensor(bits, 64)), want)
+    # fully connected only, flat input
+    fc = torch.nn.Sequential(C.LogicLayer(64, 128), C.LogicLayer(128, 80), C.GroupSum(10)).to(DEV).eval()
+    x = torch.randint(0, 2, (200, 64), device=DEV).bool()
+    with torch.no_grad():
+        assert torch.equal(CompiledLogicNet(fc)(x), fc(C.PackBitsTensor(x, 64)))

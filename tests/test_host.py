@@ -3,6 +3,7 @@ backend agrees with the oracle, wiring matches the golden vectors, argument vali
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -187,3 +188,53 @@ def test_model_construction_draws_like_the_layers_in_order():
     first = C.ConvLogicLayer(1, 1, kernel=5, padding=0, residual_init=True, complete=True, implementation="python")
     second = C.ConvLogicLayer(1, 3, kernel=3, padding=1, residual_init=True, complete=True, implementation="python")
     assert torch.equal(m.network[0].selection, first.selection) and torch.equal(m.network[1].selection, second.selection)
+
+
+# ---- CompiledLogicNet: generated C (the reference's CPU route) -------------------------------------
+@pytest.mark.parametrize("bits", [8, 64])
+def test_compiled_net_c_code_matches_eval_forward(bits, tmp_path):
+    # src/difflogic/compiled_model.py: forward(bool [N, F]) -> int32 [N, classes] = GroupSum counts of the
+    # eval-mode network; compared with this package's torch-op ("python") implementation on binary inputs
+    from convlogic_amd.difflogic import CompiledLogicNet
+    torch.manual_seed(bits)
+    dims = [12, 24, 18, 12]
+    model = torch.nn.Sequential(torch.nn.Flatten(), *[C.LogicLayer(a, b, implementation="python") for a, b in zip(dims, dims[1:])],
+                                C.GroupSum(3, tau=4.0)).eval()
+    with torch.no_grad():
+        for m in model:
+            if hasattr(m, "weights"):
+                m.weights.copy_(torch.randn_like(m.weights))
+    net = CompiledLogicNet(model, device="cpu", num_bits=bits)
+    assert net.num_inputs == 12 and net.num_classes == 3 and net.num_out_per_class == 4
+    code = net.get_c_code()
+    assert "void logic_gate_net(" in code and "void apply_logic_gate_net(bool const *inp, int *out, size_t len)" in code
+    lib = tmp_path / "net.so"
+    net.compile(save_lib_path=str(lib))
+    x = torch.randint(0, 2, (bits + 5, 12)).bool()                 # ragged last group
+    want = torch.round(model(x.float()) * 4.0).to(torch.int32)
+    assert torch.equal(net(x), want)
+    again = CompiledLogicNet.load(str(lib), num_classes=3, num_bits=bits)
+    assert torch.equal(again(x.numpy()), want)
+
+
+def test_compiled_net_gate_expressions_are_the_truth_tables():
+    from convlogic_amd.difflogic.compiled_model import GATE_EXPR
+    for i, expr in enumerate(GATE_EXPR):
+        for a in (0, 1):
+            for b in (0, 1):
+                got = eval(expr.format(a=-a, b=-b, z="0")) & 1       # all-ones / all-zeros words
+                assert got == (i >> (3 - 2 * a - b)) & 1, (i, a, b)
+
+
+def test_compiled_net_netlist_file_round_trip(tmp_path):
+    from convlogic_amd.difflogic import CompiledLogicNet
+    torch.manual_seed(1)
+    m = C.ConvLogicMnistModel(k_param=1, implementation="python")
+    net = CompiledLogicNet(m, device="cuda")
+    assert [s[0] for s in net.stages] == ["conv"] * 3 + ["fc"] * 3 and net.num_classes == 10
+    path = tmp_path / "net.npz"
+    net.save(str(path))
+    back = CompiledLogicNet.load_netlist(str(path))
+    assert len(back.stages) == 6 and back.num_classes == 10
+    for s, t in zip(net.stages, back.stages):
+        assert s[0] == t[0] and all(np.array_equal(np.asarray(u), np.asarray(v)) for u, v in zip(s[1:], t[1:]))
