@@ -495,7 +495,7 @@ __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const 
             const int c = hit[k] & 0xFFFF;
             off = (code >> 1) * row_step + (code & 1) * g.sw;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) tv[t] = xp[gp + off + taps[c * 16 + t]];
+            for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(gp + off + taps[c * 16 + t]));
         };
         int code1 = 0, code2 = 0, off0 = 0, off1 = 0;
         T gy0 = T(0), gy1 = T(0), gy2 = T(0);
@@ -609,7 +609,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
         const int pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
         T tv[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) tv[t] = xp[pos + to[t]];
+        for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(pos + to[t]));
         const TreeVals<T> v = eval_tree(tr, tv);
         T gin[7][2], gg[7];
         gg[6] = gout;
@@ -741,7 +741,7 @@ bool plan_backward_x_direct(const Geom &g, int elem, TilePlan *p, int *sample_el
     p->lds_bytes = (size_t)nw * (p->xe + kWave) * elem;
     if (p->lds_bytes > (size_t)kLdsLimit) return false;
     const int64_t se = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
-    if (se * g.n >= (1ll << 31) || (int64_t)G * g.c * I >= (1ll << 31)) return false;
+    if (se * g.n * elem >= (1ll << 32) || (int64_t)G * g.c * I >= (1ll << 31)) return false;
     if (clg_ceil_div(clg_ceil_div(g.n, G) * g.cin, nw) >= (1ll << 31)) return false;
     *sample_elems = (int)se;
     return true;
@@ -793,10 +793,10 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     // at 16.8M, 30 vs 27 us at 1.6M)
     if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_PADDED")) return false;
     const int64_t sample_elems = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
-    if (sample_elems * g.n >= (1ll << 31) || I * g.n >= (1ll << 31)) return false;
+    if (sample_elems * g.n * elem >= (1ll << 32) || I * g.n >= (1ll << 31)) return false;
     p->d_slots = make_fastdiv((uint32_t)p->chs);                    // reused as "divide by plane stride"
     ws->sample_elems = (int)sample_elems;
-    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);                   // about 8 cells per thread
+    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);                   // about 8 cells per thread (4..64 measured within 10 %)
     ws->nb = (int)(nb < 1 ? 1 : (nb > 64 ? 64 : nb));
     ws->folded_off = ((size_t)g.c * 64 * 28 * elem + 255) & ~(size_t)255;   // partials sized for 64 blocks
     ws->taps_off = (ws->folded_off + (size_t)g.c * 28 * elem + 255) & ~(size_t)255;

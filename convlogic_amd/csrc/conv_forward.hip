@@ -314,9 +314,9 @@ __global__ __launch_bounds__(256) void convblock_forward_direct_kernel(const typ
         for (int t = 0; t < 8; ++t) to[t] = taps[c * 8 + t];
         T v0[8], v1[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) v0[t] = xp[base + to[t]];
+        for (int t = 0; t < 8; ++t) v0[t] = load_at(xp, (uint32_t)(base + to[t]));
 #pragma unroll
-        for (int t = 0; t < 8; ++t) v1[t] = xp[base + row_step + to[t]];
+        for (int t = 0; t < 8; ++t) v1[t] = load_at(xp, (uint32_t)(base + row_step + to[t]));
         const T r0 = Ops::root(pr, v0), r1 = Ops::root(pr, v1);
         const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
         if (writer) Ops::pool_store(r0, r0o, r1, r1o, y + obase + (int64_t)c * I, argmax ? argmax + obase + (int64_t)c * I : nullptr, 0);
@@ -451,7 +451,7 @@ bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan 
     p->NW = 4;
     const int64_t se = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
     const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
-    if (se * g.n >= (1ll << 31) || (int64_t)g.n * g.c * I >= (1ll << 62)) return false;
+    if (se * g.n * elem >= (1ll << 32)) return false;
     d->sample_elems = (int)se;
     d->nblk = (int)clg_ceil_div((int64_t)G * p->slots, kWave);
     const int64_t sets = clg_ceil_div(g.n, G) * d->nblk, wgs_x = clg_ceil_div(sets, 4);

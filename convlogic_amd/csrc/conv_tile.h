@@ -91,6 +91,14 @@ static inline int allow_lds(K kernel, size_t bytes, const char *name)
 
 // ---- kernels shared by the paths that read taps from a padded global copy of x ------------------
 #if defined(__HIPCC__)
+// Element `index` of a buffer of fewer than 2^32 bytes: the unsigned 32-bit byte offset lets the load use a
+// scalar base with a 32-bit vector offset instead of 64-bit address arithmetic per lane.
+template <typename T>
+__device__ __forceinline__ T load_at(const T *__restrict__ base, uint32_t index)
+{
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + (size_t)(index * (uint32_t)sizeof(T)));
+}
+
 // xp = zero-padded copy of x in the shared-halo layout: sample n at n * sample_elems, plane stride chs, row
 // stride rs, pixel (iy, ix) at (iy + ph) * rs + ix + pw.  p.d_slots must hold the divisor chs.
 template <typename T>

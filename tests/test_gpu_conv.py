@@ -94,6 +94,7 @@ def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monke
     if direct == "1":
         monkeypatch.setenv("CLG_BWDX_DIRECT", "1")
         monkeypatch.setenv("CLG_FWD_DIRECT", "1")
+        monkeypatch.setenv("CLG_BWDW_PADDED", "1")
     if direct == "subset":
         monkeypatch.setenv("CLG_FWD_SUBSET", "1")
         monkeypatch.setenv("CLG_FWD_DIRECT", "0")
