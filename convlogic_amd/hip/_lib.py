@@ -98,7 +98,13 @@ def dtype_code(t):
         raise RuntimeError(f"convlogic_amd kernels support float32 and float64, got {t.dtype}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(t):
+    """hipStream_t of torch's current stream on the tensor's device, as an integer."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
