@@ -918,24 +918,29 @@ int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
 // far is remembered per kernel so that steady-state launches make no runtime call besides the launch.
 int clg_allow_lds(const void *kernel, size_t bytes, const char *name)
 {
+    constexpr int kSlots = 256;                                      // (kernel instantiation, device) pairs remembered
     static std::mutex mu;
-    static const void *known[32];
-    static size_t granted[32];
+    static const void *known[kSlots];
+    static int device_of[kSlots];
+    static size_t granted[kSlots];
     static int used = 0;
     if (bytes <= 48 * 1024) return CLG_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;                    // the attribute is kept per device
     std::lock_guard<std::mutex> lock(mu);
     int slot = -1;
     for (int i = 0; i < used; ++i)
-        if (known[i] == kernel) slot = i;
+        if (known[i] == kernel && device_of[i] == dev) slot = i;
     if (slot >= 0 && granted[slot] >= bytes) return CLG_OK;
     const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) {
         clg_set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
         return CLG_ELAUNCH;
     }
-    if (slot < 0 && used < 32) slot = used++;
+    if (slot < 0 && used < kSlots) slot = used++;
     if (slot >= 0) {
         known[slot] = kernel;
+        device_of[slot] = dev;
         granted[slot] = bytes;
     }
     return CLG_OK;
