@@ -262,8 +262,11 @@ __host__ __device__ inline Band make_band(const Geom &g, int band, int band_rows
 // of `wrows` rows x rs elements, left halo shared with the previous row's right halo) and, unless halo
 // elements can take them, one sink element per thread for masked updates.  With a hit split > 1 the
 // workgroups blockIdx.z = 0..HS-1 of one (sample group, band) take every HS-th kernel of each channel's
-// list and write partial gradient images that sum_partial_images adds in a fixed order.
-template <typename T, bool BANDED>
+// list and write partial gradient images that sum_partial_images adds in a fixed order.  Inside a workgroup,
+// p.hsw wavefronts can share one (sample group, channel) the same way: each takes every hsw-th of those
+// kernels and accumulates into its own copy of the gradient window; the copies are added in order on the
+// way out.
+template <typename T, bool BANDED, bool SHARED>
 __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
                                                   const T *__restrict__ folded, const int32_t *__restrict__ count,
                                                   const int32_t *__restrict__ hits, const int32_t *__restrict__ taps,
@@ -275,7 +278,8 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     T *gs = xs + xe4;
     const int gs_off = xe4;
     // sink of masked updates: the first (halo) row of the gradient window, or a region after it
-    const int dummy_off = p.dummy_in_halo ? gs_off + (int)(threadIdx.x & 31) : 2 * xe4 + (int)threadIdx.x;
+    const int hsw = SHARED ? p.hsw : 1;                              // SHARED = false keeps the one-owner code as lean as it was
+    const int sink_base = (1 + hsw) * xe4;
 
     const int tid = threadIdx.x, nthreads = blockDim.x;
     const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
@@ -284,7 +288,7 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     const Band bd = make_band(g, blockIdx.y, p.band_rows);
     const int chs = p.chs;                                          // plane stride of the windows
 
-    const int zero_n = 2 * xe4 + (p.dummy_in_halo ? 0 : nthreads);
+    const int zero_n = sink_base + (p.dummy_in_halo ? 0 : nthreads);
     for (int i = tid; i < zero_n; i += nthreads) xs[i] = T(0);
     __syncthreads();
     // stage the image rows that fall into the window (padded row = image row + ph)
@@ -309,7 +313,10 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
     const int groups = (s_cur + p.G - 1) / p.G;
     const int items = groups * g.cin;
     const int row_step = g.sh * p.rs;
-    for (int item = wave; item < items; item += p.NW) {
+    for (int witem = wave; witem < items * hsw; witem += p.NW) {
+        const int item = SHARED ? witem / hsw : witem, slot = SHARED ? witem - item * hsw : 0;
+        const int gw_off = gs_off + slot * xe4;                      // this wavefront's copy of the gradient window
+        const int dummy_off = p.dummy_in_halo ? gw_off + (lane & 31) : sink_base + (int)threadIdx.x;
         const int grp = item / g.cin, ch = item - grp * g.cin;
         const int s0 = grp * p.G;
         const int v_here = min(p.G, s_cur - s0) * bd.cb;
@@ -354,7 +361,7 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
                 }
             };
             CellLoads<T> cur, nxt;
-            const int hs0 = blockIdx.z, hsn = gridDim.z;
+            const int hs0 = blockIdx.z + gridDim.z * slot, hsn = gridDim.z * hsw;
             if (hs0 < nhits) issue(hs0, cur);
             for (int k = hs0; k < nhits; k += hsn) {
                 if (k + hsn < nhits) issue(k + hsn, nxt);
@@ -413,7 +420,7 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
                         for (int j = 0; j < kChunk; ++j) {
                             bool mine = live[j];
                             if (BANDED) mine = mine && ((uint32_t)(pos[j] - img0 + tr_[t]) - own_lo) < own_len;
-                            at[j] = mine ? gs_off + pos[j] + to[t] : dummy_off;
+                            at[j] = mine ? gw_off + pos[j] + to[t] : dummy_off;
                         }
 #pragma unroll
                         for (int j = 0; j < kChunk; ++j) old[j] = xs[at[j]];
@@ -433,7 +440,11 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
         const int plane = uniform(pr / orows), iy = bd.r0 + (pr - plane * orows);
         const T *row = gs + plane * chs + (iy + g.ph - bd.R0) * p.rs + g.pw;
         T *dst = dstg + ((int64_t)plane * g.h + iy) * g.w;
-        for (int ix = lane; ix < g.w; ix += kWave) dst[ix] = row[ix];
+        for (int ix = lane; ix < g.w; ix += kWave) {
+            T v = row[ix];
+            for (int k = 1; k < hsw; ++k) v += row[k * xe4 + ix];
+            dst[ix] = v;
+        }
     }
 }
 
@@ -692,13 +703,27 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     p->bands = (int)clg_ceil_div(g.h, band_rows);
     p->chs = rows_max * p->rs;
     p->xe = (int)((int64_t)G * g.cin * p->chs + g.pw);
-    p->lds_bytes = (size_t)bytes;
     p->dummy_in_halo = (p->bands == 1 && g.ph >= 1 && p->rs >= 32) ? 1 : 0;
     if (p->bands > 65535) return false;
     if (G * I < kWave / 5 && p->bands == 1) return false;            // almost empty wavefronts: gather kernel instead
+    // Few input channels leave most of the 16 wavefront slots of a workgroup empty: then several wavefronts
+    // share each gradient plane, every one with its own copy of the gradient window (at least two kernels per
+    // wavefront, windows within 96 KiB so that a second workgroup still fits on the CU).
+    const int64_t avg_hits = g.cin == 1 ? g.c : (2 * (int64_t)g.c) / g.cin;
+    const int64_t window = (int64_t)((p->xe + 3) & ~3) * elem;
+    int64_t hsw = 16 / g.cin;
+    if (const char *e = getenv("CLG_BWDX_HSW")) hsw = atoi(e);
+    if (hsw > avg_hits / 2) hsw = avg_hits / 2;
+    while (hsw > 1 && (1 + hsw) * window > 96 * 1024) --hsw;
+    if (hsw < 1 || p->bands > 1) hsw = 1;
+    p->hsw = (int)hsw;
+    p->NW = (int)(g.cin * hsw < 16 ? g.cin * hsw : 16);
+    const int64_t bytes_all = (1 + hsw) * window + (p->dummy_in_halo ? 0 : (int64_t)p->NW * kWave * elem);
+    if (bytes_all > kLdsLimit) return false;
+    p->lds_bytes = (size_t)bytes_all;
     // hit split: when (sample groups x bands) leave room for more resident workgroups, several workgroups
     // share the kernels of one image; each handles every HS-th kernel and writes a partial image
-    int64_t per_cu = kLdsLimit / (int64_t)(bytes > 1024 ? bytes : 1024);
+    int64_t per_cu = kLdsLimit / (int64_t)(bytes_all > 1024 ? bytes_all : 1024);
     if (per_cu > 20 / p->NW) per_cu = 20 / p->NW;                    // about 80 VGPRs per lane: 5 wavefronts per SIMD
     if (per_cu < 1) per_cu = 1;
     const int64_t wgs = clg_ceil_div(g.n, p->S) * p->bands;
@@ -707,8 +732,7 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     if (hs > kMaxHitSplit) hs = kMaxHitSplit;
     // every split workgroup stages the image and writes a partial image: worth it only with at least
     // about 4 kernels left per channel list (a kernel reads at most two channels)
-    const int64_t avg_hits = g.cin == 1 ? g.c : (2 * (int64_t)g.c) / g.cin;
-    if (!e_hs && hs > avg_hits / 4) hs = avg_hits / 4;
+    if (!e_hs && hs > avg_hits / (4 * hsw)) hs = avg_hits / (4 * hsw);
     if (hs < 1) hs = 1;
     p->hit_split = (int)hs;
     p->part_stride = hs > 1 ? (int64_t)g.n * g.cin * g.h * g.w : 0;
@@ -732,6 +756,7 @@ bool plan_backward_x_direct(const Geom &g, int elem, TilePlan *p, int *sample_el
     p->bands = 1;
     p->band_rows = g.h;
     p->hit_split = 1;
+    p->hsw = 1;
     p->part_stride = 0;
     p->dummy_in_halo = 0;
     p->xe = (int)(((int64_t)G * p->chs + g.ph * p->rs + g.pw + 3) & ~3ll);
@@ -843,15 +868,18 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
     T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
     T *out = p.hit_split > 1 ? part : (T *)gx;
-    if (p.bands > 1) {
-        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, true>, p.lds_bytes, "clg_convblock_backward_x")) return e;
-        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, true>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
-                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, out, g, p);
-    } else {
-        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, false>, p.lds_bytes, "clg_convblock_backward_x")) return e;
-        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, false>), grid, block, p.lds_bytes, st, (const T *)gy, (const T *)x,
-                           (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, argmax, out, g, p);
-    }
+#define CLG_BWDX_TILED(BANDED, SHARED)                                                                                          \
+    do {                                                                                                                        \
+        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, BANDED, SHARED>, p.lds_bytes, "clg_convblock_backward_x"))   \
+            return e;                                                                                                           \
+        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, BANDED, SHARED>), grid, block, p.lds_bytes, st, (const T *)gy, \
+                           (const T *)x, (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, \
+                           argmax, out, g, p);                                                                                  \
+    } while (0)
+    if (p.bands > 1) CLG_BWDX_TILED(true, false);
+    else if (p.hsw > 1) CLG_BWDX_TILED(false, true);
+    else CLG_BWDX_TILED(false, false);
+#undef CLG_BWDX_TILED
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(tiled)");
     if (p.hit_split > 1) {
         const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;

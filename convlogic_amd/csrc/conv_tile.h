@@ -30,6 +30,7 @@ struct TilePlan {
     int slots;          // per sample: (ho/2) * wo lane slots (forward) / pooled cells (input gradient)
     int band_rows, bands;  // input gradient: image rows per workgroup band, number of bands
     int hit_split;         // input gradient: workgroups sharing the kernels of one (sample, band), partial images
+    int hsw;               // input gradient: wavefronts of one workgroup sharing the kernels of one gradient plane
     int dummy_in_halo;     // input gradient: masked updates go to halo elements instead of a region of their own
     int64_t part_stride;   // input gradient: elements between partial images (0 when hit_split == 1)
     int planes;            // forward: LDS planes per sample (all input channels, or 2 per kernel of the tile)
