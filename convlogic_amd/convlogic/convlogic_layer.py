@@ -71,6 +71,35 @@ class FullConvLogicFunction(Function):
         return grad_x, grad_w, None, None, None, None, None, None, None, None, None
 
 
+class _FullConvLogicLogitsFunction(Function):
+    """Training path of the module: the complete block as a function of the LOGITS.  The softmax runs inside
+    forward, its backward is fused into the weight-gradient kernel, so a step has no separate softmax nodes
+    (same values as softmax + FullConvLogicFunction up to rounding)."""
+
+    @staticmethod
+    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+        x1, selection = x.contiguous(), selection.contiguous()
+        w_prob = torch.softmax(logits, dim=-1)
+        geo = (stride_h, stride_w, pad_h, pad_w)
+        y, argmax = convlogic_hip.full_convlogic_forward(x1, w_prob, selection, *geo, kernel_h, kernel_w)
+        ctx.save_for_backward(x1, w_prob, selection, argmax)
+        ctx.geometry = geo
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x1, w_prob, selection, argmax = ctx.saved_tensors
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        grad_x = grad_l = None
+        grad_y = grad_y.contiguous()
+        if need_w:
+            grad_x, grad_l = convlogic_hip.full_convlogic_backward_logits(grad_y, x1, w_prob, argmax, selection, *ctx.geometry,
+                                                                         need_grad_x=need_x)
+        elif need_x:
+            grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
+        return grad_x, grad_l, None, None, None, None, None, None, None
+
+
 def _pair(v):
     return (v, v) if isinstance(v, int) else tuple(v)
 
@@ -154,9 +183,12 @@ class ConvLogicLayer(nn.Module):
 
     def forward_cuda(self, x):
         x = x.contiguous()
-        w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
         sel = self.selection.contiguous()
         geo = (*self.stride, *self.padding, *self.kernel)
+        if (self.complete and self.training and not self.return_intermediate and not self.return_indices
+                and self.weights.dtype == x.dtype and self.weights.is_contiguous()):
+            return _FullConvLogicLogitsFunction.apply(x, self.weights, sel, *geo)
+        w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
         if self.complete:
             return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)
         return ConvLogicFunction.apply(x, w_prob, sel, *geo)

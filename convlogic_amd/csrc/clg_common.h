@@ -118,6 +118,21 @@ __device__ __forceinline__ T wave_sum(T v)
     }
 }
 
+// Sum over each row of 16 lanes, valid in all of its lanes (the first four steps of wave_sum).
+template <typename T>
+__device__ __forceinline__ T row16_sum(T v)
+{
+    v += dpp_zero<0xB1, 0xF>(v);
+    v += dpp_zero<0x4E, 0xF>(v);
+    v += dpp_zero<0x141, 0xF>(v);
+    v += dpp_zero<0x140, 0xF>(v);
+    return v;
+}
+// Gradient w.r.t. the logit of a 16-way softmax from the gradient g w.r.t. its probability p, the 16 gates
+// of one node sitting in the 16 lanes of a row: p_i (g_i - sum_j p_j g_j).
+template <typename T>
+__device__ __forceinline__ T softmax16_backward(T g, T p) { return p * (g - row16_sum(p * g)); }
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // selection tap: ch << 16 | row << 8 | col

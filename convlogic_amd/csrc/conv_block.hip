@@ -34,9 +34,10 @@ int clg_convblock_backward_x_generic(int dtype, const Geom &g, const void *grad_
                                      void *grad_x, hipStream_t st);
 int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
-                                     hipStream_t st);
+                                     hipStream_t st, const void *probs);
 int clg_convblock_partial_blocks(const Geom &g);
-int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name);
+int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name,
+                           const void *probs);
 
 namespace {
 
@@ -916,7 +917,7 @@ int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems,
 
 template <typename T>
 int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &ws, const void *gy, const void *x, const void *w,
-                             const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st)
+                             const int32_t *sel, const uint8_t *argmax, void *gw, void *scratch, hipStream_t st, const void *probs)
 {
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     T *partial = reinterpret_cast<T *>(base);
@@ -935,7 +936,8 @@ int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &w
                        (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p, make_fastdiv((uint32_t)I),
                        ws.sample_elems);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded)");
-    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, ws.nb, 7, st, "clg_convblock_backward_w(reduce)");
+    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, ws.nb, 7, st, "clg_convblock_backward_w(reduce)",
+                                  probs);
 }
 
 int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
@@ -1027,22 +1029,31 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
     return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the any-shape kernel
 }
 
-extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
-                                        const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
-                                        void *stream)
+// grad_w w.r.t. the gate probabilities, or -- with probs = the softmax output w -- w.r.t. the logits
+static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                     const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch, void *stream,
+                                     const void *probs, const char *name)
 {
     Geom g;
-    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w")) return e;
-    CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "clg_convblock_backward_w: null pointer argument");
+    if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
+    CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "%s: null pointer argument", name);
     TilePlan p;
     WScratch ws;
     const char *e_pad = getenv("CLG_BWDW_PADDED");
     if ((!e_pad || atoi(e_pad) != 0) && plan_backward_w(g, elem_size(dtype), &p, &ws)) {
         if (dtype == CLG_F32)
-            return launch_backward_w_padded<float>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
-        return launch_backward_w_padded<double>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+            return launch_backward_w_padded<float>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
+        return launch_backward_w_padded<double>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
     }
-    return clg_convblock_backward_w_generic(dtype, g, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream));
+    return clg_convblock_backward_w_generic(dtype, g, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
+}
+
+extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                        const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
+                                        void *stream)
+{
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w, scratch, stream, nullptr,
+                                     "clg_convblock_backward_w");
 }
 
 extern "C" int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *gg)
@@ -1062,4 +1073,18 @@ extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const 
     if (int e = clg_convblock_backward_x(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream)) return e;
     return clg_convblock_backward_w(dtype, gg, grad_y, x, w, selection, argmax, grad_w,
                                     reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream);
+}
+
+extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                             const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_logits,
+                                             void *scratch, void *stream)
+{
+    CLG_REQUIRE(scratch, "clg_convblock_backward_logits: null pointer argument");
+    const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
+    if (a < 0) return CLG_EINVAL;
+    if (grad_x != nullptr)
+        if (int e = clg_convblock_backward_x(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream)) return e;
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_logits,
+                                     reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream, w,
+                                     "clg_convblock_backward_logits");
 }

@@ -79,9 +79,11 @@ __global__ __launch_bounds__(kBlk) void conv4_backward_w_kernel(const T *__restr
     block_sum_store<T, 16, kBlk>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 16);
 }
 
-// out[row*G + q][i] = sum_k COEF[k][i] * (sum_blk partial[row][blk][q*4 + k])
+// out[row*G + q][i] = sum_k COEF[k][i] * (sum_blk partial[row][blk][q*4 + k]): the gradient w.r.t. the gate
+// probabilities; with probs (the softmax output they came from) the gradient w.r.t. the logits instead.
 template <typename T>
-__global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t rows, int nb, int G)
+__global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t rows, int nb, int G,
+                                            const T *__restrict__ probs)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= rows * G * 16) return;
@@ -94,7 +96,9 @@ __global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__
 #pragma unroll
         for (int k = 0; k < 4; ++k) s[k] += p[k];
     }
-    out[e] = coef_transpose_row<T>(i, s[0], s[1], s[2], s[3]);
+    T gi = coef_transpose_row<T>(i, s[0], s[1], s[2], s[3]);
+    if (probs != nullptr) gi = softmax16_backward(gi, probs[e]);
+    out[e] = gi;
 }
 
 // One thread per input element; every (kernel, tap) that reads the element's channel is visited in
@@ -395,11 +399,12 @@ int check_dtype(int dtype, const char *name)
 }
 
 template <typename T>
-int launch_reduce(const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name)
+int launch_reduce(const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name,
+                  const void *probs = nullptr)
 {
     const int64_t total = rows * G * 16;
     hipLaunchKernelGGL(reduce_coef_partials_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st,
-                       (const T *)partial, (T *)out, rows, nb, G);
+                       (const T *)partial, (T *)out, rows, nb, G, (const T *)probs);
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }
@@ -534,9 +539,10 @@ extern "C" int clg_tree_backward_w(int dtype, const void *grad_y, const void *x,
     CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, c * xo, nb, 1, st, "clg_tree_backward_w(reduce)"));
 }
 
-int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name)
+int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name,
+                           const void *probs)
 {
-    CLG_DISPATCH(dtype, return launch_reduce<T>(partial, out, rows, nb, G, st, name));
+    CLG_DISPATCH(dtype, return launch_reduce<T>(partial, out, rows, nb, G, st, name, probs));
 }
 
 // ---- fused block, generic entry points (called from conv_block.hip when no tiled kernel applies) ----
@@ -579,14 +585,14 @@ int clg_convblock_partial_blocks(const Geom &g) { return partial_blocks((int64_t
 
 int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
-                                     hipStream_t st)
+                                     hipStream_t st, const void *probs)
 {
     CLG_REQUIRE(g.c <= 65535, "clg_convblock_backward_w: more than 65535 logic kernels are not supported");
     const int nb = clg_convblock_partial_blocks(g);
     CLG_DISPATCH(dtype, hipLaunchKernelGGL(convblock_backward_w_generic_kernel<T>, dim3(nb, g.c), dim3(kBlk), 0, st,
                                            (const T *)grad_y, (const T *)x, (const T *)w, selection, argmax, (T *)scratch, g));
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(generic)");
-    CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, g.c, nb, 7, st, "clg_convblock_backward_w(reduce)"));
+    CLG_DISPATCH(dtype, return launch_reduce<T>(scratch, grad_w, g.c, nb, 7, st, "clg_convblock_backward_w(reduce)", probs));
 }
 
 extern "C" int clg_convblock_intermediates(int dtype, const clg_conv_geom *gg, const void *x, const void *w,

@@ -68,7 +68,7 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                              const int64_t *__restrict__ b,
                                                              const T *__restrict__ gy, T *__restrict__ gw, int out_dim,
-                                                             int64_t batch)
+                                                             int64_t batch, const T *__restrict__ probs)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
@@ -92,7 +92,11 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restri
         sa = wave_sum(sa);
         sb = wave_sum(sb);
         s1 = wave_sum(s1);
-        if (lane < 16) gw[(int64_t)j * 16 + lane] = coef_transpose_row<T>(lane, sab, sa, sb, s1);
+        if (lane < 16) {
+            T gi = coef_transpose_row<T>(lane, sab, sa, sb, s1);
+            if (probs != nullptr) gi = softmax16_backward(gi, probs[(int64_t)j * 16 + lane]);   // gradient w.r.t. the logits
+            gw[(int64_t)j * 16 + lane] = gi;
+        }
     }
 }
 
@@ -203,30 +207,44 @@ extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const 
     return CLG_OK;
 }
 
-extern "C" int clg_fc_backward_w(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
-                                 void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+static int fc_backward_w_impl(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *grad_y, void *grad_w,
+                             int64_t in_dim, int64_t out_dim, int64_t batch, void *stream, const void *probs, const char *name)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_w")) return e;
-    CLG_REQUIRE(x && a && b && grad_y && grad_w, "clg_fc_backward_w: null pointer argument");
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
+    CLG_REQUIRE(x && a && b && grad_y && grad_w, "%s: null pointer argument", name);
     const dim3 grid(grid_for(out_dim)), block(kBlock);
     hipStream_t st = clg_stream(stream);
     if (dtype == CLG_F32) {
         if (batch % 4 == 0)
             hipLaunchKernelGGL((fc_backward_w_kernel<float, 4>), grid, block, 0, st, (const float *)x, a, b,
-                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch);
+                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch, (const float *)probs);
         else
             hipLaunchKernelGGL((fc_backward_w_kernel<float, 1>), grid, block, 0, st, (const float *)x, a, b,
-                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch);
+                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch, (const float *)probs);
     } else {
         if (batch % 2 == 0)
             hipLaunchKernelGGL((fc_backward_w_kernel<double, 2>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch);
+                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch, (const double *)probs);
         else
             hipLaunchKernelGGL((fc_backward_w_kernel<double, 1>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch);
+                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch, (const double *)probs);
     }
-    CLG_CHECK_LAUNCH("clg_fc_backward_w");
+    CLG_CHECK_LAUNCH(name);
     return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_w(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *grad_y,
+                                 void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    return fc_backward_w_impl(dtype, x, a, b, grad_y, grad_w, in_dim, out_dim, batch, stream, nullptr, "clg_fc_backward_w");
+}
+
+extern "C" int clg_fc_backward_logits(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w,
+                                      const void *grad_y, void *grad_logits, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                      void *stream)
+{
+    CLG_REQUIRE(w, "clg_fc_backward_logits: null pointer argument");
+    return fc_backward_w_impl(dtype, x, a, b, grad_y, grad_logits, in_dim, out_dim, batch, stream, w, "clg_fc_backward_logits");
 }
 
 extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w,

@@ -93,6 +93,9 @@ class LogicLayer(torch.nn.Module):
         assert x.ndim == 2, x.ndim
         assert x.shape[1] == self.in_dim, (tuple(x.shape[::-1]), self.in_dim)
         xt = _feature_major(x)
+        if self.training and self.weights.dtype == xt.dtype and self.weights.is_contiguous():
+            return _LogicLayerLogitsFunction.apply(xt, self.indices_0, self.indices_1, self.weights,
+                                                   self.given_x_indices_of_y_start, self.given_x_indices_of_y).transpose(0, 1)
         w = self._gate_weights(xt.dtype)
         args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
         if self.training:
@@ -206,6 +209,29 @@ class LogicLayerCudaFunction(torch.autograd.Function):
         if ctx.needs_input_grad[3]:
             grad_w = difflogic_hip.backward_w(x, a, b, grad_y)
         return grad_x, None, None, grad_w, None, None, None
+
+
+class _LogicLayerLogitsFunction(torch.autograd.Function):
+    """Training path of the module: y[out,B] as a function of the LOGITS; the softmax runs inside forward and
+    its backward is fused into the weight-gradient kernel (same values as softmax + LogicLayerCudaFunction up
+    to rounding)."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y):
+        w = torch.softmax(logits, dim=-1)
+        ctx.save_for_backward(x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y)
+        return difflogic_hip.forward(x, a, b, w)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x, a, b, w, start, flat = ctx.saved_tensors
+        grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
+        grad_x = grad_l = None
+        if ctx.needs_input_grad[0]:
+            grad_x = difflogic_hip.backward_x(x, a, b, w, grad_y, start, flat)
+        if ctx.needs_input_grad[3]:
+            grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
+        return grad_x, None, None, grad_l, None, None
 
 
 def _contiguous_2d(t):

@@ -30,6 +30,7 @@ SIGNATURES = {
     "clg_abi_version": (_i, []),
     "clg_fc_forward": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_w": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_fc_backward_logits": (_i, [_i, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_x": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_transpose_2d": (_i, [_i, _p, _p, _i64, _i64, _p]),
     "clg_pack_bits": (_i, [_p, _p, _i64, _i64, _i, _p]),
@@ -60,6 +61,7 @@ SIGNATURES = {
     "clg_convblock_backward_w": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_w_scratch_bytes": (_i64, [_i, _GP]),
     "clg_convblock_backward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "clg_convblock_backward_logits": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_scratch_bytes": (_i64, [_i, _GP]),
 }
 

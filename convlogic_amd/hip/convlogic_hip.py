@@ -229,6 +229,23 @@ def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stri
     return gx, gw
 
 
+def full_convlogic_backward_logits(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True):
+    """-> (grad_x or None, grad_logits [C,7,16]) for weight = softmax(logits): the two gradients of the block
+    with the softmax backward fused into the final reduction of the weight gradient."""
+    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_convblock_backward_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gx = torch.empty_like(x) if need_grad_x else None
+    gl = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_convblock_backward_logits(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                            selection.data_ptr(), argmax.data_ptr(), gx.data_ptr() if need_grad_x else None,
+                                            gl.data_ptr(), scratch.data_ptr(), stream_ptr(x)))
+    return gx, gl
+
+
 # ---- input binarisation -------------------------------------------------------------------------
 def _threshold_args(x, thresholds):
     check_input(x, "x")

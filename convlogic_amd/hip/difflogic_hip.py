@@ -33,6 +33,19 @@ def backward_w(x, a, b, grad_y):
     return gw
 
 
+def backward_logits(x, a, b, w, grad_y):
+    """Gradient w.r.t. the logits [out, 16] when w = softmax(logits): backward_w and the softmax backward
+    in one kernel."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = grad_y.shape[0]
+    gl = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_backward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
+                                             grad_y.data_ptr(), gl.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return gl
+
+
 def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
     """grad_x[in, B]; difflogic_cuda.backward_x (difflogic_kernel.cu:232-269)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y"),

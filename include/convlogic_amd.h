@@ -80,6 +80,14 @@ int clg_fc_backward_x(int dtype, const void *x /*[in_dim,batch]*/, const int64_t
                       void *grad_x /*[in_dim,batch]*/, int64_t in_dim, int64_t out_dim, int64_t batch,
                       void *stream);
 
+/* clg_fc_backward_w followed by the softmax backward in the same kernel: with w = softmax(logits) the
+ * result is the gradient w.r.t. the logits, p_i (g_i - sum_j p_j g_j) per neuron.  Replaces
+ * difflogic_cuda.backward_w plus the autograd node of the softmax in LogicLayer.forward_cuda
+ * (src/difflogic/difflogic.py:138, :226-228). */
+int clg_fc_backward_logits(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w /*[out_dim,16]*/,
+                           const void *grad_y, void *grad_logits /*[out_dim,16]*/, int64_t in_dim, int64_t out_dim,
+                           int64_t batch, void *stream);
+
 /* dst[c][r] = src[r][c] for elements of elem_size 1, 2, 4 or 8 bytes (layout change between the
  * module's [batch, features] tensors and the feature-major kernels; the reference does this with
  * x.transpose(0,1).contiguous(), src/difflogic/difflogic.py:130-131). */
@@ -243,6 +251,16 @@ int clg_convblock_backward(int dtype, const clg_conv_geom *g, const void *grad_y
                            const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w, void *scratch,
                            void *stream);
 int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *g);
+
+/* Both gradients of the block for a training step that owns the softmax: grad_x as clg_convblock_backward_x
+ * (skipped when grad_x is NULL, e.g. for the first layer) and the gradient w.r.t. the LOGITS, i.e.
+ * clg_convblock_backward_w followed by the softmax backward with w = softmax(logits), fused into the
+ * final reduction.  scratch: clg_convblock_backward_scratch_bytes().  Replaces full_convlogic_backward_x +
+ * full_convlogic_backward_weight (src/convlogic/convlogic_layer.py:71-82) plus the autograd node of the
+ * softmax in ConvLogicLayer.forward_cuda (src/convlogic/convlogic_layer.py:321-323). */
+int clg_convblock_backward_logits(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                                  const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_logits,
+                                  void *scratch, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * input binarisation (the step in front of the first layer)

@@ -250,3 +250,35 @@ def test_block_errors():
         convlogic_hip.full_convlogic_forward(torch.rand(1, 1, 6, 6), layer.weights.detach().softmax(-1), layer.selection, 1, 1, 0, 0, 3, 3)
     layer = C.ConvLogicLayer(1, 1, kernel=2, padding=0, complete=True).to(DEV).eval()
     assert layer(torch.randn(1, 1, 3, 3, device=DEV)).shape == (1, 1, 1, 1)
+
+
+@pytest.mark.parametrize("shape", [(5, 3, 6, 10, 12), (64, 9, 64, 32, 32)])
+def test_block_fused_softmax_backward_matches_softmax_plus_function(shape):
+    # module training path (logits in) against softmax -> FullConvLogicFunction; the large shape takes the
+    # padded weight-gradient kernel, the small one the any-shape kernel
+    from convlogic_amd.convlogic.convlogic_layer import _FullConvLogicLogitsFunction
+    n, cin, cout, h, w = shape
+    for dtype, tol in ((torch.float32, 5e-5), (torch.float64, 1e-11)):
+        torch.manual_seed(n)
+        layer = C.ConvLogicLayer(cin, cout, padding=1, complete=True, implementation="cuda").to(DEV).to(dtype)
+        x = torch.rand(n, cin, h, w, device=DEV, dtype=dtype)
+        outs = []
+        for fused in (True, False):
+            xl = x.clone().requires_grad_(True)
+            logits = torch.randn_like(layer.weights).requires_grad_(True) if not outs else outs[0][3].detach().clone().requires_grad_(True)
+            geo = (1, 1, 1, 1, 3, 3)
+            if fused:
+                y = _FullConvLogicLogitsFunction.apply(xl, logits, layer.selection, *geo)
+            else:
+                y = C.FullConvLogicFunction.apply(xl, torch.softmax(logits, -1), layer.selection, *geo)
+            gy = torch.randn_like(y) if not outs else outs[0][4]
+            y.backward(gy)
+            outs.append((y.detach(), xl.grad, logits.grad, logits, gy))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        scale = outs[1][2].abs().max().item()
+        assert (outs[0][2] - outs[1][2]).abs().max().item() <= tol * scale
+    # first layer of a network: no input gradient requested
+    layer.train()
+    y = layer(x.detach())
+    y.sum().backward()
+    assert layer.weights.grad is not None and torch.isfinite(layer.weights.grad).all()

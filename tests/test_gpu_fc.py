@@ -145,3 +145,29 @@ def test_fc_rejects_bad_inputs():
                               torch.rand(8, 16, device=DEV).half())
     with pytest.raises(AssertionError):
         layer(torch.rand(2, 3, 8, device=DEV))
+
+
+def test_fused_softmax_backward_matches_softmax_plus_function():
+    # training path of the module (logits in, softmax inside, its backward fused into the weight-gradient
+    # kernel) against the reference-shaped route softmax -> LogicLayerCudaFunction, float32 and float64
+    from convlogic_amd.difflogic.difflogic import _LogicLayerLogitsFunction
+    for dtype, tol in ((torch.float32, 2e-5), (torch.float64, 1e-12)):
+        torch.manual_seed(7)
+        layer = C.LogicLayer(40, 96, implementation="cuda").to(DEV).to(dtype)
+        x = torch.rand(40, 33, device=DEV, dtype=dtype)
+        gy = torch.randn(96, 33, device=DEV, dtype=dtype)
+        outs = []
+        for fused in (True, False):
+            xl = x.clone().requires_grad_(True)
+            logits = layer.weights.detach().clone().requires_grad_(True)
+            tabs = (layer.indices_0, layer.indices_1)
+            csr = (layer.given_x_indices_of_y_start, layer.given_x_indices_of_y)
+            if fused:
+                y = _LogicLayerLogitsFunction.apply(xl, *tabs, logits, *csr)
+            else:
+                y = C.LogicLayerCudaFunction.apply(xl, *tabs, torch.softmax(logits, -1), *csr)
+            y.backward(gy)
+            outs.append((y.detach(), xl.grad, logits.grad))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        scale = outs[1][2].abs().max().item()
+        assert (outs[0][2] - outs[1][2]).abs().max().item() <= tol * scale
