@@ -594,7 +594,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
                                                                         const int32_t *__restrict__ taps,
                                                                         const uint8_t *__restrict__ argmax,
                                                                         T *__restrict__ partial, Geom g, TilePlan p,
-                                                                        FastDiv d_cells, int sample_elems)
+                                                                        FastDiv d_cells, int sample_elems, int tap_stride)
 {
     const int c = blockIdx.y, nb = gridDim.x;
     const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
@@ -605,7 +605,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
     for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
     int to[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) to[t] = taps[c * 8 + t];
+    for (int t = 0; t < 8; ++t) to[t] = taps[c * tap_stride + t];   // [c][8], or the first 8 of the input gradient's [c][16]
     const int row_step = g.sh * p.rs;
     const int64_t kernel_row = (int64_t)c * I;
     const int64_t sample_cells = (int64_t)g.c * I;
@@ -891,13 +891,29 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     return CLG_OK;
 }
 
+// What the direct input gradient leaves in its scratch for the weight gradient of the same call: the padded
+// copy of x, the folded coefficients and the tap offsets (first 8 of every 16) in that copy's layout.
+struct SharedPad {
+    const void *xp = nullptr, *folded = nullptr;
+    const int32_t *taps = nullptr;
+    int sample_elems = 0;
+    TilePlan p;
+};
+
 template <typename T>
 int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems, const void *gy, const void *x, const void *w,
-                             const int32_t *sel, const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
+                             const int32_t *sel, const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, SharedPad *shared)
 {
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     T *xp = reinterpret_cast<T *>(base + bwd_x_direct_xp_off(lay));
+    if (shared != nullptr) {
+        shared->xp = xp;
+        shared->folded = base;
+        shared->taps = reinterpret_cast<const int32_t *>(base + lay.taps_off);
+        shared->sample_elems = sample_elems;
+        shared->p = p;
+    }
     if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st)) return e;
     TilePlan pp = p;
     pp.d_slots = make_fastdiv((uint32_t)p.chs);                      // the pad kernel divides by the plane stride
@@ -934,10 +950,27 @@ int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &w
     const int I = (g.ho / 2) * (g.wo / 2);
     hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
                        (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p, make_fastdiv((uint32_t)I),
-                       ws.sample_elems);
+                       ws.sample_elems, 8);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded)");
     return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, ws.nb, 7, st, "clg_convblock_backward_w(reduce)",
                                   probs);
+}
+
+// weight gradient from the padded copy the input gradient of the same call has made
+template <typename T>
+int launch_backward_w_shared(const Geom &g, const SharedPad &sh, const void *gy, const uint8_t *argmax, void *gw, void *scratch,
+                             hipStream_t st, const void *probs)
+{
+    const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
+    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);
+    nb = nb < 1 ? 1 : (nb > 64 ? 64 : nb);
+    T *partial = reinterpret_cast<T *>(scratch);                      // [c][nb][28], within the any-shape kernel's [c][64][28]
+    hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
+                       (const T *)sh.xp, (const T *)sh.folded, sh.taps, argmax, partial, g, sh.p, make_fastdiv((uint32_t)I),
+                       sh.sample_elems, 16);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded, shared copy)");
+    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, (int)nb, 7, st,
+                                  "clg_convblock_backward_w(reduce)", probs);
 }
 
 int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
@@ -988,9 +1021,9 @@ extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_c
     return (int64_t)lay.total;
 }
 
-extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
-                                        const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch,
-                                        void *stream)
+static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                     const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch, void *stream,
+                                     SharedPad *shared)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x")) return e;
@@ -1004,8 +1037,9 @@ extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, cons
         return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st);
     }
     if (mode == kBwdXDirect) {
-        if (dtype == CLG_F32) return launch_backward_x_direct<float>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st);
-        return launch_backward_x_direct<double>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st);
+        if (dtype == CLG_F32)
+            return launch_backward_x_direct<float>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared);
+        return launch_backward_x_direct<double>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared);
     }
     // any other shape: per-element gather driven by the same per-channel kernel lists
     const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
@@ -1029,14 +1063,25 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
     return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the any-shape kernel
 }
 
+extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                        const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch,
+                                        void *stream)
+{
+    return convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, nullptr);
+}
+
 // grad_w w.r.t. the gate probabilities, or -- with probs = the softmax output w -- w.r.t. the logits
 static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch, void *stream,
-                                     const void *probs, const char *name)
+                                     const void *probs, const char *name, const SharedPad *shared = nullptr)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
     CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "%s: null pointer argument", name);
+    if (shared != nullptr && shared->xp != nullptr && g.c <= 65535) {
+        if (dtype == CLG_F32) return launch_backward_w_shared<float>(g, *shared, grad_y, argmax, grad_w, scratch, clg_stream(stream), probs);
+        return launch_backward_w_shared<double>(g, *shared, grad_y, argmax, grad_w, scratch, clg_stream(stream), probs);
+    }
     TilePlan p;
     WScratch ws;
     const char *e_pad = getenv("CLG_BWDW_PADDED");
@@ -1070,9 +1115,11 @@ extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const 
     CLG_REQUIRE(scratch, "clg_convblock_backward: null pointer argument");
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
-    if (int e = clg_convblock_backward_x(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream)) return e;
-    return clg_convblock_backward_w(dtype, gg, grad_y, x, w, selection, argmax, grad_w,
-                                    reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream);
+    SharedPad shared;
+    if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared)) return e;
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w,
+                                     reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream, nullptr,
+                                     "clg_convblock_backward", &shared);
 }
 
 extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -1082,9 +1129,10 @@ extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg,
     CLG_REQUIRE(scratch, "clg_convblock_backward_logits: null pointer argument");
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
+    SharedPad shared;
     if (grad_x != nullptr)
-        if (int e = clg_convblock_backward_x(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream)) return e;
+        if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared)) return e;
     return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_logits,
                                      reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream, w,
-                                     "clg_convblock_backward_logits");
+                                     "clg_convblock_backward_logits", &shared);
 }
