@@ -102,14 +102,12 @@ __global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__
 }
 
 // One thread per input element; every (kernel, tap) that reads the element's channel is visited in
-// a fixed order, so the sum is reproducible.  BLOCK = false: gradient of the 4-leaf layer
-// (grad arrives per leaf gate and conv position).  BLOCK = true: gradient of the fused block
-// (grad arrives per pooled cell and flows to the stored argmax position through the tree).
-template <typename T, bool BLOCK>
+// a fixed order, so the sum is reproducible.  Gradient of the 4-leaf layer (grad arrives per leaf gate
+// and conv position); the fused block uses convblock_backward_x_hits_kernel below.
+template <typename T>
 __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *__restrict__ gy, const T *__restrict__ x,
                                                                     const T *__restrict__ w,
                                                                     const int32_t *__restrict__ sel,
-                                                                    const uint8_t *__restrict__ argmax,
                                                                     T *__restrict__ gx, Geom g)
 {
     const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
@@ -118,7 +116,7 @@ __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *_
     const int ix = (int)(e % g.w), iy = (int)((e / g.w) % g.h);
     const int ch = (int)((e / ((int64_t)g.w * g.h)) % g.cin), n = (int)(e / ((int64_t)g.w * g.h * g.cin));
     const T *xn = x + (int64_t)n * g.cin * g.h * g.w;
-    const int P = g.ho * g.wo, wp = g.wo / 2, I = (g.ho / 2) * wp;
+    const int P = g.ho * g.wo;
     T acc = 0;
     for (int c = 0; c < g.c; ++c) {
         for (int t = 0; t < 8; ++t) {
@@ -129,25 +127,10 @@ __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *_
             const int oy = ny / g.sh, ox = nx / g.sw;
             if (oy >= g.ho || ox >= g.wo) continue;
             const int p = t >> 1;
-            if constexpr (!BLOCK) {
-                const T gl = gy[(((int64_t)n * g.c + c) * P + oy * g.wo + ox) * 4 + p];
-                const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
-                const T other = read_tap(xn, g, unpack_tap(sel[c * 8 + (t ^ 1)]), oy, ox);
-                acc += gl * ((t & 1) ? gate_db(cf, other) : gate_da(cf, other));
-            } else {
-                const int64_t cell = ((int64_t)n * g.c + c) * I + (oy >> 1) * wp + (ox >> 1);
-                if (argmax[cell] != ((oy & 1) * 2 + (ox & 1))) continue;
-                const Tree<T> tr = load_tree(w + c * 7 * 16);
-                T tap[8];
-#pragma unroll
-                for (int k = 0; k < 8; ++k) tap[k] = read_tap(xn, g, unpack_tap(sel[c * 8 + k]), oy, ox);
-                const TreeVals<T> v = eval_tree(tr, tap);
-                const T g_root = gy[cell];
-                const int m = p >> 1;  // middle gate above leaf p
-                const T g_mid = g_root * (m ? gate_db(tr.g[6], v.mid[0]) : gate_da(tr.g[6], v.mid[1]));
-                const T g_leaf = g_mid * ((p & 1) ? gate_db(tr.g[4 + m], v.leaf[p ^ 1]) : gate_da(tr.g[4 + m], v.leaf[p ^ 1]));
-                acc += g_leaf * ((t & 1) ? gate_db(tr.g[p], tap[t ^ 1]) : gate_da(tr.g[p], tap[t ^ 1]));
-            }
+            const T gl = gy[(((int64_t)n * g.c + c) * P + oy * g.wo + ox) * 4 + p];
+            const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
+            const T other = read_tap(xn, g, unpack_tap(sel[c * 8 + (t ^ 1)]), oy, ox);
+            acc += gl * ((t & 1) ? gate_db(cf, other) : gate_da(cf, other));
         }
     }
     gx[e] = acc;
@@ -453,9 +436,9 @@ extern "C" int clg_conv4_backward_x(int dtype, const clg_conv_geom *gg, const vo
     CLG_REQUIRE(grad_y && x && w && selection && grad_x, "clg_conv4_backward_x: null pointer argument");
     const int64_t total = (int64_t)g.n * g.cin * g.h * g.w;
     CLG_REQUIRE(clg_ceil_div(total, kBlk) < (1ll << 31), "clg_conv4_backward_x: input too large for one launch");
-    CLG_DISPATCH(dtype, hipLaunchKernelGGL((conv_backward_x_gather_kernel<T, false>), dim3((unsigned)clg_ceil_div(total, kBlk)),
+    CLG_DISPATCH(dtype, hipLaunchKernelGGL((conv_backward_x_gather_kernel<T>), dim3((unsigned)clg_ceil_div(total, kBlk)),
                                            dim3(kBlk), 0, clg_stream(stream), (const T *)grad_y, (const T *)x, (const T *)w,
-                                           selection, (const uint8_t *)nullptr, (T *)grad_x, g));
+                                           selection, (T *)grad_x, g));
     CLG_CHECK_LAUNCH("clg_conv4_backward_x");
     return CLG_OK;
 }
