@@ -36,6 +36,14 @@ reference checkout).  How each function is pinned (see tests/test_oracle.py):
                               pack_bits / eval_packed / group_bit_sum are
                               "parity unpinned by the reference" and pinned
                               only by the closed forms above)
+  pack_image / unpack_image   round trip; bit positions read from the definition
+  conv_block_eval_packed      no reference counterpart (new capability): defined
+                              as conv_block_forward in eval mode on {0,1} inputs
+                              and checked against it sample by sample; 16-gate
+                              truth-table test
+  thresholds_*,               closed forms: linspace(1,L,L)/(L+1); quantile
+  apply_thresholds            indices on a known ramp; strict ">" and the
+                              threshold-major channel order on a written-out image
 """
 import numpy as np
 import torch
