@@ -161,6 +161,64 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ sr
     }
 }
 
+// ---- GroupSum on feature-major activations ---------------------------------------------------
+// partial[slice][g][b] = sum over the rows f of class g that belong to the slice of x[f][b]; rows are dealt
+// to the 4 wavefronts of a workgroup and combined in LDS in a fixed order, slices by a second kernel, so
+// the sums are reproducible.
+template <typename T>
+__global__ __launch_bounds__(256) void group_sum_fm_kernel(const T *__restrict__ x, T *__restrict__ partial, int64_t class_rows,
+                                                         int64_t batch, int k, int slices)
+{
+    __shared__ T meet[4][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int g = blockIdx.y, slice = blockIdx.z;
+    const int64_t b = (int64_t)blockIdx.x * kWave + lane;
+    const int64_t r0 = class_rows * slice / slices, r1 = class_rows * (slice + 1) / slices;
+    T acc = 0;
+    if (b < batch) {
+        const T *p = x + ((int64_t)g * class_rows + r0 + wave) * batch + b;
+        int64_t r = r0 + wave;
+        for (; r + 12 < r1; r += 16) {                               // four rows of this wavefront in flight
+            const T v0 = p[0], v1 = p[4 * batch], v2 = p[8 * batch], v3 = p[12 * batch];
+            acc += (v0 + v1) + (v2 + v3);
+            p += 16 * batch;
+        }
+        for (; r < r1; r += 4) {
+            acc += *p;
+            p += 4 * batch;
+        }
+    }
+    meet[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && b < batch)
+        partial[((int64_t)slice * k + g) * batch + b] = (meet[0][lane] + meet[1][lane]) + (meet[2][lane] + meet[3][lane]);
+}
+// out[b][g] = sum over slices of partial[slice][g][b]
+template <typename T>
+__global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t batch,
+                                                             int k, int slices)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= batch * k) return;
+    const int64_t b = i / k;
+    const int g = (int)(i - b * k);
+    T acc = 0;
+    for (int s = 0; s < slices; ++s) acc += partial[((int64_t)s * k + g) * batch + b];
+    out[i] = acc;
+}
+// grad_x[f][b] = grad_out[b][class of f]; a workgroup writes 64 feature rows of one 64-sample column chunk
+template <typename T>
+__global__ __launch_bounds__(256) void group_sum_backward_fm_kernel(const T *__restrict__ grad_out, T *__restrict__ grad_x,
+                                                                  int64_t class_rows, int64_t batch, int k, int64_t bchunks)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t fb = blockIdx.x / bchunks, bc = blockIdx.x - fb * bchunks;
+    const int64_t b = bc * kWave + lane;
+    if (b >= batch) return;
+    const int64_t f0 = fb * 64, features = class_rows * k;
+    for (int64_t f = f0 + wave; f < f0 + 64 && f < features; f += 4) grad_x[f * batch + b] = grad_out[b * k + f / class_rows];
+}
+
 int grid_for(int64_t items)
 {
     const int64_t blocks = clg_ceil_div(items, kWavesPerBlock);
@@ -290,5 +348,60 @@ extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64
     default: CLG_REQUIRE(false, "clg_transpose_2d: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
     }
     CLG_CHECK_LAUNCH("clg_transpose_2d");
+    return CLG_OK;
+}
+
+extern "C" int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int64_t batch, int64_t k)
+{
+    if (features <= 0 || batch <= 0 || k <= 0 || features % k != 0) return -1;
+    return 64 * k * batch * (dtype == CLG_F64 ? 8 : 4);               // at most 64 row slices
+}
+
+extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch, int64_t features, int64_t batch, int64_t k,
+                             void *stream)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_group_sum: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
+    CLG_REQUIRE(x && out && scratch, "clg_group_sum: null pointer argument");
+    CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && k <= 65535, "clg_group_sum: features, batch and k must be positive, k <= 65535");
+    CLG_REQUIRE(features % k == 0, "in_dim (%lld) has to be divisible by k (%lld) but it is not", (long long)features, (long long)k);
+    const int64_t class_rows = features / k, bchunks = clg_ceil_div(batch, kWave);
+    CLG_REQUIRE(bchunks < (1ll << 31), "clg_group_sum: batch too large for one launch");
+    // row slices until about four workgroups per CU, at least 64 rows each
+    int64_t slices = clg_ceil_div(1024, bchunks * k);
+    if (slices > class_rows / 64) slices = class_rows / 64;
+    slices = slices < 1 ? 1 : (slices > 64 ? 64 : slices);
+    hipStream_t st = clg_stream(stream);
+    const dim3 grid((unsigned)bchunks, (unsigned)k, (unsigned)slices);
+    if (dtype == CLG_F32) {
+        hipLaunchKernelGGL(group_sum_fm_kernel<float>, grid, dim3(256), 0, st, (const float *)x, (float *)scratch, class_rows, batch, (int)k,
+                           (int)slices);
+        hipLaunchKernelGGL(group_sum_finish_kernel<float>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
+                           (const float *)scratch, (float *)out, batch, (int)k, (int)slices);
+    } else {
+        hipLaunchKernelGGL(group_sum_fm_kernel<double>, grid, dim3(256), 0, st, (const double *)x, (double *)scratch, class_rows, batch,
+                           (int)k, (int)slices);
+        hipLaunchKernelGGL(group_sum_finish_kernel<double>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
+                           (const double *)scratch, (double *)out, batch, (int)k, (int)slices);
+    }
+    CLG_CHECK_LAUNCH("clg_group_sum");
+    return CLG_OK;
+}
+
+extern "C" int clg_group_sum_backward(int dtype, const void *grad_out, void *grad_x, int64_t features, int64_t batch, int64_t k,
+                                      void *stream)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_group_sum_backward: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
+    CLG_REQUIRE(grad_out && grad_x, "clg_group_sum_backward: null pointer argument");
+    CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && features % k == 0, "clg_group_sum_backward: features must be a positive multiple of k");
+    const int64_t bchunks = clg_ceil_div(batch, kWave), blocks = clg_ceil_div(features, 64) * bchunks;
+    CLG_REQUIRE(blocks < (1ll << 31), "clg_group_sum_backward: problem too large for one launch");
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32)
+        hipLaunchKernelGGL(group_sum_backward_fm_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, (const float *)grad_out,
+                           (float *)grad_x, features / k, batch, (int)k, bchunks);
+    else
+        hipLaunchKernelGGL(group_sum_backward_fm_kernel<double>, dim3((unsigned)blocks), dim3(256), 0, st, (const double *)grad_out,
+                           (double *)grad_x, features / k, batch, (int)k, bchunks);
+    CLG_CHECK_LAUNCH("clg_group_sum_backward");
     return CLG_OK;
 }

@@ -184,10 +184,28 @@ class GroupSum(torch.nn.Module):
         if isinstance(x, PackBitsTensor):
             return x.group_sum(self.k)
         assert x.shape[-1] % self.k == 0, (x.shape, self.k)
+        if (x.is_cuda and x.dim() == 2 and x.dtype in (torch.float32, torch.float64) and x.numel() > 0
+                and x.transpose(0, 1).is_contiguous() and not x.is_contiguous()):
+            # the transposed view of a feature-major tensor, as a LogicLayer returns it: summed in that layout
+            return _GroupSumFeatureMajor.apply(x, self.k) / self.tau
         return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
 
     def extra_repr(self):
         return f"k={self.k}, tau={self.tau}"
+
+
+class _GroupSumFeatureMajor(torch.autograd.Function):
+    """Per-class sums of x [batch, features] that is a transposed view of a contiguous [features, batch]
+    tensor; the gradient comes back in the same layout (a transposed view again, no copies)."""
+
+    @staticmethod
+    def forward(ctx, x, k):
+        ctx.features = x.shape[1]
+        return difflogic_hip.group_sum(x.transpose(0, 1), k)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return difflogic_hip.group_sum_backward(grad_out.contiguous(), ctx.features).transpose(0, 1), None
 
 
 class LogicLayerCudaFunction(torch.autograd.Function):

@@ -46,6 +46,31 @@ def backward_logits(x, a, b, w, grad_y):
     return gl
 
 
+def group_sum(x_fm, k):
+    """Feature-major activations [F, B] -> per-class sums [B, k] (not divided by tau), fixed summation order."""
+    check_input(x_fm, "x")
+    features, batch = x_fm.shape
+    if features % k != 0:
+        raise ValueError(f"in_dim ({features}) has to be divisible by k ({k}) but it is not")
+    lib = _lib.load()
+    dt = dtype_code(x_fm)
+    nbytes = lib.clg_group_sum_scratch_bytes(dt, features, batch, k)
+    scratch = torch.empty((max(int(nbytes), 8),), dtype=torch.uint8, device=x_fm.device)
+    out = torch.empty((batch, k), dtype=x_fm.dtype, device=x_fm.device)
+    check(lib.clg_group_sum(dt, x_fm.data_ptr(), out.data_ptr(), scratch.data_ptr(), features, batch, k, stream_ptr(x_fm)))
+    return out
+
+
+def group_sum_backward(grad_out, features):
+    """[B, k] -> feature-major gradient [F, B]: every row of class g receives grad_out[:, g]."""
+    check_input(grad_out, "grad_out")
+    batch, k = grad_out.shape
+    gx = torch.empty((features, batch), dtype=grad_out.dtype, device=grad_out.device)
+    check(_lib.load().clg_group_sum_backward(dtype_code(grad_out), grad_out.data_ptr(), gx.data_ptr(), features, batch, k,
+                                             stream_ptr(grad_out)))
+    return gx
+
+
 def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
     """grad_x[in, B]; difflogic_cuda.backward_x (difflogic_kernel.cu:232-269)."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y"),

@@ -171,3 +171,28 @@ def test_fused_softmax_backward_matches_softmax_plus_function():
         assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
         scale = outs[1][2].abs().max().item()
         assert (outs[0][2] - outs[1][2]).abs().max().item() <= tol * scale
+
+
+@pytest.mark.parametrize("features,batch,k", [(40, 7, 4), (640, 256, 10), (65536, 100, 8), (30, 1, 3), (10240, 256, 10)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_group_sum_on_feature_major_view(features, batch, k, dtype):
+    # GroupSum behind a LogicLayer receives the transposed view of a feature-major tensor: summed by the HIP
+    # kernels in that layout (fixed order), gradient handed back as a transposed view
+    torch.manual_seed(features + batch)
+    fm = torch.rand(features, batch, device=DEV, dtype=dtype)
+    x = fm.transpose(0, 1).requires_grad_(True)
+    gs = C.GroupSum(k, tau=6.5)
+    y = gs(x)
+    ref_in = fm.transpose(0, 1).contiguous().cpu().requires_grad_(True)
+    ref = O.group_sum(ref_in, k, 6.5)
+    assert y.shape == (batch, k)
+    assert torch.allclose(y.detach().cpu(), ref.detach(), rtol=1e-5 if dtype == torch.float32 else 1e-12, atol=0)
+    g = torch.randn(batch, k, device=DEV, dtype=dtype)
+    y.backward(g)
+    ref.backward(g.cpu())
+    assert torch.allclose(x.grad.cpu(), ref_in.grad, rtol=1e-6 if dtype == torch.float32 else 1e-14, atol=0)
+    # binary activations: integer sums are exact, so the packed counts still equal tau * y
+    bits = (fm > 0.5).to(dtype)
+    counts = C.GroupSum(k, tau=1.0)(bits.transpose(0, 1))
+    assert torch.equal(counts.cpu(), bits.cpu().transpose(0, 1).reshape(batch, k, features // k).sum(-1))
+    assert torch.equal(gs(x.detach()), gs(x.detach()))             # reproducible
