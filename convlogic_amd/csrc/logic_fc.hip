@@ -64,20 +64,39 @@ __global__ __launch_bounds__(kBlock) void fc_forward_kernel(const T *__restrict_
     }
 }
 
-template <typename T, int VEC>
+// Sum over each group of LPR lanes: valid in the last 16 lanes of the group.
+template <typename T, int LPR>
+__device__ __forceinline__ T lane_group_sum(T v)
+{
+    if constexpr (LPR == 64) {
+        return wave_sum(v);
+    } else {
+        v = row16_sum(v);
+        if constexpr (LPR == 32) v += dpp_zero<0x142, 0xA>(v);   // row_bcast15: rows 1 and 3 add the row before them
+        return v;
+    }
+}
+
+// A neuron's row takes LPR lanes x VEC samples per pass, a wavefront 64/LPR neurons; the last 16 lanes of each
+// group hold the four sums and write the 16 gate gradients.
+template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                              const int64_t *__restrict__ b,
                                                              const T *__restrict__ gy, T *__restrict__ gw, int out_dim,
                                                              int64_t batch, const T *__restrict__ probs)
 {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = uniform(threadIdx.x >> 6);
-    for (int j = blockIdx.x * kWavesPerBlock + wave; j < out_dim; j += gridDim.x * kWavesPerBlock) {
+    constexpr int ROWS = kWave / LPR;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int sub = lane / LPR, l = lane % LPR;
+    for (int64_t j0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * ROWS; j0 < out_dim;
+         j0 += (int64_t)gridDim.x * kWavesPerBlock * ROWS) {
+        const bool valid = j0 + sub < out_dim;
+        const int64_t j = valid ? j0 + sub : out_dim - 1;           // every lane takes part in the reductions
         const T *xa = x + a[j] * batch;
         const T *xb = x + b[j] * batch;
-        const T *gj = gy + (int64_t)j * batch;
+        const T *gj = gy + j * batch;
         T sab = 0, sa = 0, sb = 0, s1 = 0;
-        for (int64_t s = (int64_t)lane * VEC; s < batch; s += kWave * VEC) {
+        for (int64_t s = (int64_t)l * VEC; s < batch; s += LPR * VEC) {
             const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s),
                                vg = load_vec<T, VEC>(gj + s);
 #pragma unroll
@@ -88,14 +107,15 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restri
                 s1 += vg.v[k];
             }
         }
-        sab = wave_sum(sab);
-        sa = wave_sum(sa);
-        sb = wave_sum(sb);
-        s1 = wave_sum(s1);
-        if (lane < 16) {
-            T gi = coef_transpose_row<T>(lane, sab, sa, sb, s1);
-            if (probs != nullptr) gi = softmax16_backward(gi, probs[(int64_t)j * 16 + lane]);   // gradient w.r.t. the logits
-            gw[(int64_t)j * 16 + lane] = gi;
+        sab = lane_group_sum<T, LPR>(sab);
+        sa = lane_group_sum<T, LPR>(sa);
+        sb = lane_group_sum<T, LPR>(sb);
+        s1 = lane_group_sum<T, LPR>(s1);
+        if (l >= LPR - 16) {
+            const int i = lane & 15;
+            T gi = coef_transpose_row<T>(i, sab, sa, sb, s1);
+            if (probs != nullptr) gi = softmax16_backward(gi, probs[j * 16 + i]);   // gradient w.r.t. the logits
+            if (valid) gw[j * 16 + i] = gi;
         }
     }
 }
@@ -137,6 +157,132 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restri
             }
         }
         if (live) store_vec<T, VEC>(gx + (int64_t)i * batch + s, acc);
+    }
+}
+
+// ---- folded-coefficient kernels ----------------------------------------------------------------
+// The training path folds every neuron's 16 probabilities to 4 coefficients once per step (fc_fold_kernel)
+// instead of once per wavefront that touches the neuron, and lets a wavefront carry several rows when one
+// row of `batch` samples does not fill 64 lanes: a row takes LPR = 16, 32 or 64 lanes x VEC samples per pass,
+// a wavefront 64/LPR rows.  Wiring indices and coefficients are per-lane loads (one address per row group).
+
+// probs (optional) = softmax(logits) when from_logits, folded = fold16 of the probabilities
+template <typename T>
+__global__ __launch_bounds__(256) void fc_fold_kernel(const T *__restrict__ w_in, T *__restrict__ probs,
+                                                     T *__restrict__ folded, int out_dim, int from_logits)
+{
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= out_dim) return;
+    T p[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = w_in[(int64_t)j * 16 + i];
+    if (from_logits) {
+        T m = p[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) m = p[i] > m ? p[i] : m;
+        T sum = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[i] = exp(p[i] - m);
+            sum += p[i];
+        }
+        const T inv = T(1) / sum;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) p[i] *= inv;
+    }
+    if (probs != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) probs[(int64_t)j * 16 + i] = p[i];
+    }
+    const Coef<T> c = fold16(p);
+    T *f = folded + (int64_t)j * 4;
+    f[0] = c.ab;
+    f[1] = c.a;
+    f[2] = c.b;
+    f[3] = c.one;
+}
+
+template <typename T>
+__device__ __forceinline__ Coef<T> load_coef(const T *__restrict__ f)
+{
+    Coef<T> c;
+    if constexpr (sizeof(T) == 4) {
+        const float4 v = *reinterpret_cast<const float4 *>(f);
+        c.ab = v.x, c.a = v.y, c.b = v.z, c.one = v.w;
+    } else {
+        const double2 u = *reinterpret_cast<const double2 *>(f), v = *reinterpret_cast<const double2 *>(f + 2);
+        c.ab = u.x, c.a = u.y, c.b = v.x, c.one = v.y;
+    }
+    return c;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_forward_folded_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                                 const int64_t *__restrict__ b,
+                                                                 const T *__restrict__ folded, T *__restrict__ y,
+                                                                 int out_dim, int64_t batch, int lpr_log2)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
+    const int64_t pass = (int64_t)VEC << lpr_log2;
+    for (int64_t j0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * rows; j0 < out_dim;
+         j0 += (int64_t)gridDim.x * kWavesPerBlock * rows) {
+        const int64_t j = j0 + sub;
+        if (j >= out_dim) continue;
+        const Coef<T> c = load_coef(folded + j * 4);
+        const T *xa = x + a[j] * batch;
+        const T *xb = x + b[j] * batch;
+        T *yj = y + j * batch;
+        for (int64_t s = (int64_t)l * VEC; s < batch; s += pass) {
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = gate(c, va.v[k], vb.v[k]);
+            store_vec<T, VEC>(yj + s, r);
+        }
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
+    const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
+    const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
+    T *__restrict__ gx, int in_dim, int64_t batch, int batch_chunks, int lpr_log2)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
+    const int64_t items = (int64_t)((in_dim + rows - 1) >> (6 - lpr_log2)) * batch_chunks;
+    for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < items; it += (int64_t)gridDim.x * kWavesPerBlock) {
+        const int64_t i = (it / batch_chunks) * rows + sub;
+        const int64_t s = (((it % batch_chunks) << lpr_log2) + l) * VEC;
+        if (i >= in_dim || s >= batch) continue;
+        const int64_t beg = csr_start[i], end = csr_start[i + 1];
+        Pack<T, VEC> acc;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc.v[k] = 0;
+        if (beg < end) {
+            // The chain list -> wiring and coefficients -> rows is three dependent loads deep: the list runs two
+            // consumers ahead and the tables one ahead of the rows being accumulated.
+            int64_t prev = -1, j = csr_list[beg], j_next = csr_list[beg + 1 < end ? beg + 1 : beg];
+            int64_t ia = a[j], ib = b[j];
+            Coef<T> c = load_coef(folded + j * 4);
+            for (int64_t cur = beg; cur < end; ++cur) {
+                const int64_t j_after = csr_list[cur + 2 < end ? cur + 2 : end - 1];
+                const int64_t ia_next = a[j_next], ib_next = b[j_next];
+                const Coef<T> c_next = load_coef(folded + j_next * 4);
+                // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
+                // feature twice appears twice in the list and takes the B derivative the second time.
+                const bool as_a = ia == i && !(ib == i && prev == j);
+                const T *other = x + (as_a ? ib : ia) * batch;
+                const T c_lin = as_a ? c.a : c.b;
+                const Pack<T, VEC> vo = load_vec<T, VEC>(other + s), vg = load_vec<T, VEC>(gy + j * batch + s);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc.v[k] = fma_t(fma_t(c.ab, vo.v[k], c_lin), vg.v[k], acc.v[k]);
+                prev = j, j = j_next, j_next = j_after;
+                ia = ia_next, ib = ib_next, c = c_next;
+            }
+        }
+        store_vec<T, VEC>(gx + i * batch + s, acc);
     }
 }
 
@@ -228,6 +374,13 @@ int grid_for(int64_t items)
 template <typename T>
 constexpr int vec_width() { return 16 / sizeof(T); }
 
+// log2 of the lanes one row of `batch` samples takes at `vec` samples per lane: 16, 32 or 64 lanes
+int lanes_per_row_log2(int64_t batch, int vec)
+{
+    const int64_t lanes = clg_ceil_div(batch, (int64_t)vec);
+    return lanes <= 16 ? 4 : (lanes <= 32 ? 5 : 6);
+}
+
 int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const char *name)
 {
     CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
@@ -270,23 +423,28 @@ static int fc_backward_w_impl(int dtype, const void *x, const int64_t *a, const 
 {
     if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
     CLG_REQUIRE(x && a && b && grad_y && grad_w, "%s: null pointer argument", name);
-    const dim3 grid(grid_for(out_dim)), block(kBlock);
+    const dim3 block(kBlock);
     hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_BW(T, VEC, LPR)                                                                                      \
+    hipLaunchKernelGGL((fc_backward_w_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave / LPR)))), \
+                       block, 0, st, (const T *)x, a, b, (const T *)grad_y, (T *)grad_w, (int)out_dim, batch,              \
+                       (const T *)probs)
+#define CLG_LAUNCH_BW_ROWS(T, VEC)                                                                                      \
+    do {                                                                                                               \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
+        if (lg == 4) CLG_LAUNCH_BW(T, VEC, 16);                                                                        \
+        else if (lg == 5) CLG_LAUNCH_BW(T, VEC, 32);                                                                   \
+        else CLG_LAUNCH_BW(T, VEC, 64);                                                                                \
+    } while (0)
     if (dtype == CLG_F32) {
-        if (batch % 4 == 0)
-            hipLaunchKernelGGL((fc_backward_w_kernel<float, 4>), grid, block, 0, st, (const float *)x, a, b,
-                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch, (const float *)probs);
-        else
-            hipLaunchKernelGGL((fc_backward_w_kernel<float, 1>), grid, block, 0, st, (const float *)x, a, b,
-                               (const float *)grad_y, (float *)grad_w, (int)out_dim, batch, (const float *)probs);
+        if (batch % 4 == 0) CLG_LAUNCH_BW_ROWS(float, 4);
+        else CLG_LAUNCH_BW_ROWS(float, 1);
     } else {
-        if (batch % 2 == 0)
-            hipLaunchKernelGGL((fc_backward_w_kernel<double, 2>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch, (const double *)probs);
-        else
-            hipLaunchKernelGGL((fc_backward_w_kernel<double, 1>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)grad_y, (double *)grad_w, (int)out_dim, batch, (const double *)probs);
+        if (batch % 2 == 0) CLG_LAUNCH_BW_ROWS(double, 2);
+        else CLG_LAUNCH_BW_ROWS(double, 1);
     }
+#undef CLG_LAUNCH_BW_ROWS
+#undef CLG_LAUNCH_BW
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }
@@ -329,6 +487,79 @@ extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, con
     }
 #undef CLG_LAUNCH_BX
     CLG_CHECK_LAUNCH("clg_fc_backward_x");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_fold(int dtype, int from_logits, const void *w_in, void *probs, void *folded, int64_t out_dim,
+                           void *stream)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_fc_fold: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
+    CLG_REQUIRE(w_in && folded, "clg_fc_fold: null pointer argument");
+    CLG_REQUIRE(out_dim > 0 && out_dim < (1ll << 31), "clg_fc_fold: out_dim must be in [1, 2^31-1], got %lld", (long long)out_dim);
+    const dim3 grid((unsigned)clg_ceil_div(out_dim, (int64_t)256)), block(256);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32)
+        hipLaunchKernelGGL(fc_fold_kernel<float>, grid, block, 0, st, (const float *)w_in, (float *)probs, (float *)folded,
+                           (int)out_dim, from_logits);
+    else
+        hipLaunchKernelGGL(fc_fold_kernel<double>, grid, block, 0, st, (const double *)w_in, (double *)probs,
+                           (double *)folded, (int)out_dim, from_logits);
+    CLG_CHECK_LAUNCH("clg_fc_fold");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                     void *y, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward_folded")) return e;
+    CLG_REQUIRE(x && a && b && folded && y, "clg_fc_forward_folded: null pointer argument");
+    const dim3 block(kBlock);
+    hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_FF(T, VEC)                                                                                           \
+    do {                                                                                                               \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
+        hipLaunchKernelGGL((fc_forward_folded_kernel<T, VEC>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave >> lg)))), \
+                           block, 0, st, (const T *)x, a, b, (const T *)folded, (T *)y, (int)out_dim, batch, lg);          \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_FF(float, 4);
+        else CLG_LAUNCH_FF(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_FF(double, 2);
+        else CLG_LAUNCH_FF(double, 1);
+    }
+#undef CLG_LAUNCH_FF
+    CLG_CHECK_LAUNCH("clg_fc_forward_folded");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                        const void *grad_y, const int64_t *csr_start, const int64_t *csr_list, void *grad_x,
+                                        int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_x_folded")) return e;
+    CLG_REQUIRE(x && a && b && folded && grad_y && csr_start && csr_list && grad_x,
+                "clg_fc_backward_x_folded: null pointer argument");
+    hipStream_t st = clg_stream(stream);
+    const dim3 block(kBlock);
+#define CLG_LAUNCH_BXF(T, VEC)                                                                                          \
+    do {                                                                                                               \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
+        const int chunks = (int)clg_ceil_div(batch, (int64_t)VEC << lg);                                               \
+        const int64_t items = clg_ceil_div(in_dim, (int64_t)(kWave >> lg)) * chunks;                                   \
+        hipLaunchKernelGGL((fc_backward_x_folded_kernel<T, VEC>), dim3(grid_for(items)), block, 0, st, (const T *)x, a, b, \
+                           (const T *)folded, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (int)in_dim, batch,     \
+                           chunks, lg);                                                                                \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_BXF(float, 4);
+        else CLG_LAUNCH_BXF(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_BXF(double, 2);
+        else CLG_LAUNCH_BXF(double, 1);
+    }
+#undef CLG_LAUNCH_BXF
+    CLG_CHECK_LAUNCH("clg_fc_backward_x_folded");
     return CLG_OK;
 }
 

@@ -236,17 +236,17 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y):
-        w = torch.softmax(logits, dim=-1)
-        ctx.save_for_backward(x, a, b, w, given_x_indices_of_y_start, given_x_indices_of_y)
-        return difflogic_hip.forward(x, a, b, w)
+        w, folded = difflogic_hip.fold(logits, from_logits=True)
+        ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
+        return difflogic_hip.forward_folded(x, a, b, folded)
 
     @staticmethod
     def backward(ctx, grad_y):
-        x, a, b, w, start, flat = ctx.saved_tensors
+        x, a, b, w, folded, start, flat = ctx.saved_tensors
         grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
         grad_x = grad_l = None
         if ctx.needs_input_grad[0]:
-            grad_x = difflogic_hip.backward_x(x, a, b, w, grad_y, start, flat)
+            grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)
         if ctx.needs_input_grad[3]:
             grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
         return grad_x, None, None, grad_l, None, None

@@ -46,6 +46,44 @@ def backward_logits(x, a, b, w, grad_y):
     return gl
 
 
+def fold(w_in, from_logits, want_probs=True):
+    """[out, 16] logits or probabilities -> (probabilities or None, folded coefficients [out, 4])."""
+    check_input(w_in, "w")
+    out_dim = w_in.shape[0]
+    probs = torch.empty_like(w_in) if want_probs else None
+    folded = torch.empty((out_dim, 4), dtype=w_in.dtype, device=w_in.device)
+    check(_lib.load().clg_fc_fold(dtype_code(w_in), int(bool(from_logits)), w_in.data_ptr(),
+                                  probs.data_ptr() if want_probs else 0, folded.data_ptr(), out_dim, stream_ptr(w_in)))
+    return probs, folded
+
+
+def forward_folded(x, a, b, folded):
+    """forward() with the folded coefficients [out, 4] of fold() in place of w."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = folded.shape[0]
+    y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_forward_folded(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
+                                            y.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return y
+
+
+def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
+    """backward_x() with the folded coefficients [out, 4] of fold() in place of w."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y"),
+                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
+        check_input(t, n)
+    in_dim, batch = x.shape
+    out_dim = folded.shape[0]
+    gx = torch.empty_like(x)
+    check(_lib.load().clg_fc_backward_x_folded(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
+                                               grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
+                                               given_x_indices_of_y.data_ptr(), gx.data_ptr(), in_dim, out_dim, batch,
+                                               stream_ptr(x)))
+    return gx
+
+
 def group_sum(x_fm, k):
     """Feature-major activations [F, B] -> per-class sums [B, k] (not divided by tau), fixed summation order."""
     check_input(x_fm, "x")

@@ -88,6 +88,24 @@ int clg_fc_backward_logits(int dtype, const void *x, const int64_t *a, const int
                            const void *grad_y, void *grad_logits /*[out_dim,16]*/, int64_t in_dim, int64_t out_dim,
                            int64_t batch, void *stream);
 
+/* The training step of the module folds each neuron's 16 gate probabilities to the 4 coefficients of
+ * y = c_ab*a*b + c_a*a + c_b*b + c_1 once, instead of in every wavefront that touches the neuron:
+ *   clg_fc_fold            w_in [out_dim,16] (logits when from_logits != 0, else probabilities) ->
+ *                          probs [out_dim,16] (softmax of the logits; may be NULL) and folded [out_dim,4]
+ *   clg_fc_forward_folded  clg_fc_forward with folded in place of w
+ *   clg_fc_backward_x_folded  clg_fc_backward_x with folded in place of w
+ * The two kernels give the values of clg_fc_forward / clg_fc_backward_x on the same probabilities and,
+ * when a row of `batch` samples fills fewer than 64 lanes, put 2 or 4 rows into a wavefront.  Replace the
+ * softmax of LogicLayer.forward_cuda (src/difflogic/difflogic.py:138) plus difflogic_cuda.forward /
+ * backward_x (src/difflogic/cuda/difflogic.cpp:18-19). */
+int clg_fc_fold(int dtype, int from_logits, const void *w_in /*[out_dim,16]*/, void *probs /*[out_dim,16] or NULL*/,
+                void *folded /*[out_dim,4]*/, int64_t out_dim, void *stream);
+int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
+                          void *y, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
+int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                             const void *grad_y, const int64_t *csr_start, const int64_t *csr_list, void *grad_x,
+                             int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
+
 /* GroupSum on feature-major activations x [features, batch] (what the last LogicLayer produces): out[b][g] =
  * sum of the features/k rows of class g, NOT yet divided by tau; fixed summation order (reproducible).
  * scratch: clg_group_sum_scratch_bytes().  Replaces x.reshape(..., k, F/k).sum(-1) of
