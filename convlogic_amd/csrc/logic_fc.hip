@@ -42,6 +42,21 @@ __device__ __forceinline__ void store_vec(T *p, const Pack<T, VEC> &v)
     *reinterpret_cast<V *>(p) = __builtin_bit_cast(V, v);
 }
 
+// folded = 4 coefficients per neuron, written by fc_fold_kernel
+template <typename T>
+__device__ __forceinline__ Coef<T> load_coef(const T *__restrict__ f)
+{
+    Coef<T> c;
+    if constexpr (sizeof(T) == 4) {
+        const float4 v = *reinterpret_cast<const float4 *>(f);
+        c.ab = v.x, c.a = v.y, c.b = v.z, c.one = v.w;
+    } else {
+        const double2 u = *reinterpret_cast<const double2 *>(f), v = *reinterpret_cast<const double2 *>(f + 2);
+        c.ab = u.x, c.a = u.y, c.b = v.x, c.one = v.y;
+    }
+    return c;
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                           const int64_t *__restrict__ b, const T *__restrict__ w,
@@ -105,6 +120,61 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restri
                 sa = fma_t(vg.v[k], va.v[k], sa);
                 sb = fma_t(vg.v[k], vb.v[k], sb);
                 s1 += vg.v[k];
+            }
+        }
+        sab = lane_group_sum<T, LPR>(sab);
+        sa = lane_group_sum<T, LPR>(sa);
+        sb = lane_group_sum<T, LPR>(sb);
+        s1 = lane_group_sum<T, LPR>(s1);
+        if (l >= LPR - 16) {
+            const int i = lane & 15;
+            T gi = coef_transpose_row<T>(i, sab, sa, sb, s1);
+            if (probs != nullptr) gi = softmax16_backward(gi, probs[j * 16 + i]);   // gradient w.r.t. the logits
+            if (valid) gw[j * 16 + i] = gi;
+        }
+    }
+}
+
+// Both gradients in one pass for layers in which every input feature is read by exactly one neuron operand
+// (2 out_dim = in_dim with the reference's random wiring): the input gradient of such a feature is a single
+// product, so the neuron that reads it writes its row and no gather over consumers is needed.  Same arithmetic
+// as fc_backward_w_kernel and fc_backward_x_folded_kernel; 3 row reads and 2 row writes per neuron instead of 7 and 2.
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                                const int64_t *__restrict__ b, const T *__restrict__ folded,
+                                                                const T *__restrict__ gy, T *__restrict__ gx,
+                                                                T *__restrict__ gw, int out_dim, int64_t batch,
+                                                                const T *__restrict__ probs)
+{
+    constexpr int ROWS = kWave / LPR;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int sub = lane / LPR, l = lane % LPR;
+    for (int64_t j0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * ROWS; j0 < out_dim;
+         j0 += (int64_t)gridDim.x * kWavesPerBlock * ROWS) {
+        const bool valid = j0 + sub < out_dim;
+        const int64_t j = valid ? j0 + sub : out_dim - 1;           // every lane takes part in the reductions
+        const int64_t ia = a[j], ib = b[j];
+        const Coef<T> c = load_coef(folded + j * 4);
+        const T *xa = x + ia * batch;
+        const T *xb = x + ib * batch;
+        const T *gj = gy + j * batch;
+        T sab = 0, sa = 0, sb = 0, s1 = 0;
+        for (int64_t s = (int64_t)l * VEC; s < batch; s += LPR * VEC) {
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s),
+                               vg = load_vec<T, VEC>(gj + s);
+            Pack<T, VEC> ga, gb;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                sab = fma_t(vg.v[k], va.v[k] * vb.v[k], sab);
+                sa = fma_t(vg.v[k], va.v[k], sa);
+                sb = fma_t(vg.v[k], vb.v[k], sb);
+                s1 += vg.v[k];
+                ga.v[k] = fma_t(c.ab, vb.v[k], c.a) * vg.v[k];
+                gb.v[k] = fma_t(c.ab, va.v[k], c.b) * vg.v[k];
+            }
+            if (valid) {
+                store_vec<T, VEC>(gx + ia * batch + s, ga);
+                store_vec<T, VEC>(gx + ib * batch + s, gb);
             }
         }
         sab = lane_group_sum<T, LPR>(sab);
@@ -200,20 +270,6 @@ __global__ __launch_bounds__(256) void fc_fold_kernel(const T *__restrict__ w_in
     f[1] = c.a;
     f[2] = c.b;
     f[3] = c.one;
-}
-
-template <typename T>
-__device__ __forceinline__ Coef<T> load_coef(const T *__restrict__ f)
-{
-    Coef<T> c;
-    if constexpr (sizeof(T) == 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(f);
-        c.ab = v.x, c.a = v.y, c.b = v.z, c.one = v.w;
-    } else {
-        const double2 u = *reinterpret_cast<const double2 *>(f), v = *reinterpret_cast<const double2 *>(f + 2);
-        c.ab = u.x, c.a = u.y, c.b = v.x, c.one = v.y;
-    }
-    return c;
 }
 
 template <typename T, int VEC>
@@ -560,6 +616,40 @@ extern "C" int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t 
     }
 #undef CLG_LAUNCH_BXF
     CLG_CHECK_LAUNCH("clg_fc_backward_x_folded");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                    const void *probs, const void *grad_y, void *grad_x, void *grad_w, int64_t in_dim,
+                                    int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_sole")) return e;
+    CLG_REQUIRE(x && a && b && folded && grad_y && grad_x && grad_w, "clg_fc_backward_sole: null pointer argument");
+    CLG_REQUIRE(2 * out_dim == in_dim, "clg_fc_backward_sole: needs 2*out_dim == in_dim (every input read exactly once), got %lld, %lld",
+                (long long)out_dim, (long long)in_dim);
+    const dim3 block(kBlock);
+    hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_BS(T, VEC, LPR)                                                                                         \
+    hipLaunchKernelGGL((fc_backward_sole_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave / LPR)))), \
+                       block, 0, st, (const T *)x, a, b, (const T *)folded, (const T *)grad_y, (T *)grad_x, (T *)grad_w,      \
+                       (int)out_dim, batch, (const T *)probs)
+#define CLG_LAUNCH_BS_ROWS(T, VEC)                                                                                         \
+    do {                                                                                                                  \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                    \
+        if (lg == 4) CLG_LAUNCH_BS(T, VEC, 16);                                                                           \
+        else if (lg == 5) CLG_LAUNCH_BS(T, VEC, 32);                                                                      \
+        else CLG_LAUNCH_BS(T, VEC, 64);                                                                                   \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_BS_ROWS(float, 4);
+        else CLG_LAUNCH_BS_ROWS(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_BS_ROWS(double, 2);
+        else CLG_LAUNCH_BS_ROWS(double, 1);
+    }
+#undef CLG_LAUNCH_BS_ROWS
+#undef CLG_LAUNCH_BS
+    CLG_CHECK_LAUNCH("clg_fc_backward_sole");
     return CLG_OK;
 }
 

@@ -95,7 +95,8 @@ class LogicLayer(torch.nn.Module):
         xt = _feature_major(x)
         if self.training and self.weights.dtype == xt.dtype and self.weights.is_contiguous():
             return _LogicLayerLogitsFunction.apply(xt, self.indices_0, self.indices_1, self.weights,
-                                                   self.given_x_indices_of_y_start, self.given_x_indices_of_y).transpose(0, 1)
+                                                   self.given_x_indices_of_y_start, self.given_x_indices_of_y,
+                                                   self._sole_consumers()).transpose(0, 1)
         w = self._gate_weights(xt.dtype)
         args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
         if self.training:
@@ -118,6 +119,20 @@ class LogicLayer(torch.nn.Module):
         if cached is None or cached[0] != key:
             cached = (key, self.weights.detach().argmax(-1).to(torch.uint8))
             self._gate_cache = cached
+        return cached[1]
+
+    def _sole_consumers(self):
+        """True when every input feature is read by exactly one neuron operand (the halving layers of the
+        reference's models, 2*out_dim == in_dim): both gradients then come from one kernel.  Rechecked when the
+        wiring buffers were modified in place or moved."""
+        if 2 * self.out_dim != self.in_dim:
+            return False
+        key = (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+        cached = getattr(self, "_sole_cache", None)
+        if cached is None or cached[0] != key:
+            uses = torch.bincount(torch.cat([self.indices_0, self.indices_1]), minlength=self.in_dim)
+            cached = (key, bool((uses == 1).all().item()))
+            self._sole_cache = cached
         return cached[1]
 
     def _eval_plan(self):
@@ -235,9 +250,10 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
     to rounding)."""
 
     @staticmethod
-    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y):
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False):
         w, folded = difflogic_hip.fold(logits, from_logits=True)
         ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
+        ctx.sole_consumers = sole_consumers
         return difflogic_hip.forward_folded(x, a, b, folded)
 
     @staticmethod
@@ -245,11 +261,14 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
         x, a, b, w, folded, start, flat = ctx.saved_tensors
         grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
         grad_x = grad_l = None
-        if ctx.needs_input_grad[0]:
-            grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)
-        if ctx.needs_input_grad[3]:
-            grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
-        return grad_x, None, None, grad_l, None, None
+        if ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]:
+            grad_x, grad_l = difflogic_hip.backward_sole(x, a, b, folded, w, grad_y)
+        else:
+            if ctx.needs_input_grad[0]:
+                grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)
+            if ctx.needs_input_grad[3]:
+                grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
+        return grad_x, None, None, grad_l, None, None, None
 
 
 def _contiguous_2d(t):

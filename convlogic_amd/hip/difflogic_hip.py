@@ -84,6 +84,23 @@ def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given
     return gx
 
 
+def backward_sole(x, a, b, folded, probs, grad_y):
+    """(grad_x, grad_w) in one pass for a layer whose inputs are each read by exactly one neuron operand; grad_w is
+    the gradient w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y")):
+        check_input(t, n)
+    if probs is not None:
+        check_input(probs, "w")
+    in_dim, batch = x.shape
+    out_dim = folded.shape[0]
+    gx = torch.empty_like(x)
+    gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_backward_sole(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
+                                           probs.data_ptr() if probs is not None else 0, grad_y.data_ptr(), gx.data_ptr(),
+                                           gw.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return gx, gw
+
+
 def group_sum(x_fm, k):
     """Feature-major activations [F, B] -> per-class sums [B, k] (not divided by tau), fixed summation order."""
     check_input(x_fm, "x")

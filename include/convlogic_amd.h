@@ -106,6 +106,17 @@ int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t *a, const i
                              const void *grad_y, const int64_t *csr_start, const int64_t *csr_list, void *grad_x,
                              int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
 
+/* Both gradients of a layer in which every input feature is read by exactly one neuron operand (the caller
+ * guarantees it; 2*out_dim == in_dim is checked): the neuron that reads a feature writes its grad_x row, so
+ * the pass over the CSR map is not needed.  grad_w holds the gradient w.r.t. the probabilities, or w.r.t. the
+ * logits when probs [out_dim,16] = softmax(logits) is given (NULL otherwise).  Same values as
+ * clg_fc_backward_x_folded + clg_fc_backward_w / clg_fc_backward_logits.  Replaces difflogic_cuda.backward_x
+ * and backward_w (src/difflogic/cuda/difflogic.cpp:18-19) for the halving layers of the reference's models
+ * (src/convlogic/model.py:49-55, :102-103). */
+int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
+                         const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, void *grad_x, void *grad_w,
+                         int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
+
 /* GroupSum on feature-major activations x [features, batch] (what the last LogicLayer produces): out[b][g] =
  * sum of the features/k rows of class g, NOT yet divided by tau; fixed summation order (reproducible).
  * scratch: clg_group_sum_scratch_bytes().  Replaces x.reshape(..., k, F/k).sum(-1) of

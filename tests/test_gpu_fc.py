@@ -229,3 +229,53 @@ def test_group_sum_on_feature_major_view(features, batch, k, dtype):
     counts = C.GroupSum(k, tau=1.0)(bits.transpose(0, 1))
     assert torch.equal(counts.cpu(), bits.cpu().transpose(0, 1).reshape(batch, k, features // k).sum(-1))
     assert torch.equal(gs(x.detach()), gs(x.detach()))             # reproducible
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("out_dim,batch", [(16, 8), (50, 60), (64, 128), (33, 100), (200, 256), (75, 300), (9, 33), (1, 1)])
+def test_halving_layer_gradients_come_from_one_pass(out_dim, batch, dtype):
+    # 2*out == in with the reference's random wiring reads every input exactly once: the fused kernel must give
+    # the gradients of the two separate kernels bit for bit, and the module must pick it by itself
+    from convlogic_amd.difflogic.difflogic import _LogicLayerLogitsFunction
+    torch.manual_seed(out_dim * 7 + batch)
+    in_dim = 2 * out_dim
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV).to(dtype)
+    assert layer._sole_consumers()
+    tabs = (layer.indices_0, layer.indices_1)
+    csr = (layer.given_x_indices_of_y_start, layer.given_x_indices_of_y)
+    x = torch.rand(in_dim, batch, device=DEV, dtype=dtype)
+    gy = torch.randn(out_dim, batch, device=DEV, dtype=dtype)
+    probs, folded = difflogic_hip.fold(layer.weights.detach(), from_logits=True)
+    gx, gl = difflogic_hip.backward_sole(x, *tabs, folded, probs, gy)
+    assert torch.equal(gx, difflogic_hip.backward_x_folded(x, *tabs, folded, gy, *csr))
+    assert torch.equal(gl, difflogic_hip.backward_logits(x, *tabs, probs, gy))
+    gx2, gw = difflogic_hip.backward_sole(x, *tabs, folded, None, gy)
+    assert torch.equal(gx2, gx) and torch.equal(gw, difflogic_hip.backward_w(x, *tabs, gy))
+    # through the module, against the oracle
+    xm = x.t().contiguous().requires_grad_(True)
+    layer(xm).backward(gy.t().contiguous())
+    _, gx_ref, gl_ref = _oracle_grads(xm, layer.weights, layer.indices_0, layer.indices_1, gy.t())
+    assert_grad_close(xm.grad, gx_ref.to(dtype), name="grad_x")
+    assert_grad_close(layer.weights.grad, gl_ref.to(dtype), name="grad_logits")
+
+
+def test_halving_layer_with_shared_inputs_keeps_the_gather():
+    # same sizes, but one input is wired twice and another never: the one-pass kernel would drop a term, so the
+    # module has to notice (also after an in-place rewiring of a layer it had already classified)
+    from convlogic_amd.difflogic.difflogic import _reverse_wiring
+    torch.manual_seed(11)
+    layer = C.LogicLayer(24, 12, implementation="cuda").to(DEV)
+    assert layer._sole_consumers()
+    idx0, idx1 = layer.indices_0.cpu().clone(), layer.indices_1.cpu().clone()
+    idx1[5] = idx0[2]                                                # idx0[2] now read twice, old idx1[5] never
+    layer.indices_1.copy_(idx1.to(DEV))
+    s, f = _reverse_wiring(idx0.numpy(), idx1.numpy(), 24)
+    layer.given_x_indices_of_y_start.copy_(s.to(DEV))
+    layer.given_x_indices_of_y.copy_(f.to(DEV))
+    assert not layer._sole_consumers()
+    x = torch.rand(40, 24, device=DEV, requires_grad=True)
+    gy = torch.randn(40, 12, device=DEV)
+    layer(x).backward(gy)
+    _, gx_ref, gl_ref = _oracle_grads(x, layer.weights, idx0, idx1, gy)
+    assert_grad_close(x.grad, gx_ref, name="grad_x")
+    assert_grad_close(layer.weights.grad, gl_ref, name="grad_logits")
