@@ -84,3 +84,29 @@ def test_training_step_replays_equal_eager(kind):
         want = [ex.grad] + [p.grad for p in eager.parameters()]
         for i, (got, ref) in enumerate(zip(static_grads, want)):
             assert torch.equal(got, ref), (kind, trial, i, (got - ref).abs().max().item())
+
+
+def test_graphed_step_helper_trains_like_eager_steps():
+    # GraphedStep on the CIFAR topology with an optimizer outside the graph: three steps on different batches
+    # give the same losses and parameters as three eager steps from the same start
+    torch.manual_seed(5)
+    model = C.ConvLogicCifarModel(k_param=2, input_channels=3, input_size=32, tau=10).to(DEV)
+    twin = copy.deepcopy(model)
+    batches = [(torch.randint(0, 2, (64, 3, 32, 32), device=DEV).float(), torch.randint(0, 10, (64,), device=DEV)) for _ in range(3)]
+    ce = torch.nn.functional.cross_entropy
+    step = C.GraphedStep(lambda x, y: ce(model(x), y), batches[0], model.parameters())
+    opt_g = torch.optim.SGD(model.parameters(), lr=0.1)
+    opt_e = torch.optim.SGD(twin.parameters(), lr=0.1)
+    for x, y in batches:
+        loss_g = step(x, y).clone()
+        opt_g.step()
+        torch.cuda.synchronize()
+        opt_e.zero_grad(set_to_none=True)
+        loss_e = ce(twin(x), y)
+        loss_e.backward()
+        opt_e.step()
+        assert torch.equal(loss_g, loss_e.detach())
+        for pg, pe in zip(model.parameters(), twin.parameters()):
+            assert torch.equal(pg, pe)
+    with pytest.raises(ValueError):
+        step(batches[0][0][:32], batches[0][1][:32])
