@@ -22,6 +22,9 @@
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
 int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
                                   uint8_t *argmax, hipStream_t st);
+bool clg_convblock_is_4x4(const Geom &g);
+int clg_convblock_forward_4x4(int dtype, const Geom &g, const void *x, const void *folded, const int32_t *sel, void *y, uint8_t *argmax,
+                              hipStream_t st, const char *name);
 
 namespace {
 
@@ -471,9 +474,13 @@ bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan 
 }
 
 // Which forward path a shape takes: 0 = tiled (all channels in LDS), 1 = tiled with channel subsets,
-// 2 = direct from a padded copy (needs scratch), 3 = any-shape kernel.
+// 2 = direct from a padded copy (needs scratch), 3 = any-shape kernel, 4 = one sample per lane on 4x4 images
+// (float gates; needs scratch for the folded coefficients).
 int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scratch, TilePlan *tp, DirectPlan *dp)
 {
+    bool lane_sample = have_scratch && params_per_kernel > 1 && clg_convblock_is_4x4(g);
+    if (const char *e = getenv("CLG_FWD_4X4")) lane_sample = lane_sample && atoi(e) != 0;
+    if (lane_sample) return 4;
     const bool tiled = plan_forward(g, elem, params_per_kernel, tp);
     const bool direct = have_scratch && plan_forward_direct(g, elem, params_per_kernel > 1, dp);
     // 4-byte elements: direct beats the channel-subset staging (354 -> 163 us at [256,256,16,16] -> 1024); 8-byte
@@ -601,7 +608,8 @@ extern "C" int64_t clg_convblock_forward_scratch_bytes(int dtype, const clg_conv
     TilePlan tp;
     DirectPlan dp;
     const int elem = dtype == CLG_F64 ? 8 : 4;
-    return choose_forward(g, elem, 28, true, &tp, &dp) == 2 ? (int64_t)dp.total : 0;
+    const int path = choose_forward(g, elem, 28, true, &tp, &dp);
+    return path == 2 ? (int64_t)dp.total : (path == 4 ? (int64_t)g.c * 28 * elem : 0);
 }
 
 extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
@@ -613,8 +621,20 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
     TilePlan tp;
     DirectPlan dp;
     const int elem = dtype == CLG_F64 ? 8 : 4;
-    if (choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp) != 2) return clg_convblock_forward(dtype, gg, x, w, selection, y, argmax, stream);
+    const int path = choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp);
     hipStream_t st = clg_stream(stream);
+    if (path == 4) {
+        const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
+        if (dtype == CLG_F32)
+            hipLaunchKernelGGL(convblock_w_prepare_kernel<float>, pgrid, dim3(256), 0, st, (const float *)w, selection, (float *)scratch,
+                               (int32_t *)nullptr, g.c, 0, 0);
+        else
+            hipLaunchKernelGGL(convblock_w_prepare_kernel<double>, pgrid, dim3(256), 0, st, (const double *)w, selection, (double *)scratch,
+                               (int32_t *)nullptr, g.c, 0, 0);
+        CLG_CHECK_LAUNCH("clg_convblock_forward_ws");
+        return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_ws");
+    }
+    if (path != 2) return clg_convblock_forward(dtype, gg, x, w, selection, y, argmax, stream);
     if (dtype == CLG_F32)
         return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
     return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");

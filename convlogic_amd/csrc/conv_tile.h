@@ -117,14 +117,14 @@ __global__ __launch_bounds__(256) void pad_image_kernel(const T *__restrict__ x,
     xp[e] = v;
 }
 
-// folded coefficients [c][28] (skipped when folded is null) and tap offsets [c][8] in the padded-image layout
+// folded coefficients [c][28] and tap offsets [c][8] in the padded-image layout (either is skipped when null)
 template <typename T>
 __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
                                                                 T *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
                                                                 int chs)
 {
     const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (q < (int64_t)C * 8) {
+    if (taps != nullptr && q < (int64_t)C * 8) {
         const Tap tp = unpack_tap(sel[q]);
         taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
     }

@@ -282,3 +282,30 @@ def test_block_fused_softmax_backward_matches_softmax_plus_function(shape):
     y = layer(x.detach())
     y.sum().backward()
     assert layer.weights.grad is not None and torch.isfinite(layer.weights.grad).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,cin,cout", [(32, 3, 5), (100, 24, 48), (130, 40, 17)])
+def test_block_4x4_one_sample_per_lane_vs_oracle_and_staged_path(n, cin, cout, dtype, monkeypatch):
+    # 4x4 images with at least 32 samples take the one-sample-per-lane forward: against the oracle, against the
+    # staged kernels (bit for bit, pooling choice included), with a ragged last wavefront, and with a caller-made
+    # selection whose kernels read up to eight different channels (those kernels read global memory)
+    from convlogic_amd.hip import convlogic_hip
+    torch.manual_seed(n + cin)
+    layer, x, y, idx = _run_block(n, cin, cout, 4, 4, 1, 1, 3, dtype=dtype, seed=n)
+    routed, y_ref, idx_ref, _, _, _, _, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
+    check_pool_route(idx, idx_ref, x4)
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
+    wp = torch.softmax(layer.weights.detach(), -1)
+    sel_wide = layer.selection.clone()
+    if cin >= 8:
+        taps = torch.arange(8, device=DEV, dtype=torch.int32)
+        sel_wide[1] = ((taps % cin) << 16) | ((taps % 3) << 8) | ((taps // 3) % 3)          # eight channels
+        sel_wide[cout - 1] = (((taps // 3) + 2) << 16) | ((taps % 3) << 8) | (taps % 2)     # three channels
+    for sel in (layer.selection, sel_wide):
+        args = (x.detach(), wp, sel, 1, 1, 1, 1, 3, 3)
+        y_new, a_new = convlogic_hip.full_convlogic_forward(*args)
+        monkeypatch.setenv("CLG_FWD_4X4", "0")
+        y_old, a_old = convlogic_hip.full_convlogic_forward(*args)
+        monkeypatch.delenv("CLG_FWD_4X4")
+        assert torch.equal(y_new, y_old) and torch.equal(a_new, a_old)
