@@ -82,8 +82,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
                                                               T *__restrict__ folded, int32_t *__restrict__ count,
                                                               int32_t *__restrict__ hits, int32_t *__restrict__ taps, int C,
-                                                              int cin, int fold_blocks, int rs, int chs)
+                                                              int cin, int fold_blocks, int rs, int chs, PadJob<T> pad, int pad_block0)
 {
+    if ((int)blockIdx.x >= pad_block0) {                            // tail of the launch: the padded copy of x
+        pad_image_elem(pad, (int64_t)(blockIdx.x - pad_block0) * 256 + threadIdx.x);
+        return;
+    }
     if ((int)blockIdx.x < fold_blocks) {
         const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
         if (q < (int64_t)C * 8) {                                   // tap offsets of the LDS window layout
@@ -819,7 +823,9 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     // at 16.8M, 30 vs 27 us at 1.6M)
     if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_PADDED")) return false;
     const int64_t sample_elems = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
-    if (sample_elems * g.n * elem >= (1ll << 32) || I * g.n >= (1ll << 31)) return false;
+    // the copy may be made by the tiled input gradient of the same call, whose planes keep both halo rows
+    const int64_t sample_elems_max = (int64_t)g.cin * (g.h + 2 * g.ph) * p->rs + g.ph * p->rs + g.pw;
+    if (sample_elems_max * g.n * elem >= (1ll << 32) || I * g.n >= (1ll << 31)) return false;
     p->d_slots = make_fastdiv((uint32_t)p->chs);                    // reused as "divide by plane stride"
     ws->sample_elems = (int)sample_elems;
     int64_t nb = clg_ceil_div(I * g.n, 256 * 8);                   // about 8 cells per thread (4..64 measured within 10 %)
@@ -827,21 +833,22 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     ws->folded_off = ((size_t)g.c * 64 * 28 * elem + 255) & ~(size_t)255;   // partials sized for 64 blocks
     ws->taps_off = (ws->folded_off + (size_t)g.c * 28 * elem + 255) & ~(size_t)255;
     ws->xp_off = (ws->taps_off + (size_t)g.c * 8 * 4 + 255) & ~(size_t)255;
-    ws->total = ws->xp_off + (size_t)sample_elems * g.n * elem;
+    ws->total = ws->xp_off + (size_t)sample_elems_max * g.n * elem;
     return true;
 }
 
 // folded coefficients, per-channel kernel lists and tap offsets (for LDS rows of rs, planes of chs elements)
+// (and, in the same launch, a padded copy of x when `pad` names one)
 template <typename T>
 int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const void *w, const int32_t *sel, void *scratch,
-                   hipStream_t st)
+                   hipStream_t st, const PadJob<T> &pad)
 {
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     int32_t *count = reinterpret_cast<int32_t *>(base + lay.count_off), *hits = reinterpret_cast<int32_t *>(base + lay.hits_off);
     const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), list_blocks = lay.csr ? 0 : (int)clg_ceil_div(g.cin, 4);
-    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + list_blocks)), dim3(256), 0, st, (const T *)w, sel,
-                       reinterpret_cast<T *>(base), count, lay.csr ? nullptr : hits, reinterpret_cast<int32_t *>(base + lay.taps_off),
-                       g.c, g.cin, fold_blocks, rs, chs);
+    hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + list_blocks) + pad_blocks(pad)), dim3(256), 0, st,
+                       (const T *)w, sel, reinterpret_cast<T *>(base), count, lay.csr ? nullptr : hits,
+                       reinterpret_cast<int32_t *>(base + lay.taps_off), g.c, g.cin, fold_blocks, rs, chs, pad, fold_blocks + list_blocks);
     if (lay.csr) {
         int32_t *cursor = reinterpret_cast<int32_t *>(base + lay.cursor_off), *unsorted = reinterpret_cast<int32_t *>(base + lay.unsorted_off);
         const unsigned cb = (unsigned)clg_ceil_div(g.c, 256);
@@ -858,14 +865,14 @@ int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
 
 template <typename T>
 int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, const void *x, const void *w, const int32_t *sel,
-                            const uint8_t *argmax, void *gx, void *scratch, hipStream_t st)
+                            const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, const PadJob<T> &pad)
 {
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
     T *folded = reinterpret_cast<T *>(scratch);
     int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
     int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
     int32_t *taps = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.taps_off);
-    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st)) return e;
+    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, pad)) return e;
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
     T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
     T *out = p.hit_split > 1 ? part : (T *)gx;
@@ -914,13 +921,8 @@ int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems,
         shared->sample_elems = sample_elems;
         shared->p = p;
     }
-    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st)) return e;
-    TilePlan pp = p;
-    pp.d_slots = make_fastdiv((uint32_t)p.chs);                      // the pad kernel divides by the plane stride
-    const int64_t total = (int64_t)sample_elems * g.n;
-    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, pp,
-                       make_fastdiv((uint32_t)sample_elems), make_fastdiv((uint32_t)p.rs), sample_elems, total);
-    CLG_CHECK_LAUNCH("clg_convblock_backward_x(pad)");
+    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems)))
+        return e;
     if (int e = allow_lds(convblock_backward_x_direct_kernel<T>, p.lds_bytes, "clg_convblock_backward_x")) return e;
     const int64_t items = clg_ceil_div(g.n, p.G) * g.cin;
     hipLaunchKernelGGL(convblock_backward_x_direct_kernel<T>, dim3((unsigned)clg_ceil_div(items, p.NW)), dim3(p.NW * kWave),
@@ -940,13 +942,11 @@ int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &w
     T *folded = reinterpret_cast<T *>(base + ws.folded_off);
     int32_t *taps = reinterpret_cast<int32_t *>(base + ws.taps_off);
     T *xp = reinterpret_cast<T *>(base + ws.xp_off);
-    hipLaunchKernelGGL(convblock_w_prepare_kernel<T>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
-                       (const T *)w, sel, folded, taps, g.c, p.rs, p.chs);
+    const PadJob<T> job = make_pad_job((const T *)x, xp, g, p.rs, p.chs, ws.sample_elems);
+    const unsigned prep = (unsigned)clg_ceil_div((int64_t)g.c * 8, 256);
+    hipLaunchKernelGGL((convblock_w_prepare_kernel<T, T>), dim3(prep + pad_blocks(job)), dim3(256), 0, st, (const T *)w, sel, folded, taps,
+                       g.c, p.rs, p.chs, job, (int)prep);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(prepare)");
-    const int64_t total = (int64_t)ws.sample_elems * g.n;
-    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, p,
-                       make_fastdiv((uint32_t)ws.sample_elems), make_fastdiv((uint32_t)p.rs), ws.sample_elems, total);
-    CLG_CHECK_LAUNCH("clg_convblock_backward_w(pad)");
     const int I = (g.ho / 2) * (g.wo / 2);
     hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
                        (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p, make_fastdiv((uint32_t)I),
@@ -1021,9 +1021,32 @@ extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_c
     return (int64_t)lay.total;
 }
 
+// What the tiled input gradient sets up for a padded weight gradient that follows in the same call: its prepare launch
+// also writes the padded copy (planes of p.chs elements, the layout its tap offsets are made for) into the weight
+// gradient's scratch, so that one neither folds nor computes tap offsets nor pads again.
+template <typename T>
+PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void *scratch, void *w_scratch, SharedPad *shared)
+{
+    TilePlan pw;
+    WScratch ws;
+    const char *e_pad = getenv("CLG_BWDW_PADDED");
+    if (shared == nullptr || w_scratch == nullptr || p.bands != 1 || (e_pad && atoi(e_pad) == 0) || !plan_backward_w(g, (int)sizeof(T), &pw, &ws))
+        return no_pad_job<T>();
+    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    const int sample_elems = g.cin * p.chs + g.ph * p.rs + g.pw;
+    T *xp = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(w_scratch) + ws.xp_off);
+    shared->xp = xp;
+    shared->folded = base;
+    shared->taps = reinterpret_cast<const int32_t *>(base + lay.taps_off);
+    shared->sample_elems = sample_elems;
+    shared->p = pw;
+    return make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems);
+}
+
 static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch, void *stream,
-                                     SharedPad *shared)
+                                     SharedPad *shared, void *w_scratch = nullptr)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x")) return e;
@@ -1033,8 +1056,11 @@ static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const v
     const BwdXMode mode = choose_backward_x(g, elem_size(dtype), &p, &se);
     hipStream_t st = clg_stream(stream);
     if (mode == kBwdXTiled) {
-        if (dtype == CLG_F32) return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st);
-        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st);
+        if (dtype == CLG_F32)
+            return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
+                                                  share_from_tiled<float>(g, p, x, scratch, w_scratch, shared));
+        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
+                                               share_from_tiled<double>(g, p, x, scratch, w_scratch, shared));
     }
     if (mode == kBwdXDirect) {
         if (dtype == CLG_F32)
@@ -1045,9 +1071,9 @@ static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const v
     const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     if (dtype == CLG_F32) {
-        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st)) return e;
+        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>())) return e;
     } else {
-        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st)) return e;
+        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>())) return e;
     }
     return clg_convblock_backward_x_generic(dtype, g, grad_y, x, scratch, reinterpret_cast<const int32_t *>(base + lay.count_off),
                                             reinterpret_cast<const int32_t *>(base + lay.hits_off), selection, argmax, grad_x, st);
@@ -1116,9 +1142,9 @@ extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const 
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
     SharedPad shared;
-    if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared)) return e;
-    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w,
-                                     reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream, nullptr,
+    void *w_scratch = reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll);
+    if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared, w_scratch)) return e;
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w, w_scratch, stream, nullptr,
                                      "clg_convblock_backward", &shared);
 }
 
@@ -1130,9 +1156,10 @@ extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg,
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
     SharedPad shared;
+    void *w_scratch = reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll);
     if (grad_x != nullptr)
-        if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared)) return e;
-    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_logits,
-                                     reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll), stream, w,
+        if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared, w_scratch))
+            return e;
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_logits, w_scratch, stream, w,
                                      "clg_convblock_backward_logits", &shared);
 }

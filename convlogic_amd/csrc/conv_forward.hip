@@ -501,21 +501,14 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     int32_t *taps = reinterpret_cast<int32_t *>(base + d.taps_off);
     T *xp = reinterpret_cast<T *>(base + d.xp_off);
-    const void *kernel_params = params;
-    if (Ops::kParams > 1) {                                           // float: fold the probabilities once
-        hipLaunchKernelGGL(convblock_w_prepare_kernel<P>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
-                           (const P *)params, sel, reinterpret_cast<P *>(base), taps, g.c, d.p.rs, d.p.chs);
-        kernel_params = base;
-    } else {
-        hipLaunchKernelGGL(convblock_w_prepare_kernel<P>, dim3((unsigned)clg_ceil_div((int64_t)g.c * 8, 256)), dim3(256), 0, st,
-                           (const P *)nullptr, sel, (P *)nullptr, taps, g.c, d.p.rs, d.p.chs);
-    }
-    CLG_CHECK_LAUNCH(name);
-    TilePlan pp = d.p;
-    pp.d_slots = make_fastdiv((uint32_t)d.p.chs);                     // the pad kernel divides by the plane stride
-    const int64_t total = (int64_t)d.sample_elems * g.n;
-    hipLaunchKernelGGL(pad_image_kernel<T>, dim3((unsigned)clg_ceil_div(total, 256)), dim3(256), 0, st, (const T *)x, xp, g, pp,
-                       make_fastdiv((uint32_t)d.sample_elems), make_fastdiv((uint32_t)d.p.rs), d.sample_elems, total);
+    // one launch: folded coefficients (float gates only), tap offsets and the padded copy
+    const bool fold = Ops::kParams > 1;
+    const void *kernel_params = fold ? (const void *)base : params;
+    const PadJob<T> job = make_pad_job((const T *)x, xp, g, d.p.rs, d.p.chs, d.sample_elems);
+    const unsigned prep = (unsigned)clg_ceil_div((int64_t)g.c * 8, 256);
+    hipLaunchKernelGGL((convblock_w_prepare_kernel<P, T>), dim3(prep + pad_blocks(job)), dim3(256), 0, st,
+                       fold ? (const P *)params : (const P *)nullptr, sel, fold ? reinterpret_cast<P *>(base) : (P *)nullptr, taps, g.c,
+                       d.p.rs, d.p.chs, job, (int)prep);
     CLG_CHECK_LAUNCH(name);
     const int64_t sets = clg_ceil_div(g.n, d.p.G) * d.nblk;
     hipLaunchKernelGGL(convblock_forward_direct_kernel<Ops>, dim3((unsigned)clg_ceil_div(sets, 4), (unsigned)clg_ceil_div(g.c, d.p.CT)),
@@ -626,11 +619,11 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
     if (path == 4) {
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
-            hipLaunchKernelGGL(convblock_w_prepare_kernel<float>, pgrid, dim3(256), 0, st, (const float *)w, selection, (float *)scratch,
-                               (int32_t *)nullptr, g.c, 0, 0);
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
+                               (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
         else
-            hipLaunchKernelGGL(convblock_w_prepare_kernel<double>, pgrid, dim3(256), 0, st, (const double *)w, selection, (double *)scratch,
-                               (int32_t *)nullptr, g.c, 0, 0);
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
+                               (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
         CLG_CHECK_LAUNCH("clg_convblock_forward_ws");
         return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_ws");
     }

@@ -101,35 +101,66 @@ __device__ __forceinline__ T load_at(const T *__restrict__ base, uint32_t index)
 }
 
 // xp = zero-padded copy of x in the shared-halo layout: sample n at n * sample_elems, plane stride chs, row
-// stride rs, pixel (iy, ix) at (iy + ph) * rs + ix + pw.  p.d_slots must hold the divisor chs.
+// stride rs, pixel (iy, ix) at (iy + ph) * rs + ix + pw.  A job with total = 0 does nothing.
 template <typename T>
-__global__ __launch_bounds__(256) void pad_image_kernel(const T *__restrict__ x, T *__restrict__ xp, Geom g, TilePlan p,
-                                                      FastDiv d_sample, FastDiv d_rs, int sample_elems, int64_t total)
+struct PadJob {
+    const T *x;
+    T *xp;
+    Geom g;
+    FastDiv d_sample, d_chs, d_rs;
+    int chs, rs, sample_elems;
+    int64_t total;
+};
+template <typename T>
+__device__ __forceinline__ void pad_image_elem(const PadJob<T> &j, int64_t e)
 {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= total) return;
-    const uint32_t n = fdiv((uint32_t)e, d_sample), rem = (uint32_t)e - n * (uint32_t)sample_elems;
-    const uint32_t plane = fdiv(rem, p.d_slots), r2 = rem - plane * (uint32_t)p.chs;      // d_slots holds chs here
-    const uint32_t row = fdiv(r2, d_rs), col = r2 - row * (uint32_t)p.rs;
+    if (e >= j.total) return;
+    const uint32_t n = fdiv((uint32_t)e, j.d_sample), rem = (uint32_t)e - n * (uint32_t)j.sample_elems;
+    const uint32_t plane = fdiv(rem, j.d_chs), r2 = rem - plane * (uint32_t)j.chs;
+    const uint32_t row = fdiv(r2, j.d_rs), col = r2 - row * (uint32_t)j.rs;
     T v = T(0);
-    if (plane < (uint32_t)g.cin && row >= (uint32_t)g.ph && col >= (uint32_t)g.pw)
-        v = x[(((int64_t)n * g.cin + plane) * g.h + (row - g.ph)) * g.w + (col - g.pw)];
-    xp[e] = v;
+    if (plane < (uint32_t)j.g.cin && row - (uint32_t)j.g.ph < (uint32_t)j.g.h && col >= (uint32_t)j.g.pw)   // chs may hold more rows than h + ph
+        v = j.x[(((int64_t)n * j.g.cin + plane) * j.g.h + (row - j.g.ph)) * j.g.w + (col - j.g.pw)];
+    j.xp[e] = v;
 }
 
-// folded coefficients [c][28] and tap offsets [c][8] in the padded-image layout (either is skipped when null)
 template <typename T>
-__global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
-                                                                T *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
-                                                                int chs)
+static inline PadJob<T> make_pad_job(const T *x, T *xp, const Geom &g, int rs, int chs, int sample_elems)
 {
+    PadJob<T> j;
+    j.x = x, j.xp = xp, j.g = g, j.chs = chs, j.rs = rs, j.sample_elems = sample_elems;
+    j.d_sample = make_fastdiv((uint32_t)sample_elems), j.d_chs = make_fastdiv((uint32_t)chs), j.d_rs = make_fastdiv((uint32_t)rs);
+    j.total = (int64_t)sample_elems * g.n;
+    return j;
+}
+template <typename T>
+static inline PadJob<T> no_pad_job()
+{
+    PadJob<T> j = {};
+    j.total = 0;
+    return j;
+}
+template <typename T>
+static inline unsigned pad_blocks(const PadJob<T> &j) { return (unsigned)clg_ceil_div(j.total, 256); }
+
+// folded coefficients [c][28] and tap offsets [c][8] in the padded-image layout (either is skipped when null) in the
+// first blocks of the launch, the padded copy in the blocks from pad_block0 on: one launch sets a kernel up.
+template <typename P, typename T>
+__global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const P *__restrict__ w, const int32_t *__restrict__ sel,
+                                                                P *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
+                                                                int chs, PadJob<T> pad, int pad_block0)
+{
+    if ((int)blockIdx.x >= pad_block0) {
+        pad_image_elem(pad, (int64_t)(blockIdx.x - pad_block0) * 256 + threadIdx.x);
+        return;
+    }
     const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (taps != nullptr && q < (int64_t)C * 8) {
         const Tap tp = unpack_tap(sel[q]);
         taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
     }
     if (folded != nullptr && q < (int64_t)C * 7) {
-        const Coef<T> cf = fold16(w + q * 16);
+        const Coef<P> cf = fold16(w + q * 16);
         folded[q * 4 + 0] = cf.ab;
         folded[q * 4 + 1] = cf.a;
         folded[q * 4 + 2] = cf.b;
