@@ -81,22 +81,25 @@ __global__ __launch_bounds__(kBlk) void conv4_backward_w_kernel(const T *__restr
 
 // out[row*G + q][i] = sum_k COEF[k][i] * (sum_blk partial[row][blk][q*4 + k]): the gradient w.r.t. the gate
 // probabilities; with probs (the softmax output they came from) the gradient w.r.t. the logits instead.
+// The 16 lanes of a gate split the sum: lane i adds component i & 3 over the blocks blk = i >> 2 (mod 4), the four
+// stripes meet in a butterfly (same value in both partners), and every lane then holds the four totals.
 template <typename T>
-__global__ void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t rows, int nb, int G,
-                                            const T *__restrict__ probs)
+__global__ __launch_bounds__(256) void reduce_coef_partials_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t rows,
+                                                                 int nb, int G, const T *__restrict__ probs)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= rows * G * 16) return;
-    const int i = (int)(e % 16);
-    const int q = (int)((e / 16) % G);
-    const int64_t row = e / (16 * G);
-    T s[4] = {0, 0, 0, 0};
-    for (int blk = 0; blk < nb; ++blk) {
-        const T *p = partial + ((row * nb + blk) * G + q) * 4;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) s[k] += p[k];
-    }
-    T gi = coef_transpose_row<T>(i, s[0], s[1], s[2], s[3]);
+    const int i = threadIdx.x & 15;
+    const int64_t gate = e >> 4;                                     // row * G + q; a row of 16 lanes is live or dead as a whole
+    if (gate >= rows * G) return;
+    const int64_t row = gate / G;
+    const int q = (int)(gate - row * G);
+    const T *p = partial + (row * nb * G + q) * 4 + (i & 3);
+    T acc = 0;
+    for (int blk = i >> 2; blk < nb; blk += 4) acc += p[(int64_t)blk * G * 4];
+    acc += __shfl_xor(acc, 4, 16);
+    acc += __shfl_xor(acc, 8, 16);
+    const T s0 = __shfl(acc, 0, 16), s1 = __shfl(acc, 1, 16), s2 = __shfl(acc, 2, 16), s3 = __shfl(acc, 3, 16);
+    T gi = coef_transpose_row<T>(i, s0, s1, s2, s3);
     if (probs != nullptr) gi = softmax16_backward(gi, probs[e]);
     out[e] = gi;
 }
