@@ -17,7 +17,7 @@
 // parameters and tap offsets sit in scalar registers.
 #include <stdlib.h>
 
-#include "conv_tile.h"
+#include "conv_ops.h"
 
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
 int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const void *w, const int32_t *selection, void *y,
@@ -25,117 +25,10 @@ int clg_convblock_forward_generic(int dtype, const Geom &g, const void *x, const
 bool clg_convblock_is_4x4(const Geom &g);
 int clg_convblock_forward_4x4(int dtype, const Geom &g, const void *x, const void *folded, const int32_t *sel, void *y, uint8_t *argmax,
                               hipStream_t st, const char *name);
+int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_t *gates, const int32_t *sel, uint64_t *y, hipStream_t st,
+                                  const char *name);
 
 namespace {
-
-// ---- element policies ------------------------------------------------------------------------
-template <typename T>
-struct FloatOps {
-    using Elem = T;
-    static constexpr int kParams = 28;                               // LDS elements per kernel: 7 gates x (ab, a, b, one)
-    struct Params {
-        Tree<T> tr;
-    };
-    // params = gate probabilities [c_out, 7, 16]
-    static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
-                                                        int tid, int nthreads)
-    {
-        const T *w = reinterpret_cast<const T *>(params);
-        for (int q = tid; q < ct_cur * 7; q += nthreads) {
-            const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
-            dst[q * 4 + 0] = cf.ab;
-            dst[q * 4 + 1] = cf.a;
-            dst[q * 4 + 2] = cf.b;
-            dst[q * 4 + 3] = cf.one;
-        }
-    }
-    static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
-    {
-        Params pr;
-#pragma unroll
-        for (int k = 0; k < 7; ++k) {
-            pr.tr.g[k].ab = to_sgpr(src[(lc * 7 + k) * 4 + 0]);
-            pr.tr.g[k].a = to_sgpr(src[(lc * 7 + k) * 4 + 1]);
-            pr.tr.g[k].b = to_sgpr(src[(lc * 7 + k) * 4 + 2]);
-            pr.tr.g[k].one = to_sgpr(src[(lc * 7 + k) * 4 + 3]);
-        }
-        return pr;
-    }
-    // folded = [c_out][7][4] coefficients written by convblock_w_prepare_kernel
-    static __device__ __forceinline__ Params load_global(const void *__restrict__ folded, int c)
-    {
-        const T *fc = reinterpret_cast<const T *>(folded) + (int64_t)c * 28;
-        Params pr;
-#pragma unroll
-        for (int k = 0; k < 7; ++k) pr.tr.g[k] = Coef<T>{fc[4 * k], fc[4 * k + 1], fc[4 * k + 2], fc[4 * k + 3]};
-        return pr;
-    }
-    static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8]) { return eval_tree(pr.tr, v).root; }
-    // strict > in window order (0,0),(0,1),(1,0),(1,1): the first maximum wins
-    static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
-                                                      uint8_t *__restrict__ ab, int idx)
-    {
-        Elem best = r0;
-        int code = 0;
-        if (r0o > best) { best = r0o; code = 1; }
-        if (r1 > best) { best = r1; code = 2; }
-        if (r1o > best) { best = r1o; code = 3; }
-        yb[idx] = best;
-        ab[idx] = (uint8_t)code;
-    }
-};
-
-struct BitOps {
-    using Elem = uint64_t;
-    static constexpr int kParams = 1;                                // 7 gate ids, 4 bits each
-    struct Params {
-        Masks m[7];
-    };
-    // params = gate ids uint8 [c_out, 7]
-    static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
-                                                        int tid, int nthreads)
-    {
-        const uint8_t *gid = reinterpret_cast<const uint8_t *>(params);
-        for (int q = tid; q < ct_cur; q += nthreads) {
-            uint64_t pk = 0;
-            for (int k = 0; k < 7; ++k) pk |= (uint64_t)(gid[((int64_t)c0 + q) * 7 + k] & 15) << (4 * k);
-            dst[q] = pk;
-        }
-    }
-    static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
-    {
-        const uint32_t pk = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src[lc]);
-        Params pr;
-#pragma unroll
-        for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks((pk >> (4 * k)) & 15);
-        return pr;
-    }
-    static __device__ __forceinline__ Params load_global(const void *__restrict__ gates, int c)
-    {
-        const uint8_t *gid = reinterpret_cast<const uint8_t *>(gates) + (int64_t)c * 7;
-        Params pr;
-#pragma unroll
-        for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks(gid[k] & 15);
-        return pr;
-    }
-    static __device__ __forceinline__ Elem gate64(const Masks &m, Elem a, Elem b)
-    {
-        const uint32_t lo = gate_bits(m, (uint32_t)a, (uint32_t)b), hi = gate_bits(m, (uint32_t)(a >> 32), (uint32_t)(b >> 32));
-        return ((uint64_t)hi << 32) | lo;
-    }
-    static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8])
-    {
-        Elem leaf[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) leaf[q] = gate64(pr.m[q], v[2 * q], v[2 * q + 1]);
-        return gate64(pr.m[6], gate64(pr.m[4], leaf[0], leaf[1]), gate64(pr.m[5], leaf[2], leaf[3]));
-    }
-    static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
-                                                      uint8_t *__restrict__, int idx)
-    {
-        yb[idx] = (r0 | r0o) | (r1 | r1o);
-    }
-};
 
 // ---- kernel ------------------------------------------------------------------------------------
 // ROWSTEP: elements between conv rows 2r and 2r+1 in the LDS image when known at compile time (the
@@ -584,6 +477,9 @@ extern "C" int clg_convblock_eval_packed(const clg_conv_geom *gg, const uint64_t
     CLG_REQUIRE(x != y, "clg_convblock_eval_packed: x and y must not overlap");
     TilePlan p;
     hipStream_t st = clg_stream(stream);
+    const char *e_4x4 = getenv("CLG_FWD_4X4");
+    if (clg_convblock_is_4x4(g) && (!e_4x4 || atoi(e_4x4) != 0))
+        return clg_convblock_eval_packed_4x4(g, x, gates, selection, y, st, "clg_convblock_eval_packed");
     if (plan_forward(g, 8, BitOps::kParams, &p))
         return launch_forward_tiled<BitOps>(g, p, x, gates, selection, y, nullptr, st, "clg_convblock_eval_packed");
     const int64_t blocks = clg_ceil_div((int64_t)g.n * (g.ho / 2) * (g.wo / 2), 256);

@@ -1,4 +1,5 @@
-// Fused conv-logic block on 4x4 images (3x3 kernel, stride 1, padding 1), one sample per lane.
+// Fused conv-logic block on 4x4 images (3x3 kernel, stride 1, padding 1), one sample per lane -- or, for packed
+// words, one group of 64 samples per lane (element policies of conv_ops.h).
 //
 // The last block of a network sees many channels and tiny images: a whole input plane is 16 elements, so the
 // kernels that give a workgroup an image (or a padded copy of it) spend their time in set-up, staging and barriers
@@ -8,7 +9,7 @@
 // once and stays zero), a plane arrives as four 16-byte loads per lane that are requested one kernel ahead, and the
 // 16 positions x 8 taps are LDS reads at (tap address + immediate position offset).  No barriers, no bounds checks.
 // A kernel whose taps name more than two channels (possible with a caller-made selection) reads global memory.
-#include "conv_tile.h"
+#include "conv_ops.h"
 
 namespace {
 
@@ -48,18 +49,14 @@ struct Planes {
 template <typename T>
 __device__ __forceinline__ void load_plane(T (&dst)[32], int at, const T *__restrict__ p)
 {
-    if constexpr (sizeof(T) == 4) {
+    constexpr int PER = 16 / (int)sizeof(T);                       // elements per 16-byte load
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 f = reinterpret_cast<const float4 *>(p)[q];
-            dst[at + 4 * q] = f.x, dst[at + 4 * q + 1] = f.y, dst[at + 4 * q + 2] = f.z, dst[at + 4 * q + 3] = f.w;
-        }
-    } else {
+    for (int q = 0; q < 16 / PER; ++q) {
+        const u32x4 raw = reinterpret_cast<const u32x4 *>(p)[q];
+        T part[PER];
+        __builtin_memcpy(part, &raw, 16);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const double2 f = reinterpret_cast<const double2 *>(p)[q];
-            dst[at + 2 * q] = f.x, dst[at + 2 * q + 1] = f.y;
-        }
+        for (int e = 0; e < PER; ++e) dst[at + q * PER + e] = part[e];
     }
 }
 
@@ -73,11 +70,15 @@ __device__ __forceinline__ void fetch_planes(Planes<T> &pl, const LaneTaps &tp, 
 }
 
 // grid: (64-sample blocks, kernel tiles of ct kernels); LDS: kLsWaves * 64 * kLsStride elements.
-template <typename T>
-__global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(const T *__restrict__ x, const T *__restrict__ folded,
-                                                                              const int32_t *__restrict__ sel, T *__restrict__ y,
+// params: folded coefficients [c][28] (float gates) or gate ids uint8 [c][7] (packed words, argmax = null)
+template <typename Ops>
+__global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(const typename Ops::Elem *__restrict__ x,
+                                                                              const void *__restrict__ params,
+                                                                              const int32_t *__restrict__ sel,
+                                                                              typename Ops::Elem *__restrict__ y,
                                                                               uint8_t *__restrict__ argmax, Geom g, int ct)
 {
+    using T = typename Ops::Elem;
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
     T *mine = reinterpret_cast<T *>(smem) + ((size_t)wave * kWave + lane) * kLsStride;
@@ -101,10 +102,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
                 for (int e = 0; e < 16; ++e) mine[kLsPlane + ((e >> 2) + 1) * 6 + (e & 3) + 1] = pl.v[16 + e];
             }
         }
-        Tree<T> tr;
-        const T *fc = folded + (int64_t)c * 28;
-#pragma unroll
-        for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+        const typename Ops::Params pr = Ops::load_global(params, c);
         const LaneTaps cur = tp;
         const int cn = c + kLsWaves;
         const bool more = cn < c1;
@@ -119,7 +117,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
         int codes = 0;
 #pragma unroll
         for (int cell = 0; cell < 4; ++cell) {
-            int code = 0;
+            T r[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int oy = 2 * (cell >> 1) + (q >> 1), ox = 2 * (cell & 1) + (q & 1);
@@ -135,23 +133,22 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
                         if ((unsigned)iy < 4u && (unsigned)ix < 4u && live) v[k] = xn[cur.ch[k] * 16 + iy * 4 + ix];
                     }
                 }
-                const T r = eval_tree(tr, v).root;
-                if (q == 0 || r > best[cell]) {                       // strict >: the first maximum wins
-                    best[cell] = r;
-                    code = q;
-                }
+                r[q] = Ops::root(pr, v);
             }
+            int code;
+            best[cell] = Ops::pool4(r, code);
             codes |= code << (8 * cell);
         }
         if (live) {
             const int64_t o = (n * g.c + c) * 4;
-            if constexpr (sizeof(T) == 4) {
-                *reinterpret_cast<float4 *>(y + o) = make_float4(best[0], best[1], best[2], best[3]);
-            } else {
-                *reinterpret_cast<double2 *>(y + o) = make_double2(best[0], best[1]);
-                *reinterpret_cast<double2 *>(y + o + 2) = make_double2(best[2], best[3]);
+            constexpr int PER = 16 / (int)sizeof(T);
+#pragma unroll
+            for (int q = 0; q < 4 / PER; ++q) {
+                u32x4 raw;
+                __builtin_memcpy(&raw, &best[q * PER], 16);
+                reinterpret_cast<u32x4 *>(y + o)[q] = raw;
             }
-            *reinterpret_cast<uint32_t *>(argmax + o) = (uint32_t)codes;
+            if (argmax != nullptr) *reinterpret_cast<uint32_t *>(argmax + o) = (uint32_t)codes;
         }
         if (!more) break;
         c = cn;
@@ -160,31 +157,40 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
 
 }  // namespace
 
-// The shapes this file covers: what the last block of a 32x32-input network sees.
+// The shapes this file covers: what the last block of a 32x32-input network sees (n counts 64-sample groups for packed words).
 bool clg_convblock_is_4x4(const Geom &g)
 {
     return g.h == 4 && g.w == 4 && g.kh == 3 && g.kw == 3 && g.sh == 1 && g.sw == 1 && g.ph == 1 && g.pw == 1 && g.n >= 32;
+}
+
+template <typename Ops>
+static int launch_4x4(const Geom &g, const void *x, const void *params, const int32_t *sel, void *y, uint8_t *argmax, hipStream_t st,
+                      const char *name)
+{
+    using T = typename Ops::Elem;
+    const int sblocks = (g.n + kWave - 1) / kWave;
+    int ct = 64;                                                      // 16 kernels per wavefront unless that starves the chip
+    while (ct > kLsWaves && (int64_t)sblocks * ((g.c + ct - 1) / ct) < 1024) ct >>= 1;
+    CLG_REQUIRE((g.c + ct - 1) / ct <= 65535, "%s: too many kernels for one launch (%d)", name, g.c);
+    const dim3 grid((unsigned)sblocks, (unsigned)((g.c + ct - 1) / ct)), block(kLsWaves * kWave);
+    const size_t lds = (size_t)kLsWaves * kWave * kLsStride * sizeof(T);
+    if (int e = allow_lds(convblock_forward_4x4_kernel<Ops>, lds, name)) return e;
+    hipLaunchKernelGGL(convblock_forward_4x4_kernel<Ops>, grid, block, lds, st, (const T *)x, params, sel, (T *)y, argmax, g, ct);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
 }
 
 // folded: [c][28] coefficients (convblock_w_prepare_kernel).
 int clg_convblock_forward_4x4(int dtype, const Geom &g, const void *x, const void *folded, const int32_t *sel, void *y, uint8_t *argmax,
                               hipStream_t st, const char *name)
 {
-    const int sblocks = (g.n + kWave - 1) / kWave;
-    int ct = 64;                                                      // 16 kernels per wavefront unless that starves the chip
-    while (ct > kLsWaves && (int64_t)sblocks * ((g.c + ct - 1) / ct) < 1024) ct >>= 1;
-    CLG_REQUIRE((g.c + ct - 1) / ct <= 65535, "%s: too many kernels for one launch (%d)", name, g.c);
-    const dim3 grid((unsigned)sblocks, (unsigned)((g.c + ct - 1) / ct)), block(kLsWaves * kWave);
-    const size_t lds = (size_t)kLsWaves * kWave * kLsStride * (dtype == CLG_F64 ? 8 : 4);
-    if (dtype == CLG_F32) {
-        if (int e = allow_lds(convblock_forward_4x4_kernel<float>, lds, name)) return e;
-        hipLaunchKernelGGL(convblock_forward_4x4_kernel<float>, grid, block, lds, st, (const float *)x, (const float *)folded, sel,
-                           (float *)y, argmax, g, ct);
-    } else {
-        if (int e = allow_lds(convblock_forward_4x4_kernel<double>, lds, name)) return e;
-        hipLaunchKernelGGL(convblock_forward_4x4_kernel<double>, grid, block, lds, st, (const double *)x, (const double *)folded, sel,
-                           (double *)y, argmax, g, ct);
-    }
-    CLG_CHECK_LAUNCH(name);
-    return CLG_OK;
+    if (dtype == CLG_F32) return launch_4x4<FloatOps<float>>(g, x, folded, sel, y, argmax, st, name);
+    return launch_4x4<FloatOps<double>>(g, x, folded, sel, y, argmax, st, name);
+}
+
+// gates: uint8 [c][7] gate ids; x, y: 64 samples per word.
+int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_t *gates, const int32_t *sel, uint64_t *y, hipStream_t st,
+                                  const char *name)
+{
+    return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
 }

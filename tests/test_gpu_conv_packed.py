@@ -137,3 +137,30 @@ def test_packed_block_errors():
         convlogic_hip.full_convlogic_eval_packed(x, gates[:, :4].contiguous(), layer.selection, 1, 1, 1, 1, 3, 3)
     with pytest.raises(RuntimeError, match="divisible by 2"):
         convlogic_hip.full_convlogic_eval_packed(x[:, :, :7].contiguous(), gates, layer.selection, 1, 1, 1, 1, 3, 3)
+
+
+@pytest.mark.parametrize("samples,cin,cout", [(2048, 6, 9), (2100, 24, 40), (4160, 16, 33)])
+def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
+    # from 32 word groups on, 4x4 images take the kernel that gives every lane one group of 64 samples: against the
+    # numpy oracle (bit-exact), against the staged kernel, with a ragged last wavefront and last word, and with
+    # kernels that read more than two channels
+    torch.manual_seed(samples + cin)
+    ch = torch.randint(0, cin, (cout, 2))
+    pick = torch.randint(0, 2, (cout, 8))
+    chan = torch.gather(ch, 1, pick)
+    chan[1] = torch.arange(8) % cin                                  # up to eight channels
+    chan[cout - 1, 5] = (chan[cout - 1, 0] + 1) % cin
+    chan[cout - 1, 6] = (chan[cout - 1, 0] + 2) % cin
+    sel = ((chan << 16) | (torch.randint(0, 3, (cout, 8)) << 8) | torch.randint(0, 3, (cout, 8))).to(torch.int32)
+    layer = _layer(cin, cout, 1, 1, 3, seed=3, selection=sel.to(DEV))
+    bits = torch.randint(0, 2, (samples, cin, 4, 4), device=DEV).bool()
+    gates = layer.weights.argmax(-1).to(torch.uint8)
+    words, pad = O.pack_image(bits.cpu().numpy())
+    want = O.conv_block_eval_packed(words, gates.cpu().numpy(), sel.numpy(), (1, 1), (1, 1), (3, 3))
+    p = layer(C.PackBitsTensor(bits, 64))
+    assert p.pad_len == pad and np.array_equal(p.t.cpu().numpy(), want)
+    x_words = torch.from_numpy(words).to(DEV)
+    monkeypatch.setenv("CLG_FWD_4X4", "0")
+    staged = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
+    monkeypatch.delenv("CLG_FWD_4X4")
+    assert torch.equal(staged, p.t)
