@@ -85,10 +85,12 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
         }
     }
     const int U = s_cur * p.slots;
+    const int rows_per_slot = p.one_row ? 1 : 2;                     // conv rows a lane slot covers
     for (int u = tid; u < U; u += nthreads) {
         const uint32_t s = fdiv(u, p.d_slots), r = u - s * (uint32_t)p.slots;
-        const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
-        slot[u] = make_int2((int)(s * p.planes * p.chs + (2 * rp * g.sh) * p.rs + ox * g.sw), (int)((s * g.c) * I + rp * wp + (ox >> 1)));
+        const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;        // rp: row pair, or row with one_row
+        const uint32_t oy = rp * rows_per_slot;
+        slot[u] = make_int2((int)(s * p.planes * p.chs + (oy * g.sh) * p.rs + ox * g.sw), (int)((s * g.c) * I + (oy >> 1) * wp + (ox >> 1)));
     }
     __syncthreads();
     {
@@ -122,6 +124,8 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     __syncthreads();
 
     const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
+    // lanes that pool and write: even columns, and with one position per lane even rows only
+    const bool writer_lane = !(lane & 1) && !(p.one_row && ((lane / g.wo) & 1));
     // work items = (kernel, block of 64 slots), kernel-major; every wavefront takes a contiguous range, so
     // the scalar parameters are reloaded only when its range crosses into the next kernel
     const int nblk = (U + kWave - 1) / kWave;
@@ -143,29 +147,41 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
             const bool valid = u < U;
             const int2 e = slot[valid ? u : 0];
             T v[8];
-            T r0, r1;
+            T r0, r1 = T(0);
             if (!from_global) {
 #pragma unroll
                 for (int t = 0; t < 8; ++t) v[t] = xs[e.x + to[t]];
                 r0 = Ops::root(pr, v);
+                if (!p.one_row) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
-                r1 = Ops::root(pr, v);
+                    for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
+                    r1 = Ops::root(pr, v);
+                }
             } else {
                 const uint32_t uu = valid ? u : 0;
                 const uint32_t s = fdiv(uu, p.d_slots), r = uu - s * (uint32_t)p.slots;
                 const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;
+                const uint32_t oy = rp * rows_per_slot;
                 const T *xn = x + (int64_t)(n0 + s) * g.cin * hw;
                 const int32_t *sq = sel + ((int64_t)c0 + lc) * 8;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(2 * rp), (int)ox);
+                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)oy, (int)ox);
                 r0 = Ops::root(pr, v);
+                if (!p.one_row) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(2 * rp + 1), (int)ox);
-                r1 = Ops::root(pr, v);
+                    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(oy + 1), (int)ox);
+                    r1 = Ops::root(pr, v);
+                }
             }
-            const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
-            if (valid && !(lane & 1)) Ops::pool_store(r0, r0o, r1, r1o, yb, ab, e.y);
+            const T r0o = dpp_xor1(r0);
+            T r1o;
+            if (p.one_row) {                                          // the row below sits wo lanes up (2 wo divides 64)
+                r1 = lane_up(r0, g.wo);
+                r1o = lane_up(r0o, g.wo);
+            } else {
+                r1o = dpp_xor1(r1);
+            }
+            if (valid && writer_lane) Ops::pool_store(r0, r0o, r1, r1o, yb, ab, e.y);
         }
         blk = 0;
         ++lc;
@@ -313,6 +329,15 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     if (const char *e = getenv("CLG_FWD_CT")) p->CT = atoi(e) < g.c ? atoi(e) : g.c;
     if (const char *e = getenv("CLG_FWD_NW")) p->NW = atoi(e);
     if (p->S < 1 || p->CT < 1 || p->NW < 1 || p->NW > 16) return false;
+    // A workgroup whose samples fill at most half a wavefront with (row pair, column) slots gives every conv position
+    // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64).
+    p->one_row = 0;
+    if ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
+    if (const char *e = getenv("CLG_FWD_ONE_ROW")) p->one_row = p->one_row && atoi(e) != 0;
+    if (p->one_row) {
+        p->slots = g.ho * g.wo;
+        p->d_slots = make_fastdiv((uint32_t)p->slots);
+    }
     for (;;) {
         p->planes = subset ? 2 * p->CT : g.cin;
         p->xe = (int)((int64_t)p->S * p->planes * p->chs + tail);

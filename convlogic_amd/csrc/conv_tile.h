@@ -35,6 +35,7 @@ struct TilePlan {
     int64_t part_stride;   // input gradient: elements between partial images (0 when hit_split == 1)
     int planes;            // forward: LDS planes per sample (all input channels, or 2 per kernel of the tile)
     int subset;            // forward: 1 = only the channels the kernel tile reads are staged
+    int one_row;           // forward: 1 = a lane slot is one conv position (ho * wo per sample) instead of a column of two rows
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp, d_planes;
     size_t lds_bytes;
 };
@@ -48,6 +49,21 @@ __device__ __forceinline__ T dpp_xor1(T v)
         const uint64_t u = __builtin_bit_cast(uint64_t, v);
         const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, false);
         const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, false);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+// value of the lane `delta` lanes up (ds_bpermute)
+template <typename T>
+__device__ __forceinline__ T lane_up(T v, int delta)
+{
+    const int src = (int)((threadIdx.x & 63) + delta) << 2;
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)u);
+        const uint32_t hi = __builtin_amdgcn_ds_bpermute(src, (int)(uint32_t)(u >> 32));
         return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
     }
 }
@@ -70,6 +86,7 @@ static inline void plan_common(const Geom &g, TilePlan *p)
 {
     p->rs = g.w + g.pw;
     p->chs = (g.h + g.ph) * p->rs;
+    p->one_row = 0;
     p->d_hw = make_fastdiv((uint32_t)(g.h * g.w));
     p->d_w = make_fastdiv((uint32_t)g.w);
     p->d_wo = make_fastdiv((uint32_t)g.wo);

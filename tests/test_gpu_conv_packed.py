@@ -164,3 +164,27 @@ def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
     staged = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
     monkeypatch.delenv("CLG_FWD_4X4")
     assert torch.equal(staged, p.t)
+
+
+@pytest.mark.parametrize("n,cin,cout,hw", [(70, 128, 24, 8), (5, 6, 9, 4), (33, 40, 16, 2), (3, 3, 8, 16)])
+def test_one_position_per_lane_equals_two_rows_per_lane(n, cin, cout, hw, monkeypatch):
+    # workgroups whose samples fill at most half a wavefront with (row pair, column) slots give every conv position
+    # its own lane and pool across lanes; same bits and same float values (pooling choice included) as the default
+    # mapping, and the packed result against the oracle
+    monkeypatch.setenv("CLG_FWD_4X4", "0")
+    layer = _layer(cin, cout, 1, 1, 3, seed=n)
+    bits = torch.randint(0, 2, (n * 64, cin, hw, hw), device=DEV).bool() if n <= 5 else torch.randint(0, 2, (n, cin, hw, hw), device=DEV).bool()
+    gates = layer.weights.argmax(-1).to(torch.uint8)
+    words, pad = O.pack_image(bits.cpu().numpy())
+    x_words = torch.from_numpy(words).to(DEV)
+    x = torch.rand(n, cin, hw, hw, device=DEV)
+    wp = torch.softmax(layer.weights.detach(), -1)
+    got = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("CLG_FWD_ONE_ROW", mode)
+        got[mode] = (convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3),
+                     *convlogic_hip.full_convlogic_forward(x, wp, layer.selection, 1, 1, 1, 1, 3, 3))
+    for a, b in zip(got["1"], got["0"]):
+        assert torch.equal(a, b)
+    want = O.conv_block_eval_packed(words, gates.cpu().numpy(), layer.selection.cpu().numpy(), (1, 1), (1, 1), (3, 3))
+    assert np.array_equal(got["1"][0].cpu().numpy(), want)
