@@ -36,6 +36,11 @@ int clg_convblock_backward_w_generic(int dtype, const Geom &g, const void *grad_
                                      const int32_t *selection, const uint8_t *argmax, void *grad_w, void *scratch,
                                      hipStream_t st, const void *probs);
 int clg_convblock_partial_blocks(const Geom &g);
+bool clg_convblock_is_4x4(const Geom &g);
+size_t clg_convblock_backward_4x4_tg_bytes(int dtype, const Geom &g);
+int clg_convblock_backward_4x4(int dtype, const Geom &g, const void *x, const void *folded, const int32_t *sel, const void *gy,
+                               const uint8_t *argmax, void *tg, void *gw, const void *probs, const int32_t *count, const int32_t *hits,
+                               void *gx, hipStream_t st, const char *name);
 int clg_launch_reduce_coef(int dtype, const void *partial, void *out, int64_t rows, int nb, int G, hipStream_t st, const char *name,
                            const void *probs);
 
@@ -1127,11 +1132,44 @@ extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, cons
                                      "clg_convblock_backward_w");
 }
 
+// 4x4 images with one sample per lane (conv_small.hip): scratch = prepare tables | tap gradients
+static bool backward_4x4_wanted(const Geom &g)
+{
+    const char *e = getenv("CLG_BWD_4X4");
+    return clg_convblock_is_4x4(g) && g.c <= 65535 && (!e || atoi(e) != 0);
+}
+static size_t backward_4x4_tg_off(const Geom &g, int dtype) { return (bwd_scratch_layout(g, elem_size(dtype), 1).total + 255) & ~(size_t)255; }
+
+static int convblock_backward_4x4(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w, const int32_t *selection,
+                                  const uint8_t *argmax, void *grad_x, void *grad_w, void *scratch, void *stream, const void *probs,
+                                  const char *name)
+{
+    CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "%s: null pointer argument", name);
+    const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) {
+        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>())) return e;
+    } else {
+        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>())) return e;
+    }
+    return clg_convblock_backward_4x4(dtype, g, x, base, selection, grad_y, argmax, base + backward_4x4_tg_off(g, dtype), grad_w, probs,
+                                      reinterpret_cast<const int32_t *>(base + lay.count_off),
+                                      reinterpret_cast<const int32_t *>(base + lay.hits_off), grad_x, st, name);
+}
+
 extern "C" int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *gg)
 {
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg), b = clg_convblock_backward_w_scratch_bytes(dtype, gg);
     if (a < 0 || b < 0) return -1;
-    return ((a + 255) & ~255ll) + b;
+    int64_t total = ((a + 255) & ~255ll) + b;
+    Geom g;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_scratch_bytes")) return -1;
+    if (backward_4x4_wanted(g)) {
+        const int64_t small = (int64_t)(backward_4x4_tg_off(g, dtype) + clg_convblock_backward_4x4_tg_bytes(dtype, g));
+        if (small > total) total = small;
+    }
+    return total;
 }
 
 extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -1139,6 +1177,15 @@ extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const 
                                       void *stream)
 {
     CLG_REQUIRE(scratch, "clg_convblock_backward: null pointer argument");
+    {
+        Geom g;
+        if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward")) return e;
+        if (backward_4x4_wanted(g)) {
+            CLG_REQUIRE(grad_x, "clg_convblock_backward: null pointer argument");
+            return convblock_backward_4x4(dtype, g, grad_y, x, w, selection, argmax, grad_x, grad_w, scratch, stream, nullptr,
+                                          "clg_convblock_backward");
+        }
+    }
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
     SharedPad shared;
@@ -1153,6 +1200,13 @@ extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg,
                                              void *scratch, void *stream)
 {
     CLG_REQUIRE(scratch, "clg_convblock_backward_logits: null pointer argument");
+    {
+        Geom g;
+        if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_logits")) return e;
+        if (backward_4x4_wanted(g))
+            return convblock_backward_4x4(dtype, g, grad_y, x, w, selection, argmax, grad_x, grad_logits, scratch, stream, w,
+                                          "clg_convblock_backward_logits");
+    }
     const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
     if (a < 0) return CLG_EINVAL;
     SharedPad shared;

@@ -155,6 +155,238 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
     }
 }
 
+// ---- gradients ---------------------------------------------------------------------------------
+// Two passes, both with one sample per lane and no atomics:
+//   convblock_backward_4x4_kernel      kernel-major, same plane staging as the forward: evaluates the tree at the
+//                                      pooled arg-max position of the 4 cells once, accumulates the 28 weight-gradient
+//                                      sums of its kernel over all samples (registers, then DPP and a fixed-order
+//                                      combine of the 4 wavefronts) and writes the 4 x 8 tap gradients of every
+//                                      (kernel, sample) to tg[c][n][cell][tap] (and its 4 arg-max codes to tcodes[c][n]);
+//   convblock_backward_x_4x4_kernel    channel-major: a lane owns the gradient plane of (sample, channel) in its LDS
+//                                      slice and adds the tap gradients of the kernels that read the channel, in
+//                                      increasing kernel order, taps in order -- a fixed summation order.
+// The tree and its derivatives are evaluated once per (kernel, sample, cell) for both gradients.
+
+constexpr int kGradStride = kLsPlane + 1;          // gradient plane: padded 6x6 (taps of border cells fall into the halo)
+
+template <typename T>
+__global__ __launch_bounds__(kLsWaves *kWave) void convblock_backward_4x4_kernel(
+    const T *__restrict__ x, const T *__restrict__ folded, const int32_t *__restrict__ sel, const T *__restrict__ gy,
+    const uint8_t *__restrict__ argmax, T *__restrict__ tg, uint32_t *__restrict__ tcodes, T *__restrict__ gw,
+    const T *__restrict__ probs, Geom g, int ct)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ T meet[kLsWaves][28];
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    T *mine = reinterpret_cast<T *>(smem) + ((size_t)wave * kWave + lane) * kLsStride;
+#pragma unroll
+    for (int e = 0; e < kLsStride; ++e) mine[e] = T(0);
+    const int sblocks = (g.n + kWave - 1) / kWave;
+    const int c0 = blockIdx.x * ct, c1 = min(g.c, c0 + ct);
+    for (int c = c0; c < c1; ++c) {
+        const LaneTaps tp = lane_taps(sel, c);
+        Tree<T> tr;
+        const T *fc = folded + (int64_t)c * 28;
+#pragma unroll
+        for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+        const T *ta[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ta[k] = mine + (tp.ch[k] != tp.ch0 ? kLsPlane : 0) + tp.ry[k] * 6 + tp.rx[k];
+        T acc[28];
+#pragma unroll
+        for (int k = 0; k < 28; ++k) acc[k] = T(0);
+        // the wavefronts of the workgroup deal the 64-sample blocks among themselves; planes one block ahead
+        int sb = wave;
+        Planes<T> pl;
+        {
+            const int64_t n = (int64_t)sb * kWave + lane;
+            if (sb < sblocks) fetch_planes(pl, tp, x + (n < g.n ? n : 0) * g.cin * 16, n < g.n);
+        }
+        for (; sb < sblocks; sb += kLsWaves) {
+            const int64_t n = (int64_t)sb * kWave + lane;
+            const bool live = n < g.n;
+            const T *xn = x + (live ? n : 0) * g.cin * 16;
+            if (!tp.wide) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mine[((e >> 2) + 1) * 6 + (e & 3) + 1] = live ? pl.v[e] : T(0);
+                if (tp.ch1 != tp.ch0) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) mine[kLsPlane + ((e >> 2) + 1) * 6 + (e & 3) + 1] = live ? pl.v[16 + e] : T(0);
+                }
+            }
+            const int64_t o = (n * g.c + c) * 4;
+            T gout[4] = {T(0), T(0), T(0), T(0)};
+            uint32_t codes = 0;
+            if (live) {
+#pragma unroll
+                for (int cell = 0; cell < 4; ++cell) gout[cell] = gy[o + cell];
+                codes = *reinterpret_cast<const uint32_t *>(argmax + o);
+            }
+            {
+                const int sn = sb + kLsWaves;                          // next block's planes, in flight during the cells
+                const int64_t nn = (int64_t)sn * kWave + lane;
+                if (sn < sblocks) fetch_planes(pl, tp, x + (nn < g.n ? nn : 0) * g.cin * 16, nn < g.n);
+            }
+            T gt[32];
+#pragma unroll
+            for (int cell = 0; cell < 4; ++cell) {
+                const int code = (codes >> (8 * cell)) & 3;
+                const int oy = 2 * (cell >> 1) + (code >> 1), ox = 2 * (cell & 1) + (code & 1);
+                T v[8];
+                if (!tp.wide) {
+                    const int po = oy * 6 + ox;                        // per lane: the pooled maximum's position
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) v[k] = ta[k][po];
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const int iy = oy + tp.ry[k] - 1, ix = ox + tp.rx[k] - 1;
+                        v[k] = T(0);
+                        if ((unsigned)iy < 4u && (unsigned)ix < 4u && live) v[k] = xn[tp.ch[k] * 16 + iy * 4 + ix];
+                    }
+                }
+                const TreeVals<T> tv = eval_tree(tr, v);
+                const T go = gout[cell];                               // 0 for lanes without a sample
+                const T g_m[2] = {go * gate_da(tr.g[6], tv.mid[1]), go * gate_db(tr.g[6], tv.mid[0])};
+                T g_l[4];
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    g_l[2 * m] = g_m[m] * gate_da(tr.g[4 + m], tv.leaf[2 * m + 1]);
+                    g_l[2 * m + 1] = g_m[m] * gate_db(tr.g[4 + m], tv.leaf[2 * m]);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    gt[cell * 8 + 2 * q] = g_l[q] * gate_da(tr.g[q], v[2 * q + 1]);
+                    gt[cell * 8 + 2 * q + 1] = g_l[q] * gate_db(tr.g[q], v[2 * q]);
+                }
+                // weight-gradient sums: (g a b, g a, g b, g) per gate
+                auto add = [&](int q, T gg, T a, T b) {
+                    acc[4 * q] = fma_t(gg, a * b, acc[4 * q]);
+                    acc[4 * q + 1] = fma_t(gg, a, acc[4 * q + 1]);
+                    acc[4 * q + 2] = fma_t(gg, b, acc[4 * q + 2]);
+                    acc[4 * q + 3] += gg;
+                };
+#pragma unroll
+                for (int q = 0; q < 4; ++q) add(q, g_l[q], v[2 * q], v[2 * q + 1]);
+                add(4, g_m[0], tv.leaf[0], tv.leaf[1]);
+                add(5, g_m[1], tv.leaf[2], tv.leaf[3]);
+                add(6, go, tv.mid[0], tv.mid[1]);
+            }
+            if (tg != nullptr && live) {
+                T *dst = tg + ((int64_t)c * g.n + n) * 32;
+                tcodes[(int64_t)c * g.n + n] = codes;                  // kernel-major copy: the second pass reads it coalesced
+                constexpr int PER = 16 / (int)sizeof(T);
+#pragma unroll
+                for (int q = 0; q < 32 / PER; ++q) {
+                    u32x4 raw;
+                    __builtin_memcpy(&raw, &gt[q * PER], 16);
+                    reinterpret_cast<u32x4 *>(dst)[q] = raw;
+                }
+            }
+        }
+        // 28 sums of this kernel: lanes, then the wavefronts in order
+#pragma unroll
+        for (int k = 0; k < 28; ++k) {
+            const T t = wave_sum(acc[k]);
+            if (lane == 0) meet[wave][k] = t;
+        }
+        __syncthreads();
+        if (threadIdx.x < 7 * 16) {
+            const int q = threadIdx.x >> 4, i = threadIdx.x & 15;
+            T sums[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) sums[k] = (meet[0][4 * q + k] + meet[1][4 * q + k]) + (meet[2][4 * q + k] + meet[3][4 * q + k]);
+            T gi = coef_transpose_row<T>(i, sums[0], sums[1], sums[2], sums[3]);
+            const int64_t e = ((int64_t)c * 7 + q) * 16 + i;
+            if (probs != nullptr) gi = softmax16_backward(gi, probs[e]);       // gradient w.r.t. the logits
+            gw[e] = gi;
+        }
+        __syncthreads();
+    }
+}
+
+// grid: (64-sample blocks x channels) / kLsWaves.  count[2 ch] = kernels that read the channel, count[2 ch + 1] = where
+// their list starts in hits; an entry is kernel | tap mask << 16.
+template <typename T>
+__global__ __launch_bounds__(kLsWaves *kWave) void convblock_backward_x_4x4_kernel(const T *__restrict__ tg,
+                                                                                 const int32_t *__restrict__ count,
+                                                                                 const int32_t *__restrict__ hits,
+                                                                                 const int32_t *__restrict__ sel,
+                                                                                 const uint32_t *__restrict__ tcodes,
+                                                                                 T *__restrict__ gx, Geom g)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    const int sblocks = (g.n + kWave - 1) / kWave;
+    const int item = uniform((int)blockIdx.x * kLsWaves + wave);      // channel fastest: a workgroup shares its samples
+    if (item >= sblocks * g.cin) return;
+    const int sb = item / g.cin, ch = item - sb * g.cin;
+    const int64_t n = (int64_t)sb * kWave + lane;
+    const bool live = n < g.n;
+    const int64_t ns = live ? n : 0;
+    T *plane = reinterpret_cast<T *>(smem) + ((size_t)wave * kWave + lane) * kGradStride;
+#pragma unroll
+    for (int e = 0; e < kGradStride; ++e) plane[e] = T(0);
+    const int nhits = count[2 * ch];
+    const int32_t *hit = hits + count[2 * ch + 1];
+    constexpr int PER = 16 / (int)sizeof(T);
+    auto fetch = [&](int k, T (&gt)[32], uint32_t &codes) {
+        const int c = hit[k] & 0xFFFF;
+        const T *src = tg + ((int64_t)c * g.n + ns) * 32;
+#pragma unroll
+        for (int q = 0; q < 32 / PER; ++q) {
+            const u32x4 raw = reinterpret_cast<const u32x4 *>(src)[q];
+            T part[PER];
+            __builtin_memcpy(part, &raw, 16);
+#pragma unroll
+            for (int e = 0; e < PER; ++e) gt[q * PER + e] = part[e];
+        }
+        codes = tcodes[(int64_t)c * g.n + ns];
+    };
+    T cur[32], nxt[32];
+    uint32_t cur_codes = 0, nxt_codes = 0;
+    if (nhits > 0) fetch(0, cur, cur_codes);
+    for (int k = 0; k < nhits; ++k) {
+        if (k + 1 < nhits) fetch(k + 1, nxt, nxt_codes);              // in flight during the updates of hit k
+        const int ent = hit[k];
+        const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
+        int pc[4];                                                    // padded position of every cell's maximum
+#pragma unroll
+        for (int cell = 0; cell < 4; ++cell) {
+            const int code = (cur_codes >> (8 * cell)) & 3;
+            pc[cell] = (2 * (cell >> 1) + (code >> 1)) * 6 + 2 * (cell & 1) + (code & 1);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            if ((mask >> t) & 1) {                                    // wave-uniform: tap t of kernel c reads this channel
+                const Tap tp = unpack_tap(sel[c * 8 + t]);
+                const int off = tp.ry * 6 + tp.rx;
+                T old[4];
+                // the four cells' targets of one tap are distinct elements; taps are applied one after the other
+#pragma unroll
+                for (int cell = 0; cell < 4; ++cell) old[cell] = plane[pc[cell] + off];
+#pragma unroll
+                for (int cell = 0; cell < 4; ++cell) plane[pc[cell] + off] = old[cell] + cur[cell * 8 + t];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 32; ++e) cur[e] = nxt[e];
+        cur_codes = nxt_codes;
+    }
+    if (live) {
+        T out[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) out[e] = plane[((e >> 2) + 1) * 6 + (e & 3) + 1];
+        T *dst = gx + (n * g.cin + ch) * 16;
+#pragma unroll
+        for (int q = 0; q < 16 / PER; ++q) {
+            u32x4 raw;
+            __builtin_memcpy(&raw, &out[q * PER], 16);
+            reinterpret_cast<u32x4 *>(dst)[q] = raw;
+        }
+    }
+}
+
 }  // namespace
 
 // The shapes this file covers: what the last block of a 32x32-input network sees (n counts 64-sample groups for packed words).
@@ -193,4 +425,43 @@ int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_
                                   const char *name)
 {
     return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
+}
+
+// ---- gradients: launchers (the caller has run the prepare kernel: folded coefficients and per-channel kernel lists) ----
+// tap gradients [c][n][32] followed by the arg-max codes [c][n] of the same (kernel, sample) pairs
+static size_t tg_elems_bytes(int dtype, const Geom &g) { return (size_t)g.c * g.n * 32 * (dtype == CLG_F64 ? 8 : 4); }
+size_t clg_convblock_backward_4x4_tg_bytes(int dtype, const Geom &g) { return tg_elems_bytes(dtype, g) + (size_t)g.c * g.n * 4; }
+
+template <typename T>
+static int launch_backward_4x4(const Geom &g, const void *x, const void *folded, const int32_t *sel, const void *gy, const uint8_t *argmax,
+                               void *tg, void *gw, const void *probs, const int32_t *count, const int32_t *hits, void *gx, hipStream_t st,
+                               const char *name)
+{
+    int ct = 16;                                                      // kernels per workgroup, at least ~1024 workgroups
+    while (ct > 1 && (g.c + ct - 1) / ct < 1024) ct >>= 1;
+    const size_t lds = (size_t)kLsWaves * kWave * kLsStride * sizeof(T);
+    if (int e = allow_lds(convblock_backward_4x4_kernel<T>, lds + 1024, name)) return e;
+    uint32_t *tcodes = reinterpret_cast<uint32_t *>(reinterpret_cast<unsigned char *>(tg) + tg_elems_bytes(sizeof(T) == 8 ? CLG_F64 : CLG_F32, g));
+    hipLaunchKernelGGL(convblock_backward_4x4_kernel<T>, dim3((unsigned)((g.c + ct - 1) / ct)), dim3(kLsWaves * kWave), lds, st,
+                       (const T *)x, (const T *)folded, sel, (const T *)gy, argmax, gx != nullptr ? (T *)tg : (T *)nullptr, tcodes, (T *)gw,
+                       (const T *)probs, g, ct);
+    CLG_CHECK_LAUNCH(name);
+    if (gx == nullptr) return CLG_OK;
+    const int64_t items = (int64_t)((g.n + kWave - 1) / kWave) * g.cin;
+    CLG_REQUIRE((items + kLsWaves - 1) / kLsWaves < (1ll << 31), "%s: too many (sample block, channel) pairs for one launch", name);
+    const size_t lds_x = (size_t)kLsWaves * kWave * kGradStride * sizeof(T);
+    if (int e = allow_lds(convblock_backward_x_4x4_kernel<T>, lds_x, name)) return e;
+    hipLaunchKernelGGL(convblock_backward_x_4x4_kernel<T>, dim3((unsigned)((items + kLsWaves - 1) / kLsWaves)), dim3(kLsWaves * kWave),
+                       lds_x, st, (const T *)tg, count, hits, sel, (const uint32_t *)tcodes, (T *)gx, g);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
+}
+
+// gw: gradient w.r.t. the probabilities, or w.r.t. the logits when probs (their softmax) is given; gx may be null.
+int clg_convblock_backward_4x4(int dtype, const Geom &g, const void *x, const void *folded, const int32_t *sel, const void *gy,
+                               const uint8_t *argmax, void *tg, void *gw, const void *probs, const int32_t *count, const int32_t *hits,
+                               void *gx, hipStream_t st, const char *name)
+{
+    if (dtype == CLG_F32) return launch_backward_4x4<float>(g, x, folded, sel, gy, argmax, tg, gw, probs, count, hits, gx, st, name);
+    return launch_backward_4x4<double>(g, x, folded, sel, gy, argmax, tg, gw, probs, count, hits, gx, st, name);
 }

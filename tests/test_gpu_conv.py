@@ -309,3 +309,45 @@ def test_block_4x4_one_sample_per_lane_vs_oracle_and_staged_path(n, cin, cout, d
         y_old, a_old = convlogic_hip.full_convlogic_forward(*args)
         monkeypatch.delenv("CLG_FWD_4X4")
         assert torch.equal(y_new, y_old) and torch.equal(a_new, a_old)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,cin,cout", [(32, 3, 5), (100, 24, 48), (130, 40, 17), (300, 16, 64)])
+def test_block_4x4_one_sample_per_lane_gradients(n, cin, cout, dtype, monkeypatch):
+    # gradients of 4x4 blocks from the two one-sample-per-lane passes (tap gradients per kernel, then a per-channel
+    # sum in fixed order): against the oracle through the module, and against the staged kernels through both combined
+    # entry points, with a ragged last wavefront, kernels that read up to eight channels, and without grad_x
+    from convlogic_amd.hip import convlogic_hip
+    layer, x, y, idx = _run_block(n, cin, cout, 4, 4, 1, 1, 3, dtype=dtype, seed=n + 1)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    routed, _, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
+    check_pool_route(idx, idx_ref, x4)
+    routed.backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, name="grad_logits")
+    wp = torch.softmax(layer.weights.detach(), -1)
+    sel_wide = layer.selection.clone()
+    if cin >= 8:
+        taps = torch.arange(8, device=DEV, dtype=torch.int32)
+        sel_wide[1] = ((taps % cin) << 16) | ((taps % 3) << 8) | ((taps // 3) % 3)
+        sel_wide[cout - 1] = (((taps // 3) + 2) << 16) | ((taps % 3) << 8) | (taps % 2)
+    tol = 2e-5 if dtype == torch.float32 else 1e-12
+    for sel in (layer.selection, sel_wide):
+        yy, am = convlogic_hip.full_convlogic_forward(x.detach(), wp, sel, 1, 1, 1, 1, 3, 3)
+        got, want = {}, {}
+        for store, flag in ((got, None), (want, "0")):
+            if flag is not None:
+                monkeypatch.setenv("CLG_BWD_4X4", flag)
+            store["both"] = convlogic_hip.full_convlogic_backward(gy, x.detach(), wp, am, sel, 1, 1, 1, 1)
+            store["logits"] = convlogic_hip.full_convlogic_backward_logits(gy, x.detach(), wp, am, sel, 1, 1, 1, 1)
+            store["no_gx"] = convlogic_hip.full_convlogic_backward_logits(gy, x.detach(), wp, am, sel, 1, 1, 1, 1, need_grad_x=False)
+            if flag is not None:
+                monkeypatch.delenv("CLG_BWD_4X4")
+        assert got["no_gx"][0] is None and want["no_gx"][0] is None
+        for key in ("both", "logits", "no_gx"):
+            for a, b in zip(got[key], want[key]):
+                if a is None:
+                    continue
+                scale = max(b.abs().max().item(), 1e-30)
+                assert (a - b).abs().max().item() <= tol * scale, key
