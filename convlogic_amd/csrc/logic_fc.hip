@@ -207,25 +207,49 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restri
         const int64_t s = ((it % batch_chunks) * kWave + lane) * VEC;
         const bool live = s < batch;
         const int64_t beg = csr_start[i], end = csr_start[i + 1];
-        Pack<T, VEC> acc;
+        // consumers in groups of four, one partial sum per position in the group (as fc_backward_x_folded_kernel,
+        // whose results this kernel matches bit for bit)
+        Pack<T, VEC> part[4];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc.v[k] = 0;
-        for (int64_t cur = beg; cur < end; ++cur) {
-            const int64_t j = csr_list[cur];
-            const int64_t ia = a[j], ib = b[j];
-            const Coef<T> c = fold16(w + j * 16);
-            // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
-            // feature twice appears twice in the list and takes the B derivative the second time.
-            bool as_a = ia == i;
-            if (as_a && ib == i && cur > beg && csr_list[cur - 1] == j) as_a = false;
-            const T *other = x + (as_a ? ib : ia) * batch;
-            const T c_lin = as_a ? c.a : c.b;
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
+        int64_t prev = -1;
+        for (int64_t cur = beg; cur < end; cur += 4) {
+            int64_t j[4];
+            Pack<T, VEC> vo[4], vg[4];
+            T c_ab[4], c_lin[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                j[u] = cur + u < end ? csr_list[cur + u] : -1;
+                if (j[u] >= 0) {
+                    const int64_t ia = a[j[u]], ib = b[j[u]];
+                    const Coef<T> c = fold16(w + j[u] * 16);
+                    // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
+                    // feature twice appears twice in the list and takes the B derivative the second time.
+                    const bool as_a = ia == i && !(ib == i && prev == j[u]);
+                    c_ab[u] = c.ab;
+                    c_lin[u] = as_a ? c.a : c.b;
+                    if (live) {
+                        vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
+                        vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
+                    }
+                }
+                prev = j[u];
+            }
             if (live) {
-                const Pack<T, VEC> vo = load_vec<T, VEC>(other + s), vg = load_vec<T, VEC>(gy + j * batch + s);
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) acc.v[k] = fma_t(fma_t(c.ab, vo.v[k], c_lin), vg.v[k], acc.v[k]);
+                for (int u = 0; u < 4; ++u) {
+                    if (j[u] >= 0) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
+                    }
+                }
             }
         }
+        Pack<T, VEC> acc;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
         if (live) store_vec<T, VEC>(gx + (int64_t)i * batch + s, acc);
     }
 }
@@ -313,31 +337,45 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
         const int64_t s = (((it % batch_chunks) << lpr_log2) + l) * VEC;
         if (i >= in_dim || s >= batch) continue;
         const int64_t beg = csr_start[i], end = csr_start[i + 1];
-        Pack<T, VEC> acc;
+        // Consumers in groups of four with one partial sum per position in the group, so that the rows of four
+        // consumers are in flight together; the partial sums are added as (0 + 1) + (2 + 3).
+        Pack<T, VEC> part[4];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc.v[k] = 0;
-        if (beg < end) {
-            // The chain list -> wiring and coefficients -> rows is three dependent loads deep: the list runs two
-            // consumers ahead and the tables one ahead of the rows being accumulated.
-            int64_t prev = -1, j = csr_list[beg], j_next = csr_list[beg + 1 < end ? beg + 1 : beg];
-            int64_t ia = a[j], ib = b[j];
-            Coef<T> c = load_coef(folded + j * 4);
-            for (int64_t cur = beg; cur < end; ++cur) {
-                const int64_t j_after = csr_list[cur + 2 < end ? cur + 2 : end - 1];
-                const int64_t ia_next = a[j_next], ib_next = b[j_next];
-                const Coef<T> c_next = load_coef(folded + j_next * 4);
-                // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
-                // feature twice appears twice in the list and takes the B derivative the second time.
-                const bool as_a = ia == i && !(ib == i && prev == j);
-                const T *other = x + (as_a ? ib : ia) * batch;
-                const T c_lin = as_a ? c.a : c.b;
-                const Pack<T, VEC> vo = load_vec<T, VEC>(other + s), vg = load_vec<T, VEC>(gy + j * batch + s);
+        for (int u = 0; u < 4; ++u)
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) acc.v[k] = fma_t(fma_t(c.ab, vo.v[k], c_lin), vg.v[k], acc.v[k]);
-                prev = j, j = j_next, j_next = j_after;
-                ia = ia_next, ib = ib_next, c = c_next;
+            for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
+        int64_t prev = -1;
+        for (int64_t cur = beg; cur < end; cur += 4) {
+            int64_t j[4];
+            Pack<T, VEC> vo[4], vg[4];
+            T c_ab[4], c_lin[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                j[u] = cur + u < end ? csr_list[cur + u] : -1;
+                if (j[u] >= 0) {
+                    const int64_t ia = a[j[u]], ib = b[j[u]];
+                    const Coef<T> c = load_coef(folded + j[u] * 4);
+                    // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
+                    // feature twice appears twice in the list and takes the B derivative the second time.
+                    const bool as_a = ia == i && !(ib == i && prev == j[u]);
+                    c_ab[u] = c.ab;
+                    c_lin[u] = as_a ? c.a : c.b;
+                    vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
+                    vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
+                }
+                prev = j[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (j[u] >= 0) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
+                }
             }
         }
+        Pack<T, VEC> acc;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
         store_vec<T, VEC>(gx + i * batch + s, acc);
     }
 }
