@@ -211,3 +211,33 @@ def test_compiled_netlist_runs_the_packed_kernels(tmp_path):
     x = torch.randint(0, 2, (200, 64), device=DEV).bool()
     with torch.no_grad():
         assert torch.equal(CompiledLogicNet(fc)(x), fc(C.PackBitsTensor(x, 64)))
+
+
+def test_small_network_learns_a_synthetic_task():
+    # end to end: a small CIFAR-topology network trained with Adam on a task its first block can see (which image
+    # half holds more ones) -- the loss has to fall, in eager steps and in HIP-graph replays alike
+    torch.manual_seed(0)
+    n = 256
+    x = (torch.rand(n, 3, 32, 32, device=DEV) < 0.5).float()
+    boost = torch.randint(0, 2, (n,), device=DEV)
+    x[boost == 1, :, :16] = (torch.rand(int((boost == 1).sum()), 3, 16, 32, device=DEV) < 0.8).float()
+    x[boost == 0, :, 16:] = (torch.rand(int((boost == 0).sum()), 3, 16, 32, device=DEV) < 0.8).float()
+    labels = boost * 5                                               # classes 0 and 5 of 10
+    ce = torch.nn.functional.cross_entropy
+    for graphed in (False, True):
+        torch.manual_seed(1)
+        model = C.ConvLogicCifarModel(k_param=4, input_channels=3, input_size=32, tau=4).to(DEV)
+        opt = torch.optim.Adam(model.parameters(), lr=0.05)
+        step = C.GraphedStep(lambda a, b: ce(model(a), b), (x, labels), model.parameters()) if graphed else None
+        losses = []
+        for _ in range(40):
+            if graphed:
+                loss = step(x, labels)
+            else:
+                opt.zero_grad(set_to_none=True)
+                loss = ce(model(x), labels)
+                loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        assert all(torch.isfinite(torch.tensor(losses)))
+        assert losses[-1] < 0.6 * losses[0], (graphed, losses[0], losses[-1])
