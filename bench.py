@@ -211,7 +211,6 @@ def bench_c1(steps, warmup, cpu=True):
     import torch
 
     import convlogic_amd as C
-    from oracle import convlogic_oracle as O
 
     dev = "cuda:0"
     in_dim = out_dim = 8000
@@ -252,6 +251,8 @@ def bench_c1(steps, warmup, cpu=True):
            "ms_per_step_hip_graph": graph_ms,
            "value_hip_graph": (gate_evals / (graph_ms * 1e-3) / 1e9) if graph_ms else None}
     def cpu_leg():
+        from oracle import convlogic_oracle as O            # the CPU baseline is the only user of the oracle here
+
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
         xl = x.detach().cpu().requires_grad_(True)
         ll = layer.weights.detach().cpu().requires_grad_(True)
@@ -296,7 +297,6 @@ def bench_conv(key, steps, warmup, cpu=True):
 
     import convlogic_amd as C
     from convlogic_amd.hip import convlogic_hip
-    from oracle import convlogic_oracle as O
 
     cfg = CONV[key]
     dev = "cuda:0"
@@ -353,6 +353,8 @@ def bench_conv(key, steps, warmup, cpu=True):
                              {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
                               "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked"})}
     def cpu_leg():
+        from oracle import convlogic_oracle as O            # the CPU baseline is the only user of the oracle here
+
         nb = 8                                              # bounded sample: 8 samples of the batch
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
         xl = x.detach()[:nb].cpu().requires_grad_(True)
