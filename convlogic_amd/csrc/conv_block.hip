@@ -597,7 +597,10 @@ __global__ __launch_bounds__(256) void sum_partial_images_kernel(const T *__rest
 // order by reduce_coef_partials.  Taps come from a zero-padded copy of x in global memory (written once
 // per call into scratch, same shared-halo layout as the LDS images), so the loop has no bounds checks
 // and 32-bit offsets only.
-template <typename T>
+// FIXED: the pooled cells of a sample divide the 256 threads (I = 1, 2, 4 ... 256), so a thread keeps its cell and walks
+// over samples only: cell decoding and the cell part of every offset leave the loop, and 32-bit offsets suffice (the plan
+// checks the sizes).
+template <typename T, bool FIXED>
 __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const T *__restrict__ gy, const T *__restrict__ xp,
                                                                         const T *__restrict__ folded,
                                                                         const int32_t *__restrict__ taps,
@@ -621,13 +624,30 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
     T acc[28];
 #pragma unroll
     for (int k = 0; k < 28; ++k) acc[k] = T(0);
-    for (uint32_t it = blockIdx.x * 256 + threadIdx.x; it < items; it += (uint32_t)nb * 256) {
-        const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
-        const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
-        const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
-        const int code = argmax[o];
-        const T gout = gy[o];
-        const int pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
+    // FIXED: this thread's cell, its first sample and the samples it skips per step
+    const uint32_t per_block = FIXED ? 256u / (uint32_t)I : 1u;
+    const uint32_t f_cell = FIXED ? threadIdx.x % (uint32_t)I : 0u;
+    const uint32_t f_py = fdiv(f_cell, p.d_wp), f_px = f_cell - f_py * (uint32_t)wp;
+    const uint32_t f_pos = (2 * f_py) * row_step + (2 * f_px) * g.sw;
+    const uint32_t f_out = (uint32_t)(kernel_row + f_cell);
+    const uint32_t f_n0 = blockIdx.x * per_block + threadIdx.x / (uint32_t)I, f_step = (uint32_t)nb * per_block;
+    for (uint32_t it = FIXED ? f_n0 : blockIdx.x * 256 + threadIdx.x; it < (FIXED ? (uint32_t)g.n : items);
+         it += FIXED ? f_step : (uint32_t)nb * 256) {
+        int code, pos;
+        T gout;
+        if (FIXED) {
+            const uint32_t o = it * (uint32_t)sample_cells + f_out;
+            code = load_at(argmax, o);
+            gout = load_at(gy, o);
+            pos = (int)(it * (uint32_t)sample_elems + f_pos) + (code >> 1) * row_step + (code & 1) * g.sw;
+        } else {
+            const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
+            const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+            const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
+            code = argmax[o];
+            gout = gy[o];
+            pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
+        }
         T tv[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(pos + to[t]));
@@ -819,6 +839,13 @@ struct WScratch {
     int nb, sample_elems;
     size_t folded_off, taps_off, xp_off, total;
 };
+// The padded weight-gradient kernel keeps a thread on one pooled cell when the cells of a sample divide its 256 threads
+// and grad_y / arg-max can be addressed with 32-bit byte offsets.
+bool fixed_cells(const Geom &g, int elem)
+{
+    const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
+    return I <= 256 && 256 % I == 0 && (int64_t)g.n * g.c * I * elem < (1ll << 32);
+}
 bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
 {
     if (!taps_inside(g) || g.c > 65535) return false;
@@ -953,9 +980,14 @@ int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &w
                        g.c, p.rs, p.chs, job, (int)prep);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(prepare)");
     const int I = (g.ho / 2) * (g.wo / 2);
-    hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
-                       (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p, make_fastdiv((uint32_t)I),
-                       ws.sample_elems, 8);
+    if (fixed_cells(g, (int)sizeof(T)))
+        hipLaunchKernelGGL((convblock_backward_w_padded_kernel<T, true>), dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st,
+                           (const T *)gy, (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p,
+                           make_fastdiv((uint32_t)I), ws.sample_elems, 8);
+    else
+        hipLaunchKernelGGL((convblock_backward_w_padded_kernel<T, false>), dim3((unsigned)ws.nb, (unsigned)g.c), dim3(256), 0, st,
+                           (const T *)gy, (const T *)xp, (const T *)folded, (const int32_t *)taps, argmax, partial, g, p,
+                           make_fastdiv((uint32_t)I), ws.sample_elems, 8);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded)");
     return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, ws.nb, 7, st, "clg_convblock_backward_w(reduce)",
                                   probs);
@@ -970,9 +1002,14 @@ int launch_backward_w_shared(const Geom &g, const SharedPad &sh, const void *gy,
     int64_t nb = clg_ceil_div(I * g.n, 256 * 8);
     nb = nb < 1 ? 1 : (nb > 64 ? 64 : nb);
     T *partial = reinterpret_cast<T *>(scratch);                      // [c][nb][28], within the any-shape kernel's [c][64][28]
-    hipLaunchKernelGGL(convblock_backward_w_padded_kernel<T>, dim3((unsigned)nb, (unsigned)g.c), dim3(256), 0, st, (const T *)gy,
-                       (const T *)sh.xp, (const T *)sh.folded, sh.taps, argmax, partial, g, sh.p, make_fastdiv((uint32_t)I),
-                       sh.sample_elems, 16);
+    if (fixed_cells(g, (int)sizeof(T)))
+        hipLaunchKernelGGL((convblock_backward_w_padded_kernel<T, true>), dim3((unsigned)nb, (unsigned)g.c), dim3(256), 0, st,
+                           (const T *)gy, (const T *)sh.xp, (const T *)sh.folded, sh.taps, argmax, partial, g, sh.p,
+                           make_fastdiv((uint32_t)I), sh.sample_elems, 16);
+    else
+        hipLaunchKernelGGL((convblock_backward_w_padded_kernel<T, false>), dim3((unsigned)nb, (unsigned)g.c), dim3(256), 0, st,
+                           (const T *)gy, (const T *)sh.xp, (const T *)sh.folded, sh.taps, argmax, partial, g, sh.p,
+                           make_fastdiv((uint32_t)I), sh.sample_elems, 16);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(padded, shared copy)");
     return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, partial, gw, g.c, (int)nb, 7, st,
                                   "clg_convblock_backward_w(reduce)", probs);

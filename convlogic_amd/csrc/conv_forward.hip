@@ -34,7 +34,9 @@ namespace {
 // ROWSTEP: elements between conv rows 2r and 2r+1 in the LDS image when known at compile time (the
 // second row's reads then use the immediate offset of the LDS instruction), 0 = read it from the plan.
 // SUBSET: stage two planes per kernel of the tile instead of all input channels.
-template <typename Ops, int ROWSTEP, bool SUBSET>
+// ONE_ROW: a lane slot is one conv position instead of a column of two rows (plan.one_row; compile-time so that the
+// two-row loop carries nothing of it).
+template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW>
 __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
                                                const int32_t *__restrict__ sel, typename Ops::Elem *__restrict__ y,
                                                uint8_t *__restrict__ argmax, Geom g, TilePlan p)
@@ -85,7 +87,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
         }
     }
     const int U = s_cur * p.slots;
-    const int rows_per_slot = p.one_row ? 1 : 2;                     // conv rows a lane slot covers
+    constexpr int rows_per_slot = ONE_ROW ? 1 : 2;                   // conv rows a lane slot covers
     for (int u = tid; u < U; u += nthreads) {
         const uint32_t s = fdiv(u, p.d_slots), r = u - s * (uint32_t)p.slots;
         const uint32_t rp = fdiv(r, p.d_wo), ox = r - rp * (uint32_t)g.wo;        // rp: row pair, or row with one_row
@@ -125,7 +127,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
 
     const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
     // lanes that pool and write: even columns, and with one position per lane even rows only
-    const bool writer_lane = !(lane & 1) && !(p.one_row && ((lane / g.wo) & 1));
+    const bool writer_lane = !(lane & 1) && !(ONE_ROW && ((lane / g.wo) & 1));
     // work items = (kernel, block of 64 slots), kernel-major; every wavefront takes a contiguous range, so
     // the scalar parameters are reloaded only when its range crosses into the next kernel
     const int nblk = (U + kWave - 1) / kWave;
@@ -152,7 +154,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
 #pragma unroll
                 for (int t = 0; t < 8; ++t) v[t] = xs[e.x + to[t]];
                 r0 = Ops::root(pr, v);
-                if (!p.one_row) {
+                if (!ONE_ROW) {
 #pragma unroll
                     for (int t = 0; t < 8; ++t) v[t] = xs[e.x + row_step + to[t]];
                     r1 = Ops::root(pr, v);
@@ -167,7 +169,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
 #pragma unroll
                 for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)oy, (int)ox);
                 r0 = Ops::root(pr, v);
-                if (!p.one_row) {
+                if (!ONE_ROW) {
 #pragma unroll
                     for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(oy + 1), (int)ox);
                     r1 = Ops::root(pr, v);
@@ -175,7 +177,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
             }
             const T r0o = dpp_xor1(r0);
             T r1o;
-            if (p.one_row) {                                          // the row below sits wo lanes up (2 wo divides 64)
+            if (ONE_ROW) {                                            // the row below sits wo lanes up (2 wo divides 64)
                 r1 = lane_up(r0, g.wo);
                 r1o = lane_up(r0o, g.wo);
             } else {
@@ -437,14 +439,14 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
 }
 
 // ---- launch ------------------------------------------------------------------------------------
-template <typename Ops, int ROWSTEP, bool SUBSET>
+template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW = false>
 int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
                        uint8_t *argmax, hipStream_t st, const char *name)
 {
     using T = typename Ops::Elem;
-    if (int e = allow_lds(convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET>, p.lds_bytes, name)) return e;
+    if (int e = allow_lds(convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET, ONE_ROW>, p.lds_bytes, name)) return e;
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
-    hipLaunchKernelGGL((convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
+    hipLaunchKernelGGL((convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET, ONE_ROW>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
                        params, sel, (T *)y, argmax, g, p);
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
@@ -460,6 +462,9 @@ int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const 
     case RS:                                                                                                          \
         return p.subset ? launch_forward_one<Ops, RS, true>(g, p, x, params, sel, y, argmax, st, name)                \
                         : launch_forward_one<Ops, RS, false>(g, p, x, params, sel, y, argmax, st, name)
+    if (p.one_row)                                                   // few positions per sample: the row step is not worth a variant
+        return p.subset ? launch_forward_one<Ops, 0, true, true>(g, p, x, params, sel, y, argmax, st, name)
+                        : launch_forward_one<Ops, 0, false, true>(g, p, x, params, sel, y, argmax, st, name);
     switch (g.sh * p.rs) {
         CLG_FWD_CASE(33);
         CLG_FWD_CASE(29);
