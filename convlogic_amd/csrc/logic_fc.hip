@@ -5,6 +5,8 @@
 // contiguous row segment.  The neuron index is wave-uniform: wiring indices and the 16 gate
 // probabilities come through the scalar cache and are folded to 4 coefficients in SGPR-uniform
 // registers; the per-sample work is one multiply and three FMAs.
+#include <hip/hip_fp16.h>
+
 #include "clg_common.h"
 
 namespace {
@@ -28,18 +30,81 @@ struct Pack {
     T v[VEC];
 };
 
-template <typename T, int VEC>
-__device__ __forceinline__ Pack<T, VEC> load_vec(const T *p)
+// Storage type S of a tensor and the type its values are computed in: half is a storage format only, the arithmetic
+// of such tensors runs in float32.
+template <typename S>
+struct ComputeOf { using type = S; };
+template <>
+struct ComputeOf<__half> { using type = float; };
+
+template <typename S, int VEC>
+__device__ __forceinline__ Pack<typename ComputeOf<S>::type, VEC> load_vec(const S *p)
 {
-    using V = typename VecT<T, VEC>::type;
-    const V r = *reinterpret_cast<const V *>(p);
-    return __builtin_bit_cast(Pack<T, VEC>, r);
+    using T = typename ComputeOf<S>::type;
+    if constexpr (sizeof(S) == 2) {
+        Pack<T, VEC> r;
+        if constexpr (VEC == 8) {
+            const u32x4 raw = *reinterpret_cast<const u32x4 *>(p);
+            __half h[8];
+            __builtin_memcpy(h, &raw, 16);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) r.v[k] = __half2float(h[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = __half2float(p[k]);
+        }
+        return r;
+    } else {
+        using V = typename VecT<T, VEC>::type;
+        const V r = *reinterpret_cast<const V *>(p);
+        return __builtin_bit_cast(Pack<T, VEC>, r);
+    }
 }
-template <typename T, int VEC>
-__device__ __forceinline__ void store_vec(T *p, const Pack<T, VEC> &v)
+template <typename S, int VEC>
+__device__ __forceinline__ void store_vec(S *p, const Pack<typename ComputeOf<S>::type, VEC> &v)
 {
-    using V = typename VecT<T, VEC>::type;
-    *reinterpret_cast<V *>(p) = __builtin_bit_cast(V, v);
+    using T = typename ComputeOf<S>::type;
+    if constexpr (sizeof(S) == 2) {
+        if constexpr (VEC == 8) {
+            __half h[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) h[k] = __float2half(v.v[k]);
+            u32x4 raw;
+            __builtin_memcpy(&raw, h, 16);
+            *reinterpret_cast<u32x4 *>(p) = raw;
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) p[k] = __float2half(v.v[k]);
+        }
+    } else {
+        using V = typename VecT<T, VEC>::type;
+        *reinterpret_cast<V *>(p) = __builtin_bit_cast(V, v);
+    }
+}
+template <typename S>
+__device__ __forceinline__ typename ComputeOf<S>::type load_one(const S *p)
+{
+    if constexpr (sizeof(S) == 2) return __half2float(*p);
+    else return *p;
+}
+template <typename S>
+__device__ __forceinline__ void store_one(S *p, typename ComputeOf<S>::type v)
+{
+    if constexpr (sizeof(S) == 2) *p = __float2half(v);
+    else *p = v;
+}
+// fold16 of 16 stored probabilities
+template <typename S>
+__device__ __forceinline__ Coef<typename ComputeOf<S>::type> fold16_stored(const S *__restrict__ w)
+{
+    if constexpr (sizeof(S) == 2) {
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t[i] = __half2float(w[i]);
+        return fold16(t);
+    } else {
+        return fold16(w);
+    }
 }
 
 // folded = 4 coefficients per neuron, written by fc_fold_kernel
@@ -57,24 +122,25 @@ __device__ __forceinline__ Coef<T> load_coef(const T *__restrict__ f)
     return c;
 }
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void fc_forward_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
-                                                          const int64_t *__restrict__ b, const T *__restrict__ w,
-                                                          T *__restrict__ y, int out_dim, int64_t batch)
+template <typename S, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_forward_kernel(const S *__restrict__ x, const int64_t *__restrict__ a,
+                                                          const int64_t *__restrict__ b, const S *__restrict__ w,
+                                                          S *__restrict__ y, int out_dim, int64_t batch)
 {
+    using T = typename ComputeOf<S>::type;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
     for (int j = blockIdx.x * kWavesPerBlock + wave; j < out_dim; j += gridDim.x * kWavesPerBlock) {
-        const T *xa = x + a[j] * batch;
-        const T *xb = x + b[j] * batch;
-        T *yj = y + (int64_t)j * batch;
-        const Coef<T> c = fold16(w + (int64_t)j * 16);
+        const S *xa = x + a[j] * batch;
+        const S *xb = x + b[j] * batch;
+        S *yj = y + (int64_t)j * batch;
+        const Coef<T> c = fold16_stored(w + (int64_t)j * 16);
         for (int64_t s = (int64_t)lane * VEC; s < batch; s += kWave * VEC) {
-            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
+            const Pack<T, VEC> va = load_vec<S, VEC>(xa + s), vb = load_vec<S, VEC>(xb + s);
             Pack<T, VEC> r;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r.v[k] = gate(c, va.v[k], vb.v[k]);
-            store_vec<T, VEC>(yj + s, r);
+            store_vec<S, VEC>(yj + s, r);
         }
     }
 }
@@ -94,12 +160,13 @@ __device__ __forceinline__ T lane_group_sum(T v)
 
 // A neuron's row takes LPR lanes x VEC samples per pass, a wavefront 64/LPR neurons; the last 16 lanes of each
 // group hold the four sums and write the 16 gate gradients.
-template <typename T, int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+template <typename S, int VEC, int LPR>
+__global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const S *__restrict__ x, const int64_t *__restrict__ a,
                                                              const int64_t *__restrict__ b,
-                                                             const T *__restrict__ gy, T *__restrict__ gw, int out_dim,
-                                                             int64_t batch, const T *__restrict__ probs)
+                                                             const S *__restrict__ gy, S *__restrict__ gw, int out_dim,
+                                                             int64_t batch, const S *__restrict__ probs)
 {
+    using T = typename ComputeOf<S>::type;
     constexpr int ROWS = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int sub = lane / LPR, l = lane % LPR;
@@ -107,13 +174,13 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restri
          j0 += (int64_t)gridDim.x * kWavesPerBlock * ROWS) {
         const bool valid = j0 + sub < out_dim;
         const int64_t j = valid ? j0 + sub : out_dim - 1;           // every lane takes part in the reductions
-        const T *xa = x + a[j] * batch;
-        const T *xb = x + b[j] * batch;
-        const T *gj = gy + j * batch;
+        const S *xa = x + a[j] * batch;
+        const S *xb = x + b[j] * batch;
+        const S *gj = gy + j * batch;
         T sab = 0, sa = 0, sb = 0, s1 = 0;
         for (int64_t s = (int64_t)l * VEC; s < batch; s += LPR * VEC) {
-            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s),
-                               vg = load_vec<T, VEC>(gj + s);
+            const Pack<T, VEC> va = load_vec<S, VEC>(xa + s), vb = load_vec<S, VEC>(xb + s),
+                               vg = load_vec<S, VEC>(gj + s);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 sab = fma_t(vg.v[k], va.v[k] * vb.v[k], sab);
@@ -129,8 +196,8 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const T *__restri
         if (l >= LPR - 16) {
             const int i = lane & 15;
             T gi = coef_transpose_row<T>(i, sab, sa, sb, s1);
-            if (probs != nullptr) gi = softmax16_backward(gi, probs[j * 16 + i]);   // gradient w.r.t. the logits
-            if (valid) gw[j * 16 + i] = gi;
+            if (probs != nullptr) gi = softmax16_backward(gi, load_one(probs + j * 16 + i));   // gradient w.r.t. the logits
+            if (valid) store_one(gw + j * 16 + i, gi);
         }
     }
 }
@@ -190,15 +257,16 @@ __global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__res
     }
 }
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
-                                                             const int64_t *__restrict__ b, const T *__restrict__ w,
-                                                             const T *__restrict__ gy,
+template <typename S, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const S *__restrict__ x, const int64_t *__restrict__ a,
+                                                             const int64_t *__restrict__ b, const S *__restrict__ w,
+                                                             const S *__restrict__ gy,
                                                              const int64_t *__restrict__ csr_start,
                                                              const int64_t *__restrict__ csr_list,
-                                                             T *__restrict__ gx, int in_dim, int64_t batch,
+                                                             S *__restrict__ gx, int in_dim, int64_t batch,
                                                              int batch_chunks)
 {
+    using T = typename ComputeOf<S>::type;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
     const int64_t items = (int64_t)in_dim * batch_chunks;
@@ -224,15 +292,15 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restri
                 j[u] = cur + u < end ? csr_list[cur + u] : -1;
                 if (j[u] >= 0) {
                     const int64_t ia = a[j[u]], ib = b[j[u]];
-                    const Coef<T> c = fold16(w + j[u] * 16);
+                    const Coef<T> c = fold16_stored(w + j[u] * 16);
                     // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
                     // feature twice appears twice in the list and takes the B derivative the second time.
                     const bool as_a = ia == i && !(ib == i && prev == j[u]);
                     c_ab[u] = c.ab;
                     c_lin[u] = as_a ? c.a : c.b;
                     if (live) {
-                        vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
-                        vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
+                        vo[u] = load_vec<S, VEC>(x + (as_a ? ib : ia) * batch + s);
+                        vg[u] = load_vec<S, VEC>(gy + j[u] * batch + s);
                     }
                 }
                 prev = j[u];
@@ -250,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const T *__restri
         Pack<T, VEC> acc;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
-        if (live) store_vec<T, VEC>(gx + (int64_t)i * batch + s, acc);
+        if (live) store_vec<S, VEC>(gx + (int64_t)i * batch + s, acc);
     }
 }
 
@@ -475,9 +543,13 @@ int lanes_per_row_log2(int64_t batch, int vec)
     return lanes <= 16 ? 4 : (lanes <= 32 ? 5 : 6);
 }
 
-int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const char *name)
+int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const char *name, bool half_ok = false)
 {
-    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
+    if (half_ok)
+        CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64 || dtype == CLG_F16, "%s: dtype must be CLG_F32, CLG_F64 or CLG_F16, got %d",
+                    name, dtype);
+    else
+        CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
     CLG_REQUIRE(in_dim > 0 && out_dim > 0 && batch > 0, "%s: in_dim, out_dim and batch must be positive (%lld, %lld, %lld)",
                 name, (long long)in_dim, (long long)out_dim, (long long)batch);
     CLG_REQUIRE(in_dim < (1ll << 31) && out_dim < (1ll << 31), "%s: in_dim/out_dim above 2^31-1 are not supported", name);
@@ -489,25 +561,23 @@ int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const ch
 extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
                               int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward")) return e;
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward", true)) return e;
     CLG_REQUIRE(x && a && b && w && y, "clg_fc_forward: null pointer argument");
     const dim3 grid(grid_for(out_dim)), block(kBlock);
     hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_F(S, VEC) \
+    hipLaunchKernelGGL((fc_forward_kernel<S, VEC>), grid, block, 0, st, (const S *)x, a, b, (const S *)w, (S *)y, (int)out_dim, batch)
     if (dtype == CLG_F32) {
-        if (batch % 4 == 0)
-            hipLaunchKernelGGL((fc_forward_kernel<float, 4>), grid, block, 0, st, (const float *)x, a, b, (const float *)w,
-                               (float *)y, (int)out_dim, batch);
-        else
-            hipLaunchKernelGGL((fc_forward_kernel<float, 1>), grid, block, 0, st, (const float *)x, a, b, (const float *)w,
-                               (float *)y, (int)out_dim, batch);
+        if (batch % 4 == 0) CLG_LAUNCH_F(float, 4);
+        else CLG_LAUNCH_F(float, 1);
+    } else if (dtype == CLG_F64) {
+        if (batch % 2 == 0) CLG_LAUNCH_F(double, 2);
+        else CLG_LAUNCH_F(double, 1);
     } else {
-        if (batch % 2 == 0)
-            hipLaunchKernelGGL((fc_forward_kernel<double, 2>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)w, (double *)y, (int)out_dim, batch);
-        else
-            hipLaunchKernelGGL((fc_forward_kernel<double, 1>), grid, block, 0, st, (const double *)x, a, b,
-                               (const double *)w, (double *)y, (int)out_dim, batch);
+        if (batch % 8 == 0) CLG_LAUNCH_F(__half, 8);
+        else CLG_LAUNCH_F(__half, 1);
     }
+#undef CLG_LAUNCH_F
     CLG_CHECK_LAUNCH("clg_fc_forward");
     return CLG_OK;
 }
@@ -515,7 +585,7 @@ extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const 
 static int fc_backward_w_impl(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *grad_y, void *grad_w,
                              int64_t in_dim, int64_t out_dim, int64_t batch, void *stream, const void *probs, const char *name)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, name, true)) return e;
     CLG_REQUIRE(x && a && b && grad_y && grad_w, "%s: null pointer argument", name);
     const dim3 block(kBlock);
     hipStream_t st = clg_stream(stream);
@@ -533,9 +603,12 @@ static int fc_backward_w_impl(int dtype, const void *x, const int64_t *a, const 
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_BW_ROWS(float, 4);
         else CLG_LAUNCH_BW_ROWS(float, 1);
-    } else {
+    } else if (dtype == CLG_F64) {
         if (batch % 2 == 0) CLG_LAUNCH_BW_ROWS(double, 2);
         else CLG_LAUNCH_BW_ROWS(double, 1);
+    } else {
+        if (batch % 8 == 0) CLG_LAUNCH_BW_ROWS(__half, 8);
+        else CLG_LAUNCH_BW_ROWS(__half, 1);
     }
 #undef CLG_LAUNCH_BW_ROWS
 #undef CLG_LAUNCH_BW
@@ -561,7 +634,7 @@ extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, con
                                  const void *grad_y, const int64_t *csr_start, const int64_t *csr_list, void *grad_x,
                                  int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_x")) return e;
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_x", true)) return e;
     CLG_REQUIRE(x && a && b && w && grad_y && csr_start && csr_list && grad_x, "clg_fc_backward_x: null pointer argument");
     hipStream_t st = clg_stream(stream);
     const dim3 block(kBlock);
@@ -575,9 +648,12 @@ extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, con
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_BX(float, 4);
         else CLG_LAUNCH_BX(float, 1);
-    } else {
+    } else if (dtype == CLG_F64) {
         if (batch % 2 == 0) CLG_LAUNCH_BX(double, 2);
         else CLG_LAUNCH_BX(double, 1);
+    } else {
+        if (batch % 8 == 0) CLG_LAUNCH_BX(__half, 8);
+        else CLG_LAUNCH_BX(__half, 1);
     }
 #undef CLG_LAUNCH_BX
     CLG_CHECK_LAUNCH("clg_fc_backward_x");

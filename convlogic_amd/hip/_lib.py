@@ -11,8 +11,9 @@ import torch
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, "libconvlogic_amd.so")
 
-CLG_F32, CLG_F64 = 0, 1
+CLG_F32, CLG_F64, CLG_F16 = 0, 1, 2
 _DTYPES = {torch.float32: CLG_F32, torch.float64: CLG_F64}
+_DTYPES_FC = {**_DTYPES, torch.float16: CLG_F16}       # LogicLayer forward / backward_w / backward_x also store half
 
 _p, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
 
@@ -100,11 +101,12 @@ def check(rc):
         raise RuntimeError(load().clg_last_error().decode())
 
 
-def dtype_code(t):
+def dtype_code(t, half_ok=False):
     try:
-        return _DTYPES[t.dtype]
+        return (_DTYPES_FC if half_ok else _DTYPES)[t.dtype]
     except KeyError:
-        raise RuntimeError(f"convlogic_amd kernels support float32 and float64, got {t.dtype}") from None
+        kinds = "float32, float64 and float16" if half_ok else "float32 and float64"
+        raise RuntimeError(f"convlogic_amd: this kernel supports {kinds}, got {t.dtype}") from None
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)

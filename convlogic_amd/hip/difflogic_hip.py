@@ -16,7 +16,7 @@ def forward(x, a, b, w):
     out_dim = w.shape[0]
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     if y.numel():
-        check(_lib.load().clg_fc_forward(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(), y.data_ptr(),
+        check(_lib.load().clg_fc_forward(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(), y.data_ptr(),
                                          in_dim, out_dim, batch, stream_ptr(x)))
     return y
 
@@ -28,7 +28,7 @@ def backward_w(x, a, b, grad_y):
     in_dim, batch = x.shape
     out_dim = grad_y.shape[0]
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
-    check(_lib.load().clg_fc_backward_w(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), grad_y.data_ptr(),
+    check(_lib.load().clg_fc_backward_w(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), grad_y.data_ptr(),
                                         gw.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
     return gw
 
@@ -134,7 +134,7 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
     in_dim, batch = x.shape
     out_dim = w.shape[0]
     gx = torch.empty_like(x)
-    check(_lib.load().clg_fc_backward_x(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
+    check(_lib.load().clg_fc_backward_x(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
                                         grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
                                         given_x_indices_of_y.data_ptr(), gx.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
     return gx

@@ -14,7 +14,7 @@
  * it stands in for.
  *
  * Conventions
- *   dtype           CLG_F32 or CLG_F64 (all float tensors of a call share it)
+ *   dtype           CLG_F32 or CLG_F64 (all float tensors of a call share it); CLG_F16 where an entry point says so
  *   gate weights w  [..., 16] probabilities per gate (softmax or one-hot), gate ids
  *                   as in src/difflogic/functional.py:7-24
  *   selection       int32 [C, 8], tap = ch << 16 | row << 8 | col
@@ -32,6 +32,7 @@ extern "C" {
 
 #define CLG_F32 0
 #define CLG_F64 1
+#define CLG_F16 2 /* IEEE half as a storage format of clg_fc_forward / _backward_w / _backward_x (arithmetic in float32) */
 
 #define CLG_OK 0
 #define CLG_EINVAL (-1)  /* rejected argument (shape, dtype, null pointer, limit) */
@@ -55,7 +56,8 @@ typedef struct clg_conv_geom {
 
 /* y[j][s] = sum_i w[j][i] * op_i(x[a[j]][s], x[b[j]][s]).
  * Replaces difflogic_cuda.forward -- src/difflogic/cuda/difflogic.cpp:17,
- * logic_layer_cuda_forward src/difflogic/cuda/difflogic_kernel.cu:89-126. */
+ * logic_layer_cuda_forward src/difflogic/cuda/difflogic_kernel.cu:89-126.  dtype may be CLG_F16 here and in
+ * clg_fc_backward_w / clg_fc_backward_x (the reference dispatches these three for half as well, :108,146,249). */
 int clg_fc_forward(int dtype, const void *x /*[in_dim,batch]*/, const int64_t *a /*[out_dim]*/,
                    const int64_t *b /*[out_dim]*/, const void *w /*[out_dim,16]*/, void *y /*[out_dim,batch]*/,
                    int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
