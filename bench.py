@@ -35,6 +35,26 @@ def _avg_ms(pairs):
     return sum(a.elapsed_time(b) for a, b in pairs) / max(len(pairs), 1)
 
 
+def _launch_stats(pairs):
+    """median and minimum of the per-launch durations next to the average the roofline uses"""
+    t = sorted(a.elapsed_time(b) for a, b in pairs)
+    return {"median_launch_ms": t[len(t) // 2], "min_launch_ms": t[0]} if t else {}
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+VALU_LANE_OPS_PER_S = 256 * 64 * 2.4e9    # 256 CUs x 64 lanes x 2.4 GHz: one non-packed fp32 lane operation per lane and cycle
+
+
 def _timed(step, steps, warmup):
     """warmup untimed steps, then exactly `steps` steps between two device synchronisations."""
     import torch
@@ -150,7 +170,7 @@ def bench_c2(steps, warmup, cpu=True):
         "gate_evals_per_s": samples * width * nl / sec,
         "roofline": {"bound": "hbm", "kernel": "eval_packed_walk_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": C2_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": alg_bytes,
-                     "avg_launch_ms": kernel_ms, "launches_timed": len(pairs),
+                     "avg_launch_ms": kernel_ms, **_launch_stats(pairs), "launches_timed": len(pairs),
                      "plain_copy_GBps_same_size": copy_gbs},
     }
     if cpu:
@@ -190,9 +210,25 @@ def cpu_c2(layers, x0):
         el = time.perf_counter() - t0
         if el > 10.0 or reps >= 2000:
             break
-    return {"value": words * 64 * reps / el, "unit": "samples/s", "cores": threads, "kind": "port",
-            "sample": f"full C2 workload (3 layers x {width} neurons x {words * 64} samples), {reps} passes in {el:.1f} s, "
-                      f"oracle/packed_oracle.c with OpenMP"}
+    res = {"value": words * 64 * reps / el, "unit": "samples/s", "cores": threads, "kind": "port",
+           "sample": f"full C2 workload (3 layers x {width} neurons x {words * 64} samples), {reps} passes in {el:.1f} s, "
+                     f"oracle/packed_oracle.c with OpenMP", "cpu_model": _cpu_model(), "host_cores": os.cpu_count()}
+    try:                                                     # the same on one thread, for about 3 s
+        omp = ctypes.CDLL("libgomp.so.1")
+        omp.omp_set_num_threads(1)
+        one_pass()
+        reps1, t0 = 0, time.perf_counter()
+        while True:
+            one_pass()
+            reps1 += 1
+            el1 = time.perf_counter() - t0
+            if el1 > 3.0:
+                break
+        omp.omp_set_num_threads(threads)
+        res["value_one_thread"] = words * 64 * reps1 / el1
+    except (OSError, AttributeError):
+        pass
+    return res
 
 
 # ------------------------------------------------------------------------------------------------
@@ -351,7 +387,11 @@ def bench_conv(key, steps, warmup, cpu=True):
            "value_hip_graph": (gate_evals / (graph_ms * 1e-3) / 1e9) if graph_ms else None, "kernel_ms": ms, "kernels_only_Ggate_evals_per_s": gate_evals / (total_ms * 1e-3) / 1e9,
            "roofline": _roof("convblock fwd + bwd_x + bwd_w kernels", alg_f + alg_b, total_ms,
                              {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
-                              "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked"})}
+                              # lane-operation floor of the forward: 3 FMAs per gate evaluation, non-packed fp32
+                              "valu_floor_forward_ms": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3,
+                              "valu_frac_forward": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3 / ms["fwd"],
+                              "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
+                                      "the lane-operation floor (39.3 T fp32 lane-ops/s) beside it"})}
     def cpu_leg():
         from oracle import convlogic_oracle as O            # the CPU baseline is the only user of the oracle here
 
