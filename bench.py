@@ -496,6 +496,19 @@ def bench_c5(steps, warmup, cpu=True):
                                "ms_network_only": net_ms, "ms_with_threshold_pack": el * 1e3,
                                "note": "float32 images [65536,3,32,32] resident in HBM -> thresholds + bit packing -> 4 packed blocks, "
                                        "flatten, 3 packed LogicLayers, per-class counts"}
+    # the same at the training batch (256 samples = 4 words per feature): latency of the launch chain
+    small = vb[:n].contiguous()
+    ev = _events(max(steps, 5))
+    with torch.no_grad():
+        for _ in range(2):
+            model(binarize.pack_thresholds(small, thr))
+        torch.cuda.synchronize()
+        for a_, b_ in ev:
+            a_.record()
+            model(binarize.pack_thresholds(small, thr))
+            b_.record()
+        torch.cuda.synchronize()
+    out["packed_inference"]["ms_at_256_samples_with_threshold_pack"] = _avg_ms(ev)
     if cpu:
         out["_cpu"] = lambda: _cpu_c5(model, x, labels, ge // n)
     return out
