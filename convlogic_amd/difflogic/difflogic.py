@@ -164,8 +164,9 @@ class LogicLayer(torch.nn.Module):
 
 
 class _FeatureMajor(torch.autograd.Function):
-    """[batch, features] -> contiguous [features, batch] through the tiled HIP transpose; the gradient
-    is handed back as a transposed view."""
+    """[batch, features] -> contiguous [features, batch] through the tiled HIP transpose, and the same for the
+    gradient on the way back: whoever receives it (a leaf's .grad, Flatten, a conv block) wants it contiguous, and
+    a transposed view would be copied there by a generic strided kernel."""
 
     @staticmethod
     def forward(ctx, x):
@@ -173,6 +174,8 @@ class _FeatureMajor(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad):
+        if grad.is_cuda and grad.is_contiguous() and grad.element_size() in (1, 2, 4, 8):
+            return difflogic_hip.transpose(grad)
         return grad.transpose(0, 1)
 
 
