@@ -449,23 +449,25 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
 }
 
 // ---- 2-D transpose through a padded LDS tile -------------------------------------------------
-template <typename T>
+// TILE x TILE elements per workgroup of 256 threads; the 32 x 32 tile gives small matrices four times as many workgroups.
+template <typename T, int TILE>
 __global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t rows,
                                                       int64_t cols)
 {
-    __shared__ T tile[64][65];
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    __shared__ T tile[TILE][TILE + 1];
+    constexpr int RPP = 256 / TILE;                                  // tile rows covered per pass
+    const int tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+    const int64_t r0 = (int64_t)blockIdx.y * TILE, c0 = (int64_t)blockIdx.x * TILE;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        const int64_t r = r0 + ty + 4 * k, c = c0 + tx;
-        if (r < rows && c < cols) tile[ty + 4 * k][tx] = src[r * cols + c];
+    for (int k = 0; k < TILE / RPP; ++k) {
+        const int64_t r = r0 + ty + RPP * k, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + RPP * k][tx] = src[r * cols + c];
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        const int64_t c = c0 + ty + 4 * k, r = r0 + tx;
-        if (r < rows && c < cols) dst[c * rows + r] = tile[tx][ty + 4 * k];
+    for (int k = 0; k < TILE / RPP; ++k) {
+        const int64_t c = c0 + ty + RPP * k, r = r0 + tx;
+        if (r < rows && c < cols) dst[c * rows + r] = tile[tx][ty + RPP * k];
     }
 }
 
@@ -771,17 +773,25 @@ extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64
 {
     CLG_REQUIRE(src && dst, "clg_transpose_2d: null pointer argument");
     CLG_REQUIRE(rows > 0 && cols > 0, "clg_transpose_2d: rows and cols must be positive");
-    const int64_t gx = clg_ceil_div(cols, 64), gy = clg_ceil_div(rows, 64);
+    const bool small = clg_ceil_div(cols, 64) * clg_ceil_div(rows, 64) < 2048;     // few 64 x 64 tiles: take 32 x 32 ones
+    const int tile = small ? 32 : 64;
+    const int64_t gx = clg_ceil_div(cols, tile), gy = clg_ceil_div(rows, tile);
     CLG_REQUIRE(gy <= 65535, "clg_transpose_2d: more than 65535*64 rows are not supported");
     const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
     hipStream_t st = clg_stream(stream);
+#define CLG_TRANSPOSE(U)                                                                                                \
+    do {                                                                                                               \
+        if (small) hipLaunchKernelGGL((transpose_kernel<U, 32>), grid, block, 0, st, (const U *)src, (U *)dst, rows, cols); \
+        else hipLaunchKernelGGL((transpose_kernel<U, 64>), grid, block, 0, st, (const U *)src, (U *)dst, rows, cols);   \
+    } while (0)
     switch (elem_size) {
-    case 1: hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, block, 0, st, (const uint8_t *)src, (uint8_t *)dst, rows, cols); break;
-    case 2: hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, block, 0, st, (const uint16_t *)src, (uint16_t *)dst, rows, cols); break;
-    case 4: hipLaunchKernelGGL(transpose_kernel<uint32_t>, grid, block, 0, st, (const uint32_t *)src, (uint32_t *)dst, rows, cols); break;
-    case 8: hipLaunchKernelGGL(transpose_kernel<uint64_t>, grid, block, 0, st, (const uint64_t *)src, (uint64_t *)dst, rows, cols); break;
+    case 1: CLG_TRANSPOSE(uint8_t); break;
+    case 2: CLG_TRANSPOSE(uint16_t); break;
+    case 4: CLG_TRANSPOSE(uint32_t); break;
+    case 8: CLG_TRANSPOSE(uint64_t); break;
     default: CLG_REQUIRE(false, "clg_transpose_2d: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
     }
+#undef CLG_TRANSPOSE
     CLG_CHECK_LAUNCH("clg_transpose_2d");
     return CLG_OK;
 }
