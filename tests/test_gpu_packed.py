@@ -93,6 +93,50 @@ def test_eval_packed_config2_row_shape_properties():
     assert torch.equal(~got_c, got)
 
 
+def test_eval_packed_config2_full_size_properties():
+    # BASELINE config 2 at full size: 64000 -> 64000 neurons, 65536 samples in 1024 int64 words per feature (524 MB per
+    # tensor), through the module path (walk-ordered kernel).  Checked by properties the size does not change:
+    # pass-through gates reproduce the wired input rows (against torch's own gather), the walk-ordered kernel equals
+    # the plain one on random gates, and complemented gates on complemented inputs complement the output.
+    torch.manual_seed(2)
+    width, words = 64000, 1024
+    x = torch.randint(-2**63, 2**63 - 1, (width, words), dtype=torch.int64, device=DEV)
+    layer = C.LogicLayer(width, width, implementation="cuda").to(DEV).eval()
+    packed = C.PackBitsTensor.__new__(C.PackBitsTensor)
+    packed.bit_count, packed.pad_len, packed.t = 64, 0, x
+    with torch.no_grad():
+        layer.weights.zero_()
+        layer.weights[: width // 2, 3] = 1.0                        # gate 3: A
+        layer.weights[width // 2:, 5] = 1.0                         # gate 5: B
+        out = layer(packed).t
+        assert torch.equal(out[: width // 2], x[layer.indices_0[: width // 2]])
+        assert torch.equal(out[width // 2:], x[layer.indices_1[width // 2:]])
+        del out
+        layer.weights.copy_(torch.randn_like(layer.weights))
+        gate = layer.weights.argmax(-1).to(torch.uint8)
+        packed.t = x
+        walked = layer(packed).t
+        plain = difflogic_hip.eval(x, layer.indices_0, layer.indices_1, gate)
+        assert torch.equal(walked, plain)
+        del plain
+        comp = torch.tensor([15 - ((g & 8) >> 3 | (g & 4) >> 1 | (g & 2) << 1 | (g & 1) << 3) for g in range(16)],
+                            dtype=torch.uint8, device=DEV)
+        got_c = difflogic_hip.eval(~x, layer.indices_0, layer.indices_1, comp[gate.long()])
+        assert torch.equal(~got_c, walked)
+        # per-class counts of the full tensor: every sample's ten counts sum to the number of set bits in its column
+        counts = difflogic_hip.groupbitsum(walked, 0, 10)
+        assert counts.shape == (65536, 10) and int(counts.sum().item()) == _popcount_sum(walked)
+
+
+def _popcount_sum(words):
+    """number of set bits of an int64 tensor, on the GPU, 16 bits at a time through a lookup table"""
+    table = torch.tensor([bin(i).count("1") for i in range(65536)], dtype=torch.int64, device=words.device)
+    total = 0
+    for shift in (0, 16, 32, 48):
+        total += int(table[((words >> shift) & 0xFFFF)].sum().item())
+    return total
+
+
 def test_packed_errors():
     x = torch.zeros(8, 4, dtype=torch.bool, device=DEV)
     with pytest.raises(ValueError):
