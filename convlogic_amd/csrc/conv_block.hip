@@ -631,26 +631,8 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
     const uint32_t f_pos = (2 * f_py) * row_step + (2 * f_px) * g.sw;
     const uint32_t f_out = (uint32_t)(kernel_row + f_cell);
     const uint32_t f_n0 = blockIdx.x * per_block + threadIdx.x / (uint32_t)I, f_step = (uint32_t)nb * per_block;
-    for (uint32_t it = FIXED ? f_n0 : blockIdx.x * 256 + threadIdx.x; it < (FIXED ? (uint32_t)g.n : items);
-         it += FIXED ? f_step : (uint32_t)nb * 256) {
-        int code, pos;
-        T gout;
-        if (FIXED) {
-            const uint32_t o = it * (uint32_t)sample_cells + f_out;
-            code = load_at(argmax, o);
-            gout = load_at(gy, o);
-            pos = (int)(it * (uint32_t)sample_elems + f_pos) + (code >> 1) * row_step + (code & 1) * g.sw;
-        } else {
-            const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
-            const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
-            const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
-            code = argmax[o];
-            gout = gy[o];
-            pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
-        }
-        T tv[8];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(pos + to[t]));
+    // tree, upstream gradients and the 28 sums of one pooled cell
+    auto accumulate = [&](const T (&tv)[8], T gout) {
         const TreeVals<T> v = eval_tree(tr, tv);
         T gin[7][2], gg[7];
         gg[6] = gout;
@@ -676,6 +658,31 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
             acc[4 * k + 1] = fma_t(gg[k], gin[k][0], acc[4 * k + 1]);
             acc[4 * k + 2] = fma_t(gg[k], gin[k][1], acc[4 * k + 2]);
             acc[4 * k + 3] += gg[k];
+        }
+    };
+    if (FIXED) {
+        for (uint32_t it = f_n0; it < (uint32_t)g.n; it += f_step) {
+            const uint32_t o = it * (uint32_t)sample_cells + f_out;
+            const int code = load_at(argmax, o);
+            const T gout = load_at(gy, o);
+            const int pos = (int)(it * (uint32_t)sample_elems + f_pos) + (code >> 1) * row_step + (code & 1) * g.sw;
+            T tv[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(pos + to[t]));
+            accumulate(tv, gout);
+        }
+    } else {
+        for (uint32_t it = blockIdx.x * 256 + threadIdx.x; it < items; it += (uint32_t)nb * 256) {
+            const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
+            const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
+            const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
+            const int code = argmax[o];
+            const T gout = gy[o];
+            const int pos = (int)(n * (uint32_t)sample_elems) + (int)((2 * py + (code >> 1)) * row_step + (2 * px + (code & 1)) * g.sw);
+            T tv[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) tv[t] = load_at(xp, (uint32_t)(pos + to[t]));
+            accumulate(tv, gout);
         }
     }
     block_sum_store<T, 28, 256>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 28);
@@ -841,6 +848,14 @@ struct WScratch {
 };
 // The padded weight-gradient kernel keeps a thread on one pooled cell when the cells of a sample divide its 256 threads
 // and grad_y / arg-max can be addressed with 32-bit byte offsets.
+// Pooled cells a thread of the padded weight-gradient kernel sums before the block reduction (28 wavefront sums per
+// block): 16 when a kernel has at least 64 Ki cells (89 vs 92 us at [256,9,32,32] -> 256), else 8 (25.5 vs 29 us at
+// [256,32,16,16] -> 128, where more would leave too few workgroups).
+int cells_per_thread(int64_t cells_per_kernel)
+{
+    if (const char *e = getenv("CLG_BWDW_CELLS")) return atoi(e) > 0 ? atoi(e) : 8;
+    return cells_per_kernel >= 65536 ? 16 : 8;
+}
 bool fixed_cells(const Geom &g, int elem)
 {
     const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
@@ -860,7 +875,7 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     if (sample_elems_max * g.n * elem >= (1ll << 32) || I * g.n >= (1ll << 31)) return false;
     p->d_slots = make_fastdiv((uint32_t)p->chs);                    // reused as "divide by plane stride"
     ws->sample_elems = (int)sample_elems;
-    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);                   // about 8 cells per thread (4..64 measured within 10 %)
+    int64_t nb = clg_ceil_div(I * g.n, 256 * cells_per_thread(I * g.n));
     ws->nb = (int)(nb < 1 ? 1 : (nb > 64 ? 64 : nb));
     ws->folded_off = ((size_t)g.c * 64 * 28 * elem + 255) & ~(size_t)255;   // partials sized for 64 blocks
     ws->taps_off = (ws->folded_off + (size_t)g.c * 28 * elem + 255) & ~(size_t)255;
@@ -999,7 +1014,7 @@ int launch_backward_w_shared(const Geom &g, const SharedPad &sh, const void *gy,
                              hipStream_t st, const void *probs)
 {
     const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
-    int64_t nb = clg_ceil_div(I * g.n, 256 * 8);
+    int64_t nb = clg_ceil_div(I * g.n, 256 * cells_per_thread(I * g.n));
     nb = nb < 1 ? 1 : (nb > 64 ? 64 : nb);
     T *partial = reinterpret_cast<T *>(scratch);                      // [c][nb][28], within the any-shape kernel's [c][64][28]
     if (fixed_cells(g, (int)sizeof(T)))
