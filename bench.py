@@ -590,9 +590,19 @@ def bench_large(steps, warmup, cpu=True):
         opt.step()
 
     sec = _timed(step, max(3, steps // 4), max(2, warmup // 2))
+
+    # the same step without the optimizer: what the kernels of this repository take (AdamW is torch's foreach implementation,
+    # the reference's default, `src/convlogic/model.py:180`)
+    def step_no_opt(_k):
+        for p in model.parameters():
+            p.grad = None
+        torch.nn.functional.cross_entropy(model(x), labels).backward()
+
+    sec_no_opt = _timed(step_no_opt, max(3, steps // 4), 2)
     return {"workload": f"cifar10_l topology: ConvLogicCifarModel k={k}, {cin} input channels, batch {n}, float32 training step "
                         "(fwd + CE loss + bwd + AdamW), residual init",
             "metric": "convlogic_fwd_bwd_Ggate_evals_per_s", "value": ge / sec / 1e9, "unit": "Ggate-evals/s", "ms_per_step": sec * 1e3,
+            "ms_per_step_without_optimizer": sec_no_opt * 1e3,
             "dtype": "f32", "parameters": sum(p.numel() for p in model.parameters()),
             "roofline": _roof("whole training step incl. AdamW (all kernels)", alg, sec * 1e3),
             "reference_anchor": "not a published kernel number: the reference README quotes ~45 s per epoch on an RTX 4090 for this model, "
@@ -686,7 +696,7 @@ def main():
             "roofline": primary["roofline"], "cpu_baseline": primary.get("cpu_baseline"),
             "device": torch.cuda.get_device_name(0), "host_cores": os.cpu_count()}
     for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s", "kernels", "packed_inference",
-                  "ms_per_step_hip_graph", "value_hip_graph"):
+                  "ms_per_step_hip_graph", "value_hip_graph", "ms_per_step_without_optimizer", "parameters", "reference_anchor"):
         if extra in primary:
             line[extra] = primary[extra]
     if also:
