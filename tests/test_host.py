@@ -41,6 +41,21 @@ def test_c_abi_rejects_bad_arguments_without_gpu():
     assert b"divisible by 2" in lib.clg_last_error()
 
 
+def test_missing_library_fails_loudly_and_product_never_imports_the_oracle(monkeypatch):
+    # no silent fallback: without the built library the "cuda" implementation raises, naming the build step
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "convlogic_amd", "no_such_library.so"))
+    assert not _lib.available()
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
+    # and nothing under the package imports, opens or names the oracle
+    for folder, _, files in os.walk(os.path.join(ROOT, "convlogic_amd")):
+        for name in files:
+            if name.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(folder, name)).read()
+                assert "oracle" not in text, os.path.join(folder, name)
+
+
 @pytest.mark.parametrize("i", range(16))
 def test_bin_op_matches_oracle(i):
     a, b = torch.rand(20, dtype=torch.float64), torch.rand(20, dtype=torch.float64)
