@@ -635,7 +635,7 @@ def bench_stream(steps, warmup, cpu=True):
     batch, feats = 8192, 64000
     t = torch.randint(0, 2, (batch, feats), device=dev, dtype=torch.uint8).bool()
     ms = timed(lambda: difflogic_hip.tensor_packbits_sample_major(t, 64))
-    res.append(dict(_roof("pack_bits_sm_kernel", batch * feats + batch * feats // 8, ms),
+    res.append(dict(_roof("pack_bits_tile_kernel", batch * feats + batch * feats // 8, ms),
                     workload=f"PackBitsTensor: bool [{batch},{feats}] -> int64 words [{feats},{batch // 64}]"))
     del t
     words = torch.randint(-2**63, 2**63 - 1, (feats, 1024), device=dev, dtype=torch.int64)

@@ -16,7 +16,10 @@ TORCH_WORD = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
 
 @pytest.mark.parametrize("bits", [8, 16, 32, 64])
 @pytest.mark.parametrize("batch,features", [(1, 1), (7, 3), (64, 5), (100, 130), (129, 257), (1000, 33), (4096, 16), (70, 48),
-                                            (257, 1024), (64, 4112), (5, 32)])
+                                            (257, 1024), (64, 4112), (5, 32),
+                                            # 8..15 and >= 16 groups of 64 samples with 16 | features: the LDS-transposing kernels,
+                                            # ragged last group, last word and last feature tile
+                                            (1000, 48), (600, 160), (1030, 32), (520, 4112), (2049, 528)])
 def test_pack_bits_both_layouts(bits, batch, features):
     rng = np.random.default_rng(batch * 7 + features)
     t = rng.integers(0, 2, (batch, features)).astype(bool)
