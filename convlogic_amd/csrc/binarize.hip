@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void threshold_pack_kernel(const float *__rest
     }
 #pragma unroll
     for (int l = 0; l < kLevelsPerPass; ++l)
-        if (l0 + l < levels) words[(g * levels + l0 + l) * plane_elems + e] = w[l];
+        if (l0 + l < levels) __builtin_nontemporal_store(w[l], &words[(g * levels + l0 + l) * plane_elems + e]);
 }
 
 __global__ __launch_bounds__(256) void threshold_float_kernel(const float *__restrict__ x, const float *__restrict__ thr,
