@@ -279,10 +279,9 @@ __global__ __launch_bounds__(256) void pack_bits_smv_kernel(const uint8_t *__res
 // row with consecutive lanes and streaming stores.  The 8-byte stores of the kernel above, scattered over rows, cost a
 // third of its time (155 us against 100 us without them on bool [8192, 64000]).
 template <int FL, int SG>
-__global__ __launch_bounds__(256) void pack_bits_tile_kernel(const uint8_t *__restrict__ t, uint8_t *__restrict__ out,
+__global__ __launch_bounds__(FL *SG) void pack_bits_tile_kernel(const uint8_t *__restrict__ t, uint8_t *__restrict__ out,
                                                            int64_t features, int64_t batch, int64_t row_bytes)
 {
-    static_assert(FL * SG == 256, "one thread per (feature lane, sample group)");
     __shared__ uint64_t tile[FL * 16][SG + 1];
     const int fl = threadIdx.x % FL, sg = threadIdx.x / FL;
     const int64_t f0 = ((int64_t)blockIdx.x * FL + fl) * 16;
@@ -329,7 +328,7 @@ __global__ __launch_bounds__(256) void pack_bits_tile_kernel(const uint8_t *__re
     }
     __syncthreads();
     const int64_t frow0 = (int64_t)blockIdx.x * FL * 16, grp0 = (int64_t)blockIdx.y * SG;
-    for (int idx = threadIdx.x; idx < FL * 16 * SG; idx += 256) {
+    for (int idx = threadIdx.x; idx < FL * 16 * SG; idx += FL * SG) {
         const int row = idx / SG, w = idx % SG;
         const int64_t f = frow0 + row, byte0 = (grp0 + w) * 8;
         if (f >= features || byte0 >= row_bytes) continue;
@@ -583,14 +582,15 @@ extern "C" int clg_pack_bits_sample_major(const uint8_t *t, void *words, int64_t
     const int64_t groups = clg_ceil_div(batch, 64);
     if (features % 16 == 0 && ((uintptr_t)t & 15) == 0 && ((uintptr_t)words & 7) == 0 && groups <= 65535) {
         // 16 features per lane, 2 groups per thread: best of 4..16 features x 2..16 groups (3.8 TB/s on bool [8192, 64000])
-        // from 16 (8) groups of 64 samples on, the words go through LDS and leave as 128 (64) contiguous bytes per feature
-        // row: 155 -> 133 us on bool [8192, 64000], 101 -> 60 us on [65536, 4096]; CLG_PACK_TILE=0 keeps the direct stores
+        // from 8 groups of 64 samples on, the words go through LDS and leave as 64 (8..15 groups) or 128 contiguous bytes per
+        // feature row: 155 -> 121 us on bool [8192, 64000], 101 -> 52 us on [65536, 4096] with 32 feature lanes x 16 groups
+        // (512 threads; 16 x 16 and 64 x 8 are 8 % slower); CLG_PACK_TILE=0 keeps the direct stores
         const char *e_tile = getenv("CLG_PACK_TILE");
-        const int tile = e_tile ? atoi(e_tile) : (groups >= 16 ? 16 : 8);
-        if (tile == 16 && groups >= 16)
-            hipLaunchKernelGGL((pack_bits_tile_kernel<16, 16>), dim3((unsigned)clg_ceil_div(features, 16 * 16), (unsigned)clg_ceil_div(groups, 16)),
-                               dim3(256), 0, clg_stream(stream), t, (uint8_t *)words, features, batch, row_bytes);
-        else if (tile >= 8 && groups >= 8)
+        const bool tiled = !e_tile || atoi(e_tile) != 0;
+        if (tiled && groups >= 16)
+            hipLaunchKernelGGL((pack_bits_tile_kernel<32, 16>), dim3((unsigned)clg_ceil_div(features, 32 * 16), (unsigned)clg_ceil_div(groups, 16)),
+                               dim3(512), 0, clg_stream(stream), t, (uint8_t *)words, features, batch, row_bytes);
+        else if (tiled && groups >= 8)
             hipLaunchKernelGGL((pack_bits_tile_kernel<32, 8>), dim3((unsigned)clg_ceil_div(features, 32 * 16), (unsigned)clg_ceil_div(groups, 8)),
                                dim3(256), 0, clg_stream(stream), t, (uint8_t *)words, features, batch, row_bytes);
         else
