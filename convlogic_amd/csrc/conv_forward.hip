@@ -35,7 +35,7 @@ namespace {
 // second row's reads then use the immediate offset of the LDS instruction), 0 = read it from the plan.
 // SUBSET: stage two planes per kernel of the tile instead of all input channels.
 // ONE_ROW: a lane slot is one conv position instead of a column of two rows (plan.one_row; compile-time so that the
-// two-row loop carries nothing of it).
+// two-row loop carries nothing of it); ROWSTEP is then wo if that is 8 or 4 (and all channels are staged), else 0.
 template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW>
 __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
                                                const int32_t *__restrict__ sel, typename Ops::Elem *__restrict__ y,
@@ -134,6 +134,57 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     const int items = ct_cur * nblk;
     const int per = (items + p.NW - 1) / p.NW;
     const int first = wave * per, last = min(items, first + per);
+    if constexpr (ONE_ROW && !SUBSET) {
+        // One block of lane slots (at most 64 positions per workgroup), so an item is a kernel.  The wavefront holds few
+        // instructions in flight per kernel (parameters -> tap reads -> gates -> pooling), and the workgroup's LDS
+        // image keeps other workgroups off the CU: two kernels per step double what is in flight.
+        const bool valid = lane < U;
+        const int2 e = slot[valid ? lane : 0];
+        const bool store_lane = valid && writer_lane;
+        const int64_t obase = ((int64_t)n0 * g.c + c0) * I + e.y;
+        // the row below sits wo lanes up: a DPP row shift when ROWSTEP names wo (8 or 4), else ds_bpermute
+        auto below = [&](T v) {
+            if constexpr (ROWSTEP == 8 || ROWSTEP == 4) return row_up<ROWSTEP>(v);
+            else return lane_up(v, g.wo);
+        };
+        constexpr int K = 2;                                          // 3 and 4 measured the same
+        for (int lc = first; lc < last; lc += K) {
+            int lk[K];
+            typename Ops::Params pr[K];
+            T v[K][8], r[K], ro[K], r1[K], r1o[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                lk[k] = min(lc + k, last - 1);
+                pr[k] = Ops::load(coef, lk[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[k][t] = xs[e.x + toff[lk[k] * 8 + t]];    // offsets stay vector values
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                r[k] = Ops::root(pr[k], v[k]);
+                ro[k] = dpp_xor1(r[k]);
+                if constexpr (Ops::kOrPool) {                         // the row first, then one exchange with the row below
+                    ro[k] = Ops::join(pr[k], r[k], ro[k]);
+                    r1o[k] = below(ro[k]);
+                } else {
+                    r1[k] = below(r[k]);
+                    r1o[k] = below(ro[k]);
+                }
+            }
+            if (store_lane) {
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (k > 0 && lc + k >= last) continue;
+                    if constexpr (Ops::kOrPool) y[obase + lk[k] * I] = Ops::join_last(pr[k], ro[k], r1o[k]);
+                    else Ops::pool_store(r[k], ro[k], r1[k], r1o[k], y + obase, argmax ? argmax + obase : nullptr, lk[k] * I);
+                }
+            }
+        }
+        return;
+    }
     int lc = first / nblk, blk = first - lc * nblk;
     for (int item = first; item < last;) {
         const typename Ops::Params pr = Ops::load(coef, lc);
@@ -175,15 +226,27 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
                     r1 = Ops::root(pr, v);
                 }
             }
-            const T r0o = dpp_xor1(r0);
-            T r1o;
-            if (ONE_ROW) {                                            // the row below sits wo lanes up (2 wo divides 64)
-                r1 = lane_up(r0, g.wo);
-                r1o = lane_up(r0o, g.wo);
+            if constexpr (Ops::kOrPool) {                             // OR pool: any order, one exchange per direction
+                T m;
+                if (ONE_ROW) {
+                    m = Ops::join(pr, r0, dpp_xor1(r0));
+                    m = Ops::join_last(pr, m, lane_up(m, g.wo));
+                } else {
+                    m = Ops::join(pr, r0, r1);
+                    m = Ops::join_last(pr, m, dpp_xor1(m));
+                }
+                if (valid && writer_lane) yb[e.y] = m;
             } else {
-                r1o = dpp_xor1(r1);
+                const T r0o = dpp_xor1(r0);
+                T r1o;
+                if (ONE_ROW) {                                        // the row below sits wo lanes up (2 wo divides 64)
+                    r1 = lane_up(r0, g.wo);
+                    r1o = lane_up(r0o, g.wo);
+                } else {
+                    r1o = dpp_xor1(r1);
+                }
+                if (valid && writer_lane) Ops::pool_store(r0, r0o, r1, r1o, yb, ab, e.y);
             }
-            if (valid && writer_lane) Ops::pool_store(r0, r0o, r1, r1o, yb, ab, e.y);
         }
         blk = 0;
         ++lc;
@@ -232,8 +295,13 @@ __global__ __launch_bounds__(256) void convblock_forward_direct_kernel(const typ
 #pragma unroll
         for (int t = 0; t < 8; ++t) v1[t] = load_at(xp, (uint32_t)(base + row_step + to[t]));
         const T r0 = Ops::root(pr, v0), r1 = Ops::root(pr, v1);
-        const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
-        if (writer) Ops::pool_store(r0, r0o, r1, r1o, y + obase + (int64_t)c * I, argmax ? argmax + obase + (int64_t)c * I : nullptr, 0);
+        if constexpr (Ops::kOrPool) {
+            const T m = Ops::join(pr, r0, r1), pooled = Ops::join_last(pr, m, dpp_xor1(m));
+            if (writer) y[obase + (int64_t)c * I] = pooled;
+        } else {
+            const T r0o = dpp_xor1(r0), r1o = dpp_xor1(r1);
+            if (writer) Ops::pool_store(r0, r0o, r1, r1o, y + obase + (int64_t)c * I, argmax ? argmax + obase + (int64_t)c * I : nullptr, 0);
+        }
     }
 }
 
@@ -248,16 +316,14 @@ __global__ __launch_bounds__(256) void convblock_packed_generic_kernel(const uin
     if (item >= (int64_t)g.n * I) return;
     const int n = (int)(item / I), cell = (int)(item - (int64_t)n * I);
     const int py = cell / wp, px = cell - py * wp;
-    BitOps::Params pr;
-#pragma unroll
-    for (int k = 0; k < 7; ++k) pr.m[k] = gate_masks(gid[(int64_t)c * 7 + k] & 15);
+    const BitOps::Params pr = BitOps::load_global(gid, c);
     const uint64_t *xn = x + (int64_t)n * g.cin * g.h * g.w;
     uint64_t acc = 0;
     for (int q = 0; q < 4; ++q) {
         uint64_t v[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t]), 2 * py + (q >> 1), 2 * px + (q & 1));
-        acc |= BitOps::root(pr, v);
+        acc |= BitOps::root_true(pr, v);
     }
     y[((int64_t)n * g.c + c) * I + cell] = acc;
 }
@@ -465,9 +531,12 @@ int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const 
     case RS:                                                                                                          \
         return p.subset ? launch_forward_one<Ops, RS, true>(g, p, x, params, sel, y, argmax, st, name)                \
                         : launch_forward_one<Ops, RS, false>(g, p, x, params, sel, y, argmax, st, name)
-    if (p.one_row)                                                   // few positions per sample: the row step is not worth a variant
-        return p.subset ? launch_forward_one<Ops, 0, true, true>(g, p, x, params, sel, y, argmax, st, name)
-                        : launch_forward_one<Ops, 0, false, true>(g, p, x, params, sel, y, argmax, st, name);
+    if (p.one_row) {                                                 // ROWSTEP names wo when a DPP row shift reaches the row below
+        if (p.subset) return launch_forward_one<Ops, 0, true, true>(g, p, x, params, sel, y, argmax, st, name);
+        if (g.wo == 8) return launch_forward_one<Ops, 8, false, true>(g, p, x, params, sel, y, argmax, st, name);
+        if (g.wo == 4) return launch_forward_one<Ops, 4, false, true>(g, p, x, params, sel, y, argmax, st, name);
+        return launch_forward_one<Ops, 0, false, true>(g, p, x, params, sel, y, argmax, st, name);
+    }
     switch (g.sh * p.rs) {
         CLG_FWD_CASE(33);
         CLG_FWD_CASE(29);
@@ -513,8 +582,16 @@ extern "C" int clg_convblock_eval_packed(const clg_conv_geom *gg, const uint64_t
     const char *e_4x4 = getenv("CLG_FWD_4X4");
     if (clg_convblock_is_4x4(g) && (!e_4x4 || atoi(e_4x4) != 0))
         return clg_convblock_eval_packed_4x4(g, x, gates, selection, y, st, "clg_convblock_eval_packed");
-    if (plan_forward(g, 8, BitOps::kParams, &p))
+    if (plan_forward(g, 8, BitOps::kParams, &p)) {
+        // one position per lane: a wavefront meets every kernel once, so the gates take the form without vector masks
+        if (p.one_row && !p.subset) {
+            const char *name = "clg_convblock_eval_packed";
+            if (g.wo == 8) return launch_forward_one<BitOpsAnf, 8, false, true>(g, p, x, gates, selection, y, nullptr, st, name);
+            if (g.wo == 4) return launch_forward_one<BitOpsAnf, 4, false, true>(g, p, x, gates, selection, y, nullptr, st, name);
+            return launch_forward_one<BitOpsAnf, 0, false, true>(g, p, x, gates, selection, y, nullptr, st, name);
+        }
         return launch_forward_tiled<BitOps>(g, p, x, gates, selection, y, nullptr, st, "clg_convblock_eval_packed");
+    }
     const int64_t blocks = clg_ceil_div((int64_t)g.n * (g.ho / 2) * (g.wo / 2), 256);
     CLG_REQUIRE(g.c <= 65535 && blocks < (1ll << 31), "clg_convblock_eval_packed: problem too large for one launch");
     hipLaunchKernelGGL(convblock_packed_generic_kernel, dim3((unsigned)blocks, (unsigned)g.c), dim3(256), 0, st, x, gates, selection, y,

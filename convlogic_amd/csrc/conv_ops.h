@@ -12,6 +12,7 @@ template <typename T>
 struct FloatOps {
     using Elem = T;
     static constexpr int kParams = 28;                               // LDS elements per kernel: 7 gates x (ab, a, b, one)
+    static constexpr bool kOrPool = false;
     struct Params {
         Tree<T> tr;
     };
@@ -63,7 +64,7 @@ struct FloatOps {
         ab[idx] = (uint8_t)code;
     }
     // the same rule on the four values of a window in a register array
-    static __device__ __forceinline__ Elem pool4(const Elem (&r)[4], int &code)
+    static __device__ __forceinline__ Elem pool4(const Params &, const Elem (&r)[4], int &code)
     {
         Elem best = r[0];
         code = 0;
@@ -78,9 +79,13 @@ struct FloatOps {
     }
 };
 
+// Packed samples, gates as three bitwise multiplexers with the truth table as all-ones / all-zeros masks: two of the
+// four masks of a gate have to sit in vector registers (one scalar operand per instruction), which pays when a
+// wavefront evaluates a kernel at many positions.
 struct BitOps {
     using Elem = uint64_t;
     static constexpr int kParams = 1;                                // 7 gate ids, 4 bits each
+    static constexpr bool kOrPool = true;                            // the pool is an OR: any order, no arg-max
     struct Params {
         Masks m[7];
     };
@@ -123,15 +128,113 @@ struct BitOps {
         for (int q = 0; q < 4; ++q) leaf[q] = gate64(pr.m[q], v[2 * q], v[2 * q + 1]);
         return gate64(pr.m[6], gate64(pr.m[4], leaf[0], leaf[1]), gate64(pr.m[5], leaf[2], leaf[3]));
     }
-    static __device__ __forceinline__ void pool_store(Elem r0, Elem r0o, Elem r1, Elem r1o, Elem *__restrict__ yb,
-                                                      uint8_t *__restrict__, int idx)
-    {
-        yb[idx] = (r0 | r0o) | (r1 | r1o);
-    }
-    static __device__ __forceinline__ Elem pool4(const Elem (&r)[4], int &code)
+    static __device__ __forceinline__ Elem root_true(const Params &pr, const Elem (&v)[8]) { return root(pr, v); }
+    static __device__ __forceinline__ Elem join(const Params &, Elem a, Elem b) { return a | b; }
+    static __device__ __forceinline__ Elem join_last(const Params &, Elem a, Elem b) { return a | b; }
+    static __device__ __forceinline__ Elem pool4(const Params &, const Elem (&r)[4], int &code)
     {
         code = 0;
         return (r[0] | r[1]) | (r[2] | r[3]);
+    }
+};
+
+// The same for kernels that a wavefront evaluates at ONE position before it moves on (no room to amortise vector
+// masks): a gate is its algebraic normal form  y = c0 ^ (c1 & a) ^ (c2 & b) ^ (c3 & a & b)  with the constant
+// c0 moved into the truth table of the gate that consumes y (an input that arrives inverted permutes the table), so a
+// gate costs three 3-input bit operations with one scalar mask each; the root's c0 is applied once at the end.
+// tree_code(): the 7 gate ids of a kernel -> bits 3k..3k+2 = (c1, c2, c3) of gate k, bit 21 = c0 of the root.
+__host__ __device__ inline uint32_t tree_code(const uint8_t *gid)
+{
+    uint32_t code = 0;
+    int inv[7];                                                      // gate k delivers its true output xor inv[k]
+#pragma unroll
+    for (int k = 0; k < 7; ++k) {
+        const int id = gid[k] & 15;
+        const int pa = k < 4 ? 0 : inv[2 * (k - 4)], pb = k < 4 ? 0 : inv[2 * (k - 4) + 1];
+        // truth table entry for (a, b) = bit 3 - 2a - b of the gate id
+        const int f00 = (id >> (3 - 2 * pa - pb)) & 1, f01 = (id >> (3 - 2 * pa - (pb ^ 1))) & 1;
+        const int f10 = (id >> (3 - 2 * (pa ^ 1) - pb)) & 1, f11 = (id >> (3 - 2 * (pa ^ 1) - (pb ^ 1))) & 1;
+        inv[k] = f00;
+        code |= (uint32_t)((f00 ^ f10) | ((f00 ^ f01) << 1) | ((f00 ^ f01 ^ f10 ^ f11) << 2)) << (3 * k);
+    }
+    return code | ((uint32_t)inv[6] << 21);
+}
+
+struct BitOpsAnf {
+    using Elem = uint64_t;
+    static constexpr int kParams = 1;                                // tree_code of the kernel
+    static constexpr bool kOrPool = true;                            // the pool is an OR: any order, no arg-max
+    struct Params {
+        uint32_t c1[7], c2[7], c3[7], inv;                           // all-ones / all-zeros
+    };
+    static __device__ __forceinline__ Params unpack(uint32_t code)
+    {
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            pr.c1[k] = 0u - ((code >> (3 * k)) & 1u);
+            pr.c2[k] = 0u - ((code >> (3 * k + 1)) & 1u);
+            pr.c3[k] = 0u - ((code >> (3 * k + 2)) & 1u);
+        }
+        pr.inv = 0u - ((code >> 21) & 1u);
+        return pr;
+    }
+    // params = gate ids uint8 [c_out, 7]
+    static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
+                                                        int tid, int nthreads)
+    {
+        const uint8_t *gid = reinterpret_cast<const uint8_t *>(params);
+        for (int q = tid; q < ct_cur; q += nthreads) dst[q] = tree_code(gid + ((int64_t)c0 + q) * 7);
+    }
+    static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
+    {
+        return unpack((uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src[lc]));
+    }
+    static __device__ __forceinline__ Params load_global(const void *__restrict__ gates, int c)
+    {
+        return unpack(tree_code(reinterpret_cast<const uint8_t *>(gates) + (int64_t)c * 7));
+    }
+    static __device__ __forceinline__ uint32_t gate32(const Params &pr, int k, uint32_t a, uint32_t b)
+    {
+        // v_bitop3_b32 with the table spelled out (0xF0 = first, 0xCC = second, 0xAA = third operand), so that every
+        // instruction carries exactly one scalar mask
+        const uint32_t t = __builtin_amdgcn_bitop3_b32(a, b, pr.c3[k], 0xF0 & 0xCC & 0xAA);
+        const uint32_t u = __builtin_amdgcn_bitop3_b32(t, a, pr.c1[k], 0xF0 ^ (0xCC & 0xAA));
+        return __builtin_amdgcn_bitop3_b32(u, b, pr.c2[k], 0xF0 ^ (0xCC & 0xAA));
+    }
+    static __device__ __forceinline__ uint32_t root32(const Params &pr, const Elem (&v)[8], int shift)
+    {
+        uint32_t leaf[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) leaf[q] = gate32(pr, q, (uint32_t)(v[2 * q] >> shift), (uint32_t)(v[2 * q + 1] >> shift));
+        return gate32(pr, 6, gate32(pr, 4, leaf[0], leaf[1]), gate32(pr, 5, leaf[2], leaf[3]));
+    }
+    // The root WITHOUT its constant: the true value is root(...) ^ pr.inv.  The 2x2 OR pool takes the constant along:
+    // join() of raw values stays raw (OR of the true values = AND of the raw ones when they are inverted), join_last()
+    // delivers the true pooled value -- one bit operation each, where the plain form needs an XOR per position.
+    static __device__ __forceinline__ Elem root(const Params &pr, const Elem (&v)[8])
+    {
+        return ((uint64_t)root32(pr, v, 32) << 32) | root32(pr, v, 0);
+    }
+    static __device__ __forceinline__ Elem root_true(const Params &pr, const Elem (&v)[8])
+    {
+        return root(pr, v) ^ (((uint64_t)pr.inv << 32) | pr.inv);
+    }
+    template <int TABLE>
+    static __device__ __forceinline__ Elem join_as(const Params &pr, Elem a, Elem b)
+    {
+        const uint32_t lo = __builtin_amdgcn_bitop3_b32((uint32_t)a, (uint32_t)b, pr.inv, TABLE);
+        const uint32_t hi = __builtin_amdgcn_bitop3_b32((uint32_t)(a >> 32), (uint32_t)(b >> 32), pr.inv, TABLE);
+        return ((uint64_t)hi << 32) | lo;
+    }
+    // inv ? a & b : a | b      (0xF0 = a, 0xCC = b, 0xAA = inv)
+    static __device__ __forceinline__ Elem join(const Params &pr, Elem a, Elem b) { return join_as<0xD4>(pr, a, b); }
+    // inv ? ~(a & b) : a | b
+    static __device__ __forceinline__ Elem join_last(const Params &pr, Elem a, Elem b) { return join_as<0x7E>(pr, a, b); }
+    static __device__ __forceinline__ Elem pool4(const Params &pr, const Elem (&r)[4], int &code)
+    {
+        code = 0;
+        return join_last(pr, join(pr, r[0], r[1]), join(pr, r[2], r[3]));
     }
 };
 

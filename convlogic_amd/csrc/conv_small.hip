@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
                 r[q] = Ops::root(pr, v);
             }
             int code;
-            best[cell] = Ops::pool4(r, code);
+            best[cell] = Ops::pool4(pr, r, code);
             codes |= code << (8 * cell);
         }
         if (live) {

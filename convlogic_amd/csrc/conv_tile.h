@@ -68,6 +68,22 @@ __device__ __forceinline__ T lane_up(T v, int delta)
     }
 }
 
+// value of the lane DELTA lanes up inside a row of 16 lanes, as a DPP row shift (no LDS round trip); lanes whose
+// source falls outside the row read 0
+template <int DELTA, typename T>
+__device__ __forceinline__ T row_up(T v)
+{
+    static_assert(DELTA > 0 && DELTA < 16, "row shift");
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + DELTA, 0xF, 0xF, true));
+    } else {
+        const uint64_t u = __builtin_bit_cast(uint64_t, v);
+        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0x100 + DELTA, 0xF, 0xF, true);
+        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0x100 + DELTA, 0xF, 0xF, true);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ T to_sgpr(T v)
 {
