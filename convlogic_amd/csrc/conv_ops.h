@@ -128,6 +128,14 @@ struct BitOps {
         for (int q = 0; q < 4; ++q) leaf[q] = gate64(pr.m[q], v[2 * q], v[2 * q + 1]);
         return gate64(pr.m[6], gate64(pr.m[4], leaf[0], leaf[1]), gate64(pr.m[5], leaf[2], leaf[3]));
     }
+    // the same tree on 32 samples
+    static __device__ __forceinline__ uint32_t root32(const Params &pr, const uint32_t (&v)[8])
+    {
+        uint32_t leaf[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) leaf[q] = gate_bits(pr.m[q], v[2 * q], v[2 * q + 1]);
+        return gate_bits(pr.m[6], gate_bits(pr.m[4], leaf[0], leaf[1]), gate_bits(pr.m[5], leaf[2], leaf[3]));
+    }
     static __device__ __forceinline__ Elem root_true(const Params &pr, const Elem (&v)[8]) { return root(pr, v); }
     static __device__ __forceinline__ Elem join(const Params &, Elem a, Elem b) { return a | b; }
     static __device__ __forceinline__ Elem join_last(const Params &, Elem a, Elem b) { return a | b; }

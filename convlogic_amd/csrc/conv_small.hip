@@ -9,6 +9,8 @@
 // once and stays zero), a plane arrives as four 16-byte loads per lane that are requested one kernel ahead, and the
 // 16 positions x 8 taps are LDS reads at (tap address + immediate position offset).  No barriers, no bounds checks.
 // A kernel whose taps name more than two channels (possible with a caller-made selection) reads global memory.
+#include <stdlib.h>
+
 #include "conv_ops.h"
 
 namespace {
@@ -149,6 +151,102 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
                 reinterpret_cast<u32x4 *>(y + o)[q] = raw;
             }
             if (argmax != nullptr) *reinterpret_cast<uint32_t *>(argmax + o) = (uint32_t)codes;
+        }
+        if (!more) break;
+        c = cn;
+    }
+}
+
+// Packed words, one group of 64 samples per lane, evaluated as two halves of 32 samples: the lane's LDS slice holds
+// 4-byte elements, so a workgroup takes half the LDS of the 8-byte variant and two of them share a CU (the kernel is
+// bound by what a wavefront has in flight, not by arithmetic).  Order per kernel: low halves to LDS, evaluate, high
+// halves to LDS, request the next kernel's planes, evaluate, store 64-bit words.
+__global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_kernel(const uint64_t *__restrict__ x,
+                                                                                  const uint8_t *__restrict__ gates,
+                                                                                  const int32_t *__restrict__ sel,
+                                                                                  uint64_t *__restrict__ y, Geom g, int ct)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
+    uint32_t *mine = reinterpret_cast<uint32_t *>(smem) + ((size_t)wave * kWave + lane) * kLsStride;
+    const int64_t n = (int64_t)blockIdx.x * kWave + lane;
+    const bool live = n < g.n;
+    const uint64_t *xn = x + (live ? n : 0) * g.cin * 16;
+#pragma unroll
+    for (int e = 0; e < kLsStride; ++e) mine[e] = 0u;
+    const int c0 = blockIdx.y * ct, c1 = min(g.c, c0 + ct);
+    int c = c0 + wave;
+    if (c >= c1) return;
+    LaneTaps tp = lane_taps(sel, c);
+    Planes<uint64_t> pl;
+    fetch_planes(pl, tp, xn, live);
+    while (true) {
+        const BitOps::Params pr = BitOps::load_global(gates, c);
+        const LaneTaps cur = tp;
+        const int cn = c + kLsWaves;
+        const bool more = cn < c1;
+        const uint32_t *ta[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ta[k] = mine + (cur.ch[k] != cur.ch0 ? kLsPlane : 0) + cur.ry[k] * 6 + cur.rx[k];
+        if (cur.wide) {
+            // taps in more than two channels (caller-made selection): 64-bit words straight from global memory, cell by
+            // cell in a real loop so that the rare case costs no registers
+            if (more) {
+                tp = lane_taps(sel, cn);
+                fetch_planes(pl, tp, xn, live);
+            }
+#pragma unroll 1
+            for (int cell = 0; cell < 4; ++cell) {
+                uint64_t pooled = 0;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int oy = 2 * (cell >> 1) + (q >> 1), ox = 2 * (cell & 1) + (q & 1);
+                    uint64_t v[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const int iy = oy + cur.ry[k] - 1, ix = ox + cur.rx[k] - 1;
+                        v[k] = 0;
+                        if ((unsigned)iy < 4u && (unsigned)ix < 4u && live) v[k] = xn[cur.ch[k] * 16 + iy * 4 + ix];
+                    }
+                    pooled |= BitOps::root(pr, v);
+                }
+                if (live) y[(n * g.c + c) * 4 + cell] = pooled;
+            }
+        } else {
+            uint64_t best[4] = {0, 0, 0, 0};
+#pragma unroll 1
+            for (int half = 0; half < 2; ++half) {                    // a real loop: unrolled, the two passes pile up in registers
+                if (live) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) mine[((e >> 2) + 1) * 6 + (e & 3) + 1] = (uint32_t)(pl.v[e] >> (32 * half));
+                    if (cur.ch1 != cur.ch0) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) mine[kLsPlane + ((e >> 2) + 1) * 6 + (e & 3) + 1] = (uint32_t)(pl.v[16 + e] >> (32 * half));
+                    }
+                }
+                if (half == 1 && more) {                              // in flight while the high halves are evaluated
+                    tp = lane_taps(sel, cn);
+                    fetch_planes(pl, tp, xn, live);
+                }
+#pragma unroll
+                for (int cell = 0; cell < 4; ++cell) {
+                    uint32_t pooled = 0;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int oy = 2 * (cell >> 1) + (q >> 1), ox = 2 * (cell & 1) + (q & 1);
+                        uint32_t v[8];
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) v[k] = ta[k][oy * 6 + ox];
+                        pooled |= BitOps::root32(pr, v);
+                    }
+                    best[cell] |= (uint64_t)pooled << (32 * half);
+                }
+            }
+            if (live) {
+                u32x4 *out = reinterpret_cast<u32x4 *>(y + (n * g.c + c) * 4);
+                out[0] = u32x4{(uint32_t)best[0], (uint32_t)(best[0] >> 32), (uint32_t)best[1], (uint32_t)(best[1] >> 32)};
+                out[1] = u32x4{(uint32_t)best[2], (uint32_t)(best[2] >> 32), (uint32_t)best[3], (uint32_t)(best[3] >> 32)};
+            }
         }
         if (!more) break;
         c = cn;
@@ -424,7 +522,18 @@ int clg_convblock_forward_4x4(int dtype, const Geom &g, const void *x, const voi
 int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_t *gates, const int32_t *sel, uint64_t *y, hipStream_t st,
                                   const char *name)
 {
-    return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
+    const char *e_half = getenv("CLG_PACKED_4X4_HALVES");            // 0: one 64-bit pass per kernel (measurement)
+    if (e_half && atoi(e_half) == 0) return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
+    const int sblocks = (g.n + kWave - 1) / kWave;
+    int ct = 64;
+    while (ct > kLsWaves && (int64_t)sblocks * ((g.c + ct - 1) / ct) < 2048) ct >>= 1;
+    CLG_REQUIRE((g.c + ct - 1) / ct <= 65535, "%s: too many kernels for one launch (%d)", name, g.c);
+    const size_t lds = (size_t)kLsWaves * kWave * kLsStride * sizeof(uint32_t);
+    if (int e = allow_lds(convblock_eval_packed_4x4_kernel, lds, name)) return e;
+    hipLaunchKernelGGL(convblock_eval_packed_4x4_kernel, dim3((unsigned)sblocks, (unsigned)((g.c + ct - 1) / ct)), dim3(kLsWaves * kWave), lds,
+                       st, x, gates, sel, y, g, ct);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
 }
 
 // ---- gradients: launchers (the caller has run the prepare kernel: folded coefficients and per-channel kernel lists) ----
