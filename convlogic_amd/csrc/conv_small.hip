@@ -71,20 +71,20 @@ __device__ __forceinline__ void fetch_planes(Planes<T> &pl, const LaneTaps &tp, 
     if (tp.ch1 != tp.ch0) load_plane(pl.v, 16, xn + tp.ch1 * 16);
 }
 
-// grid: (64-sample blocks, kernel tiles of ct kernels); LDS: kLsWaves * 64 * kLsStride elements.
+// grid: (64-sample blocks from sample n_first on, kernel tiles of ct kernels); LDS: kLsWaves * 64 * kLsStride elements.
 // params: folded coefficients [c][28] (float gates) or gate ids uint8 [c][7] (packed words, argmax = null)
 template <typename Ops>
 __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(const typename Ops::Elem *__restrict__ x,
                                                                               const void *__restrict__ params,
                                                                               const int32_t *__restrict__ sel,
                                                                               typename Ops::Elem *__restrict__ y,
-                                                                              uint8_t *__restrict__ argmax, Geom g, int ct)
+                                                                              uint8_t *__restrict__ argmax, Geom g, int ct, int n_first)
 {
     using T = typename Ops::Elem;
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
     T *mine = reinterpret_cast<T *>(smem) + ((size_t)wave * kWave + lane) * kLsStride;
-    const int64_t n = (int64_t)blockIdx.x * kWave + lane;
+    const int64_t n = (int64_t)n_first + (int64_t)blockIdx.x * kWave + lane;
     const bool live = n < g.n;
     const T *xn = x + (live ? n : 0) * g.cin * 16;
 #pragma unroll
@@ -159,30 +159,60 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
 
 // Packed words, one group of 64 samples per lane, evaluated as two halves of 32 samples: the lane's LDS slice holds
 // 4-byte elements, so a workgroup takes half the LDS of the 8-byte variant and two of them share a CU (the kernel is
-// bound by what a wavefront has in flight, not by arithmetic).  Order per kernel: low halves to LDS, evaluate, high
-// halves to LDS, request the next kernel's planes, evaluate, store 64-bit words.
+// bound by what a wavefront has in flight, not by arithmetic).  The planes are fetched by the wavefront together:
+// 8 lanes read the 128 contiguous bytes of one group's plane (8 lines per load instruction instead of 64) and every
+// lane writes its two words into the slice of the lane that owns the group.  Order per kernel: low halves to LDS,
+// evaluate, high halves to LDS, request the next kernel's planes, evaluate, store 64-bit words.
+struct PackedPlanes {
+    u32x4 raw[2][8];                               // [plane][load]: words 2 piece, 2 piece + 1 of group 8 load + lane / 8
+};
+
 __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_kernel(const uint64_t *__restrict__ x,
                                                                                   const uint8_t *__restrict__ gates,
                                                                                   const int32_t *__restrict__ sel,
-                                                                                  uint64_t *__restrict__ y, Geom g, int ct)
+                                                                                  uint64_t *__restrict__ y, Geom g, int ct,
+                                                                                  int ctiles, int sblocks)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
-    uint32_t *mine = reinterpret_cast<uint32_t *>(smem) + ((size_t)wave * kWave + lane) * kLsStride;
-    const int64_t n = (int64_t)blockIdx.x * kWave + lane;
-    const bool live = n < g.n;
-    const uint64_t *xn = x + (live ? n : 0) * g.cin * 16;
+    // Workgroups go round the 8 XCDs by their linear index; an XCD takes the blocks of 64 groups  xcd, xcd + 8, ...
+    // one after the other with all kernel tiles of a block in a row, so that the block's planes (cin x 8 KiB) are
+    // served by that XCD's L2 while the kernels pick channels at random.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int sblock = xcd + 8 * (slot / ctiles), tile = slot - (slot / ctiles) * ctiles;
+    if (sblock >= sblocks) return;
+    uint32_t *slices = reinterpret_cast<uint32_t *>(smem) + (size_t)wave * kWave * kLsStride;   // of this wavefront
+    uint32_t *mine = slices + lane * kLsStride;
+    const int64_t n = (int64_t)sblock * kWave + lane;
+    constexpr bool live = true;                                      // the host sends full blocks of 64 groups only
+    const uint64_t *xn = x + n * g.cin * 16;
 #pragma unroll
     for (int e = 0; e < kLsStride; ++e) mine[e] = 0u;
-    const int c0 = blockIdx.y * ct, c1 = min(g.c, c0 + ct);
+    const int c0 = tile * ct, c1 = min(g.c, c0 + ct);
     int c = c0 + wave;
     if (c >= c1) return;
-    LaneTaps tp = lane_taps(sel, c);
-    Planes<uint64_t> pl;
-    fetch_planes(pl, tp, xn, live);
+    // shared fetch: load j covers groups 8 j .. 8 j + 7 of the wavefront, this lane takes 16 bytes (words 2 piece and
+    // 2 piece + 1) of group 8 j + sub
+    const int piece = lane & 7, sub = lane >> 3;
+    const uint64_t *xw = x + ((int64_t)sblock * kWave + sub) * g.cin * 16 + 2 * piece;   // load j: + 8 j groups
+    const int64_t group_step = (int64_t)8 * g.cin * 16;
+    uint32_t *put = slices + sub * kLsStride + ((piece >> 1) + 1) * 6 + 2 * (piece & 1) + 1;   // + 8 j slices, + plane
+    PackedPlanes pl;
+    // Only the channels of the next kernel are looked at ahead of time (its taps are read again when its turn comes:
+    // scalar registers are scarce next to 28 gate masks).  Both planes are always fetched and written, also when a
+    // kernel reads one channel only: one code path, so the registers of `pl` need no copies where paths meet.
+    auto fetch = [&](int kernel) {
+        const LaneTaps t = lane_taps(sel, kernel);
+        if (t.wide) return;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pl.raw[0][j] = *reinterpret_cast<const u32x4 *>(xw + j * group_step + t.ch0 * 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pl.raw[1][j] = *reinterpret_cast<const u32x4 *>(xw + j * group_step + t.ch1 * 16);
+    };
+    fetch(c);
     while (true) {
         const BitOps::Params pr = BitOps::load_global(gates, c);
-        const LaneTaps cur = tp;
+        const LaneTaps cur = lane_taps(sel, c);
         const int cn = c + kLsWaves;
         const bool more = cn < c1;
         const uint32_t *ta[8];
@@ -191,10 +221,7 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
         if (cur.wide) {
             // taps in more than two channels (caller-made selection): 64-bit words straight from global memory, cell by
             // cell in a real loop so that the rare case costs no registers
-            if (more) {
-                tp = lane_taps(sel, cn);
-                fetch_planes(pl, tp, xn, live);
-            }
+            if (more) fetch(cn);
 #pragma unroll 1
             for (int cell = 0; cell < 4; ++cell) {
                 uint64_t pooled = 0;
@@ -216,18 +243,24 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
             uint64_t best[4] = {0, 0, 0, 0};
 #pragma unroll 1
             for (int half = 0; half < 2; ++half) {                    // a real loop: unrolled, the two passes pile up in registers
-                if (live) {
+                // the lanes write into each other's slices: LDS serves a wavefront's instructions in order, the fences
+                // keep the compiler from moving this lane's reads across the writes
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) mine[((e >> 2) + 1) * 6 + (e & 3) + 1] = (uint32_t)(pl.v[e] >> (32 * half));
-                    if (cur.ch1 != cur.ch0) {
+                for (int j = 0; j < 8; ++j) {
+                    uint32_t *dst = put + 8 * j * kLsStride;
+                    dst[0] = half ? pl.raw[0][j].y : pl.raw[0][j].x;
+                    dst[1] = half ? pl.raw[0][j].w : pl.raw[0][j].z;
+                }
 #pragma unroll
-                        for (int e = 0; e < 16; ++e) mine[kLsPlane + ((e >> 2) + 1) * 6 + (e & 3) + 1] = (uint32_t)(pl.v[16 + e] >> (32 * half));
-                    }
+                for (int j = 0; j < 8; ++j) {
+                    uint32_t *dst = put + 8 * j * kLsStride + kLsPlane;
+                    dst[0] = half ? pl.raw[1][j].y : pl.raw[1][j].x;
+                    dst[1] = half ? pl.raw[1][j].w : pl.raw[1][j].z;
                 }
-                if (half == 1 && more) {                              // in flight while the high halves are evaluated
-                    tp = lane_taps(sel, cn);
-                    fetch_planes(pl, tp, xn, live);
-                }
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
                 for (int cell = 0; cell < 4; ++cell) {
                     uint32_t pooled = 0;
@@ -242,6 +275,7 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
                     best[cell] |= (uint64_t)pooled << (32 * half);
                 }
             }
+            if (more) fetch(cn);
             if (live) {
                 u32x4 *out = reinterpret_cast<u32x4 *>(y + (n * g.c + c) * 4);
                 out[0] = u32x4{(uint32_t)best[0], (uint32_t)(best[0] >> 32), (uint32_t)best[1], (uint32_t)(best[1] >> 32)};
@@ -495,17 +529,17 @@ bool clg_convblock_is_4x4(const Geom &g)
 
 template <typename Ops>
 static int launch_4x4(const Geom &g, const void *x, const void *params, const int32_t *sel, void *y, uint8_t *argmax, hipStream_t st,
-                      const char *name)
+                      const char *name, int n_first = 0)
 {
     using T = typename Ops::Elem;
-    const int sblocks = (g.n + kWave - 1) / kWave;
+    const int sblocks = (g.n - n_first + kWave - 1) / kWave;
     int ct = 64;                                                      // 16 kernels per wavefront unless that starves the chip
     while (ct > kLsWaves && (int64_t)sblocks * ((g.c + ct - 1) / ct) < 1024) ct >>= 1;
     CLG_REQUIRE((g.c + ct - 1) / ct <= 65535, "%s: too many kernels for one launch (%d)", name, g.c);
     const dim3 grid((unsigned)sblocks, (unsigned)((g.c + ct - 1) / ct)), block(kLsWaves * kWave);
     const size_t lds = (size_t)kLsWaves * kWave * kLsStride * sizeof(T);
     if (int e = allow_lds(convblock_forward_4x4_kernel<Ops>, lds, name)) return e;
-    hipLaunchKernelGGL(convblock_forward_4x4_kernel<Ops>, grid, block, lds, st, (const T *)x, params, sel, (T *)y, argmax, g, ct);
+    hipLaunchKernelGGL(convblock_forward_4x4_kernel<Ops>, grid, block, lds, st, (const T *)x, params, sel, (T *)y, argmax, g, ct, n_first);
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }
@@ -524,14 +558,21 @@ int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_
 {
     const char *e_half = getenv("CLG_PACKED_4X4_HALVES");            // 0: one 64-bit pass per kernel (measurement)
     if (e_half && atoi(e_half) == 0) return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
-    const int sblocks = (g.n + kWave - 1) / kWave;
+    // full blocks of 64 groups go to the half-word kernel, what is left of the batch to the 64-bit one
+    const int sblocks = g.n / kWave;
+    if (sblocks * kWave < g.n) {
+        if (int e = launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name, sblocks * kWave)) return e;
+        if (sblocks == 0) return CLG_OK;
+    }
     int ct = 64;
     while (ct > kLsWaves && (int64_t)sblocks * ((g.c + ct - 1) / ct) < 2048) ct >>= 1;
-    CLG_REQUIRE((g.c + ct - 1) / ct <= 65535, "%s: too many kernels for one launch (%d)", name, g.c);
+    const int ctiles = (g.c + ct - 1) / ct;
+    const int64_t wgs = (int64_t)8 * ((sblocks + 7) / 8) * ctiles;
+    CLG_REQUIRE(wgs < (1ll << 31), "%s: problem too large for one launch", name);
     const size_t lds = (size_t)kLsWaves * kWave * kLsStride * sizeof(uint32_t);
     if (int e = allow_lds(convblock_eval_packed_4x4_kernel, lds, name)) return e;
-    hipLaunchKernelGGL(convblock_eval_packed_4x4_kernel, dim3((unsigned)sblocks, (unsigned)((g.c + ct - 1) / ct)), dim3(kLsWaves * kWave), lds,
-                       st, x, gates, sel, y, g, ct);
+    hipLaunchKernelGGL(convblock_eval_packed_4x4_kernel, dim3((unsigned)wgs), dim3(kLsWaves * kWave), lds, st, x, gates, sel, y, g, ct, ctiles,
+                       sblocks);
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }

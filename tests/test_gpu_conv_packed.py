@@ -139,11 +139,12 @@ def test_packed_block_errors():
         convlogic_hip.full_convlogic_eval_packed(x[:, :, :7].contiguous(), gates, layer.selection, 1, 1, 1, 1, 3, 3)
 
 
-@pytest.mark.parametrize("samples,cin,cout", [(2048, 6, 9), (2100, 24, 40), (4160, 16, 33)])
+@pytest.mark.parametrize("samples,cin,cout", [(2048, 6, 9), (2100, 24, 40), (4160, 16, 33), (8192, 12, 21)])
 def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
-    # from 32 word groups on, 4x4 images take the kernel that gives every lane one group of 64 samples: against the
-    # numpy oracle (bit-exact), against the staged kernel, with a ragged last wavefront and last word, and with
-    # kernels that read more than two channels
+    # from 32 word groups on, 4x4 images take the kernels that give every lane one group of 64 samples (full blocks of
+    # 64 groups: two passes of 32 samples with planes fetched by the wavefront together; the rest of the batch: one
+    # 64-bit pass): against the numpy oracle (bit-exact), against the staged kernel and the 64-bit pass alone, with a
+    # ragged last wavefront and last word, and with kernels that read more than two channels
     torch.manual_seed(samples + cin)
     ch = torch.randint(0, cin, (cout, 2))
     pick = torch.randint(0, 2, (cout, 8))
@@ -164,6 +165,9 @@ def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
     staged = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
     monkeypatch.delenv("CLG_FWD_4X4")
     assert torch.equal(staged, p.t)
+    monkeypatch.setenv("CLG_PACKED_4X4_HALVES", "0")
+    whole = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
+    assert torch.equal(whole, p.t)
 
 
 @pytest.mark.parametrize("n,cin,cout,hw", [(70, 128, 24, 8), (5, 6, 9, 4), (33, 40, 16, 2), (3, 3, 8, 16)])
