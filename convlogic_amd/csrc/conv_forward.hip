@@ -398,13 +398,11 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     if (const char *e = getenv("CLG_FWD_NW")) p->NW = atoi(e);
     if (p->S < 1 || p->CT < 1 || p->NW < 1 || p->NW > 16) return false;
     // A workgroup whose samples fill at most half a wavefront with (row pair, column) slots gives every conv position
-    // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64).
-    // Measured on [*,128,8,8] -> 512: packed words 174 -> 140 us, float32 38 -> 42 us (its kernel is bound by the prologue
-    // and loses the compile-time row step), so 4-byte elements keep two rows per lane.
+    // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64), two
+    // kernels per step.  Measured on [*,128,8,8] -> 512: packed words 174 -> 102 us, float32 39 -> 37 us.
     p->one_row = 0;
-    if (elem == 8 && (int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
-    if (const char *e = getenv("CLG_FWD_ONE_ROW"))                   // 0: never, 1: default rule, 2: also for 4-byte elements
-        p->one_row = atoi(e) == 2 ? ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) : (p->one_row && atoi(e) != 0);
+    if ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
+    if (const char *e = getenv("CLG_FWD_ONE_ROW")) p->one_row = p->one_row && atoi(e) != 0;   // 0: never
     if (p->one_row) {
         p->slots = g.ho * g.wo;
         p->d_slots = make_fastdiv((uint32_t)p->slots);

@@ -44,11 +44,11 @@ template <typename T>
 __device__ __forceinline__ T dpp_xor1(T v)
 {
     if constexpr (sizeof(T) == 4) {
-        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
     } else {
         const uint64_t u = __builtin_bit_cast(uint64_t, v);
-        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, false);
-        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, false);
+        const uint32_t lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, 0xB1, 0xF, 0xF, true);
+        const uint32_t hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), 0xB1, 0xF, 0xF, true);
         return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
     }
 }

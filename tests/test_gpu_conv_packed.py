@@ -185,7 +185,7 @@ def test_one_position_per_lane_equals_two_rows_per_lane(n, cin, cout, hw, monkey
     wp = torch.softmax(layer.weights.detach(), -1)
     got = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("CLG_FWD_ONE_ROW", "2" if mode == "1" else "0")       # 2: float32 too (off by default there)
+        monkeypatch.setenv("CLG_FWD_ONE_ROW", mode)                   # 0: every shape keeps two rows per lane
         got[mode] = (convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3),
                      *convlogic_hip.full_convlogic_forward(x, wp, layer.selection, 1, 1, 1, 1, 3, 3))
     for a, b in zip(got["1"], got["0"]):
