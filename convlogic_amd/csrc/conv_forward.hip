@@ -147,7 +147,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
             if constexpr (ROWSTEP == 8 || ROWSTEP == 4) return row_up<ROWSTEP>(v);
             else return lane_up(v, g.wo);
         };
-        constexpr int K = 2;                                          // 3 and 4 measured the same
+        constexpr int K = 2;                                          // 1: 2 % slower, 4: the same
         for (int lc = first; lc < last; lc += K) {
             int lk[K];
             typename Ops::Params pr[K];

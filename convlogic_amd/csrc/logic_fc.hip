@@ -506,7 +506,7 @@ __global__ __launch_bounds__(256) void group_sum_fm_kernel(const T *__restrict__
 // out[b][g] = sum over slices of partial[slice][g][b]
 template <typename T>
 __global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t batch,
-                                                             int k, int slices)
+                                                             int k, int slices, T inv_tau)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= batch * k) return;
@@ -514,19 +514,19 @@ __global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restri
     const int g = (int)(i - b * k);
     T acc = 0;
     for (int s = 0; s < slices; ++s) acc += partial[((int64_t)s * k + g) * batch + b];
-    out[i] = acc;
+    out[i] = acc * inv_tau;
 }
-// grad_x[f][b] = grad_out[b][class of f]; a workgroup writes 64 feature rows of one 64-sample column chunk
+// grad_x[f][b] = grad_out[b][class of f] * (1 / tau); a workgroup writes 64 feature rows of one 64-sample column chunk
 template <typename T>
 __global__ __launch_bounds__(256) void group_sum_backward_fm_kernel(const T *__restrict__ grad_out, T *__restrict__ grad_x,
-                                                                  int64_t class_rows, int64_t batch, int k, int64_t bchunks)
+                                                                  int64_t class_rows, int64_t batch, int k, int64_t bchunks, T inv_tau)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int64_t fb = blockIdx.x / bchunks, bc = blockIdx.x - fb * bchunks;
     const int64_t b = bc * kWave + lane;
     if (b >= batch) return;
     const int64_t f0 = fb * 64, features = class_rows * k;
-    for (int64_t f = f0 + wave; f < f0 + 64 && f < features; f += 4) grad_x[f * batch + b] = grad_out[b * k + f / class_rows];
+    for (int64_t f = f0 + wave; f < f0 + 64 && f < features; f += 4) grad_x[f * batch + b] = grad_out[b * k + f / class_rows] * inv_tau;
 }
 
 int grid_for(int64_t items)
@@ -803,8 +803,9 @@ extern "C" int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int6
 }
 
 extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch, int64_t features, int64_t batch, int64_t k,
-                             void *stream)
+                             double tau, void *stream)
 {
+    CLG_REQUIRE(tau != 0.0, "clg_group_sum: tau must not be zero");
     CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_group_sum: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
     CLG_REQUIRE(x && out && scratch, "clg_group_sum: null pointer argument");
     CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && k <= 65535, "clg_group_sum: features, batch and k must be positive, k <= 65535");
@@ -821,20 +822,21 @@ extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch,
         hipLaunchKernelGGL(group_sum_fm_kernel<float>, grid, dim3(256), 0, st, (const float *)x, (float *)scratch, class_rows, batch, (int)k,
                            (int)slices);
         hipLaunchKernelGGL(group_sum_finish_kernel<float>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
-                           (const float *)scratch, (float *)out, batch, (int)k, (int)slices);
+                           (const float *)scratch, (float *)out, batch, (int)k, (int)slices, 1.0f / (float)tau);
     } else {
         hipLaunchKernelGGL(group_sum_fm_kernel<double>, grid, dim3(256), 0, st, (const double *)x, (double *)scratch, class_rows, batch,
                            (int)k, (int)slices);
         hipLaunchKernelGGL(group_sum_finish_kernel<double>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
-                           (const double *)scratch, (double *)out, batch, (int)k, (int)slices);
+                           (const double *)scratch, (double *)out, batch, (int)k, (int)slices, 1.0 / tau);
     }
     CLG_CHECK_LAUNCH("clg_group_sum");
     return CLG_OK;
 }
 
 extern "C" int clg_group_sum_backward(int dtype, const void *grad_out, void *grad_x, int64_t features, int64_t batch, int64_t k,
-                                      void *stream)
+                                      double tau, void *stream)
 {
+    CLG_REQUIRE(tau != 0.0, "clg_group_sum_backward: tau must not be zero");
     CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_group_sum_backward: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
     CLG_REQUIRE(grad_out && grad_x, "clg_group_sum_backward: null pointer argument");
     CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && features % k == 0, "clg_group_sum_backward: features must be a positive multiple of k");
@@ -843,10 +845,10 @@ extern "C" int clg_group_sum_backward(int dtype, const void *grad_out, void *gra
     hipStream_t st = clg_stream(stream);
     if (dtype == CLG_F32)
         hipLaunchKernelGGL(group_sum_backward_fm_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, (const float *)grad_out,
-                           (float *)grad_x, features / k, batch, (int)k, bchunks);
+                           (float *)grad_x, features / k, batch, (int)k, bchunks, 1.0f / (float)tau);
     else
         hipLaunchKernelGGL(group_sum_backward_fm_kernel<double>, dim3((unsigned)blocks), dim3(256), 0, st, (const double *)grad_out,
-                           (double *)grad_x, features / k, batch, (int)k, bchunks);
+                           (double *)grad_x, features / k, batch, (int)k, bchunks, 1.0 / tau);
     CLG_CHECK_LAUNCH("clg_group_sum_backward");
     return CLG_OK;
 }

@@ -205,7 +205,7 @@ class GroupSum(torch.nn.Module):
         if (x.is_cuda and x.dim() == 2 and x.dtype in (torch.float32, torch.float64) and x.numel() > 0
                 and x.transpose(0, 1).is_contiguous() and not x.is_contiguous()):
             # the transposed view of a feature-major tensor, as a LogicLayer returns it: summed in that layout
-            return _GroupSumFeatureMajor.apply(x, self.k) / self.tau
+            return _GroupSumFeatureMajor.apply(x, self.k, self.tau)
         return x.reshape(*x.shape[:-1], self.k, x.shape[-1] // self.k).sum(-1) / self.tau
 
     def extra_repr(self):
@@ -213,17 +213,19 @@ class GroupSum(torch.nn.Module):
 
 
 class _GroupSumFeatureMajor(torch.autograd.Function):
-    """Per-class sums of x [batch, features] that is a transposed view of a contiguous [features, batch]
-    tensor; the gradient comes back in the same layout (a transposed view again, no copies)."""
+    """Per-class sums / tau of x [batch, features] that is a transposed view of a contiguous [features, batch]
+    tensor; the gradient comes back in the same layout (a transposed view again, no copies).  The division by
+    tau happens inside the two kernels (as a product with 1 / tau, which is what torch computes for `sum / tau` on the
+    device)."""
 
     @staticmethod
-    def forward(ctx, x, k):
-        ctx.features = x.shape[1]
-        return difflogic_hip.group_sum(x.transpose(0, 1), k)
+    def forward(ctx, x, k, tau):
+        ctx.features, ctx.tau = x.shape[1], tau
+        return difflogic_hip.group_sum(x.transpose(0, 1), k, tau)
 
     @staticmethod
     def backward(ctx, grad_out):
-        return difflogic_hip.group_sum_backward(grad_out.contiguous(), ctx.features).transpose(0, 1), None
+        return difflogic_hip.group_sum_backward(grad_out.contiguous(), ctx.features, ctx.tau).transpose(0, 1), None, None
 
 
 class LogicLayerCudaFunction(torch.autograd.Function):

@@ -15,7 +15,7 @@ CLG_F32, CLG_F64, CLG_F16 = 0, 1, 2
 _DTYPES = {torch.float32: CLG_F32, torch.float64: CLG_F64}
 _DTYPES_FC = {**_DTYPES, torch.float16: CLG_F16}       # LogicLayer forward / backward_w / backward_x also store half
 
-_p, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+_p, _i, _i64, _f64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_double
 
 
 class ConvGeom(ctypes.Structure):
@@ -37,8 +37,8 @@ SIGNATURES = {
     "clg_fc_backward_x_folded": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_sole": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_group_sum_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
-    "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _p]),
-    "clg_group_sum_backward": (_i, [_i, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _f64, _p]),
+    "clg_group_sum_backward": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_fc_backward_x": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_transpose_2d": (_i, [_i, _p, _p, _i64, _i64, _p]),
     "clg_pack_bits": (_i, [_p, _p, _i64, _i64, _i, _p]),

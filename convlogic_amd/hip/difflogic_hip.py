@@ -101,8 +101,8 @@ def backward_sole(x, a, b, folded, probs, grad_y):
     return gx, gw
 
 
-def group_sum(x_fm, k):
-    """Feature-major activations [F, B] -> per-class sums [B, k] (not divided by tau), fixed summation order."""
+def group_sum(x_fm, k, tau=1.0):
+    """Feature-major activations [F, B] -> per-class sums [B, k] divided by tau, fixed summation order."""
     check_input(x_fm, "x")
     features, batch = x_fm.shape
     if features % k != 0:
@@ -112,17 +112,17 @@ def group_sum(x_fm, k):
     nbytes = lib.clg_group_sum_scratch_bytes(dt, features, batch, k)
     scratch = torch.empty((max(int(nbytes), 8),), dtype=torch.uint8, device=x_fm.device)
     out = torch.empty((batch, k), dtype=x_fm.dtype, device=x_fm.device)
-    check(lib.clg_group_sum(dt, x_fm.data_ptr(), out.data_ptr(), scratch.data_ptr(), features, batch, k, stream_ptr(x_fm)))
+    check(lib.clg_group_sum(dt, x_fm.data_ptr(), out.data_ptr(), scratch.data_ptr(), features, batch, k, float(tau), stream_ptr(x_fm)))
     return out
 
 
-def group_sum_backward(grad_out, features):
-    """[B, k] -> feature-major gradient [F, B]: every row of class g receives grad_out[:, g]."""
+def group_sum_backward(grad_out, features, tau=1.0):
+    """[B, k] -> feature-major gradient [F, B]: every row of class g receives grad_out[:, g] / tau."""
     check_input(grad_out, "grad_out")
     batch, k = grad_out.shape
     gx = torch.empty((features, batch), dtype=grad_out.dtype, device=grad_out.device)
     check(_lib.load().clg_group_sum_backward(dtype_code(grad_out), grad_out.data_ptr(), gx.data_ptr(), features, batch, k,
-                                             stream_ptr(grad_out)))
+                                             float(tau), stream_ptr(grad_out)))
     return gx
 
 

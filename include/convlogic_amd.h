@@ -120,15 +120,16 @@ int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64
                          int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
 
 /* GroupSum on feature-major activations x [features, batch] (what the last LogicLayer produces): out[b][g] =
- * sum of the features/k rows of class g, NOT yet divided by tau; fixed summation order (reproducible).
- * scratch: clg_group_sum_scratch_bytes().  Replaces x.reshape(..., k, F/k).sum(-1) of
+ * (sum of the features/k rows of class g) * (1 / tau), the reciprocal rounded to dtype as torch's division of a
+ * device tensor by a scalar does; fixed summation order (reproducible).
+ * scratch: clg_group_sum_scratch_bytes().  Replaces x.reshape(..., k, F/k).sum(-1) / tau of
  * src/difflogic/difflogic.py:203-208 without the transposed copy. */
 int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int64_t batch, int64_t k);
 int clg_group_sum(int dtype, const void *x, void *out /*[batch,k]*/, void *scratch, int64_t features, int64_t batch,
-                  int64_t k, void *stream);
-/* Its backward: grad_x[f][b] = grad_out[b][f / (features/k)] (grad_out already divided by tau). */
+                  int64_t k, double tau, void *stream);
+/* Its backward: grad_x[f][b] = grad_out[b][f / (features/k)] * (1 / tau). */
 int clg_group_sum_backward(int dtype, const void *grad_out /*[batch,k]*/, void *grad_x /*[features,batch]*/,
-                           int64_t features, int64_t batch, int64_t k, void *stream);
+                           int64_t features, int64_t batch, int64_t k, double tau, void *stream);
 
 /* dst[c][r] = src[r][c] for elements of elem_size 1, 2, 4 or 8 bytes (layout change between the
  * module's [batch, features] tensors and the feature-major kernels; the reference does this with
