@@ -448,6 +448,97 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
     }
 }
 
+// Both gradients in one pass for any wiring, as long as one pass of LPR lanes x VEC samples covers the batch: the
+// wavefront that owns input i walks its consumers (as fc_backward_x_folded_kernel) and, on the visit that reaches a
+// consumer through its FIRST operand -- which happens exactly once per neuron, and has the neuron's gy row, its first
+// operand row (x[i]) and its second operand row in registers -- also forms the four sums of the weight gradient
+// (as fc_backward_w_kernel: same lanes, same order, same reduction) and writes the neuron's 16 gate gradients.
+// Saves the second pass over gy and the operand rows that a separate weight-gradient kernel makes.
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
+    const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
+    const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
+    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int64_t batch, const T *__restrict__ probs)
+{
+    constexpr int ROWS = kWave / LPR;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int sub = lane / LPR, l = lane % LPR;
+    const int64_t groups = (in_dim + ROWS - 1) / ROWS;
+    const int64_t s = (int64_t)l * VEC;
+    for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < groups; it += (int64_t)gridDim.x * kWavesPerBlock) {
+        const bool row_ok = it * ROWS + sub < in_dim;
+        const int64_t i = row_ok ? it * ROWS + sub : in_dim - 1;
+        const bool live = row_ok && s < batch;                       // lanes beyond the batch add zeros to the sums
+        const int64_t beg = csr_start[i], end = row_ok ? csr_start[i + 1] : beg;
+        Pack<T, VEC> xi;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) xi.v[k] = 0;
+        if (live) xi = load_vec<T, VEC>(x + i * batch + s);
+        Pack<T, VEC> part[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
+        int64_t prev = -1;
+        for (int64_t cur = beg; cur < end; cur += 4) {               // the lanes of a row group leave the loop together
+            int64_t j[4];
+            Pack<T, VEC> vo[4], vg[4];
+            T c_ab[4], c_lin[4];
+            bool first[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                j[u] = cur + u < end ? csr_list[cur + u] : -1;
+                first[u] = false;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) vo[u].v[k] = vg[u].v[k] = 0;
+                if (j[u] >= 0) {
+                    const int64_t ia = a[j[u]], ib = b[j[u]];
+                    const Coef<T> c = load_coef(folded + j[u] * 4);
+                    const bool as_a = ia == i && !(ib == i && prev == j[u]);   // see fc_backward_x_folded_kernel
+                    first[u] = as_a;
+                    c_ab[u] = c.ab;
+                    c_lin[u] = as_a ? c.a : c.b;
+                    if (live) {
+                        vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
+                        vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
+                    }
+                }
+                prev = j[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (j[u] < 0) continue;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
+                if (first[u]) {                                      // uniform over the row group
+                    T sab = 0, sa = 0, sb = 0, s1 = 0;
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        sab = fma_t(vg[u].v[k], xi.v[k] * vo[u].v[k], sab);
+                        sa = fma_t(vg[u].v[k], xi.v[k], sa);
+                        sb = fma_t(vg[u].v[k], vo[u].v[k], sb);
+                        s1 += vg[u].v[k];
+                    }
+                    sab = lane_group_sum<T, LPR>(sab);
+                    sa = lane_group_sum<T, LPR>(sa);
+                    sb = lane_group_sum<T, LPR>(sb);
+                    s1 = lane_group_sum<T, LPR>(s1);
+                    if (l >= LPR - 16) {
+                        const int q = lane & 15;
+                        T gi = coef_transpose_row<T>(q, sab, sa, sb, s1);
+                        if (probs != nullptr) gi = softmax16_backward(gi, probs[j[u] * 16 + q]);
+                        gw[j[u] * 16 + q] = gi;
+                    }
+                }
+            }
+        }
+        Pack<T, VEC> acc;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
+        if (live) store_vec<T, VEC>(gx + i * batch + s, acc);
+    }
+}
+
 // ---- 2-D transpose through a padded LDS tile -------------------------------------------------
 // TILE x TILE elements per workgroup of 256 threads; the 32 x 32 tile gives small matrices four times as many workgroups.
 template <typename T, int TILE>
@@ -766,6 +857,54 @@ extern "C" int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, 
 #undef CLG_LAUNCH_BS_ROWS
 #undef CLG_LAUNCH_BS
     CLG_CHECK_LAUNCH("clg_fc_backward_sole");
+    return CLG_OK;
+}
+
+// largest batch one pass of a wavefront row covers: 64 lanes x VEC samples
+static int64_t fused_batch_limit(int dtype, int64_t batch)
+{
+    const int vec = dtype == CLG_F32 ? (batch % 4 == 0 ? 4 : 1) : (batch % 2 == 0 ? 2 : 1);
+    return (int64_t)kWave * vec;
+}
+
+extern "C" int clg_fc_backward_fused_fits(int dtype, int64_t batch)
+{
+    return (dtype == CLG_F32 || dtype == CLG_F64) && batch > 0 && batch <= fused_batch_limit(dtype, batch) ? 1 : 0;
+}
+
+extern "C" int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                     const void *probs, const void *grad_y, const int64_t *csr_start, const int64_t *csr_list,
+                                     void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_fused")) return e;
+    CLG_REQUIRE(x && a && b && folded && grad_y && csr_start && csr_list && grad_x && grad_w,
+                "clg_fc_backward_fused: null pointer argument");
+    CLG_REQUIRE(batch <= fused_batch_limit(dtype, batch),
+                "clg_fc_backward_fused: batch %lld exceeds what one pass covers (%lld); use clg_fc_backward_x_folded and "
+                "clg_fc_backward_logits", (long long)batch, (long long)fused_batch_limit(dtype, batch));
+    const dim3 block(kBlock);
+    hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_BF(T, VEC, LPR)                                                                                         \
+    hipLaunchKernelGGL((fc_backward_fused_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(in_dim, (int64_t)(kWave / LPR)))), \
+                       block, 0, st, (const T *)x, a, b, (const T *)folded, (const T *)grad_y, csr_start, csr_list,          \
+                       (T *)grad_x, (T *)grad_w, (int)in_dim, batch, (const T *)probs)
+#define CLG_LAUNCH_BF_ROWS(T, VEC)                                                                                         \
+    do {                                                                                                                  \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                    \
+        if (lg == 4) CLG_LAUNCH_BF(T, VEC, 16);                                                                           \
+        else if (lg == 5) CLG_LAUNCH_BF(T, VEC, 32);                                                                      \
+        else CLG_LAUNCH_BF(T, VEC, 64);                                                                                   \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_BF_ROWS(float, 4);
+        else CLG_LAUNCH_BF_ROWS(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_BF_ROWS(double, 2);
+        else CLG_LAUNCH_BF_ROWS(double, 1);
+    }
+#undef CLG_LAUNCH_BF_ROWS
+#undef CLG_LAUNCH_BF
+    CLG_CHECK_LAUNCH("clg_fc_backward_fused");
     return CLG_OK;
 }
 

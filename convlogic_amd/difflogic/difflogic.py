@@ -268,6 +268,8 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
         grad_x = grad_l = None
         if ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]:
             grad_x, grad_l = difflogic_hip.backward_sole(x, a, b, folded, w, grad_y)
+        elif ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and difflogic_hip.backward_fused_fits(x):
+            grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, grad_y, start, flat)
         else:
             if ctx.needs_input_grad[0]:
                 grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)

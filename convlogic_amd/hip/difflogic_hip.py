@@ -101,6 +101,31 @@ def backward_sole(x, a, b, folded, probs, grad_y):
     return gx, gw
 
 
+def backward_fused_fits(x):
+    """True when backward_fused() covers the batch of feature-major x [in, B] in one pass."""
+    return bool(_lib.load().clg_fc_backward_fused_fits(dtype_code(x), x.shape[1]))
+
+
+def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
+    """(grad_x, grad_w) of a layer with any wiring in one pass (see backward_fused_fits); grad_w is the gradient
+    w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities.  Same values as
+    backward_x_folded() + backward_w() / backward_logits()."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y"),
+                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
+        check_input(t, n)
+    if probs is not None:
+        check_input(probs, "w")
+    in_dim, batch = x.shape
+    out_dim = folded.shape[0]
+    gx = torch.empty_like(x)
+    gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_backward_fused(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
+                                            probs.data_ptr() if probs is not None else None, grad_y.data_ptr(),
+                                            given_x_indices_of_y_start.data_ptr(), given_x_indices_of_y.data_ptr(),
+                                            gx.data_ptr(), gw.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
+    return gx, gw
+
+
 def group_sum(x_fm, k, tau=1.0):
     """Feature-major activations [F, B] -> per-class sums [B, k] divided by tau, fixed summation order."""
     check_input(x_fm, "x")

@@ -119,6 +119,18 @@ int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64
                          const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, void *grad_x, void *grad_w,
                          int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
 
+/* Both gradients of a layer with ANY wiring in one pass, for batches that one pass of a wavefront row covers
+ * (clg_fc_backward_fused_fits() != 0: batch <= 256 for float32 batches divisible by 4, 128 for float64 batches divisible
+ * by 2, 64 otherwise): the walk of clg_fc_backward_x_folded also forms each neuron's weight-gradient sums on the visit
+ * through the neuron's first operand.  grad_x and grad_w as clg_fc_backward_x_folded + clg_fc_backward_w /
+ * clg_fc_backward_logits (probs given), bit for bit.  Replaces difflogic_cuda.backward_x + backward_w
+ * (src/difflogic/cuda/difflogic_kernel.cu:153-269) in the module's training path. */
+int clg_fc_backward_fused_fits(int dtype, int64_t batch);
+int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
+                          const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, const int64_t *csr_start,
+                          const int64_t *csr_list, void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch,
+                          void *stream);
+
 /* GroupSum on feature-major activations x [features, batch] (what the last LogicLayer produces): out[b][g] =
  * (sum of the features/k rows of class g) * (1 / tau), the reciprocal rounded to dtype as torch's division of a
  * device tensor by a scalar does; fixed summation order (reproducible).

@@ -11,6 +11,18 @@ from tests.gpu_util import DEV, assert_grad_close
 pytestmark = pytest.mark.gpu
 
 
+def _layer_with(idx0, idx1, in_dim, dtype):
+    """A LogicLayer on the device with the given wiring (and the consumer lists that go with it)."""
+    from convlogic_amd.difflogic.difflogic import _reverse_wiring
+    layer = C.LogicLayer(in_dim, idx0.numel(), implementation="cuda")
+    layer.indices_0.copy_(idx0)
+    layer.indices_1.copy_(idx1)
+    start, flat = _reverse_wiring(idx0.numpy(), idx1.numpy(), in_dim)
+    layer.given_x_indices_of_y_start.copy_(start)
+    layer.given_x_indices_of_y.copy_(flat)
+    return layer.to(DEV).to(dtype)
+
+
 def _oracle_grads(x, logits, idx0, idx1, gy):
     xl = x.detach().cpu().clone().requires_grad_(True)
     ll = logits.detach().cpu().clone().requires_grad_(True)
@@ -206,6 +218,35 @@ def test_folded_kernels_equal_probability_kernels(in_dim, out_dim, batch, dtype)
     xa, xb = xl[layer.indices_0.cpu()], xl[layer.indices_1.cpu()]
     sums = torch.stack([(gl * xa * xb).sum(1), (gl * xa).sum(1), (gl * xb).sum(1), gl.sum(1)], 1)      # [out, 4]
     assert_grad_close(gw, (sums @ O.COEF).to(dtype), name="grad_w")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(24, 50, 8), (24, 50, 60), (40, 97, 100), (64, 131, 128), (30, 75, 256),
+                                                  (70, 40, 64), (7, 9, 33), (3, 5, 1), (8000, 8000, 256), (16, 8, 12)])
+def test_fused_backward_equals_the_two_kernels(in_dim, out_dim, batch, dtype):
+    # one walk over the consumer lists gives both gradients: bit for bit what the input-gradient kernel and the
+    # weight-gradient kernel give separately (w.r.t. the probabilities and w.r.t. the logits), for 16 / 32 / 64 lanes
+    # per row, inputs without consumers, and neurons that read the same feature twice
+    torch.manual_seed(in_dim * 3 + out_dim + batch)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV).to(dtype)
+    a, b = layer.indices_0.clone(), layer.indices_1.clone()
+    b[::5] = a[::5]                                                  # some neurons wired to one feature twice
+    layer = _layer_with(a.cpu(), b.cpu(), in_dim, dtype)
+    tabs = (layer.indices_0, layer.indices_1)
+    csr = (layer.given_x_indices_of_y_start, layer.given_x_indices_of_y)
+    x = torch.rand(in_dim, batch, device=DEV, dtype=dtype)
+    gy = torch.randn(out_dim, batch, device=DEV, dtype=dtype)
+    probs, folded = difflogic_hip.fold(layer.weights.detach(), from_logits=True)
+    fits = difflogic_hip.backward_fused_fits(x)
+    assert fits == (batch <= (256 if dtype == torch.float32 and batch % 4 == 0 else 128 if dtype == torch.float64 and batch % 2 == 0 else 64))
+    if not fits:
+        with pytest.raises(RuntimeError, match="exceeds what one pass covers"):
+            difflogic_hip.backward_fused(x, *tabs, folded, probs, gy, *csr)
+        return
+    gx_ref = difflogic_hip.backward_x_folded(x, *tabs, folded, gy, *csr)
+    for p_arg, gw_ref in ((None, difflogic_hip.backward_w(x, *tabs, gy)), (probs, difflogic_hip.backward_logits(x, *tabs, probs, gy))):
+        gx, gw = difflogic_hip.backward_fused(x, *tabs, folded, p_arg, gy, *csr)
+        assert torch.equal(gx, gx_ref) and torch.equal(gw, gw_ref)
 
 
 @pytest.mark.parametrize("features,batch,k", [(40, 7, 4), (640, 256, 10), (65536, 100, 8), (30, 1, 3), (10240, 256, 10)])
