@@ -55,10 +55,15 @@ def _cpu_model():
 VALU_LANE_OPS_PER_S = 256 * 64 * 2.4e9    # 256 CUs x 64 lanes x 2.4 GHz: one non-packed fp32 lane operation per lane and cycle
 
 
-def _timed(step, steps, warmup):
-    """warmup untimed steps, then exactly `steps` steps between two device synchronisations."""
+def _timed(step, steps, warmup, settle=0.0):
+    """warmup untimed steps, then exactly `steps` steps between two device synchronisations.  settle: keep taking
+    untimed steps until that many seconds have passed -- the sub-millisecond workloads are bound by the host in
+    eager mode, and a host that has just started runs them up to 40 % slower than a few hundred steps later."""
     import torch
+    t_start = time.perf_counter()
     for _ in range(warmup):
+        step(None)
+    while time.perf_counter() - t_start < settle:
         step(None)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -267,7 +272,7 @@ def bench_c1(steps, warmup, cpu=True):
         if k is not None:
             pairs[k][1].record()
 
-    sec = _timed(step, steps, warmup)
+    sec = _timed(step, steps, warmup, settle=0.5)
     gate_evals = batch * out_dim
     import copy
 
@@ -349,7 +354,7 @@ def bench_conv(key, steps, warmup, cpu=True):
         y = layer(x)
         y.backward(gy)
 
-    sec = _timed(step, steps, warmup)
+    sec = _timed(step, steps, warmup, settle=0.5)
     gate_evals = n * k * h * w * 7
     import copy
 
@@ -448,7 +453,7 @@ def bench_c5(steps, warmup, cpu=True):
             p.grad = None
         torch.nn.functional.cross_entropy(model(x), labels).backward()
 
-    sec = _timed(step, steps, warmup)
+    sec = _timed(step, steps, warmup, settle=0.5)
     import copy
 
     def leaves():
