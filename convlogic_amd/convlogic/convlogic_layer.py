@@ -77,13 +77,19 @@ class _FullConvLogicLogitsFunction(Function):
     (same values as softmax + FullConvLogicFunction up to rounding)."""
 
     @staticmethod
-    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
         x1, selection = x.contiguous(), selection.contiguous()
         w_prob = torch.softmax(logits, dim=-1)
         geo = (stride_h, stride_w, pad_h, pad_w)
+        ctx.geometry, ctx.kernel = geo, (kernel_h, kernel_w)
+        if feature_major and convlogic_hip.feature_major_supported(x1, logits.shape[0], *geo, kernel_h, kernel_w):
+            # y in memory as [C, Ho/2, Wo/2, N], handed out as the [N, C, Ho/2, Wo/2] view of it: nn.Flatten and the
+            # LogicLayer behind it then work on that memory without a transposed copy, and so does the way back
+            y_fm, argmax = convlogic_hip.full_convlogic_forward_fm(x1, w_prob, selection, *geo, kernel_h, kernel_w)
+            ctx.save_for_backward(x1, w_prob, selection, argmax)
+            return y_fm.permute(3, 0, 1, 2)
         y, argmax = convlogic_hip.full_convlogic_forward(x1, w_prob, selection, *geo, kernel_h, kernel_w)
         ctx.save_for_backward(x1, w_prob, selection, argmax)
-        ctx.geometry = geo
         return y
 
     @staticmethod
@@ -91,13 +97,19 @@ class _FullConvLogicLogitsFunction(Function):
         x1, w_prob, selection, argmax = ctx.saved_tensors
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         grad_x = grad_l = None
+        grad_fm = grad_y.permute(1, 2, 3, 0)
+        if (need_w and not grad_y.is_contiguous() and grad_fm.is_contiguous()
+                and convlogic_hip.feature_major_supported(x1, w_prob.shape[0], *ctx.geometry, *ctx.kernel)):
+            grad_x, grad_l = convlogic_hip.full_convlogic_backward_fm(grad_fm, x1, w_prob, argmax, selection, *ctx.geometry,
+                                                                     need_grad_x=need_x)
+            return grad_x, grad_l, None, None, None, None, None, None, None, None
         grad_y = grad_y.contiguous()
         if need_w:
             grad_x, grad_l = convlogic_hip.full_convlogic_backward_logits(grad_y, x1, w_prob, argmax, selection, *ctx.geometry,
                                                                          need_grad_x=need_x)
         elif need_x:
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
-        return grad_x, grad_l, None, None, None, None, None, None, None
+        return grad_x, grad_l, None, None, None, None, None, None, None, None
 
 
 def _pair(v):
@@ -187,7 +199,7 @@ class ConvLogicLayer(nn.Module):
         geo = (*self.stride, *self.padding, *self.kernel)
         if (self.complete and self.training and not self.return_intermediate and not self.return_indices
                 and self.weights.dtype == x.dtype and self.weights.is_contiguous()):
-            return _FullConvLogicLogitsFunction.apply(x, self.weights, sel, *geo)
+            return _FullConvLogicLogitsFunction.apply(x, self.weights, sel, *geo, getattr(self, "feature_major_output", False))
         w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
         if self.complete:
             return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)

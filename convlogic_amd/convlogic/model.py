@@ -35,6 +35,9 @@ class ConvLogicCifarModel(nn.Module):
         flat = widths[-1] * side * side
         m = self.extra_layers
         dims = [flat, m * flat * 10, m * flat * 5, m * (flat * 10) // 4]
+        # the last block feeds nn.Flatten and a LogicLayer, which reads feature-major memory: when the block's kernels
+        # can write that layout (4x4 images on the GPU) its output is the [N, C, 2, 2] view of a [C, 2, 2, N] tensor
+        blocks[-1].feature_major_output = implementation == "cuda"
         self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
 
     def forward(self, x):

@@ -1247,6 +1247,21 @@ extern "C" int clg_convblock_backward(int dtype, const clg_conv_geom *gg, const 
                                      "clg_convblock_backward", &shared);
 }
 
+extern "C" int clg_convblock_fm_supported(int dtype, const clg_conv_geom *gg);
+
+extern "C" int clg_convblock_backward_fm(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                         const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w,
+                                         int wrt_logits, void *scratch, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_fm")) return e;
+    CLG_REQUIRE(clg_convblock_fm_supported(dtype, gg), "clg_convblock_backward_fm: needs 4x4 images, a 3x3 kernel, stride 1, padding 1 "
+                "and at least 32 samples (clg_convblock_fm_supported)");
+    g.y_fm = 1;
+    return convblock_backward_4x4(dtype, g, grad_y, x, w, selection, argmax, grad_x, grad_w, scratch, stream, wrt_logits ? w : nullptr,
+                                  "clg_convblock_backward_fm");
+}
+
 extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
                                              const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_logits,
                                              void *scratch, void *stream)

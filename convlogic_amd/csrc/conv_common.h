@@ -5,6 +5,7 @@
 
 struct Geom {
     int n, cin, h, w, c, sh, sw, ph, pw, kh, kw, ho, wo;
+    int y_fm;   // 1: the block's output and its gradient are laid out [c, ho/2, wo/2, n] (4x4 kernels only), else [n, c, ho/2, wo/2]
 };
 
 static inline int clg_make_geom(const clg_conv_geom *g, Geom *out, const char *name)
@@ -22,7 +23,7 @@ static inline int clg_make_geom(const clg_conv_geom *g, Geom *out, const char *n
                 "%s: Invalid output shape: H_out=%d, W_out=%d", name, ho, wo);
     CLG_REQUIRE((int64_t)g->c_in * g->h * g->w < (1ll << 31) && (int64_t)g->c_out * ho * wo * 4 < (1ll << 31),
                 "%s: one sample must hold fewer than 2^31 elements", name);
-    *out = Geom{g->n, g->c_in, g->h, g->w, g->c_out, g->stride_h, g->stride_w, g->pad_h, g->pad_w, g->kernel_h, g->kernel_w, ho, wo};
+    *out = Geom{g->n, g->c_in, g->h, g->w, g->c_out, g->stride_h, g->stride_w, g->pad_h, g->pad_w, g->kernel_h, g->kernel_w, ho, wo, 0};
     return CLG_OK;
 }
 

@@ -637,6 +637,38 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
     return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
 }
 
+// Which shapes the feature-major variants take: the one-sample-per-lane kernels for 4x4 images (conv_small.hip).
+extern "C" int clg_convblock_fm_supported(int dtype, const clg_conv_geom *gg)
+{
+    Geom g;
+    if (gg == nullptr || (dtype != CLG_F32 && dtype != CLG_F64)) return 0;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_fm_supported")) return 0;
+    const char *e_fwd = getenv("CLG_FWD_4X4"), *e_bwd = getenv("CLG_BWD_4X4");
+    if ((e_fwd && atoi(e_fwd) == 0) || (e_bwd && atoi(e_bwd) == 0)) return 0;
+    return clg_convblock_is_4x4(g) && g.c <= 65535 ? 1 : 0;
+}
+
+extern "C" int clg_convblock_forward_fm(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                        void *y, uint8_t *argmax, void *scratch, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_forward_fm")) return e;
+    CLG_REQUIRE(x && w && selection && y && argmax && scratch, "clg_convblock_forward_fm: null pointer argument");
+    CLG_REQUIRE(clg_convblock_fm_supported(dtype, gg), "clg_convblock_forward_fm: needs 4x4 images, a 3x3 kernel, stride 1, padding 1 and "
+                "at least 32 samples (clg_convblock_fm_supported)");
+    g.y_fm = 1;
+    hipStream_t st = clg_stream(stream);
+    const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
+    if (dtype == CLG_F32)
+        hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
+                           (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
+    else
+        hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
+                           (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
+    CLG_CHECK_LAUNCH("clg_convblock_forward_fm");
+    return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_fm");
+}
+
 extern "C" int64_t clg_convblock_eval_packed_scratch_bytes(const clg_conv_geom *gg)
 {
     Geom g;

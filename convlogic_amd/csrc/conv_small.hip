@@ -143,12 +143,17 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
         }
         if (live) {
             const int64_t o = (n * g.c + c) * 4;
-            constexpr int PER = 16 / (int)sizeof(T);
+            if (g.y_fm) {                                             // [c, 2, 2, n]: the lanes' samples are neighbours
 #pragma unroll
-            for (int q = 0; q < 4 / PER; ++q) {
-                u32x4 raw;
-                __builtin_memcpy(&raw, &best[q * PER], 16);
-                reinterpret_cast<u32x4 *>(y + o)[q] = raw;
+                for (int cell = 0; cell < 4; ++cell) y[((int64_t)c * 4 + cell) * g.n + n] = best[cell];
+            } else {
+                constexpr int PER = 16 / (int)sizeof(T);
+#pragma unroll
+                for (int q = 0; q < 4 / PER; ++q) {
+                    u32x4 raw;
+                    __builtin_memcpy(&raw, &best[q * PER], 16);
+                    reinterpret_cast<u32x4 *>(y + o)[q] = raw;
+                }
             }
             if (argmax != nullptr) *reinterpret_cast<uint32_t *>(argmax + o) = (uint32_t)codes;
         }
@@ -351,7 +356,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_backward_4x4_kernel
             uint32_t codes = 0;
             if (live) {
 #pragma unroll
-                for (int cell = 0; cell < 4; ++cell) gout[cell] = gy[o + cell];
+                for (int cell = 0; cell < 4; ++cell) gout[cell] = g.y_fm ? gy[((int64_t)c * 4 + cell) * g.n + n] : gy[o + cell];
                 codes = *reinterpret_cast<const uint32_t *>(argmax + o);
             }
             {

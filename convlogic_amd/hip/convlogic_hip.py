@@ -246,6 +246,48 @@ def full_convlogic_backward_logits(grad_y, x, weight, argmax, selection, stride_
     return gx, gl
 
 
+def feature_major_supported(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """True when the block on x can write its output feature-major (full_convlogic_forward_fm)."""
+    if not (x.is_cuda and x.dim() == 4 and x.dtype in (torch.float32, torch.float64)):
+        return False
+    g = _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    return bool(_lib.load().clg_convblock_fm_supported(dtype_code(x), ctypes.byref(g)))
+
+
+def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """full_convlogic_forward() with y laid out [C, Ho/2, Wo/2, N] (contiguous); argmax stays [N,C,Ho/2,Wo/2]."""
+    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    y = torch.empty((g.c_out, ho // 2, wo // 2, g.n), dtype=x.dtype, device=x.device)
+    argmax = torch.empty((g.n, g.c_out, ho // 2, wo // 2), dtype=torch.uint8, device=x.device)
+    lib = _lib.load()
+    scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
+    check(lib.clg_convblock_forward_fm(dtype_code(x), ctypes.byref(g), x.data_ptr(), weight.data_ptr(), selection.data_ptr(),
+                                       y.data_ptr(), argmax.data_ptr(), scratch.data_ptr() if scratch is not None else None,
+                                       stream_ptr(x)))
+    return y, argmax
+
+
+def full_convlogic_backward_fm(grad_y_fm, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True,
+                               wrt_logits=True):
+    """-> (grad_x or None, grad_w [C,7,16]) from grad_y laid out [C, Ho/2, Wo/2, N]; grad_w is the gradient w.r.t. the
+    logits (weight = their softmax) or, with wrt_logits=False, w.r.t. the probabilities."""
+    for t, n in ((grad_y_fm, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom_from_out(x, grad_y_fm.shape[0], 2 * grad_y_fm.shape[1], 2 * grad_y_fm.shape[2], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    scratch = _scratch(lib.clg_convblock_backward_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gx = torch.empty_like(x) if need_grad_x else None
+    gw = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_convblock_backward_fm(dt, ctypes.byref(g), grad_y_fm.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                        selection.data_ptr(), argmax.data_ptr(), gx.data_ptr() if need_grad_x else None,
+                                        gw.data_ptr(), 1 if wrt_logits else 0, scratch.data_ptr(), stream_ptr(x)))
+    return gx, gw
+
+
 # ---- input binarisation -------------------------------------------------------------------------
 def _threshold_args(x, thresholds):
     check_input(x, "x")

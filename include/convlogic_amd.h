@@ -317,6 +317,22 @@ int clg_convblock_backward_logits(int dtype, const clg_conv_geom *g, const void 
                                   const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_logits,
                                   void *scratch, void *stream);
 
+/* The complete block with its output (and the output's gradient) laid out feature-major, [c_out, ho/2, wo/2, n] -- the
+ * layout the LogicLayer behind nn.Flatten reads, so that neither direction needs a transposed copy.  For the shapes of
+ * clg_convblock_fm_supported() != 0 (4x4 images, 3x3 kernel, stride 1, padding 1, n >= 32: the last block of a
+ * 32x32-input network); argmax, x and grad_x keep their layouts.  Scratch: clg_convblock_forward_scratch_bytes /
+ * clg_convblock_backward_scratch_bytes.  grad_w: gradient w.r.t. the logits when wrt_logits != 0 (w = their softmax),
+ * else w.r.t. the probabilities w; grad_x may be NULL.  Same values as clg_convblock_forward_ws /
+ * clg_convblock_backward(_logits) on the permuted tensors.  Replaces full_convlogic_forward / _backward_x /
+ * _backward_weight (src/convlogic/cuda/convlogic.cpp:29-37) plus the copies around
+ * x.transpose(0, 1).contiguous() in LogicLayer.forward_cuda (src/difflogic/difflogic.py:130-141). */
+int clg_convblock_fm_supported(int dtype, const clg_conv_geom *g);
+int clg_convblock_forward_fm(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection,
+                             void *y /*[c_out,ho/2,wo/2,n]*/, uint8_t *argmax, void *scratch, void *stream);
+int clg_convblock_backward_fm(int dtype, const clg_conv_geom *g, const void *grad_y /*[c_out,ho/2,wo/2,n]*/, const void *x,
+                              const void *w, const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w,
+                              int wrt_logits, void *scratch, void *stream);
+
 /* ---------------------------------------------------------------------------------
  * input binarisation (the step in front of the first layer)
  * --------------------------------------------------------------------------------- */

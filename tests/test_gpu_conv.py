@@ -351,3 +351,49 @@ def test_block_4x4_one_sample_per_lane_gradients(n, cin, cout, dtype, monkeypatc
                     continue
                 scale = max(b.abs().max().item(), 1e-30)
                 assert (a - b).abs().max().item() <= tol * scale, key
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,cin,cout", [(32, 3, 5), (100, 24, 48), (130, 40, 17)])
+def test_block_4x4_feature_major_output(n, cin, cout, dtype):
+    # the last block of a 32x32-input network can lay its output out [C, 2, 2, N] for the LogicLayer behind nn.Flatten:
+    # same values as the [N, C, 2, 2] kernels bit for bit, forward and both gradients, and the module chain
+    # block -> Flatten -> LogicLayer then runs without transposed copies in either direction
+    from convlogic_amd.hip import convlogic_hip
+    torch.manual_seed(n * 7 + cin)
+    layer = C.ConvLogicLayer(cin, cout, padding=1, complete=True, implementation="cuda").to(DEV).to(dtype)
+    x = torch.rand(n, cin, 4, 4, device=DEV, dtype=dtype)
+    wp = torch.softmax(layer.weights.detach(), -1)
+    geo = (1, 1, 1, 1)
+    assert convlogic_hip.feature_major_supported(x, cout, *geo, 3, 3)
+    assert not convlogic_hip.feature_major_supported(x[:8], cout, *geo, 3, 3)           # fewer than 32 samples
+    assert not convlogic_hip.feature_major_supported(torch.rand(n, cin, 8, 8, device=DEV, dtype=dtype), cout, *geo, 3, 3)
+    y, am = convlogic_hip.full_convlogic_forward(x, wp, layer.selection, *geo, 3, 3)
+    y_fm, am_fm = convlogic_hip.full_convlogic_forward_fm(x, wp, layer.selection, *geo, 3, 3)
+    assert y_fm.shape == (cout, 2, 2, n) and torch.equal(y_fm.permute(3, 0, 1, 2), y) and torch.equal(am_fm, am)
+    gy = torch.randn_like(y)
+    gy_fm = gy.permute(1, 2, 3, 0).contiguous()
+    for need_x in (True, False):
+        gx, gl = convlogic_hip.full_convlogic_backward_logits(gy, x, wp, am, layer.selection, *geo, need_grad_x=need_x)
+        gx_fm, gl_fm = convlogic_hip.full_convlogic_backward_fm(gy_fm, x, wp, am, layer.selection, *geo, need_grad_x=need_x)
+        assert torch.equal(gl, gl_fm) and (gx is None and gx_fm is None or torch.equal(gx, gx_fm))
+    _, gw = convlogic_hip.full_convlogic_backward(gy, x, wp, am, layer.selection, *geo)
+    _, gw_fm = convlogic_hip.full_convlogic_backward_fm(gy_fm, x, wp, am, layer.selection, *geo, wrt_logits=False)
+    assert torch.equal(gw, gw_fm)
+    with pytest.raises(RuntimeError, match="clg_convblock_fm_supported"):
+        convlogic_hip.full_convlogic_forward_fm(x[:8].contiguous(), wp, layer.selection, *geo, 3, 3)
+    # module chain: the same losses and gradients with and without the layout
+    head = C.LogicLayer(cout * 4, cout * 8, implementation="cuda").to(DEV).to(dtype)
+    gout = torch.randn(n, cout * 8, device=DEV, dtype=dtype)
+    grads = {}
+    for fm in (False, True):
+        layer.feature_major_output = fm
+        xin = x.clone().requires_grad_(True)
+        layer.weights.grad = head.weights.grad = None
+        h = layer(xin)
+        assert h.shape == (n, cout, 2, 2) and h.is_contiguous() != fm
+        out = head(torch.flatten(h, 1))
+        out.backward(gout)
+        grads[fm] = (out.detach(), xin.grad, layer.weights.grad.clone(), head.weights.grad.clone())
+    for a, b in zip(grads[False], grads[True]):
+        assert torch.equal(a, b)
