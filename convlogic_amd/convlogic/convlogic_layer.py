@@ -216,7 +216,8 @@ class ConvLogicLayer(nn.Module):
             raise RuntimeError("packed evaluation needs implementation='cuda'")
         assert x.image and x.t.dim() == 4 and x.t.shape[1] == self.in_channels, (x.image, tuple(x.t.shape), self.in_channels)
         x.t = convlogic_hip.full_convlogic_eval_packed(x.t.contiguous(), self._eval_gates(), self.selection.contiguous(),
-                                                       *self.stride, *self.padding, *self.kernel)
+                                                       *self.stride, *self.padding, *self.kernel,
+                                                       feature_major=getattr(self, "feature_major_output", False))
         return x
 
     def _eval_gates(self):

@@ -669,6 +669,27 @@ extern "C" int clg_convblock_forward_fm(int dtype, const clg_conv_geom *gg, cons
     return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_fm");
 }
 
+extern "C" int clg_convblock_eval_packed_fm_supported(const clg_conv_geom *gg)
+{
+    Geom g;
+    if (gg == nullptr || clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed_fm_supported")) return 0;
+    const char *e_4x4 = getenv("CLG_FWD_4X4");
+    return clg_convblock_is_4x4(g) && (!e_4x4 || atoi(e_4x4) != 0) ? 1 : 0;
+}
+
+extern "C" int clg_convblock_eval_packed_fm(const clg_conv_geom *gg, const uint64_t *x, const uint8_t *gates, const int32_t *selection,
+                                            uint64_t *y, void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed_fm")) return e;
+    CLG_REQUIRE(x && gates && selection && y, "clg_convblock_eval_packed_fm: null pointer argument");
+    CLG_REQUIRE(x != y, "clg_convblock_eval_packed_fm: x and y must not overlap");
+    CLG_REQUIRE(clg_convblock_eval_packed_fm_supported(gg), "clg_convblock_eval_packed_fm: needs 4x4 images, a 3x3 kernel, stride 1, "
+                "padding 1 and at least 32 word groups (clg_convblock_eval_packed_fm_supported)");
+    g.y_fm = 1;
+    return clg_convblock_eval_packed_4x4(g, x, gates, selection, y, clg_stream(stream), "clg_convblock_eval_packed_fm");
+}
+
 extern "C" int64_t clg_convblock_eval_packed_scratch_bytes(const clg_conv_geom *gg)
 {
     Geom g;

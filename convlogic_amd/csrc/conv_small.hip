@@ -242,7 +242,7 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
                     }
                     pooled |= BitOps::root(pr, v);
                 }
-                if (live) y[(n * g.c + c) * 4 + cell] = pooled;
+                if (live) y[g.y_fm ? ((int64_t)c * 4 + cell) * g.n + n : (n * g.c + c) * 4 + cell] = pooled;
             }
         } else {
             uint64_t best[4] = {0, 0, 0, 0};
@@ -282,9 +282,14 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
             }
             if (more) fetch(cn);
             if (live) {
-                u32x4 *out = reinterpret_cast<u32x4 *>(y + (n * g.c + c) * 4);
-                out[0] = u32x4{(uint32_t)best[0], (uint32_t)(best[0] >> 32), (uint32_t)best[1], (uint32_t)(best[1] >> 32)};
-                out[1] = u32x4{(uint32_t)best[2], (uint32_t)(best[2] >> 32), (uint32_t)best[3], (uint32_t)(best[3] >> 32)};
+                if (g.y_fm) {                                         // [c, 2, 2, groups]: the lanes' groups are neighbours
+#pragma unroll
+                    for (int cell = 0; cell < 4; ++cell) y[((int64_t)c * 4 + cell) * g.n + n] = best[cell];
+                } else {
+                    u32x4 *out = reinterpret_cast<u32x4 *>(y + (n * g.c + c) * 4);
+                    out[0] = u32x4{(uint32_t)best[0], (uint32_t)(best[0] >> 32), (uint32_t)best[1], (uint32_t)(best[1] >> 32)};
+                    out[1] = u32x4{(uint32_t)best[2], (uint32_t)(best[2] >> 32), (uint32_t)best[3], (uint32_t)(best[3] >> 32)};
+                }
             }
         }
         if (!more) break;

@@ -57,10 +57,15 @@ class PackBitsTensor:
 
     def flatten(self, start_dim=0, end_dim=-1, **kwargs):
         """nn.Flatten is a no-op on feature-major packed activations (src/difflogic/packbitstensor.py:26-31);
-        a group-major image batch becomes feature-major here (one 8-byte transpose)."""
+        a group-major image batch becomes feature-major here (one 8-byte transpose, or a view when the last
+        block already wrote its words feature-major)."""
         if self.image:
             groups = self.t.shape[0]
-            self.t = difflogic_hip.transpose(self.t.reshape(groups, -1))
+            by_feature = self.t.permute(*range(1, self.t.dim()), 0)
+            if by_feature.is_contiguous():                           # a block that wrote [C, H, W, G]: already feature-major
+                self.t = by_feature.reshape(-1, groups)
+            else:
+                self.t = difflogic_hip.transpose(self.t.reshape(groups, -1))
             self.image = False
         return self
 

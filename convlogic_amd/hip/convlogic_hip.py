@@ -139,11 +139,13 @@ def full_convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_
     return y, argmax
 
 
-def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
     """Packed-bit inference of the fused block.  x: int64 words [G, C_in, H, W], 64 samples per word
     (bit s of group g = sample 64 g + s); gates: uint8 [C, 7] arg-max gate ids; -> int64 [G, C, Ho/2, Wo/2].
     Equals the eval-mode float block on binary inputs (src/convlogic/convlogic_layer.py:231-316,321-325);
-    the reference has no packed conv kernel."""
+    the reference has no packed conv kernel.  feature_major: where the kernels can (4x4 images, at least 32
+    groups), the result is the [G, C, Ho/2, Wo/2] VIEW of a contiguous [C, Ho/2, Wo/2, G] tensor -- the layout
+    PackBitsTensor.flatten() needs, which then takes a view instead of transposing."""
     for t, n in ((x, "x"), (gates, "gates"), (selection, "selection")):
         check_input(t, n)
     if x.dtype != torch.int64 or gates.dtype != torch.uint8 or x.dim() != 4:
@@ -152,8 +154,13 @@ def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, p
         raise RuntimeError(f"full_convlogic_eval_packed expects gate ids of shape [C, 7], got {tuple(gates.shape)}")
     g = _geom(x, gates.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
-    y = torch.empty((g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2), dtype=torch.int64, device=x.device)
     lib = _lib.load()
+    if feature_major and lib.clg_convblock_eval_packed_fm_supported(ctypes.byref(g)):
+        y = torch.empty((g.c_out, ho // 2, wo // 2, g.n), dtype=torch.int64, device=x.device)
+        check(lib.clg_convblock_eval_packed_fm(ctypes.byref(g), x.data_ptr(), gates.data_ptr(), selection.data_ptr(), y.data_ptr(),
+                                               stream_ptr(x)))
+        return y.permute(3, 0, 1, 2)
+    y = torch.empty((g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2), dtype=torch.int64, device=x.device)
     scratch = _scratch(lib.clg_convblock_eval_packed_scratch_bytes(ctypes.byref(g)), x.device)
     check(lib.clg_convblock_eval_packed_ws(ctypes.byref(g), x.data_ptr(), gates.data_ptr(), selection.data_ptr(), y.data_ptr(),
                                            scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))

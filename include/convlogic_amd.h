@@ -327,6 +327,11 @@ int clg_convblock_backward_logits(int dtype, const clg_conv_geom *g, const void 
  * _backward_weight (src/convlogic/cuda/convlogic.cpp:29-37) plus the copies around
  * x.transpose(0, 1).contiguous() in LogicLayer.forward_cuda (src/difflogic/difflogic.py:130-141). */
 int clg_convblock_fm_supported(int dtype, const clg_conv_geom *g);
+/* The same for packed words: y laid out [c_out, ho/2, wo/2, groups], which IS the feature-major [features, words] layout
+ * of clg_fc_eval_packed (feature = (c, y, x) in nn.Flatten order), so PackBitsTensor.flatten needs no transpose. */
+int clg_convblock_eval_packed_fm_supported(const clg_conv_geom *g);
+int clg_convblock_eval_packed_fm(const clg_conv_geom *g, const uint64_t *x, const uint8_t *gates, const int32_t *selection,
+                                 uint64_t *y /*[c_out,ho/2,wo/2,groups]*/, void *stream);
 int clg_convblock_forward_fm(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection,
                              void *y /*[c_out,ho/2,wo/2,n]*/, uint8_t *argmax, void *scratch, void *stream);
 int clg_convblock_backward_fm(int dtype, const clg_conv_geom *g, const void *grad_y /*[c_out,ho/2,wo/2,n]*/, const void *x,

@@ -170,6 +170,34 @@ def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
     assert torch.equal(whole, p.t)
 
 
+@pytest.mark.parametrize("samples,cin,cout", [(2048, 6, 9), (4160, 16, 33), (8192, 12, 21), (1000, 6, 9)])
+def test_packed_block_4x4_feature_major_output(samples, cin, cout):
+    # the last block can write its words [C, 2, 2, G]: the same words as the [G, C, 2, 2] kernels, flatten() then takes a
+    # view instead of a transpose, and the packed LogicLayer behind it gives the same result; batches below 32 groups
+    # (the 1000-sample case) keep the group-major kernels and the transpose
+    torch.manual_seed(samples + cout)
+    layer = _layer(cin, cout, 1, 1, 3, seed=5)
+    bits = torch.randint(0, 2, (samples, cin, 4, 4), device=DEV).bool()
+    gates = layer.weights.argmax(-1).to(torch.uint8)
+    x_words = C.PackBitsTensor(bits, 64).t
+    plain = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
+    fm = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3, feature_major=True)
+    groups = x_words.shape[0]
+    assert fm.shape == plain.shape and torch.equal(fm, plain)
+    assert fm.is_contiguous() == (groups < 32) and (groups < 32 or fm.permute(1, 2, 3, 0).is_contiguous())
+    head = C.LogicLayer(cout * 4, cout * 8, implementation="cuda").to(DEV).eval()
+    outs = []
+    for flag in (False, True):
+        layer.feature_major_output = flag
+        p = layer(C.PackBitsTensor(bits, 64))
+        before = p.t.data_ptr()
+        p.flatten()
+        assert p.t.shape == (cout * 4, groups) and p.t.is_contiguous() and not p.image
+        assert (p.t.data_ptr() == before) == (flag and groups >= 32)           # a view of the block's output, or a transposed copy
+        outs.append(head(p).t.clone())
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("n,cin,cout,hw", [(70, 128, 24, 8), (5, 6, 9, 4), (33, 40, 16, 2), (3, 3, 8, 16)])
 def test_one_position_per_lane_equals_two_rows_per_lane(n, cin, cout, hw, monkeypatch):
     # workgroups whose samples fill at most half a wavefront with (row pair, column) slots give every conv position
