@@ -78,19 +78,17 @@ class _FullConvLogicLogitsFunction(Function):
 
     @staticmethod
     def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
-        x1, selection = x.contiguous(), selection.contiguous()
-        w_prob = torch.softmax(logits, dim=-1)
+        x1, selection, logits = x.contiguous(), selection.contiguous(), logits.contiguous()
         geo = (stride_h, stride_w, pad_h, pad_w)
         ctx.geometry, ctx.kernel = geo, (kernel_h, kernel_w)
-        if feature_major and convlogic_hip.feature_major_supported(x1, logits.shape[0], *geo, kernel_h, kernel_w):
-            # y in memory as [C, Ho/2, Wo/2, N], handed out as the [N, C, Ho/2, Wo/2] view of it: nn.Flatten and the
-            # LogicLayer behind it then work on that memory without a transposed copy, and so does the way back
-            y_fm, argmax = convlogic_hip.full_convlogic_forward_fm(x1, w_prob, selection, *geo, kernel_h, kernel_w)
-            ctx.save_for_backward(x1, w_prob, selection, argmax)
-            return y_fm.permute(3, 0, 1, 2)
-        y, argmax = convlogic_hip.full_convlogic_forward(x1, w_prob, selection, *geo, kernel_h, kernel_w)
+        # y in memory as [C, Ho/2, Wo/2, N] where asked for and possible, handed out as the [N, C, Ho/2, Wo/2] view of it:
+        # nn.Flatten and the LogicLayer behind it then work on that memory without a transposed copy, and so does the
+        # way back
+        fm = feature_major and convlogic_hip.feature_major_supported(x1, logits.shape[0], *geo, kernel_h, kernel_w)
+        y, argmax, w_prob = convlogic_hip.full_convlogic_forward_logits(x1, logits.detach(), selection, *geo, kernel_h, kernel_w,
+                                                                        feature_major=fm)
         ctx.save_for_backward(x1, w_prob, selection, argmax)
-        return y
+        return y.permute(3, 0, 1, 2) if fm else y
 
     @staticmethod
     def backward(ctx, grad_y):

@@ -55,6 +55,27 @@ __device__ __forceinline__ Coef<T> fold16(const T *__restrict__ w)
     return c;
 }
 
+// softmax of 16 logits (maximum subtracted, one reciprocal), as clg_fc_fold computes it
+template <typename T>
+__device__ __forceinline__ void softmax16(const T *__restrict__ logits, T (&p)[16])
+{
+    T m = logits[0];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        p[i] = logits[i];
+        m = p[i] > m ? p[i] : m;
+    }
+    T sum = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        p[i] = exp(p[i] - m);
+        sum += p[i];
+    }
+    const T inv = T(1) / sum;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] *= inv;
+}
+
 template <typename T>
 __device__ __forceinline__ T fma_t(T a, T b, T c);
 template <>

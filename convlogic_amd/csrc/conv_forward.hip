@@ -39,7 +39,7 @@ namespace {
 template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW>
 __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
                                                const int32_t *__restrict__ sel, typename Ops::Elem *__restrict__ y,
-                                               uint8_t *__restrict__ argmax, Geom g, TilePlan p)
+                                               uint8_t *__restrict__ argmax, Geom g, TilePlan p, void *__restrict__ probs_out)
 {
     using T = typename Ops::Elem;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -58,7 +58,8 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     const int hw = g.h * g.w;
 
     for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
-    Ops::stage_params(coef, params, c0, ct_cur, tid, nthreads);
+    // logits in (plan.w_logits): every workgroup takes the softmax of its kernels, the first sample block writes it out
+    Ops::stage_params(coef, params, c0, ct_cur, tid, nthreads, p.w_logits != 0, blockIdx.x == 0 ? probs_out : nullptr);
     if (!SUBSET) {
         for (int q = tid; q < ct_cur * 8; q += nthreads) {
             const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
@@ -400,6 +401,7 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     // A workgroup whose samples fill at most half a wavefront with (row pair, column) slots gives every conv position
     // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64), two
     // kernels per step.  Measured on [*,128,8,8] -> 512: packed words 174 -> 102 us, float32 39 -> 32 us.
+    p->w_logits = 0;
     p->one_row = 0;
     if ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
     if (const char *e = getenv("CLG_FWD_ONE_ROW")) p->one_row = p->one_row && atoi(e) != 0;   // 0: never
@@ -482,7 +484,8 @@ int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scr
 
 template <typename Ops, typename P>
 int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, const void *params, const int32_t *sel, void *y,
-                          uint8_t *argmax, void *scratch, hipStream_t st, const char *name)
+                          uint8_t *argmax, void *scratch, hipStream_t st, const char *name, bool from_logits = false,
+                          void *probs_out = nullptr)
 {
     using T = typename Ops::Elem;
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
@@ -495,7 +498,7 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
     const unsigned prep = (unsigned)clg_ceil_div((int64_t)g.c * 8, 256);
     hipLaunchKernelGGL((convblock_w_prepare_kernel<P, T>), dim3(prep + pad_blocks(job)), dim3(256), 0, st,
                        fold ? (const P *)params : (const P *)nullptr, sel, fold ? reinterpret_cast<P *>(base) : (P *)nullptr, taps, g.c,
-                       d.p.rs, d.p.chs, job, (int)prep);
+                       d.p.rs, d.p.chs, job, (int)prep, fold && from_logits ? 1 : 0, reinterpret_cast<P *>(probs_out));
     CLG_CHECK_LAUNCH(name);
     const int64_t sets = clg_ceil_div(g.n, d.p.G) * d.nblk;
     hipLaunchKernelGGL(convblock_forward_direct_kernel<Ops>, dim3((unsigned)clg_ceil_div(sets, 4), (unsigned)clg_ceil_div(g.c, d.p.CT)),
@@ -508,13 +511,13 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
 // ---- launch ------------------------------------------------------------------------------------
 template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW = false>
 int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
-                       uint8_t *argmax, hipStream_t st, const char *name)
+                       uint8_t *argmax, hipStream_t st, const char *name, void *probs_out = nullptr)
 {
     using T = typename Ops::Elem;
     if (int e = allow_lds(convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET, ONE_ROW>, p.lds_bytes, name)) return e;
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)clg_ceil_div(g.c, p.CT));
     hipLaunchKernelGGL((convblock_forward_tiled_kernel<Ops, ROWSTEP, SUBSET, ONE_ROW>), grid, dim3(p.NW * kWave), p.lds_bytes, st, (const T *)x,
-                       params, sel, (T *)y, argmax, g, p);
+                       params, sel, (T *)y, argmax, g, p, probs_out);
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }
@@ -523,17 +526,17 @@ int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const vo
 // instantiation; everything else reads the step from the plan.
 template <typename Ops>
 int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
-                         uint8_t *argmax, hipStream_t st, const char *name)
+                         uint8_t *argmax, hipStream_t st, const char *name, void *probs_out = nullptr)
 {
 #define CLG_FWD_CASE(RS)                                                                                              \
     case RS:                                                                                                          \
-        return p.subset ? launch_forward_one<Ops, RS, true>(g, p, x, params, sel, y, argmax, st, name)                \
-                        : launch_forward_one<Ops, RS, false>(g, p, x, params, sel, y, argmax, st, name)
+        return p.subset ? launch_forward_one<Ops, RS, true>(g, p, x, params, sel, y, argmax, st, name, probs_out)                \
+                        : launch_forward_one<Ops, RS, false>(g, p, x, params, sel, y, argmax, st, name, probs_out)
     if (p.one_row) {                                                 // ROWSTEP names wo when a DPP row shift reaches the row below
-        if (p.subset) return launch_forward_one<Ops, 0, true, true>(g, p, x, params, sel, y, argmax, st, name);
-        if (g.wo == 8) return launch_forward_one<Ops, 8, false, true>(g, p, x, params, sel, y, argmax, st, name);
-        if (g.wo == 4) return launch_forward_one<Ops, 4, false, true>(g, p, x, params, sel, y, argmax, st, name);
-        return launch_forward_one<Ops, 0, false, true>(g, p, x, params, sel, y, argmax, st, name);
+        if (p.subset) return launch_forward_one<Ops, 0, true, true>(g, p, x, params, sel, y, argmax, st, name, probs_out);
+        if (g.wo == 8) return launch_forward_one<Ops, 8, false, true>(g, p, x, params, sel, y, argmax, st, name, probs_out);
+        if (g.wo == 4) return launch_forward_one<Ops, 4, false, true>(g, p, x, params, sel, y, argmax, st, name, probs_out);
+        return launch_forward_one<Ops, 0, false, true>(g, p, x, params, sel, y, argmax, st, name, probs_out);
     }
     switch (g.sh * p.rs) {
         CLG_FWD_CASE(33);
@@ -542,8 +545,8 @@ int launch_forward_tiled(const Geom &g, const TilePlan &p, const void *x, const 
         CLG_FWD_CASE(9);
         CLG_FWD_CASE(5);
     default:
-        return p.subset ? launch_forward_one<Ops, 0, true>(g, p, x, params, sel, y, argmax, st, name)
-                        : launch_forward_one<Ops, 0, false>(g, p, x, params, sel, y, argmax, st, name);
+        return p.subset ? launch_forward_one<Ops, 0, true>(g, p, x, params, sel, y, argmax, st, name, probs_out)
+                        : launch_forward_one<Ops, 0, false>(g, p, x, params, sel, y, argmax, st, name, probs_out);
     }
 #undef CLG_FWD_CASE
 }
@@ -635,6 +638,82 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
     if (dtype == CLG_F32)
         return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
     return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, "clg_convblock_forward_ws");
+}
+
+namespace {
+// probabilities of a [rows, 16] logit table: for the any-shape forward, whose kernel takes probabilities
+template <typename T>
+__global__ __launch_bounds__(256) void softmax16_rows_kernel(const T *__restrict__ logits, T *__restrict__ probs, int64_t rows)
+{
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= rows) return;
+    T pr[16];
+    softmax16(logits + q * 16, pr);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) probs[q * 16 + i] = pr[i];
+}
+}  // namespace
+
+// Forward of the complete block with options (flags: CLG_FWD_W_LOGITS, CLG_FWD_Y_FEATURE_MAJOR).
+extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                        void *y, uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream)
+{
+    const char *name = "clg_convblock_forward_ex";
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
+    CLG_REQUIRE(x && w && selection && y && argmax, "%s: null pointer argument", name);
+    CLG_REQUIRE((flags & ~(CLG_FWD_W_LOGITS | CLG_FWD_Y_FEATURE_MAJOR)) == 0, "%s: unknown flags 0x%x", name, flags);
+    const bool logits = (flags & CLG_FWD_W_LOGITS) != 0, fm = (flags & CLG_FWD_Y_FEATURE_MAJOR) != 0;
+    CLG_REQUIRE(!logits || probs_out, "%s: CLG_FWD_W_LOGITS needs probs_out [c_out, 7, 16]", name);
+    CLG_REQUIRE(!fm || (scratch && clg_convblock_fm_supported(dtype, gg)), "%s: CLG_FWD_Y_FEATURE_MAJOR needs scratch and a shape for "
+                "which clg_convblock_fm_supported() holds (4x4 images, 3x3 kernel, stride 1, padding 1, n >= 32)", name);
+    TilePlan tp;
+    DirectPlan dp;
+    const int elem = dtype == CLG_F64 ? 8 : 4;
+    const int path = fm ? 4 : choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp);
+    hipStream_t st = clg_stream(stream);
+    if (path == 4) {
+        g.y_fm = fm ? 1 : 0;
+        const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
+        if (dtype == CLG_F32)
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
+                               (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
+                               (float *)probs_out);
+        else
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
+                               (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
+                               (double *)probs_out);
+        CLG_CHECK_LAUNCH(name);
+        return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, name);
+    }
+    if (path == 2) {
+        if (dtype == CLG_F32)
+            return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
+        return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
+    }
+    // The staged kernels take the softmax per workgroup while they set their gate parameters up (measured against a
+    // small launch of its own: C3 graph step 63.7 vs 66.7 us, C5 451 vs 459 us, C4 the same); the any-shape kernel
+    // gets its probabilities from that small launch.
+    const bool staged = path == 0 || path == 1;
+    bool in_kernel = staged && logits;
+    if (const char *e = getenv("CLG_FWD_SOFTMAX_IN_KERNEL")) in_kernel = staged && logits && atoi(e) != 0;
+    if (logits && !in_kernel) {
+        const int64_t rows = (int64_t)g.c * 7;
+        if (dtype == CLG_F32)
+            hipLaunchKernelGGL(softmax16_rows_kernel<float>, dim3((unsigned)clg_ceil_div(rows, 256)), dim3(256), 0, st, (const float *)w,
+                               (float *)probs_out, rows);
+        else
+            hipLaunchKernelGGL(softmax16_rows_kernel<double>, dim3((unsigned)clg_ceil_div(rows, 256)), dim3(256), 0, st, (const double *)w,
+                               (double *)probs_out, rows);
+        CLG_CHECK_LAUNCH(name);
+        w = probs_out;
+    }
+    if (staged) {
+        tp.w_logits = in_kernel ? 1 : 0;
+        if (dtype == CLG_F32) return launch_forward_tiled<FloatOps<float>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
+        return launch_forward_tiled<FloatOps<double>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
+    }
+    return clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, st);
 }
 
 // Which shapes the feature-major variants take: the one-sample-per-lane kernels for 4x4 images (conv_small.hip).

@@ -16,13 +16,27 @@ struct FloatOps {
     struct Params {
         Tree<T> tr;
     };
-    // params = gate probabilities [c_out, 7, 16]
+    // params = gate probabilities [c_out, 7, 16], or the logits (from_logits): then the softmax is taken here and, where
+    // probs_out is given, written out for the backward pass
     static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
-                                                        int tid, int nthreads)
+                                                        int tid, int nthreads, bool from_logits = false, void *probs_out = nullptr)
     {
         const T *w = reinterpret_cast<const T *>(params);
         for (int q = tid; q < ct_cur * 7; q += nthreads) {
-            const Coef<T> cf = fold16(w + ((int64_t)c0 * 7 + q) * 16);
+            const T *row = w + ((int64_t)c0 * 7 + q) * 16;
+            T pr[16];
+            if (from_logits) {
+                softmax16(row, pr);
+                if (probs_out != nullptr) {
+                    T *po = reinterpret_cast<T *>(probs_out) + ((int64_t)c0 * 7 + q) * 16;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) po[i] = pr[i];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) pr[i] = row[i];
+            }
+            const Coef<T> cf = fold16(pr);
             dst[q * 4 + 0] = cf.ab;
             dst[q * 4 + 1] = cf.a;
             dst[q * 4 + 2] = cf.b;
@@ -105,7 +119,7 @@ struct BitOps {
     };
     // params = gate ids uint8 [c_out, 7]
     static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
-                                                        int tid, int nthreads)
+                                                        int tid, int nthreads, bool = false, void * = nullptr)
     {
         const uint8_t *gid = reinterpret_cast<const uint8_t *>(params);
         for (int q = tid; q < ct_cur; q += nthreads) {
@@ -204,7 +218,7 @@ struct BitOpsAnf {
     }
     // params = gate ids uint8 [c_out, 7]
     static __device__ __forceinline__ void stage_params(Elem *__restrict__ dst, const void *__restrict__ params, int c0, int ct_cur,
-                                                        int tid, int nthreads)
+                                                        int tid, int nthreads, bool = false, void * = nullptr)
     {
         const uint8_t *gid = reinterpret_cast<const uint8_t *>(params);
         for (int q = tid; q < ct_cur; q += nthreads) dst[q] = tree_code(gid + ((int64_t)c0 + q) * 7);

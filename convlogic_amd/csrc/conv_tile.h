@@ -36,6 +36,7 @@ struct TilePlan {
     int planes;            // forward: LDS planes per sample (all input channels, or 2 per kernel of the tile)
     int subset;            // forward: 1 = only the channels the kernel tile reads are staged
     int one_row;           // forward: 1 = a lane slot is one conv position (ho * wo per sample) instead of a column of two rows
+    int w_logits;          // forward: 1 = the gate parameters handed to the kernel are logits (softmax taken while staging them)
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp, d_planes;
     size_t lds_bytes;
 };
@@ -178,10 +179,12 @@ static inline unsigned pad_blocks(const PadJob<T> &j) { return (unsigned)clg_cei
 
 // folded coefficients [c][28] and tap offsets [c][8] in the padded-image layout (either is skipped when null) in the
 // first blocks of the launch, the padded copy in the blocks from pad_block0 on: one launch sets a kernel up.
+// from_logits: w holds the logits, whose softmax goes to probs_out.
 template <typename P, typename T>
 __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const P *__restrict__ w, const int32_t *__restrict__ sel,
                                                                 P *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
-                                                                int chs, PadJob<T> pad, int pad_block0)
+                                                                int chs, PadJob<T> pad, int pad_block0, int from_logits = 0,
+                                                                P *__restrict__ probs_out = nullptr)
 {
     if ((int)blockIdx.x >= pad_block0) {
         pad_image_elem(pad, (int64_t)(blockIdx.x - pad_block0) * 256 + threadIdx.x);
@@ -193,7 +196,18 @@ __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const P *__res
         taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
     }
     if (folded != nullptr && q < (int64_t)C * 7) {
-        const Coef<P> cf = fold16(w + q * 16);
+        P pr[16];
+        if (from_logits) {                                           // w holds logits: softmax here, written out for the backward pass
+            softmax16(w + q * 16, pr);
+            if (probs_out != nullptr) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) probs_out[q * 16 + i] = pr[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) pr[i] = w[q * 16 + i];
+        }
+        const Coef<P> cf = fold16(pr);
         folded[q * 4 + 0] = cf.ab;
         folded[q * 4 + 1] = cf.a;
         folded[q * 4 + 2] = cf.b;

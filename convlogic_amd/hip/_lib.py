@@ -73,6 +73,7 @@ SIGNATURES = {
     "clg_convblock_backward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_logits": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_fm_supported": (_i, [_i, _GP]),
+    "clg_convblock_forward_ex": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _i, _p, _p]),
     "clg_convblock_eval_packed_fm_supported": (_i, [_GP]),
     "clg_convblock_eval_packed_fm": (_i, [_GP, _p, _p, _p, _p, _p]),
     "clg_convblock_forward_fm": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p]),

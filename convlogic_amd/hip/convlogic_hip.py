@@ -277,6 +277,26 @@ def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, p
     return y, argmax
 
 
+def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
+    """full_convlogic_forward() from the LOGITS [C, 7, 16]: the softmax is taken inside the launch that sets the gate
+    parameters up.  -> (y, argmax, probs); with feature_major (where feature_major_supported) y is laid out
+    [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm()."""
+    for t, n in ((x, "x"), (logits, "weights"), (selection, "selection")):
+        check_input(t, n)
+    g = _geom(x, logits.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    ho, wo = _out_size(g)
+    shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
+    y = torch.empty((g.c_out, shape[2], shape[3], g.n) if feature_major else shape, dtype=x.dtype, device=x.device)
+    argmax = torch.empty(shape, dtype=torch.uint8, device=x.device)
+    probs = torch.empty_like(logits)
+    lib = _lib.load()
+    scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
+    check(lib.clg_convblock_forward_ex(dtype_code(x), ctypes.byref(g), x.data_ptr(), logits.data_ptr(), selection.data_ptr(),
+                                       y.data_ptr(), argmax.data_ptr(), probs.data_ptr(), 1 | (2 if feature_major else 0),
+                                       scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))
+    return y, argmax, probs
+
+
 def full_convlogic_backward_fm(grad_y_fm, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True,
                                wrt_logits=True):
     """-> (grad_x or None, grad_w [C,7,16]) from grad_y laid out [C, Ho/2, Wo/2, N]; grad_w is the gradient w.r.t. the

@@ -327,6 +327,14 @@ int clg_convblock_backward_logits(int dtype, const clg_conv_geom *g, const void 
  * _backward_weight (src/convlogic/cuda/convlogic.cpp:29-37) plus the copies around
  * x.transpose(0, 1).contiguous() in LogicLayer.forward_cuda (src/difflogic/difflogic.py:130-141). */
 int clg_convblock_fm_supported(int dtype, const clg_conv_geom *g);
+/* clg_convblock_forward_ws with options.  CLG_FWD_W_LOGITS: w holds the LOGITS [c_out, 7, 16]; their softmax is taken
+ * while the gate parameters are set up (no separate softmax launch) and written to probs_out [c_out, 7, 16] for the
+ * backward entry points -- replaces torch.softmax(self.weights) + full_convlogic_forward of ConvLogicLayer.forward_cuda
+ * (src/convlogic/convlogic_layer.py:318-329).  CLG_FWD_Y_FEATURE_MAJOR: y laid out as for clg_convblock_forward_fm. */
+#define CLG_FWD_W_LOGITS 1
+#define CLG_FWD_Y_FEATURE_MAJOR 2
+int clg_convblock_forward_ex(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection, void *y,
+                             uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream);
 /* The same for packed words: y laid out [c_out, ho/2, wo/2, groups], which IS the feature-major [features, words] layout
  * of clg_fc_eval_packed (feature = (c, y, x) in nn.Flatten order), so PackBitsTensor.flatten needs no transpose. */
 int clg_convblock_eval_packed_fm_supported(const clg_conv_geom *g);

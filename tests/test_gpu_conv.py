@@ -274,9 +274,16 @@ def test_block_fused_softmax_backward_matches_softmax_plus_function(shape):
             gy = torch.randn_like(y) if not outs else outs[0][4]
             y.backward(gy)
             outs.append((y.detach(), xl.grad, logits.grad, logits, gy))
-        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
-        scale = outs[1][2].abs().max().item()
-        assert (outs[0][2] - outs[1][2]).abs().max().item() <= tol * scale
+        # the forward launch takes its own softmax of the logits (one reciprocal per row), so the two routes agree to
+        # rounding, not bit for bit
+        assert (outs[0][0] - outs[1][0]).abs().max().item() <= (2e-6 if dtype == torch.float32 else 1e-14)
+        # (a pooled cell whose two best positions tie to rounding may route its gradient to the other one)
+        for k in (1, 2):
+            diff, ref = (outs[0][k] - outs[1][k]).abs(), outs[1][k]
+            off = (diff > tol * ref.abs().max().item()).float().mean().item()
+            assert k == 2 or off <= 2e-3, (k, off)                   # input gradient: a flip moves up to 8 elements
+            assert (diff.norm() / ref.norm()).item() <= 1e-2, (k, (diff.norm() / ref.norm()).item())
+            assert diff.max().item() <= 5e-2 * ref.abs().max().item(), k
     # first layer of a network: no input gradient requested
     layer.train()
     y = layer(x.detach())
@@ -397,3 +404,31 @@ def test_block_4x4_feature_major_output(n, cin, cout, dtype):
         grads[fm] = (out.detach(), xin.grad, layer.weights.grad.clone(), head.weights.grad.clone())
     for a, b in zip(grads[False], grads[True]):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape,env", [((6, 3, 12, 12, 10), {}), ((70, 40, 8, 8, 24), {}), ((5, 24, 8, 8, 16), {"CLG_FWD_SUBSET": "1", "CLG_FWD_DIRECT": "0"}),
+                                       ((6, 12, 16, 16, 20), {"CLG_FWD_DIRECT": "1"}), ((100, 24, 4, 4, 48), {}),
+                                       ((3, 2, 11, 15, 4), {})])
+def test_forward_from_logits_takes_the_softmax_inside(shape, env, dtype, monkeypatch):
+    # the training path hands the logits to the forward launch: the probabilities it writes out equal torch's softmax to
+    # rounding, and the block output is bit for bit what the probability entry point gives on those probabilities --
+    # on the staged kernels (all channels, channel subsets, one position per lane), the padded-copy kernel, the 4x4
+    # kernels (both output layouts) and the any-shape kernel (stride 2 here)
+    from convlogic_amd.hip import convlogic_hip
+    n, cin, h, w, cout = shape
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    stride = 2 if h == 11 else 1
+    torch.manual_seed(n + cin + h)
+    layer = C.ConvLogicLayer(cin, cout, stride=stride, padding=1, complete=True, implementation="cuda").to(DEV).to(dtype)
+    x = torch.rand(n, cin, h, w, device=DEV, dtype=dtype)
+    logits = layer.weights.detach()
+    geo = (stride, stride, 1, 1, 3, 3)
+    y, am, probs = convlogic_hip.full_convlogic_forward_logits(x, logits, layer.selection, *geo)
+    assert (probs - torch.softmax(logits, -1)).abs().max().item() <= (1e-6 if dtype == torch.float32 else 1e-14)
+    y_ref, am_ref = convlogic_hip.full_convlogic_forward(x, probs, layer.selection, *geo)
+    assert torch.equal(y, y_ref) and torch.equal(am, am_ref)
+    if convlogic_hip.feature_major_supported(x, cout, *geo):
+        y_fm, am_fm, probs_fm = convlogic_hip.full_convlogic_forward_logits(x, logits, layer.selection, *geo, feature_major=True)
+        assert torch.equal(y_fm.permute(3, 0, 1, 2), y) and torch.equal(am_fm, am) and torch.equal(probs_fm, probs)
