@@ -691,11 +691,12 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
             return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
         return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
     }
-    // The staged kernels take the softmax per workgroup while they set their gate parameters up (measured against a
-    // small launch of its own: C3 graph step 63.7 vs 66.7 us, C5 451 vs 459 us, C4 the same); the any-shape kernel
-    // gets its probabilities from that small launch.
+    // The staged kernels take the softmax per workgroup while they set their gate parameters up, as long as that is at
+    // most two rows of 16 logits per thread (C3 graph step 66.7 -> 63.7 us against a small launch of its own; with the
+    // 512 kernels of [256,128,8,8] -> 512 in one tile it is four rows and costs 7 us where the launch costs 3); beyond
+    // that, and for the any-shape kernel, the probabilities come from that small launch.
     const bool staged = path == 0 || path == 1;
-    bool in_kernel = staged && logits;
+    bool in_kernel = staged && logits && clg_ceil_div((int64_t)tp.CT * 7, (int64_t)tp.NW * kWave) <= 2;
     if (const char *e = getenv("CLG_FWD_SOFTMAX_IN_KERNEL")) in_kernel = staged && logits && atoi(e) != 0;
     if (logits && !in_kernel) {
         const int64_t rows = (int64_t)g.c * 7;
