@@ -149,6 +149,19 @@ __device__ __forceinline__ T row16_sum(T v)
     v += dpp_zero<0x140, 0xF>(v);
     return v;
 }
+// Maximum over each row of 16 lanes, valid in all of its lanes.
+template <typename T>
+__device__ __forceinline__ T row16_max(T v)
+{
+    T o = dpp_zero<0xB1, 0xF>(v);
+    v = o > v ? o : v;
+    o = dpp_zero<0x4E, 0xF>(v);
+    v = o > v ? o : v;
+    o = dpp_zero<0x141, 0xF>(v);
+    v = o > v ? o : v;
+    o = dpp_zero<0x140, 0xF>(v);
+    return o > v ? o : v;
+}
 // Gradient w.r.t. the logit of a 16-way softmax from the gradient g w.r.t. its probability p, the 16 gates
 // of one node sitting in the 16 lanes of a row: p_i (g_i - sum_j p_j g_j).
 template <typename T>

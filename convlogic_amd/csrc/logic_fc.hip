@@ -391,6 +391,63 @@ __global__ __launch_bounds__(kBlock) void fc_forward_folded_kernel(const T *__re
     }
 }
 
+// Forward from the LOGITS: the 16 lanes of every lane row hold the 16 logits of the row group's neuron, take the
+// softmax with DPP reductions (maximum, sum, one reciprocal) and fold it to the 4 coefficients as four 16-lane dot
+// products with the integer patterns of fold16; the first row writes probabilities and coefficients out for the
+// backward pass.  One launch instead of fold + forward; the reductions ride on a kernel that waits for memory.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void fc_forward_logits_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                                 const int64_t *__restrict__ b,
+                                                                 const T *__restrict__ logits, T *__restrict__ probs,
+                                                                 T *__restrict__ folded, T *__restrict__ y, int out_dim,
+                                                                 int64_t batch, int lpr_log2)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
+    const int q = lane & 15;
+    // fold16 as dot products with integer patterns; c_1 = sum of gates 8..15
+    constexpr int kAb[16] = {0, 1, -1, 0, -1, 0, -2, -1, 1, 2, 0, 1, 0, 1, -1, 0};
+    constexpr int kA[16] = {0, 0, 1, 1, 0, 0, 1, 1, -1, -1, 0, 0, -1, -1, 0, 0};
+    constexpr int kB[16] = {0, 0, 0, 0, 1, 1, 1, 1, -1, -1, -1, -1, 0, 0, 0, 0};
+    int ab = 0, aa = 0, bb = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {                                    // selects, not a table in memory
+        ab = q == i ? kAb[i] : ab;
+        aa = q == i ? kA[i] : aa;
+        bb = q == i ? kB[i] : bb;
+    }
+    const T w_ab = (T)ab, w_a = (T)aa, w_b = (T)bb, w_1 = q >= 8 ? T(1) : T(0);
+    const int64_t pass = (int64_t)VEC << lpr_log2;
+    for (int64_t j0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * rows; j0 < out_dim;
+         j0 += (int64_t)gridDim.x * kWavesPerBlock * rows) {
+        const bool valid = j0 + sub < out_dim;
+        const int64_t j = valid ? j0 + sub : out_dim - 1;            // every lane takes part in the reductions
+        const T lg = logits[j * 16 + q];
+        const T e = exp(lg - row16_max(lg));
+        const T p = e * (T(1) / row16_sum(e));
+        Coef<T> c;
+        c.ab = row16_sum(p * w_ab);
+        c.a = row16_sum(p * w_a);
+        c.b = row16_sum(p * w_b);
+        c.one = row16_sum(p * w_1);
+        if (valid && l < 16) {
+            probs[j * 16 + q] = p;
+            if (q < 4) folded[j * 4 + q] = q == 0 ? c.ab : (q == 1 ? c.a : (q == 2 ? c.b : c.one));
+        }
+        if (!valid) continue;
+        const T *xa = x + a[j] * batch;
+        const T *xb = x + b[j] * batch;
+        T *yj = y + j * batch;
+        for (int64_t s = (int64_t)l * VEC; s < batch; s += pass) {
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = gate(c, va.v[k], vb.v[k]);
+            store_vec<T, VEC>(yj + s, r);
+        }
+    }
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
@@ -793,6 +850,33 @@ extern "C" int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a,
     }
 #undef CLG_LAUNCH_FF
     CLG_CHECK_LAUNCH("clg_fc_forward_folded");
+    return CLG_OK;
+}
+
+extern "C" int clg_fc_forward_logits(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *logits,
+                                     void *probs, void *folded, void *y, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                     void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward_logits")) return e;
+    CLG_REQUIRE(x && a && b && logits && probs && folded && y, "clg_fc_forward_logits: null pointer argument");
+    const dim3 block(kBlock);
+    hipStream_t st = clg_stream(stream);
+#define CLG_LAUNCH_FL(T, VEC)                                                                                           \
+    do {                                                                                                               \
+        const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
+        hipLaunchKernelGGL((fc_forward_logits_kernel<T, VEC>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave >> lg)))), \
+                           block, 0, st, (const T *)x, a, b, (const T *)logits, (T *)probs, (T *)folded, (T *)y,           \
+                           (int)out_dim, batch, lg);                                                                   \
+    } while (0)
+    if (dtype == CLG_F32) {
+        if (batch % 4 == 0) CLG_LAUNCH_FL(float, 4);
+        else CLG_LAUNCH_FL(float, 1);
+    } else {
+        if (batch % 2 == 0) CLG_LAUNCH_FL(double, 2);
+        else CLG_LAUNCH_FL(double, 1);
+    }
+#undef CLG_LAUNCH_FL
+    CLG_CHECK_LAUNCH("clg_fc_forward_logits");
     return CLG_OK;
 }
 

@@ -262,10 +262,10 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False):
-        w, folded = difflogic_hip.fold(logits, from_logits=True)
+        y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach())
         ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.sole_consumers = sole_consumers
-        return difflogic_hip.forward_folded(x, a, b, folded)
+        return y
 
     @staticmethod
     def backward(ctx, grad_y):

@@ -69,6 +69,23 @@ def forward_folded(x, a, b, folded):
     return y
 
 
+def forward_logits(x, a, b, logits):
+    """fold(from_logits=True) + forward_folded() in one launch -> (y [out, B], probs [out, 16], folded [out, 4])."""
+    for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "w")):
+        check_input(t, n)
+    if logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.dtype not in _lib._DTYPES:
+        raise RuntimeError(f"forward_logits expects float32/float64 logits [out, 16] of x's dtype, got {tuple(logits.shape)} {logits.dtype}")
+    in_dim, batch = x.shape
+    out_dim = logits.shape[0]
+    y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
+    probs = torch.empty_like(logits)
+    folded = torch.empty((out_dim, 4), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_forward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), logits.data_ptr(),
+                                            probs.data_ptr(), folded.data_ptr(), y.data_ptr(), in_dim, out_dim, batch,
+                                            stream_ptr(x)))
+    return y, probs, folded
+
+
 def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
     """backward_x() with the folded coefficients [out, 4] of fold() in place of w."""
     for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y"),

@@ -119,6 +119,15 @@ int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64
                          const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, void *grad_x, void *grad_w,
                          int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
 
+/* clg_fc_fold (from logits) + clg_fc_forward_folded in one launch: y from the LOGITS [out_dim, 16]; their softmax goes to
+ * probs [out_dim, 16] and its 4 folded coefficients per neuron to folded [out_dim, 4] for the backward entry points
+ * (the 16 lanes of a lane row hold a neuron's logits; sums are DPP trees, so probs agree with clg_fc_fold to rounding).
+ * Replaces torch.softmax(self.weights) + difflogic_cuda.forward of LogicLayer.forward_cuda
+ * (src/difflogic/difflogic.py:130-141) in the module's training path. */
+int clg_fc_forward_logits(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *logits,
+                          void *probs /*[out_dim,16]*/, void *folded /*[out_dim,4]*/, void *y, int64_t in_dim, int64_t out_dim,
+                          int64_t batch, void *stream);
+
 /* Both gradients of a layer with ANY wiring in one pass, for batches that one pass of a wavefront row covers
  * (clg_fc_backward_fused_fits() != 0: batch <= 256 for float32 batches divisible by 4, 128 for float64 batches divisible
  * by 2, 64 otherwise): the walk of clg_fc_backward_x_folded also forms each neuron's weight-gradient sums on the visit

@@ -249,6 +249,28 @@ def test_fused_backward_equals_the_two_kernels(in_dim, out_dim, batch, dtype):
         assert torch.equal(gx, gx_ref) and torch.equal(gw, gw_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(24, 50, 8), (40, 97, 100), (64, 131, 128), (30, 75, 256), (30, 75, 300),
+                                                  (7, 9, 33), (3, 5, 1), (8000, 8000, 256)])
+def test_forward_from_logits_folds_inside(in_dim, out_dim, batch, dtype):
+    # one launch for softmax + fold + forward: probabilities against torch's softmax, coefficients against the oracle's
+    # fold of those probabilities, and y bit for bit what the folded forward gives on the coefficients written out
+    torch.manual_seed(in_dim + 2 * out_dim + batch)
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV).to(dtype)
+    tabs = (layer.indices_0, layer.indices_1)
+    x = torch.rand(in_dim, batch, device=DEV, dtype=dtype)
+    logits = (torch.randn(out_dim, 16, device=DEV, dtype=dtype) * 3).contiguous()
+    y, probs, folded = difflogic_hip.forward_logits(x, *tabs, logits)
+    eps = 1e-6 if dtype == torch.float32 else 1e-14
+    assert (probs - torch.softmax(logits, -1)).abs().max().item() <= eps
+    assert (folded.cpu().double() - O.fold_coefficients(probs.cpu().double())).abs().max().item() <= 16 * eps
+    assert torch.equal(y, difflogic_hip.forward_folded(x, *tabs, folded))
+    want = O.logic_fc_forward(x.T.cpu(), layer.indices_0.cpu(), layer.indices_1.cpu(), torch.softmax(logits.cpu(), -1))
+    assert (y.T.cpu() - want).abs().max().item() <= (1e-5 if dtype == torch.float32 else 1e-12)
+    with pytest.raises(RuntimeError):
+        difflogic_hip.forward_logits(x, *tabs, logits[:, :8].contiguous())
+
+
 @pytest.mark.parametrize("features,batch,k", [(40, 7, 4), (640, 256, 10), (65536, 100, 8), (30, 1, 3), (10240, 256, 10)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_group_sum_on_feature_major_view(features, batch, k, dtype):
