@@ -432,3 +432,29 @@ def test_forward_from_logits_takes_the_softmax_inside(shape, env, dtype, monkeyp
     if convlogic_hip.feature_major_supported(x, cout, *geo):
         y_fm, am_fm, probs_fm = convlogic_hip.full_convlogic_forward_logits(x, logits, layer.selection, *geo, feature_major=True)
         assert torch.equal(y_fm.permute(3, 0, 1, 2), y) and torch.equal(am_fm, am) and torch.equal(probs_fm, probs)
+
+
+def test_forward_ex_rejects_bad_options():
+    # the options entry point: unknown flags, logits without a place for the probabilities, the feature-major layout on a
+    # shape its kernels do not take
+    import ctypes
+    from convlogic_amd.hip import _lib, convlogic_hip
+    lib = _lib.load()
+    layer = C.ConvLogicLayer(3, 4, padding=1, complete=True, implementation="cuda").to(DEV)
+    x = torch.rand(2, 3, 8, 8, device=DEV)
+    g = convlogic_hip._geom(x, 4, 1, 1, 1, 1, 3, 3)
+    y = torch.empty(2, 4, 4, 4, device=DEV)
+    am = torch.empty(2, 4, 4, 4, device=DEV, dtype=torch.uint8)
+    probs = torch.empty_like(layer.weights)
+    scratch = torch.empty(1 << 16, device=DEV, dtype=torch.uint8)
+
+    def call(flags, probs_ptr):
+        return lib.clg_convblock_forward_ex(0, ctypes.byref(g), x.data_ptr(), layer.weights.data_ptr(), layer.selection.data_ptr(),
+                                            y.data_ptr(), am.data_ptr(), probs_ptr, flags, scratch.data_ptr(), None)
+
+    assert call(8, probs.data_ptr()) != 0 and b"unknown flags" in lib.clg_last_error()
+    assert call(1, None) != 0 and b"probs_out" in lib.clg_last_error()
+    assert call(2, probs.data_ptr()) != 0 and b"clg_convblock_fm_supported" in lib.clg_last_error()
+    assert call(1, probs.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert (probs - torch.softmax(layer.weights.detach(), -1)).abs().max().item() <= 1e-6

@@ -157,6 +157,11 @@ def test_fc_rejects_bad_inputs():
                               torch.rand(8, 16, device=DEV).bfloat16())
     with pytest.raises(RuntimeError):                                   # half is a format of the reference-shaped kernels only
         difflogic_hip.fold(torch.rand(8, 16, device=DEV).half(), from_logits=True)
+    with pytest.raises(RuntimeError):                                   # ... and so are the logits-in forward and the one-pass backward
+        difflogic_hip.forward_logits(torch.rand(8, 4, device=DEV).half(), layer.indices_0, layer.indices_1,
+                                     torch.rand(8, 16, device=DEV).half())
+    with pytest.raises(RuntimeError):
+        difflogic_hip.forward_logits(torch.rand(8, 4, device=DEV), layer.indices_0, layer.indices_1, torch.rand(8, 16, device=DEV).double())
     with pytest.raises(AssertionError):
         layer(torch.rand(2, 3, 8, device=DEV))
 
