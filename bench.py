@@ -239,6 +239,11 @@ def cpu_c2(layers, x0):
 # ------------------------------------------------------------------------------------------------
 # float workloads: forward + backward
 # ------------------------------------------------------------------------------------------------
+# HBM bytes of one training step of the block (all its kernels), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
+# a plain copy of known size in the same runs (profiles/convblock_c4_c3_hbm_traffic_pmc.txt): recorded, not taken live.
+CONV_TRAFFIC_BYTES = {"c4": 369.7e6, "c3": 36.8e6}
+
+
 def _roof(name, alg_bytes, ms, extra=None):
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     r = {"bound": "hbm", "kernel": name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -395,6 +400,7 @@ def bench_conv(key, steps, warmup, cpu=True):
                               # lane-operation floor of the forward: 3 FMAs per gate evaluation, non-packed fp32
                               "valu_floor_forward_ms": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3,
                               "valu_frac_forward": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3 / ms["fwd"],
+                              "traffic": CONV_TRAFFIC_BYTES.get(key),
                               "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
                                       "the lane-operation floor (39.3 T fp32 lane-ops/s) beside it"})}
     def cpu_leg():
