@@ -27,6 +27,35 @@ def test_library_exports_every_declared_symbol():
     assert lib.clg_last_error() == b""
 
 
+def test_ctypes_signatures_match_the_header_prototypes():
+    # every prototype of the header, argument by argument, against the ctypes declaration that calls it: a pointer
+    # passed where the library reads an int64 (or an argument too few) would not fail at load time
+    import ctypes
+    header = open(os.path.join(ROOT, "include", "convlogic_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", " ", header, flags=re.S)              # comments, also the ones inside argument lists
+    header = re.sub(r"//[^\n]*", " ", header)
+    protos = re.findall(r"\b(const char \*|int64_t|int)\s*(clg_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", header)
+    assert {name for _, name, _ in protos} == set(_lib.SIGNATURES)
+
+    def ctype_of(decl):
+        decl = " ".join(decl.split())
+        if decl == "void":
+            return None
+        if "*" in decl:
+            return _lib._GP if "clg_conv_geom" in decl else ctypes.c_void_p
+        base = decl.rsplit(" ", 1)[0] if " " in decl else decl        # drop the parameter name
+        return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "double": ctypes.c_double}[base.replace("const ", "")]
+
+    results = {"const char *": ctypes.c_char_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int}
+    for ret, name, args in protos:
+        want = [t for t in (ctype_of(a) for a in args.split(",")) if t is not None]
+        res, got = _lib.SIGNATURES[name]
+        assert res is results[ret], name
+        assert len(got) == len(want), (name, len(got), len(want))
+        for k, (g, w) in enumerate(zip(got, want)):
+            assert g is w, (name, k, g, w)
+
+
 def test_c_abi_rejects_bad_arguments_without_gpu():
     lib = _lib.load()
     assert lib.clg_fc_forward(7, 0, 0, 0, 0, 0, 4, 4, 4, None) == -1
