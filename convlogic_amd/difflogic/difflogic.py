@@ -92,11 +92,14 @@ class LogicLayer(torch.nn.Module):
             assert x.is_cuda, f"x must be a CUDA tensor, got device: {x.device}"
         assert x.ndim == 2, x.ndim
         assert x.shape[1] == self.in_dim, (tuple(x.shape[::-1]), self.in_dim)
+        if self.training and self.weights.dtype == x.dtype and self.weights.is_contiguous():
+            # a sample-major batch is transposed inside the Function (and its gradient on the way back): one autograd
+            # node per layer instead of two
+            inside = _transposes_with_kernel(x)
+            return _LogicLayerLogitsFunction.apply(x if inside else _feature_major(x), self.indices_0, self.indices_1,
+                                                   self.weights, self.given_x_indices_of_y_start,
+                                                   self.given_x_indices_of_y, self._sole_consumers(), inside).transpose(0, 1)
         xt = _feature_major(x)
-        if self.training and self.weights.dtype == xt.dtype and self.weights.is_contiguous():
-            return _LogicLayerLogitsFunction.apply(xt, self.indices_0, self.indices_1, self.weights,
-                                                   self.given_x_indices_of_y_start, self.given_x_indices_of_y,
-                                                   self._sole_consumers()).transpose(0, 1)
         w = self._gate_weights(xt.dtype)
         args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
         if self.training:
@@ -179,13 +182,20 @@ class _FeatureMajor(torch.autograd.Function):
         return grad.transpose(0, 1)
 
 
+def _transposes_with_kernel(x):
+    """True for a dense sample-major device tensor whose feature-major copy the tiled HIP transpose makes (a
+    transposed view of a feature-major tensor needs no copy at all)."""
+    return (x.is_cuda and x.dim() == 2 and x.is_contiguous() and not x.transpose(0, 1).is_contiguous()
+            and x.element_size() in (1, 2, 4, 8))
+
+
 def _feature_major(x):
     """[batch, features] -> contiguous [features, batch].  A transposed view of a feature-major
     tensor (what the previous LogicLayer returned) is used as is, without a copy."""
     xt = x.transpose(0, 1)
     if xt.is_contiguous():
         return xt
-    if x.is_cuda and x.is_contiguous() and x.element_size() in (1, 2, 4, 8):
+    if _transposes_with_kernel(x):
         return _FeatureMajor.apply(x)
     return xt.contiguous()
 
@@ -261,10 +271,14 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
     to rounding)."""
 
     @staticmethod
-    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False):
+    def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False,
+                sample_major_input=False):
+        if sample_major_input:                                       # x is [B, in]: its gradient goes back in that layout
+            x = difflogic_hip.transpose(x)
         y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach())
         ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.sole_consumers = sole_consumers
+        ctx.sample_major_input = sample_major_input
         return y
 
     @staticmethod
@@ -282,7 +296,9 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
                 grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)
             if ctx.needs_input_grad[3]:
                 grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
-        return grad_x, None, None, grad_l, None, None, None
+        if ctx.sample_major_input and grad_x is not None:
+            grad_x = difflogic_hip.transpose(grad_x)
+        return grad_x, None, None, grad_l, None, None, None, None
 
 
 def _contiguous_2d(t):
