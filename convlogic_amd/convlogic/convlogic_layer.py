@@ -146,6 +146,32 @@ class ConvLogicLayer(nn.Module):
         self.register_buffer("selection", selection)
         assert selection.shape == (out_channels, 8)
         assert self.weights.shape[-1] == 16, f"Expected 16 logic functions, got {self.weights.shape[-1]}"
+        self._check_selection()
+
+    def _check_selection(self):
+        """The kernels size their tiles from the geometry and read taps without bounds checks on the channel, row and
+        column a tap names: a selection outside (in_channels, kernel) must raise here instead of faulting the GPU.
+        Checked at construction, on the first launch and whenever the buffer was modified in place (version counter)
+        or replaced; writes through `.data` bypass the counter -- call invalidate() after those."""
+        sel = self.selection
+        key = (sel._version, sel.data_ptr())
+        if getattr(self, "_selection_checked", None) == key:
+            return
+        if sel.dtype != torch.int32 or tuple(sel.shape) != (self.out_channels, 8):
+            raise ValueError(f"selection must be int32 [{self.out_channels}, 8], got {sel.dtype} {tuple(sel.shape)}")
+        ch, row, col = self.unpack_selection(sel)
+        if sel.numel() and (int(ch.max()) >= self.in_channels or int(row.max()) >= self.kernel[0] or int(col.max()) >= self.kernel[1]):
+            raise ValueError(f"selection names a tap outside {self.in_channels} input channels and a "
+                             f"{self.kernel[0]}x{self.kernel[1]} receptive field")
+        self._selection_checked = key
+
+    def invalidate(self):
+        """Forces the next call to check the selection buffer again (after a write through `.data`)."""
+        self._selection_checked = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.invalidate()
 
     def forward(self, x):
         if isinstance(x, PackBitsTensor):
@@ -192,13 +218,17 @@ class ConvLogicLayer(nn.Module):
         return PoolLogicLayer()(level)
 
     def forward_cuda(self, x):
+        self._check_selection()
+        if x.dim() != 4 or x.shape[1] != self.in_channels:          # the taps index channels of x without bounds checks
+            raise RuntimeError(f"Expected x of shape [N, {self.in_channels}, H, W], got {tuple(x.shape)}")
         x = x.contiguous()
         sel = self.selection.contiguous()
         geo = (*self.stride, *self.padding, *self.kernel)
         if (self.complete and self.training and not self.return_intermediate and not self.return_indices
                 and self.weights.dtype == x.dtype and self.weights.is_contiguous()):
             return _FullConvLogicLogitsFunction.apply(x, self.weights, sel, *geo, getattr(self, "feature_major_output", False))
-        w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
+        # the kernels read the probabilities in x's element type (the bindings reject any other)
+        w_prob = gate_probabilities(self.weights, self.training, x.dtype).to(x.dtype).contiguous()
         if self.complete:
             return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)
         return ConvLogicFunction.apply(x, w_prob, sel, *geo)
@@ -213,19 +243,17 @@ class ConvLogicLayer(nn.Module):
         if self.implementation != "cuda":
             raise RuntimeError("packed evaluation needs implementation='cuda'")
         assert x.image and x.t.dim() == 4 and x.t.shape[1] == self.in_channels, (x.image, tuple(x.t.shape), self.in_channels)
+        self._check_selection()
         x.t = convlogic_hip.full_convlogic_eval_packed(x.t.contiguous(), self._eval_gates(), self.selection.contiguous(),
                                                        *self.stride, *self.padding, *self.kernel,
                                                        feature_major=getattr(self, "feature_major_output", False))
         return x
 
     def _eval_gates(self):
-        """uint8 [C, 7] arg-max gate ids, recomputed only after the logits changed."""
-        key = (self.weights._version, self.weights.data_ptr())
-        cached = getattr(self, "_gate_cache", None)
-        if cached is None or cached[0] != key:
-            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8).contiguous())
-            self._gate_cache = cached
-        return cached[1]
+        """uint8 [C, 7] arg-max gate ids, taken from the logits on every call (one small launch; nothing cached that an
+        in-place update of `weights.data` could leave stale)."""
+        from ..hip import difflogic_hip
+        return difflogic_hip.gate_argmax(self.weights.detach().contiguous())
 
     def extra_repr(self):
         return f"in_channels={self.in_channels}, out_channels={self.out_channels}, groups={self.groups}"

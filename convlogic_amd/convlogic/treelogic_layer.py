@@ -66,7 +66,8 @@ class TreeLogicLayer(nn.Module):
         raise ValueError(f"Unknown implementation {self.implementation!r}")
 
     def forward_cuda(self, x):
-        w_prob = gate_probabilities(self.weights, self.training, x.dtype).contiguous()
+        # the kernels read the probabilities in x's element type (the bindings reject any other)
+        w_prob = gate_probabilities(self.weights, self.training, x.dtype).to(x.dtype).contiguous()
         return TreeLogicFunction.apply(x, w_prob)
 
     def forward_python(self, x):

@@ -27,6 +27,24 @@ void clg_set_error(const char *fmt, ...);
         }                                                                           \
     } while (0)
 
+// ---- host side: tuning knobs ---------------------------------------------------------------
+// Environment variables CLG_<name>, for measurement and for forcing a code path in tests (unset = the measured
+// optimum).  They are read ONCE per process, on the first lookup, so a launch costs no getenv(); clg_reload_knobs()
+// (C ABI) reads them again after the environment was changed.
+#define CLG_KNOBS(X)                                                                                                   \
+    X(BWDW_CELLS) X(BWDW_PADDED) X(BWDX_BANDS) X(BWDX_CSR) X(BWDX_DIRECT) X(BWDX_HSW) X(BWDX_SPLIT) X(BWD_4X4)         \
+    X(EVAL_CHUNK_BYTES) X(EVAL_NPW) X(EVAL_WALK_R) X(EVAL_WALK_SEG) X(FWD_4X4) X(FWD_CT) X(FWD_DIRECT) X(FWD_NW)       \
+    X(FWD_ONE_ROW) X(FWD_S) X(FWD_SOFTMAX_IN_KERNEL) X(FWD_SUBSET) X(GSUM_SLICES) X(PACKED_4X4_HALVES) X(PACK_TILE)    \
+    X(FC_SAMPLE_MAJOR) X(BWDW_LDS)
+enum ClgKnob {
+#define CLG_KNOB_ENUM(name) K_##name,
+    CLG_KNOBS(CLG_KNOB_ENUM)
+#undef CLG_KNOB_ENUM
+    K_COUNT
+};
+// value of the variable as read at the last (re)load, or nullptr when it was not set
+const char *clg_knob(ClgKnob k);
+
 static inline int64_t clg_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline hipStream_t clg_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -64,7 +64,7 @@ struct BwdScratch {
 constexpr int kMaxHitSplit = 16;
 bool hits_compressed(const Geom &g)
 {
-    if (const char *e = getenv("CLG_BWDX_CSR")) return atoi(e) != 0;
+    if (const char *e = clg_knob(K_BWDX_CSR)) return atoi(e) != 0;
     return (int64_t)g.cin * g.c > (1ll << 20);
 }
 BwdScratch bwd_scratch_layout(const Geom &g, int elem, int hit_split)
@@ -724,7 +724,7 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
         // One band (the whole image) unless it does not fit: the time of this kernel is set by the
         // dependent chain of steps per visited kernel, which every band would repeat (measured: bands
         // never paid off, not even at 256 wavefronts in flight).  CLG_BWDX_BANDS overrides for tuning.
-        const char *e_b = getenv("CLG_BWDX_BANDS");
+        const char *e_b = clg_knob(K_BWDX_BANDS);
         int64_t want = e_b ? atoi(e_b) : 1;
         if (want > g.h / 4) want = g.h / 4;
         if (want < 1) want = 1;
@@ -749,7 +749,7 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     const int64_t avg_hits = g.cin == 1 ? g.c : (2 * (int64_t)g.c) / g.cin;
     const int64_t window = (int64_t)((p->xe + 3) & ~3) * elem;
     int64_t hsw = 16 / g.cin;
-    if (const char *e = getenv("CLG_BWDX_HSW")) hsw = atoi(e);
+    if (const char *e = clg_knob(K_BWDX_HSW)) hsw = atoi(e);
     if (hsw > avg_hits / 2) hsw = avg_hits / 2;
     while (hsw > 1 && (1 + hsw) * window > 96 * 1024) --hsw;
     if (hsw < 1 || p->bands > 1) hsw = 1;
@@ -764,7 +764,7 @@ bool plan_backward_x(const Geom &g, int elem, TilePlan *p)
     if (per_cu > 20 / p->NW) per_cu = 20 / p->NW;                    // about 80 VGPRs per lane: 5 wavefronts per SIMD
     if (per_cu < 1) per_cu = 1;
     const int64_t wgs = clg_ceil_div(g.n, p->S) * p->bands;
-    const char *e_hs = getenv("CLG_BWDX_SPLIT");
+    const char *e_hs = clg_knob(K_BWDX_SPLIT);
     int64_t hs = e_hs ? atoi(e_hs) : (256 * per_cu) / wgs;
     if (hs > kMaxHitSplit) hs = kMaxHitSplit;
     // every split workgroup stages the image and writes a partial image: worth it only with at least
@@ -826,7 +826,7 @@ BwdXMode choose_backward_x(const Geom &g, int elem, TilePlan *p, int *sample_ele
     // 74 vs 164 us at [256,64,16,16] -> 256; few channels with long lists stay tiled: 141 vs 248 us at C4).
     const int64_t owners = clg_ceil_div(g.n, pd.G) * g.cin, avg_hits = (2 * (int64_t)g.c) / g.cin;
     bool use_direct = direct && (!tiled || lanes(pd) >= 2 * lanes(pt) || (owners >= 4096 && avg_hits <= 16));
-    if (const char *e = getenv("CLG_BWDX_DIRECT")) use_direct = direct && (atoi(e) != 0 || !tiled);
+    if (const char *e = clg_knob(K_BWDX_DIRECT)) use_direct = direct && (atoi(e) != 0 || !tiled);
     if (use_direct) {
         *p = pd;
         *sample_elems = se;
@@ -853,7 +853,7 @@ struct WScratch {
 // [256,32,16,16] -> 128, where more would leave too few workgroups).
 int cells_per_thread(int64_t cells_per_kernel)
 {
-    if (const char *e = getenv("CLG_BWDW_CELLS")) return atoi(e) > 0 ? atoi(e) : 8;
+    if (const char *e = clg_knob(K_BWDW_CELLS)) return atoi(e) > 0 ? atoi(e) : 8;
     return cells_per_kernel >= 65536 ? 16 : 8;
 }
 bool fixed_cells(const Geom &g, int elem)
@@ -868,7 +868,7 @@ bool plan_backward_w(const Geom &g, int elem, TilePlan *p, WScratch *ws)
     const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
     // the padded copy costs two extra launches: it pays from about 8M pooled values (measured 102 vs 124 us
     // at 16.8M, 30 vs 27 us at 1.6M)
-    if ((int64_t)g.n * g.c * I < (8ll << 20) && !getenv("CLG_BWDW_PADDED")) return false;
+    if ((int64_t)g.n * g.c * I < (8ll << 20) && !clg_knob(K_BWDW_PADDED)) return false;
     const int64_t sample_elems = (int64_t)g.cin * p->chs + g.ph * p->rs + g.pw;
     // the copy may be made by the tiled input gradient of the same call, whose planes keep both halo rows
     const int64_t sample_elems_max = (int64_t)g.cin * (g.h + 2 * g.ph) * p->rs + g.ph * p->rs + g.pw;
@@ -1086,7 +1086,7 @@ PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void
 {
     TilePlan pw;
     WScratch ws;
-    const char *e_pad = getenv("CLG_BWDW_PADDED");
+    const char *e_pad = clg_knob(K_BWDW_PADDED);
     if (shared == nullptr || w_scratch == nullptr || p.bands != 1 || (e_pad && atoi(e_pad) == 0) || !plan_backward_w(g, (int)sizeof(T), &pw, &ws))
         return no_pad_job<T>();
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
@@ -1167,7 +1167,7 @@ static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const v
     }
     TilePlan p;
     WScratch ws;
-    const char *e_pad = getenv("CLG_BWDW_PADDED");
+    const char *e_pad = clg_knob(K_BWDW_PADDED);
     if ((!e_pad || atoi(e_pad) != 0) && plan_backward_w(g, elem_size(dtype), &p, &ws)) {
         if (dtype == CLG_F32)
             return launch_backward_w_padded<float>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
@@ -1187,7 +1187,7 @@ extern "C" int clg_convblock_backward_w(int dtype, const clg_conv_geom *gg, cons
 // 4x4 images with one sample per lane (conv_small.hip): scratch = prepare tables | tap gradients
 static bool backward_4x4_wanted(const Geom &g)
 {
-    const char *e = getenv("CLG_BWD_4X4");
+    const char *e = clg_knob(K_BWD_4X4);
     return clg_convblock_is_4x4(g) && g.c <= 65535 && (!e || atoi(e) != 0);
 }
 static size_t backward_4x4_tg_off(const Geom &g, int dtype) { return (bwd_scratch_layout(g, elem_size(dtype), 1).total + 255) & ~(size_t)255; }

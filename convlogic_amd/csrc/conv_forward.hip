@@ -375,7 +375,7 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     // Staging all channels wins whenever it fits with reasonable lane use (measured on 8x8 and 16x16 layers
     // with 32..128 input channels); the two-planes-per-kernel staging is for what is left.
     bool subset = sb > 0 && (sa == 0 || ua < 0.4);
-    if (const char *e = getenv("CLG_FWD_SUBSET")) subset = sb > 0 && (atoi(e) != 0 || sa == 0);
+    if (const char *e = clg_knob(K_FWD_SUBSET)) subset = sb > 0 && (atoi(e) != 0 || sa == 0);
     const double util = subset ? ub : ua;
     if ((subset ? sb : sa) == 0 || util < 0.4) return false;
     p->subset = subset ? 1 : 0;
@@ -394,9 +394,9 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
         p->CT = (int)ct;
     }
     // measurement overrides
-    if (const char *e = getenv("CLG_FWD_S")) p->S = atoi(e) < g.n ? atoi(e) : g.n;
-    if (const char *e = getenv("CLG_FWD_CT")) p->CT = atoi(e) < g.c ? atoi(e) : g.c;
-    if (const char *e = getenv("CLG_FWD_NW")) p->NW = atoi(e);
+    if (const char *e = clg_knob(K_FWD_S)) p->S = atoi(e) < g.n ? atoi(e) : g.n;
+    if (const char *e = clg_knob(K_FWD_CT)) p->CT = atoi(e) < g.c ? atoi(e) : g.c;
+    if (const char *e = clg_knob(K_FWD_NW)) p->NW = atoi(e);
     if (p->S < 1 || p->CT < 1 || p->NW < 1 || p->NW > 16) return false;
     // A workgroup whose samples fill at most half a wavefront with (row pair, column) slots gives every conv position
     // a lane of its own instead (the pooling partner one row down is wo lanes up, so 2 wo has to divide 64), two
@@ -404,7 +404,7 @@ bool plan_forward(const Geom &g, int elem, int params_per_kernel, TilePlan *p)
     p->w_logits = 0;
     p->one_row = 0;
     if ((int64_t)p->S * p->slots * 2 <= kWave && g.wo <= 32 && (g.wo & (g.wo - 1)) == 0) p->one_row = 1;
-    if (const char *e = getenv("CLG_FWD_ONE_ROW")) p->one_row = p->one_row && atoi(e) != 0;   // 0: never
+    if (const char *e = clg_knob(K_FWD_ONE_ROW)) p->one_row = p->one_row && atoi(e) != 0;   // 0: never
     if (p->one_row) {
         p->slots = g.ho * g.wo;
         p->d_slots = make_fastdiv((uint32_t)p->slots);
@@ -451,7 +451,7 @@ bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan 
     int64_t ct = g.c;
     while (ct > 16 && wgs_x * clg_ceil_div(g.c, ct) < 4096) ct = (ct + 1) / 2;
     ct = clg_ceil_div(g.c, clg_ceil_div(g.c, ct));
-    if (const char *e = getenv("CLG_FWD_CT")) ct = atoi(e) < g.c ? atoi(e) : g.c;
+    if (const char *e = clg_knob(K_FWD_CT)) ct = atoi(e) < g.c ? atoi(e) : g.c;
     if (ct < 1) ct = 1;
     p->CT = (int)ct;
     if (wgs_x >= (1ll << 31) || clg_ceil_div(g.c, ct) > 65535) return false;
@@ -468,7 +468,7 @@ bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan 
 int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scratch, TilePlan *tp, DirectPlan *dp)
 {
     bool lane_sample = have_scratch && params_per_kernel > 1 && clg_convblock_is_4x4(g);
-    if (const char *e = getenv("CLG_FWD_4X4")) lane_sample = lane_sample && atoi(e) != 0;
+    if (const char *e = clg_knob(K_FWD_4X4)) lane_sample = lane_sample && atoi(e) != 0;
     if (lane_sample) return 4;
     const bool tiled = plan_forward(g, elem, params_per_kernel, tp);
     const bool direct = have_scratch && plan_forward_direct(g, elem, params_per_kernel > 1, dp);
@@ -476,7 +476,7 @@ int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scr
     // elements load twice the bytes per tap and stay on the staged kernels (200 vs 329 us at [256,4096,4,4] -> 8192)
     // (4x4 images: the padded copy is 1.6x the image and both paths tie, 30 vs 35 us at [256,512,4,4] -> 1024).
     bool use_direct = direct && (!tiled || (tp->subset && elem == 4 && g.h * g.w >= 64));
-    if (const char *e = getenv("CLG_FWD_DIRECT")) use_direct = direct && (atoi(e) != 0 || !tiled);
+    if (const char *e = clg_knob(K_FWD_DIRECT)) use_direct = direct && (atoi(e) != 0 || !tiled);
     if (use_direct) return 2;
     if (tiled) return tp->subset ? 1 : 0;
     return 3;
@@ -580,7 +580,7 @@ extern "C" int clg_convblock_eval_packed(const clg_conv_geom *gg, const uint64_t
     CLG_REQUIRE(x != y, "clg_convblock_eval_packed: x and y must not overlap");
     TilePlan p;
     hipStream_t st = clg_stream(stream);
-    const char *e_4x4 = getenv("CLG_FWD_4X4");
+    const char *e_4x4 = clg_knob(K_FWD_4X4);
     if (clg_convblock_is_4x4(g) && (!e_4x4 || atoi(e_4x4) != 0))
         return clg_convblock_eval_packed_4x4(g, x, gates, selection, y, st, "clg_convblock_eval_packed");
     if (plan_forward(g, 8, BitOps::kParams, &p)) {
@@ -697,7 +697,7 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     // that, and for the any-shape kernel, the probabilities come from that small launch.
     const bool staged = path == 0 || path == 1;
     bool in_kernel = staged && logits && clg_ceil_div((int64_t)tp.CT * 7, (int64_t)tp.NW * kWave) <= 2;
-    if (const char *e = getenv("CLG_FWD_SOFTMAX_IN_KERNEL")) in_kernel = staged && logits && atoi(e) != 0;
+    if (const char *e = clg_knob(K_FWD_SOFTMAX_IN_KERNEL)) in_kernel = staged && logits && atoi(e) != 0;
     if (logits && !in_kernel) {
         const int64_t rows = (int64_t)g.c * 7;
         if (dtype == CLG_F32)
@@ -723,7 +723,7 @@ extern "C" int clg_convblock_fm_supported(int dtype, const clg_conv_geom *gg)
     Geom g;
     if (gg == nullptr || (dtype != CLG_F32 && dtype != CLG_F64)) return 0;
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_fm_supported")) return 0;
-    const char *e_fwd = getenv("CLG_FWD_4X4"), *e_bwd = getenv("CLG_BWD_4X4");
+    const char *e_fwd = clg_knob(K_FWD_4X4), *e_bwd = clg_knob(K_BWD_4X4);
     if ((e_fwd && atoi(e_fwd) == 0) || (e_bwd && atoi(e_bwd) == 0)) return 0;
     return clg_convblock_is_4x4(g) && g.c <= 65535 ? 1 : 0;
 }
@@ -753,7 +753,7 @@ extern "C" int clg_convblock_eval_packed_fm_supported(const clg_conv_geom *gg)
 {
     Geom g;
     if (gg == nullptr || clg_convblock_check(gg, &g, CLG_F64, "clg_convblock_eval_packed_fm_supported")) return 0;
-    const char *e_4x4 = getenv("CLG_FWD_4X4");
+    const char *e_4x4 = clg_knob(K_FWD_4X4);
     return clg_convblock_is_4x4(g) && (!e_4x4 || atoi(e_4x4) != 0) ? 1 : 0;
 }
 

@@ -566,7 +566,7 @@ int clg_convblock_forward_4x4(int dtype, const Geom &g, const void *x, const voi
 int clg_convblock_eval_packed_4x4(const Geom &g, const uint64_t *x, const uint8_t *gates, const int32_t *sel, uint64_t *y, hipStream_t st,
                                   const char *name)
 {
-    const char *e_half = getenv("CLG_PACKED_4X4_HALVES");            // 0: one 64-bit pass per kernel (measurement)
+    const char *e_half = clg_knob(K_PACKED_4X4_HALVES);            // 0: one 64-bit pass per kernel (measurement)
     if (e_half && atoi(e_half) == 0) return launch_4x4<BitOps>(g, x, gates, sel, y, nullptr, st, name);
     // full blocks of 64 groups go to the half-word kernel, what is left of the batch to the 64-bit one
     const int sblocks = g.n / kWave;

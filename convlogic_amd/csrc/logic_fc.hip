@@ -677,6 +677,26 @@ __global__ __launch_bounds__(256) void group_sum_backward_fm_kernel(const T *__r
     for (int64_t f = f0 + wave; f < f0 + 64 && f < features; f += 4) grad_x[f * batch + b] = grad_out[b * k + f / class_rows] * inv_tau;
 }
 
+// gate[r] = index of the first maximum of the 16 logits of row r (a NaN counts as the maximum, as in torch.argmax)
+template <typename S>
+__global__ __launch_bounds__(256) void gate_argmax_kernel(const S *__restrict__ logits, uint8_t *__restrict__ gate, int64_t rows)
+{
+    using T = typename ComputeOf<S>::type;
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    T best = load_one(logits + r * 16);
+    int at = 0;
+#pragma unroll
+    for (int i = 1; i < 16; ++i) {
+        const T v = load_one(logits + r * 16 + i);
+        if (v > best || (v != v && best == best)) {
+            best = v;
+            at = i;
+        }
+    }
+    gate[r] = (uint8_t)at;
+}
+
 int grid_for(int64_t items)
 {
     const int64_t blocks = clg_ceil_div(items, kWavesPerBlock);
@@ -707,6 +727,21 @@ int check_fc(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch, const ch
 }
 
 }  // namespace
+
+extern "C" int clg_gate_argmax(int dtype, const void *logits, uint8_t *gate, int64_t rows, void *stream)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64 || dtype == CLG_F16, "clg_gate_argmax: dtype must be CLG_F32, CLG_F64 or CLG_F16, got %d",
+                dtype);
+    CLG_REQUIRE(logits && gate, "clg_gate_argmax: null pointer argument");
+    CLG_REQUIRE(rows > 0 && rows < (1ll << 39), "clg_gate_argmax: rows must be in 1..2^39-1");
+    const dim3 grid((unsigned)clg_ceil_div(rows, 256)), block(256);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) hipLaunchKernelGGL(gate_argmax_kernel<float>, grid, block, 0, st, (const float *)logits, gate, rows);
+    else if (dtype == CLG_F64) hipLaunchKernelGGL(gate_argmax_kernel<double>, grid, block, 0, st, (const double *)logits, gate, rows);
+    else hipLaunchKernelGGL(gate_argmax_kernel<__half>, grid, block, 0, st, (const __half *)logits, gate, rows);
+    CLG_CHECK_LAUNCH("clg_gate_argmax");
+    return CLG_OK;
+}
 
 extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *w, void *y,
                               int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)

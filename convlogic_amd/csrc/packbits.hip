@@ -515,7 +515,7 @@ void launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_
     // column chunks of at most 4 KiB per row: both uses of a row segment fall inside one chunk pass,
     // so the working set of a pass (in_dim x 4 KiB) can stay in the last-level cache (measured best on
     // 64000 x 8 KiB rows among 0.5..8 KiB).  CLG_EVAL_CHUNK_BYTES / CLG_EVAL_NPW override for tuning.
-    const char *e_chunk = getenv("CLG_EVAL_CHUNK_BYTES"), *e_npw = getenv("CLG_EVAL_NPW");
+    const char *e_chunk = clg_knob(K_EVAL_CHUNK_BYTES), *e_npw = clg_knob(K_EVAL_NPW);
     const int max_chunk_vecs = (e_chunk ? atoi(e_chunk) : 4096) / (int)sizeof(V);
     const int chunk_vecs = row_vecs < max_chunk_vecs ? (int)row_vecs : max_chunk_vecs;
     const int chunks = (int)clg_ceil_div(row_vecs, chunk_vecs);
@@ -585,7 +585,7 @@ extern "C" int clg_pack_bits_sample_major(const uint8_t *t, void *words, int64_t
         // from 8 groups of 64 samples on, the words go through LDS and leave as 64 (8..15 groups) or 128 contiguous bytes per
         // feature row: 155 -> 121 us on bool [8192, 64000], 101 -> 52 us on [65536, 4096] with 32 feature lanes x 16 groups
         // (512 threads; 16 x 16 and 64 x 8 are 8 % slower); CLG_PACK_TILE=0 keeps the direct stores
-        const char *e_tile = getenv("CLG_PACK_TILE");
+        const char *e_tile = clg_knob(K_PACK_TILE);
         const bool tiled = !e_tile || atoi(e_tile) != 0;
         if (tiled && groups >= 16)
             hipLaunchKernelGGL((pack_bits_tile_kernel<32, 16>), dim3((unsigned)clg_ceil_div(features, 32 * 16), (unsigned)clg_ceil_div(groups, 16)),
@@ -624,7 +624,7 @@ extern "C" int clg_group_bit_sum(int elem_size, const void *x, int32_t *out, int
         // words); rows are sliced only beyond the counter range of 2^14 - 8 rows per workgroup.
         const int64_t row_words = row_bytes / 8;
         const int64_t col_blocks = clg_ceil_div(row_words, kWave);
-        const char *e_sl = getenv("CLG_GSUM_SLICES");
+        const char *e_sl = clg_knob(K_GSUM_SLICES);
         int64_t slices = e_sl ? atoi(e_sl) : 1;
         if (slices > class_rows / (64 * kCountWaves)) slices = class_rows / (64 * kCountWaves);
         const int64_t need = clg_ceil_div(class_rows, (1 << kCountPlanes) - 8);
@@ -725,7 +725,7 @@ extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const in
     // short or unaligned rows gain nothing from carrying a row in registers
     if ((align & 15) != 0 || row_bytes < 1024) return clg_fc_eval_packed(elem_size, x, a, b, gate, y, in_dim, out_dim, words, stream);
     const int64_t row_vecs = row_bytes / 16;
-    const char *e_r = getenv("CLG_EVAL_WALK_R"), *e_l = getenv("CLG_EVAL_WALK_SEG");
+    const char *e_r = clg_knob(K_EVAL_WALK_R), *e_l = clg_knob(K_EVAL_WALK_SEG);
     int R = e_r ? atoi(e_r) : 4;
     while (R > 1 && (int64_t)kWave * (R / 2) >= row_vecs) R /= 2;
     const int seg = e_l ? atoi(e_l) : 8;

@@ -92,7 +92,9 @@ class LogicLayer(torch.nn.Module):
             assert x.is_cuda, f"x must be a CUDA tensor, got device: {x.device}"
         assert x.ndim == 2, x.ndim
         assert x.shape[1] == self.in_dim, (tuple(x.shape[::-1]), self.in_dim)
-        if self.training and self.weights.dtype == x.dtype and self.weights.is_contiguous():
+        self._check_wiring()
+        if (self.training and self.weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
+                and self.weights.is_contiguous()):
             # a sample-major batch is transposed inside the Function (and its gradient on the way back): one autograd
             # node per layer instead of two
             inside = _transposes_with_kernel(x)
@@ -116,13 +118,36 @@ class LogicLayer(torch.nn.Module):
         return x
 
     def _eval_gates(self):
-        """uint8 arg-max gate id per neuron, recomputed only after the logits changed."""
-        key = (self.weights._version, self.weights.data_ptr())
-        cached = getattr(self, "_gate_cache", None)
-        if cached is None or cached[0] != key:
-            cached = (key, self.weights.detach().argmax(-1).to(torch.uint8))
-            self._gate_cache = cached
-        return cached[1]
+        """uint8 arg-max gate id per neuron, taken from the logits on every call as the reference does
+        (src/difflogic/difflogic.py:161): one small launch, and no cache that an in-place update of
+        `weights.data` (EMA swaps, legacy optimisers) could leave stale."""
+        return difflogic_hip.gate_argmax(self.weights.detach())
+
+    def _wiring_key(self):
+        return (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+
+    def _check_wiring(self):
+        """The kernels index x with indices_0 / indices_1 without bounds checks: an index outside [0, in_dim) must
+        raise here instead of faulting the GPU.  Checked on the first launch and again whenever the buffers were
+        modified in place (version counter) or replaced; writes through `.data` bypass the counter -- call
+        invalidate() after those."""
+        key = self._wiring_key()
+        if getattr(self, "_wiring_checked", None) != key:
+            for name, idx in (("indices_0", self.indices_0), ("indices_1", self.indices_1)):
+                if idx.dtype != torch.int64 or tuple(idx.shape) != (self.out_dim,):
+                    raise ValueError(f"{name} must be int64 [{self.out_dim}], got {idx.dtype} {tuple(idx.shape)}")
+                if idx.numel() and (int(idx.min()) < 0 or int(idx.max()) >= self.in_dim):
+                    raise ValueError(f"{name} holds an input index outside [0, {self.in_dim})")
+            self._wiring_checked = key
+
+    def invalidate(self):
+        """Drops everything derived from the wiring buffers (range check, consumer analysis, packed walk plan).  Needed
+        only after writing indices_0 / indices_1 through `.data`, which the version counters do not see."""
+        self._wiring_checked = self._sole_cache = self._plan_cache = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.invalidate()
 
     def _sole_consumers(self):
         """True when every input feature is read by exactly one neuron operand (the halving layers of the
@@ -130,7 +155,7 @@ class LogicLayer(torch.nn.Module):
         wiring buffers were modified in place or moved."""
         if 2 * self.out_dim != self.in_dim:
             return False
-        key = (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+        key = self._wiring_key()
         cached = getattr(self, "_sole_cache", None)
         if cached is None or cached[0] != key:
             uses = torch.bincount(torch.cat([self.indices_0, self.indices_1]), minlength=self.in_dim)
@@ -141,7 +166,8 @@ class LogicLayer(torch.nn.Module):
     def _eval_plan(self):
         """Walk order of the wiring graph for the packed evaluation kernel; rebuilt when the wiring
         buffers were modified in place or moved to another device."""
-        key = (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+        self._check_wiring()
+        key = self._wiring_key()
         cached = getattr(self, "_plan_cache", None)
         if cached is None or cached[0] != key:
             cached = (key, difflogic_hip.eval_plan(self.indices_0, self.indices_1, self.in_dim))

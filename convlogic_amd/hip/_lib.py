@@ -29,6 +29,8 @@ _GP = ctypes.POINTER(ConvGeom)
 SIGNATURES = {
     "clg_last_error": (ctypes.c_char_p, []),
     "clg_abi_version": (_i, []),
+    "clg_reload_knobs": (None, []),
+    "clg_gate_argmax": (_i, [_i, _p, _p, _i64, _p]),
     "clg_fc_forward": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_w": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_logits": (_i, [_i, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
@@ -128,10 +130,22 @@ def stream_ptr(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def check_input(t, name):
-    """Same contract as the reference's CHECK_INPUT (src/common/cuda_utils.cuh:9-13)."""
+def check_input(t, name, dtype=None, shape=None):
+    """Same contract as the reference's CHECK_INPUT (src/common/cuda_utils.cuh:9-13); with dtype / shape also what its
+    typed packed_accessor<scalar_t, N> arguments enforce: the kernels read raw pointers, so a tensor of another
+    element type or size would be read out of bounds instead of raising."""
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a CUDA tensor")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
     return t
+
+
+def check_same_device(ref, *tensors):
+    for t in tensors:
+        if t is not None and t.device != ref.device:
+            raise RuntimeError(f"all tensors must be on one device, got {ref.device} and {t.device}")

@@ -24,6 +24,40 @@ def _out_size(g):
     return (g.h + 2 * g.pad_h - g.kernel_h) // g.stride_h + 1, (g.w + 2 * g.pad_w - g.kernel_w) // g.stride_w + 1
 
 
+def _conv_args(x, weight, selection, gates):
+    """x [N, C_in, H, W] float, weight [C, gates, 16] of x's dtype, selection int32 [C, 8]: everything on x's device."""
+    check_input(x, "x")
+    if x.dim() != 4:
+        raise RuntimeError(f"Expected x to be 4D (N, C, H, W), but got {x.dim()}")
+    c = weight.shape[0] if weight.dim() else -1
+    check_input(weight, "weights", x.dtype, (c, gates, 16))
+    _selection_arg(x, selection, c)
+    _lib.check_same_device(x, weight)
+
+
+def _selection_arg(x, selection, c):
+    check_input(selection, "selection", torch.int32, (c, 8))
+    _lib.check_same_device(x, selection)
+
+
+def _grad_args(grad_y, x, shape):
+    check_input(grad_y, "grad_y", x.dtype, shape)
+    _lib.check_same_device(x, grad_y)
+
+
+def _block_grad_args(grad_y, x, weight, argmax, selection, feature_major=False):
+    """Arguments of the fused block's backward entry points: grad_y [N, C, Ho/2, Wo/2] (or [C, Ho/2, Wo/2, N]) of x's
+    dtype, argmax uint8 [N, C, Ho/2, Wo/2] with codes 0..3, weights [C, 7, 16], selection int32 [C, 8]."""
+    _conv_args(x, weight, selection, 7)
+    if grad_y.dim() != 4:
+        raise RuntimeError(f"Expected grad_y to be 4D, but got {grad_y.dim()}")
+    n, c = x.shape[0], weight.shape[0]
+    hp, wp = (grad_y.shape[1], grad_y.shape[2]) if feature_major else (grad_y.shape[2], grad_y.shape[3])
+    _grad_args(grad_y, x, (c, hp, wp, n) if feature_major else (n, c, hp, wp))
+    check_input(argmax, "argmax", torch.uint8, (n, c, hp, wp))
+    _lib.check_same_device(x, argmax)
+
+
 def _scratch(nbytes, device):
     if nbytes < 0:
         raise RuntimeError(_lib.load().clg_last_error().decode())
@@ -33,8 +67,7 @@ def _scratch(nbytes, device):
 # ---- split layer ------------------------------------------------------------------------------
 def convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
     """[N,C,Ho,Wo,4]; src/convlogic/cuda/convlogic_kernel.cu:67-106."""
-    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, weight, selection, 4)
     g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     y = torch.empty((g.n, g.c_out, max(ho, 0), max(wo, 0), 4), dtype=x.dtype, device=x.device)
@@ -45,8 +78,10 @@ def convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_w, ke
 
 def convlogic_backward_x(grad_y, x, weight, selection, stride_h, stride_w, pad_h, pad_w):
     """src/convlogic/cuda/convlogic_kernel.cu:321-359 (deterministic here)."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, weight, selection, 4)
+    if grad_y.dim() != 5:
+        raise RuntimeError(f"Expected grad_y to be 5D (N, C, Ho, Wo, 4), but got {grad_y.dim()}")
+    _grad_args(grad_y, x, (x.shape[0], weight.shape[0], grad_y.shape[2], grad_y.shape[3], 4))
     g = _geom_from_out(x, grad_y.shape[1], grad_y.shape[2], grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     gx = torch.empty_like(x)
     check(_lib.load().clg_conv4_backward_x(dtype_code(x), ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
@@ -56,8 +91,11 @@ def convlogic_backward_x(grad_y, x, weight, selection, stride_h, stride_w, pad_h
 
 def convlogic_backward_weight(grad_y, x, selection, stride_h, stride_w, pad_h, pad_w):
     """[C,4,16]; src/convlogic/cuda/convlogic_kernel.cu:197-248."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (selection, "selection")):
-        check_input(t, n)
+    check_input(x, "x")
+    if x.dim() != 4 or grad_y.dim() != 5:
+        raise RuntimeError(f"Expected x 4D and grad_y 5D (N, C, Ho, Wo, 4), but got {x.dim()} and {grad_y.dim()}")
+    _grad_args(grad_y, x, (x.shape[0], grad_y.shape[1], grad_y.shape[2], grad_y.shape[3], 4))
+    _selection_arg(x, selection, grad_y.shape[1])
     g = _geom_from_out(x, grad_y.shape[1], grad_y.shape[2], grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -81,9 +119,9 @@ def _tree_dims(x, xo):
 def treelogic_forward(x, weights):
     """[N,C,H,W,Xout]; src/convlogic/cuda/treelogic_kernel.cu:46-85."""
     check_input(x, "x")
-    check_input(weights, "weights")
-    xo = weights.shape[1]
+    xo = weights.shape[1] if weights.dim() == 3 else -1
     n, c, pos = _tree_dims(x, xo)
+    check_input(weights, "weights", x.dtype, (c, xo, 16))
     y = torch.empty(x.shape[:4] + (xo,), dtype=x.dtype, device=x.device)
     if y.numel():
         check(_lib.load().clg_tree_forward(dtype_code(x), x.data_ptr(), weights.data_ptr(), y.data_ptr(), n, c, pos, xo,
@@ -93,10 +131,11 @@ def treelogic_forward(x, weights):
 
 def treelogic_backward_x(grad_y, x, weights):
     """src/convlogic/cuda/treelogic_kernel.cu:252-285."""
-    for t, n_ in ((grad_y, "grad_y"), (x, "x"), (weights, "weights")):
-        check_input(t, n_)
-    xo = weights.shape[1]
+    check_input(x, "x")
+    xo = weights.shape[1] if weights.dim() == 3 else -1
     n, c, pos = _tree_dims(x, xo)
+    check_input(weights, "weights", x.dtype, (c, xo, 16))
+    check_input(grad_y, "grad_y", x.dtype, tuple(x.shape[:4]) + (xo,))
     gx = torch.empty_like(x)
     if gx.numel():
         check(_lib.load().clg_tree_backward_x(dtype_code(x), grad_y.data_ptr(), x.data_ptr(), weights.data_ptr(), gx.data_ptr(),
@@ -106,10 +145,10 @@ def treelogic_backward_x(grad_y, x, weights):
 
 def treelogic_backward_weight(grad_y, x):
     """[C,Xout,16]; src/convlogic/cuda/treelogic_kernel.cu:160-206."""
-    check_input(grad_y, "grad_y")
     check_input(x, "x")
-    xo = grad_y.shape[4]
+    xo = grad_y.shape[4] if grad_y.dim() == 5 else -1
     n, c, pos = _tree_dims(x, xo)
+    check_input(grad_y, "grad_y", x.dtype, tuple(x.shape[:4]) + (xo,))
     lib = _lib.load()
     dt = dtype_code(x)
     scratch = _scratch(lib.clg_tree_backward_w_scratch_bytes(dt, n, c, pos, xo), x.device)
@@ -124,8 +163,7 @@ def full_convlogic_forward(x, weight, selection, stride_h, stride_w, pad_h, pad_
     """-> (y [N,C,Ho/2,Wo/2], argmax uint8 [N,C,Ho/2,Wo/2] = dy*2+dx of the pooled maximum).
     src/convlogic/cuda/full_convlogic_kernel.cu:147-231; the leaf / middle gate planes the reference
     also returns are not materialised (see full_convlogic_intermediates)."""
-    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, weight, selection, 7)
     g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
@@ -146,12 +184,14 @@ def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, p
     the reference has no packed conv kernel.  feature_major: where the kernels can (4x4 images, at least 32
     groups), the result is the [G, C, Ho/2, Wo/2] VIEW of a contiguous [C, Ho/2, Wo/2, G] tensor -- the layout
     PackBitsTensor.flatten() needs, which then takes a view instead of transposing."""
-    for t, n in ((x, "x"), (gates, "gates"), (selection, "selection")):
-        check_input(t, n)
+    check_input(x, "x")
+    check_input(gates, "gates")
     if x.dtype != torch.int64 or gates.dtype != torch.uint8 or x.dim() != 4:
         raise RuntimeError("full_convlogic_eval_packed expects int64 words [G, C, H, W] and uint8 gate ids [C, 7]")
     if gates.dim() != 2 or gates.shape[1] != 7:
         raise RuntimeError(f"full_convlogic_eval_packed expects gate ids of shape [C, 7], got {tuple(gates.shape)}")
+    _selection_arg(x, selection, gates.shape[0])
+    _lib.check_same_device(x, gates)
     g = _geom(x, gates.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     lib = _lib.load()
@@ -170,8 +210,7 @@ def full_convlogic_eval_packed(x, gates, selection, stride_h, stride_w, pad_h, p
 def full_convlogic_intermediates(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
     """-> (x2 [N,C,Ho,Wo,4], x3 [N,C,Ho,Wo,2]), the second and third result of the reference's
     full_convlogic_forward (full_convlogic_kernel.cu:172,194)."""
-    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, weight, selection, 7)
     g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     x2 = torch.empty((g.n, g.c_out, ho, wo, 4), dtype=x.dtype, device=x.device)
@@ -194,8 +233,7 @@ def argmax_to_indices(argmax, wo):
 
 def full_convlogic_backward_x(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
     """src/convlogic/cuda/full_convlogic_kernel.cu:365-461 (deterministic here)."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
-        check_input(t, n)
+    _block_grad_args(grad_y, x, weight, argmax, selection)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -208,8 +246,7 @@ def full_convlogic_backward_x(grad_y, x, weight, argmax, selection, stride_h, st
 
 def full_convlogic_backward_weight(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
     """[C,7,16]; src/convlogic/cuda/full_convlogic_kernel.cu:616-701."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
-        check_input(t, n)
+    _block_grad_args(grad_y, x, weight, argmax, selection)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -223,8 +260,7 @@ def full_convlogic_backward_weight(grad_y, x, weight, argmax, selection, stride_
 def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w):
     """-> (grad_x, grad_w [C,7,16]) in one call (the pair of calls of
     src/convlogic/convlogic_layer.py:76-81, one scratch buffer, one transition into the library)."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
-        check_input(t, n)
+    _block_grad_args(grad_y, x, weight, argmax, selection)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -239,8 +275,7 @@ def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stri
 def full_convlogic_backward_logits(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True):
     """-> (grad_x or None, grad_logits [C,7,16]) for weight = softmax(logits): the two gradients of the block
     with the softmax backward fused into the final reduction of the weight gradient."""
-    for t, n in ((grad_y, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
-        check_input(t, n)
+    _block_grad_args(grad_y, x, weight, argmax, selection)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -263,8 +298,7 @@ def feature_major_supported(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h
 
 def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
     """full_convlogic_forward() with y laid out [C, Ho/2, Wo/2, N] (contiguous); argmax stays [N,C,Ho/2,Wo/2]."""
-    for t, n in ((x, "x"), (weight, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, weight, selection, 7)
     g = _geom(x, weight.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     y = torch.empty((g.c_out, ho // 2, wo // 2, g.n), dtype=x.dtype, device=x.device)
@@ -281,8 +315,7 @@ def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_
     """full_convlogic_forward() from the LOGITS [C, 7, 16]: the softmax is taken inside the launch that sets the gate
     parameters up.  -> (y, argmax, probs); with feature_major (where feature_major_supported) y is laid out
     [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm()."""
-    for t, n in ((x, "x"), (logits, "weights"), (selection, "selection")):
-        check_input(t, n)
+    _conv_args(x, logits, selection, 7)
     g = _geom(x, logits.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
@@ -301,8 +334,7 @@ def full_convlogic_backward_fm(grad_y_fm, x, weight, argmax, selection, stride_h
                                wrt_logits=True):
     """-> (grad_x or None, grad_w [C,7,16]) from grad_y laid out [C, Ho/2, Wo/2, N]; grad_w is the gradient w.r.t. the
     logits (weight = their softmax) or, with wrt_logits=False, w.r.t. the probabilities."""
-    for t, n in ((grad_y_fm, "grad_y"), (x, "x"), (weight, "weights"), (argmax, "argmax"), (selection, "selection")):
-        check_input(t, n)
+    _block_grad_args(grad_y_fm, x, weight, argmax, selection, feature_major=True)
     g = _geom_from_out(x, grad_y_fm.shape[0], 2 * grad_y_fm.shape[1], 2 * grad_y_fm.shape[2], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)

@@ -6,14 +6,31 @@ from . import _lib
 from ._lib import check, check_input, dtype_code, stream_ptr
 
 _WORD_DTYPE = {8: torch.int8, 16: torch.int16, 32: torch.int32, 64: torch.int64}
+_I64 = torch.int64
+
+
+def _wiring(x, a, b, out_dim):
+    """x [in, B] with the wiring a, b int64 [out] on x's device -> (in_dim, batch)."""
+    check_input(x, "x")
+    if x.dim() != 2:
+        raise RuntimeError(f"x must be 2-D [in_dim, batch], got {tuple(x.shape)}")
+    check_input(a, "a", _I64, (out_dim,))
+    check_input(b, "b", _I64, (out_dim,))
+    _lib.check_same_device(x, a, b)
+    return x.shape
+
+
+def _reverse_map(x, start, flat, out_dim):
+    check_input(start, "given_x_indices_of_y_start", _I64, (x.shape[0] + 1,))
+    check_input(flat, "given_x_indices_of_y", _I64, (2 * out_dim,))
+    _lib.check_same_device(x, start, flat)
 
 
 def forward(x, a, b, w):
     """y[out, B]; difflogic_cuda.forward (src/difflogic/cuda/difflogic_kernel.cu:89-126)."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = w.shape[0]
+    out_dim = w.shape[0] if w.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(w, "w", x.dtype, (out_dim, 16))
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     if y.numel():
         check(_lib.load().clg_fc_forward(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(), y.data_ptr(),
@@ -23,10 +40,9 @@ def forward(x, a, b, w):
 
 def backward_w(x, a, b, grad_y):
     """grad_w[out, 16]; difflogic_cuda.backward_w (difflogic_kernel.cu:128-173)."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (grad_y, "grad_y")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = grad_y.shape[0]
+    out_dim = grad_y.shape[0] if grad_y.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_w(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), grad_y.data_ptr(),
                                         gw.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
@@ -36,10 +52,10 @@ def backward_w(x, a, b, grad_y):
 def backward_logits(x, a, b, w, grad_y):
     """Gradient w.r.t. the logits [out, 16] when w = softmax(logits): backward_w and the softmax backward
     in one kernel."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = grad_y.shape[0]
+    out_dim = grad_y.shape[0] if grad_y.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(w, "w", x.dtype, (out_dim, 16))
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
     gl = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
                                              grad_y.data_ptr(), gl.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
@@ -49,6 +65,8 @@ def backward_logits(x, a, b, w, grad_y):
 def fold(w_in, from_logits, want_probs=True):
     """[out, 16] logits or probabilities -> (probabilities or None, folded coefficients [out, 4])."""
     check_input(w_in, "w")
+    if w_in.dim() != 2 or w_in.shape[1] != 16:
+        raise RuntimeError(f"w must have shape [out_dim, 16], got {tuple(w_in.shape)}")
     out_dim = w_in.shape[0]
     probs = torch.empty_like(w_in) if want_probs else None
     folded = torch.empty((out_dim, 4), dtype=w_in.dtype, device=w_in.device)
@@ -59,10 +77,9 @@ def fold(w_in, from_logits, want_probs=True):
 
 def forward_folded(x, a, b, folded):
     """forward() with the folded coefficients [out, 4] of fold() in place of w."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = folded.shape[0]
+    out_dim = folded.shape[0] if folded.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(folded, "folded", x.dtype, (out_dim, 4))
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_forward_folded(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
                                             y.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
@@ -71,12 +88,11 @@ def forward_folded(x, a, b, folded):
 
 def forward_logits(x, a, b, logits):
     """fold(from_logits=True) + forward_folded() in one launch -> (y [out, B], probs [out, 16], folded [out, 4])."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (logits, "w")):
-        check_input(t, n)
     if logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.dtype not in _lib._DTYPES:
         raise RuntimeError(f"forward_logits expects float32/float64 logits [out, 16] of x's dtype, got {tuple(logits.shape)} {logits.dtype}")
-    in_dim, batch = x.shape
     out_dim = logits.shape[0]
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(logits, "w")
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     probs = torch.empty_like(logits)
     folded = torch.empty((out_dim, 4), dtype=x.dtype, device=x.device)
@@ -88,11 +104,11 @@ def forward_logits(x, a, b, logits):
 
 def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
     """backward_x() with the folded coefficients [out, 4] of fold() in place of w."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y"),
-                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = folded.shape[0]
+    out_dim = folded.shape[0] if folded.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(folded, "folded", x.dtype, (out_dim, 4))
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
+    _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
     gx = torch.empty_like(x)
     check(_lib.load().clg_fc_backward_x_folded(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
                                                grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
@@ -104,12 +120,12 @@ def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given
 def backward_sole(x, a, b, folded, probs, grad_y):
     """(grad_x, grad_w) in one pass for a layer whose inputs are each read by exactly one neuron operand; grad_w is
     the gradient w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y")):
-        check_input(t, n)
+    out_dim = folded.shape[0] if folded.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(folded, "folded", x.dtype, (out_dim, 4))
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
     if probs is not None:
-        check_input(probs, "w")
-    in_dim, batch = x.shape
-    out_dim = folded.shape[0]
+        check_input(probs, "w", x.dtype, (out_dim, 16))
     gx = torch.empty_like(x)
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_sole(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
@@ -127,13 +143,13 @@ def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, g
     """(grad_x, grad_w) of a layer with any wiring in one pass (see backward_fused_fits); grad_w is the gradient
     w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities.  Same values as
     backward_x_folded() + backward_w() / backward_logits()."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (folded, "folded"), (grad_y, "grad_y"),
-                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
-        check_input(t, n)
+    out_dim = folded.shape[0] if folded.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(folded, "folded", x.dtype, (out_dim, 4))
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
+    _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
     if probs is not None:
-        check_input(probs, "w")
-    in_dim, batch = x.shape
-    out_dim = folded.shape[0]
+        check_input(probs, "w", x.dtype, (out_dim, 16))
     gx = torch.empty_like(x)
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_fused(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
@@ -146,6 +162,8 @@ def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, g
 def group_sum(x_fm, k, tau=1.0):
     """Feature-major activations [F, B] -> per-class sums [B, k] divided by tau, fixed summation order."""
     check_input(x_fm, "x")
+    if x_fm.dim() != 2:
+        raise RuntimeError(f"x must be 2-D [features, batch], got {tuple(x_fm.shape)}")
     features, batch = x_fm.shape
     if features % k != 0:
         raise ValueError(f"in_dim ({features}) has to be divisible by k ({k}) but it is not")
@@ -161,6 +179,8 @@ def group_sum(x_fm, k, tau=1.0):
 def group_sum_backward(grad_out, features, tau=1.0):
     """[B, k] -> feature-major gradient [F, B]: every row of class g receives grad_out[:, g] / tau."""
     check_input(grad_out, "grad_out")
+    if grad_out.dim() != 2 or grad_out.shape[1] < 1 or features % grad_out.shape[1] != 0:
+        raise RuntimeError(f"grad_out must be [batch, k] with k dividing {features}, got {tuple(grad_out.shape)}")
     batch, k = grad_out.shape
     gx = torch.empty((features, batch), dtype=grad_out.dtype, device=grad_out.device)
     check(_lib.load().clg_group_sum_backward(dtype_code(grad_out), grad_out.data_ptr(), gx.data_ptr(), features, batch, k,
@@ -170,11 +190,11 @@ def group_sum_backward(grad_out, features, tau=1.0):
 
 def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
     """grad_x[in, B]; difflogic_cuda.backward_x (difflogic_kernel.cu:232-269)."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (grad_y, "grad_y"),
-                 (given_x_indices_of_y_start, "given_x_indices_of_y_start"), (given_x_indices_of_y, "given_x_indices_of_y")):
-        check_input(t, n)
-    in_dim, batch = x.shape
-    out_dim = w.shape[0]
+    out_dim = w.shape[0] if w.dim() else -1
+    in_dim, batch = _wiring(x, a, b, out_dim)
+    check_input(w, "w", x.dtype, (out_dim, 16))
+    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
+    _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
     gx = torch.empty_like(x)
     check(_lib.load().clg_fc_backward_x(dtype_code(x, half_ok=True), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
                                         grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
@@ -185,6 +205,8 @@ def backward_x(x, a, b, w, grad_y, given_x_indices_of_y_start, given_x_indices_o
 def transpose(x):
     """Contiguous transposed copy of a 2-D tensor through the tiled HIP transpose."""
     check_input(x, "x")
+    if x.dim() != 2:
+        raise RuntimeError(f"transpose expects a 2-D tensor, got {tuple(x.shape)}")
     rows, cols = x.shape
     out = torch.empty((cols, rows), dtype=x.dtype, device=x.device)
     if out.numel():
@@ -195,16 +217,27 @@ def transpose(x):
 def eval(x, a, b, w):  # noqa: A001 - name of the reference binding
     """Packed-bit layer evaluation; difflogic_cuda.eval (difflogic_kernel.cu:295-330).
     x: integer words [in, W]; w: uint8 gate ids [out]."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w")):
-        check_input(t, n)
-    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8:
-        raise RuntimeError("eval expects int8/16/32/64 words and uint8 gate ids")
-    in_dim, words = x.shape
+    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8 or w.dim() != 1:
+        raise RuntimeError("eval expects int8/16/32/64 words and uint8 gate ids [out]")
     out_dim = w.shape[0]
+    in_dim, words = _wiring(x, a, b, out_dim)
+    check_input(w, "w")
     y = torch.empty((out_dim, words), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_eval_packed(x.element_size(), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
                                          y.data_ptr(), in_dim, out_dim, words, stream_ptr(x)))
     return y
+
+
+def gate_argmax(logits):
+    """uint8 index of the first maximum over the last dimension (16 gates) of float logits [..., 16]."""
+    check_input(logits, "weights")
+    if logits.dim() < 1 or logits.shape[-1] != 16:
+        raise RuntimeError(f"expected logits [..., 16], got {tuple(logits.shape)}")
+    gate = torch.empty(logits.shape[:-1], dtype=torch.uint8, device=logits.device)
+    if gate.numel():
+        check(_lib.load().clg_gate_argmax(dtype_code(logits, half_ok=True), logits.data_ptr(), gate.data_ptr(), gate.numel(),
+                                          stream_ptr(logits)))
+    return gate
 
 
 def eval_plan(a, b, in_dim):
@@ -220,13 +253,13 @@ def eval_plan(a, b, in_dim):
 def eval_planned(x, a, b, w, plan):
     """eval() in the order of `plan` (from eval_plan for the same a, b): identical result, about half
     the input traffic."""
-    for t, n in ((x, "x"), (a, "a"), (b, "b"), (w, "w"), (plan, "plan")):
-        check_input(t, n)
-    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8 or plan.dtype != torch.int32:
-        raise RuntimeError("eval_planned expects int8/16/32/64 words, uint8 gate ids and an int32 plan")
-    in_dim, words = x.shape
+    if x.dtype not in _WORD_DTYPE.values() or w.dtype != torch.uint8 or plan.dtype != torch.int32 or w.dim() != 1:
+        raise RuntimeError("eval_planned expects int8/16/32/64 words, uint8 gate ids [out] and an int32 plan")
     out_dim = w.shape[0]
-    if plan.shape[0] != out_dim:
+    in_dim, words = _wiring(x, a, b, out_dim)
+    check_input(w, "w")
+    check_input(plan, "plan")
+    if tuple(plan.shape) != (out_dim,):
         raise RuntimeError("plan does not match the number of neurons")
     y = torch.empty((out_dim, words), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_eval_packed_planned(x.element_size(), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
@@ -268,6 +301,8 @@ def tensor_packbits_sample_major(t, bit_count):
 def groupbitsum(b, pad_len, k):
     """int32 [samples, k]; difflogic_cuda.groupbitsum (difflogic.cpp:22-33, difflogic_kernel.cu:450-482)."""
     check_input(b, "b")
+    if b.dim() != 2 or b.dtype not in _WORD_DTYPE.values():
+        raise RuntimeError(f"groupbitsum expects int8/16/32/64 words [features, words], got {tuple(b.shape)} {b.dtype}")
     features, words = b.shape
     if features % k != 0:
         raise ValueError(f"in_dim ({features}) has to be divisible by k ({k}) but it is not")

@@ -43,6 +43,10 @@ const char *clg_last_error(void);
 /* ABI version of this library (bumped on incompatible changes). */
 int clg_abi_version(void);
 
+/* The CLG_* environment variables (tuning and path-forcing knobs) are read once per process; this reads them again
+ * after the environment was changed.  Not synchronised with calls on other threads.  No counterpart in the reference. */
+void clg_reload_knobs(void);
+
 /* Geometry of a logic convolution (src/convlogic/convlogic_layer.py:94-109,192-193). */
 typedef struct clg_conv_geom {
     int32_t n, c_in, h, w;   /* input  [n, c_in, h, w]            */
@@ -190,6 +194,11 @@ int clg_fc_eval_packed(int elem_size, const void *x /*[in_dim,words]*/, const in
  * reference's eval path. */
 int clg_fc_eval_plan(const int64_t *a_host /*[out_dim]*/, const int64_t *b_host /*[out_dim]*/, int64_t in_dim,
                      int64_t out_dim, int32_t *plan_host /*[out_dim]*/);
+
+/* gate[r] = index of the first maximum of the 16 logits of row r, for rows = out_dim (LogicLayer) or c_out * 7
+ * (fused block); dtype CLG_F32, CLG_F64 or CLG_F16.  Replaces self.weights.argmax(-1).to(torch.uint8) of
+ * LogicLayer.forward_cuda_eval (src/difflogic/difflogic.py:161), taken on every packed call as there. */
+int clg_gate_argmax(int dtype, const void *logits /*[rows,16]*/, uint8_t *gate /*[rows]*/, int64_t rows, void *stream);
 
 /* Same result as clg_fc_eval_packed, evaluated in plan order: the shared input row of consecutive
  * neurons stays in registers, so every input row is fetched about once instead of twice.  plan is

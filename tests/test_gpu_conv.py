@@ -7,7 +7,7 @@ import torch
 import convlogic_amd as C
 from convlogic_amd.hip import convlogic_hip
 from oracle import convlogic_oracle as O
-from tests.gpu_util import DEV, assert_grad_close, block_oracle, check_pool_route
+from tests.gpu_util import DEV, assert_grad_close, block_oracle, check_pool_route, set_knobs
 
 pytestmark = pytest.mark.gpu
 
@@ -92,14 +92,14 @@ def test_block_forward_backward_small(stride, pad, kernel, binary, direct, monke
     # "1" forces the kernels that read taps from a padded global copy of x (forward and input gradient);
     # "subset" forces the forward staging of two LDS planes per kernel
     if direct == "1":
-        monkeypatch.setenv("CLG_BWDX_DIRECT", "1")
-        monkeypatch.setenv("CLG_FWD_DIRECT", "1")
-        monkeypatch.setenv("CLG_BWDW_PADDED", "1")
+        set_knobs(monkeypatch, CLG_BWDX_DIRECT="1")
+        set_knobs(monkeypatch, CLG_FWD_DIRECT="1")
+        set_knobs(monkeypatch, CLG_BWDW_PADDED="1")
     if direct == "subset":
-        monkeypatch.setenv("CLG_FWD_SUBSET", "1")
-        monkeypatch.setenv("CLG_FWD_DIRECT", "0")
+        set_knobs(monkeypatch, CLG_FWD_SUBSET="1")
+        set_knobs(monkeypatch, CLG_FWD_DIRECT="0")
     if binary:
-        monkeypatch.setenv("CLG_BWDX_CSR", "1")                    # compressed channel -> kernel lists (wide layers)
+        set_knobs(monkeypatch, CLG_BWDX_CSR="1")                    # compressed channel -> kernel lists (wide layers)
     n, cin, cout, h, w = 3, 3, 6, 8 + pad, 10 + pad
     if ((h + 2 * pad - kernel) // stride + 1) % 2:
         h += stride
@@ -312,9 +312,9 @@ def test_block_4x4_one_sample_per_lane_vs_oracle_and_staged_path(n, cin, cout, d
     for sel in (layer.selection, sel_wide):
         args = (x.detach(), wp, sel, 1, 1, 1, 1, 3, 3)
         y_new, a_new = convlogic_hip.full_convlogic_forward(*args)
-        monkeypatch.setenv("CLG_FWD_4X4", "0")
+        set_knobs(monkeypatch, CLG_FWD_4X4="0")
         y_old, a_old = convlogic_hip.full_convlogic_forward(*args)
-        monkeypatch.delenv("CLG_FWD_4X4")
+        set_knobs(monkeypatch, CLG_FWD_4X4=None)
         assert torch.equal(y_new, y_old) and torch.equal(a_new, a_old)
 
 
@@ -345,12 +345,12 @@ def test_block_4x4_one_sample_per_lane_gradients(n, cin, cout, dtype, monkeypatc
         got, want = {}, {}
         for store, flag in ((got, None), (want, "0")):
             if flag is not None:
-                monkeypatch.setenv("CLG_BWD_4X4", flag)
+                set_knobs(monkeypatch, CLG_BWD_4X4=flag)
             store["both"] = convlogic_hip.full_convlogic_backward(gy, x.detach(), wp, am, sel, 1, 1, 1, 1)
             store["logits"] = convlogic_hip.full_convlogic_backward_logits(gy, x.detach(), wp, am, sel, 1, 1, 1, 1)
             store["no_gx"] = convlogic_hip.full_convlogic_backward_logits(gy, x.detach(), wp, am, sel, 1, 1, 1, 1, need_grad_x=False)
             if flag is not None:
-                monkeypatch.delenv("CLG_BWD_4X4")
+                set_knobs(monkeypatch, CLG_BWD_4X4=None)
         assert got["no_gx"][0] is None and want["no_gx"][0] is None
         for key in ("both", "logits", "no_gx"):
             for a, b in zip(got[key], want[key]):
@@ -418,7 +418,7 @@ def test_forward_from_logits_takes_the_softmax_inside(shape, env, dtype, monkeyp
     from convlogic_amd.hip import convlogic_hip
     n, cin, h, w, cout = shape
     for k, v in env.items():
-        monkeypatch.setenv(k, v)
+        set_knobs(monkeypatch, **{k: v})
     stride = 2 if h == 11 else 1
     torch.manual_seed(n + cin + h)
     layer = C.ConvLogicLayer(cin, cout, stride=stride, padding=1, complete=True, implementation="cuda").to(DEV).to(dtype)
@@ -458,3 +458,36 @@ def test_forward_ex_rejects_bad_options():
     assert call(1, probs.data_ptr()) == 0
     torch.cuda.synchronize()
     assert (probs - torch.softmax(layer.weights.detach(), -1)).abs().max().item() <= 1e-6
+
+
+def test_block_bindings_reject_mismatched_tensors():
+    # float32 probabilities with a float64 x, an int64 selection, a wrong gate count: RuntimeError before any launch
+    layer = C.ConvLogicLayer(3, 4, padding=1, complete=True, implementation="cuda").to(DEV)
+    x = torch.rand(2, 3, 8, 8, device=DEV)
+    w = torch.softmax(layer.weights.detach(), -1)
+    geo = (1, 1, 1, 1, 3, 3)
+    with pytest.raises(RuntimeError, match="dtype"):
+        convlogic_hip.full_convlogic_forward(x.double(), w, layer.selection, *geo)
+    with pytest.raises(RuntimeError, match="dtype"):
+        convlogic_hip.full_convlogic_forward(x, w, layer.selection.long(), *geo)
+    with pytest.raises(RuntimeError, match="shape"):
+        convlogic_hip.full_convlogic_forward(x, w[:, :4].contiguous(), layer.selection, *geo)
+    with pytest.raises(RuntimeError, match="shape"):
+        convlogic_hip.convlogic_forward(x, w, layer.selection, *geo)          # the split layer takes 4 gates
+    y, am = convlogic_hip.full_convlogic_forward(x, w, layer.selection, *geo)
+    with pytest.raises(RuntimeError, match="dtype"):
+        convlogic_hip.full_convlogic_backward(torch.rand_like(y), x, w, am.int(), layer.selection, 1, 1, 1, 1)
+    with pytest.raises(RuntimeError, match="shape"):
+        convlogic_hip.full_convlogic_backward(torch.rand(2, 4, 4, 5, device=DEV), x, w, am, layer.selection, 1, 1, 1, 1)
+    # the modules cast the probabilities to x's element type themselves: float32 weights, float64 input
+    yd = layer(x.double())
+    assert yd.dtype == torch.float64 and (yd.float() - layer(x)).abs().max().item() <= 1e-5
+    tree = C.TreeLogicLayer(4, 4, implementation="cuda").to(DEV)
+    xt = torch.rand(2, 4, 3, 3, 4, device=DEV)
+    assert (tree(xt.double()).float() - tree(xt)).abs().max().item() <= 1e-5
+    # a selection that names a channel the input does not have, and an input with the wrong channel count
+    with pytest.raises(RuntimeError, match="Expected x of shape"):
+        layer(torch.rand(2, 2, 8, 8, device=DEV))
+    layer.selection[0, 0] = (7 << 16) | (1 << 8) | 1
+    with pytest.raises(ValueError, match="selection names a tap outside"):
+        layer(x)

@@ -8,7 +8,7 @@ import torch
 import convlogic_amd as C
 from convlogic_amd.hip import convlogic_hip
 from oracle import convlogic_oracle as O
-from tests.gpu_util import DEV
+from tests.gpu_util import DEV, set_knobs
 
 pytestmark = pytest.mark.gpu
 GEOMS = [(1, 1, 3), (2, 2, 4), (1, 0, 3), (2, 1, 3), (1, 2, 5)]
@@ -37,10 +37,10 @@ def _fit_even(h, w, stride, pad, kernel):
 @pytest.mark.parametrize("subset", [None, "1", "direct"])
 def test_packed_block_small_vs_oracle(stride, pad, kernel, n, subset, monkeypatch):
     if subset == "1":
-        monkeypatch.setenv("CLG_FWD_SUBSET", "1")          # two LDS planes per kernel instead of all channels
-        monkeypatch.setenv("CLG_FWD_DIRECT", "0")
+        set_knobs(monkeypatch, CLG_FWD_SUBSET="1")          # two LDS planes per kernel instead of all channels
+        set_knobs(monkeypatch, CLG_FWD_DIRECT="0")
     if subset == "direct":
-        monkeypatch.setenv("CLG_FWD_DIRECT", "1")          # taps from a padded global copy, no LDS
+        set_knobs(monkeypatch, CLG_FWD_DIRECT="1")          # taps from a padded global copy, no LDS
     cin, cout = 3, 6
     h, w = _fit_even(8 + pad, 10 + pad, stride, pad, kernel)
     layer = _layer(cin, cout, stride, pad, kernel, seed=n + stride)
@@ -77,10 +77,10 @@ def test_packed_block_equals_float_eval_path(shape):
 
 @pytest.mark.parametrize("subset", ["0", "1"])
 def test_selection_with_more_than_two_channels_per_kernel(subset, monkeypatch):
-    monkeypatch.setenv("CLG_FWD_DIRECT", "0")
+    set_knobs(monkeypatch, CLG_FWD_DIRECT="0")
     # a caller-made selection may name up to 8 channels per kernel; the two-planes-per-kernel staging then
     # reads those kernels' taps from global memory (float and packed)
-    monkeypatch.setenv("CLG_FWD_SUBSET", subset)
+    set_knobs(monkeypatch, CLG_FWD_SUBSET=subset)
     torch.manual_seed(2)
     cin, cout, h, w = 12, 10, 8, 8
     ch = torch.randint(0, cin, (cout, 8))
@@ -161,11 +161,11 @@ def test_packed_block_4x4_one_group_per_lane(samples, cin, cout, monkeypatch):
     p = layer(C.PackBitsTensor(bits, 64))
     assert p.pad_len == pad and np.array_equal(p.t.cpu().numpy(), want)
     x_words = torch.from_numpy(words).to(DEV)
-    monkeypatch.setenv("CLG_FWD_4X4", "0")
+    set_knobs(monkeypatch, CLG_FWD_4X4="0")
     staged = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
-    monkeypatch.delenv("CLG_FWD_4X4")
+    set_knobs(monkeypatch, CLG_FWD_4X4=None)
     assert torch.equal(staged, p.t)
-    monkeypatch.setenv("CLG_PACKED_4X4_HALVES", "0")
+    set_knobs(monkeypatch, CLG_PACKED_4X4_HALVES="0")
     whole = convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3)
     assert torch.equal(whole, p.t)
 
@@ -203,7 +203,7 @@ def test_one_position_per_lane_equals_two_rows_per_lane(n, cin, cout, hw, monkey
     # workgroups whose samples fill at most half a wavefront with (row pair, column) slots give every conv position
     # its own lane and pool across lanes; same bits and same float values (pooling choice included) as the default
     # mapping, and the packed result against the oracle
-    monkeypatch.setenv("CLG_FWD_4X4", "0")
+    set_knobs(monkeypatch, CLG_FWD_4X4="0")
     layer = _layer(cin, cout, 1, 1, 3, seed=n)
     bits = torch.randint(0, 2, (n * 64, cin, hw, hw), device=DEV).bool() if n <= 5 else torch.randint(0, 2, (n, cin, hw, hw), device=DEV).bool()
     gates = layer.weights.argmax(-1).to(torch.uint8)
@@ -213,7 +213,7 @@ def test_one_position_per_lane_equals_two_rows_per_lane(n, cin, cout, hw, monkey
     wp = torch.softmax(layer.weights.detach(), -1)
     got = {}
     for mode in ("1", "0"):
-        monkeypatch.setenv("CLG_FWD_ONE_ROW", mode)                   # 0: every shape keeps two rows per lane
+        set_knobs(monkeypatch, CLG_FWD_ONE_ROW=mode)                   # 0: every shape keeps two rows per lane
         got[mode] = (convlogic_hip.full_convlogic_eval_packed(x_words, gates, layer.selection, 1, 1, 1, 1, 3, 3),
                      *convlogic_hip.full_convlogic_forward(x, wp, layer.selection, 1, 1, 1, 1, 3, 3))
     for a, b in zip(got["1"], got["0"]):

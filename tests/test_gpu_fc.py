@@ -383,3 +383,87 @@ def test_fc_half_storage(in_dim, out_dim, batch):
     layer.eval()
     yb = layer(torch.randint(0, 2, (batch, in_dim), device=DEV).half())
     assert torch.all((yb == 0) | (yb == 1))
+
+
+def test_fc_half_layer_trains_on_half_input():
+    # layer.half() with a float16 batch (the reference dispatches forward / backward for half,
+    # src/difflogic/cuda/difflogic_kernel.cu:108,146,249, with w = softmax(weights).to(x.dtype)): forward and both
+    # gradients against the float32 oracle on the half-rounded tensors
+    torch.manual_seed(21)
+    layer = C.LogicLayer(48, 64, implementation="cuda").to(DEV).half()
+    x = torch.rand(40, 48, device=DEV).half().requires_grad_(True)
+    gy = torch.randn(40, 64, device=DEV).half()
+    y = layer(x)
+    assert y.dtype == torch.float16
+    y.backward(gy)
+    assert layer.weights.grad is not None and layer.weights.grad.dtype == torch.float16
+    xl = x.detach().float().cpu().requires_grad_(True)
+    ll = layer.weights.detach().float().cpu().requires_grad_(True)
+    w = torch.softmax(ll, -1)
+    y_ref = O.logic_fc_forward(xl, layer.indices_0.cpu(), layer.indices_1.cpu(), w)
+    y_ref.backward(gy.float().cpu())
+    assert (y.detach().float().cpu() - y_ref.detach()).abs().max().item() <= 2e-3
+    assert (x.grad.float().cpu() - xl.grad).abs().max().item() <= 4e-3 * xl.grad.abs().max().item() + 1e-3
+    assert (layer.weights.grad.float().cpu() - ll.grad).abs().max().item() <= 1e-2 * ll.grad.abs().max().item() + 1e-3
+
+
+def test_fc_bindings_reject_mismatched_tensors():
+    # the kernels read raw pointers: a tensor of another element type or shape must raise, as the reference's typed
+    # accessors do, instead of being read out of bounds
+    layer = C.LogicLayer(16, 24, implementation="cuda").to(DEV)
+    xt = torch.rand(16, 8, device=DEV)
+    a, b = layer.indices_0, layer.indices_1
+    w = torch.softmax(layer.weights.detach(), -1)
+    with pytest.raises(RuntimeError, match="dtype"):
+        difflogic_hip.forward(xt.double(), a, b, w)                  # float32 probabilities with float64 x
+    with pytest.raises(RuntimeError, match="dtype"):
+        difflogic_hip.forward(xt, a.int(), b, w)                     # int32 wiring
+    with pytest.raises(RuntimeError, match="shape"):
+        difflogic_hip.forward(xt, a[:-1].contiguous(), b, w)
+    with pytest.raises(RuntimeError, match="shape"):
+        difflogic_hip.backward_w(xt, a, b, torch.rand(24, 9, device=DEV))
+    with pytest.raises(RuntimeError, match="shape"):
+        difflogic_hip.backward_x(xt, a, b, w, torch.rand(24, 8, device=DEV), layer.given_x_indices_of_y_start[:-1].contiguous(),
+                                 layer.given_x_indices_of_y)
+    with pytest.raises(RuntimeError):
+        difflogic_hip.eval(torch.zeros(16, 4, dtype=torch.int64, device=DEV), a, b, torch.zeros(24, dtype=torch.int64, device=DEV))
+
+
+def test_fc_rewired_out_of_range_raises_instead_of_launching():
+    layer = C.LogicLayer(16, 24, implementation="cuda").to(DEV)
+    x = torch.rand(8, 16, device=DEV)
+    layer(x)
+    layer.indices_0[5] = 16
+    with pytest.raises(ValueError, match="indices_0"):
+        layer(x)
+    layer.eval()
+    with pytest.raises(ValueError, match="indices_0"):
+        layer(C.PackBitsTensor(x > 0.5, 64))
+
+
+def test_packed_gates_follow_in_place_weight_updates():
+    # the arg-max gates of the packed path are taken from the logits on every call: an update through `.data`
+    # (EMA swap, legacy optimiser), which no version counter sees, must change the evaluated network
+    torch.manual_seed(23)
+    layer = C.LogicLayer(32, 48, implementation="cuda").to(DEV).eval()
+    bits = torch.randint(0, 2, (100, 32), device=DEV).bool()
+    before = layer(C.PackBitsTensor(bits, 64)).t.clone()
+    new = torch.randn_like(layer.weights)
+    layer.weights.data.copy_(new)
+    after = layer(C.PackBitsTensor(bits, 64)).t
+    words, _ = O.pack_bits(bits.cpu().numpy().T, 64)
+    import numpy as np
+    want = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(),
+                         new.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(after.cpu().numpy(), want) and not torch.equal(before, after)
+    # ties and the first-maximum rule of the arg-max kernel
+    logits = torch.zeros(5, 16, device=DEV)
+    logits[1, 7] = logits[1, 9] = 2.0
+    logits[2, 15] = 1.0
+    logits[3] = -1.0
+    logits[4, 3] = float("nan")
+    got = difflogic_hip.gate_argmax(logits)
+    assert got.tolist() == [0, 7, 15, 0, 3] and got.dtype == torch.uint8
+    assert torch.equal(difflogic_hip.gate_argmax(new).long(), new.argmax(-1))
+    assert torch.equal(difflogic_hip.gate_argmax(new.double()).long(), new.argmax(-1))
+    assert torch.equal(difflogic_hip.gate_argmax(new.half()).long(), new.half().argmax(-1))

@@ -34,7 +34,7 @@ def test_ctypes_signatures_match_the_header_prototypes():
     header = open(os.path.join(ROOT, "include", "convlogic_amd.h")).read()
     header = re.sub(r"/\*.*?\*/", " ", header, flags=re.S)              # comments, also the ones inside argument lists
     header = re.sub(r"//[^\n]*", " ", header)
-    protos = re.findall(r"\b(const char \*|int64_t|int)\s*(clg_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", header)
+    protos = re.findall(r"\b(const char \*|int64_t|int|void)\s*(clg_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", header)
     assert {name for _, name, _ in protos} == set(_lib.SIGNATURES)
 
     def ctype_of(decl):
@@ -46,7 +46,7 @@ def test_ctypes_signatures_match_the_header_prototypes():
         base = decl.rsplit(" ", 1)[0] if " " in decl else decl        # drop the parameter name
         return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "double": ctypes.c_double}[base.replace("const ", "")]
 
-    results = {"const char *": ctypes.c_char_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int}
+    results = {"const char *": ctypes.c_char_p, "int64_t": ctypes.c_int64, "int": ctypes.c_int, "void": None}
     for ret, name, args in protos:
         want = [t for t in (ctype_of(a) for a in args.split(",")) if t is not None]
         res, got = _lib.SIGNATURES[name]
@@ -196,6 +196,44 @@ def test_constructor_validation():
     assert set(layer.state_dict()) == {"weights", "selection"}
     fc = C.LogicLayer(4, 4, implementation="python")
     assert set(fc.state_dict()) == {"weights", "indices_0", "indices_1"}
+
+
+def test_bad_selection_and_wiring_raise_on_the_host():
+    # a tap outside the input channels / receptive field, or a wiring index outside the input features, would be an
+    # out-of-range access inside a kernel: both are rejected on the host (ValueError), also after in-place edits
+    good = C.ConvLogicLayer(2, 3, kernel=3, implementation="python").selection
+    for bad_tap in ((5 << 16) | (1 << 8) | 1, (1 << 16) | (3 << 8) | 1, (1 << 16) | (1 << 8) | 7):
+        bad = good.clone()
+        bad[1, 4] = bad_tap
+        with pytest.raises(ValueError, match="selection names a tap outside"):
+            C.ConvLogicLayer(2, 3, kernel=3, selection=bad, implementation="python")
+    with pytest.raises(ValueError, match="int32"):
+        C.ConvLogicLayer(2, 3, kernel=3, selection=good.long(), implementation="python")
+    layer = C.ConvLogicLayer(2, 3, kernel=3, selection=good.clone(), implementation="python")
+    layer._check_selection()
+    layer.selection[0, 0] = 9 << 16                              # in-place edit: seen through the version counter
+    with pytest.raises(ValueError):
+        layer._check_selection()
+    layer.selection.data[0, 0] = good[0, 0]                      # .data writes bypass it ...
+    layer.invalidate()                                            # ... and need an explicit invalidate()
+    layer._check_selection()
+
+    fc = C.LogicLayer(6, 8, implementation="python")
+    fc._check_wiring()
+    fc.indices_1[3] = 6
+    with pytest.raises(ValueError, match="indices_1"):
+        fc._check_wiring()
+    fc.indices_1[3] = 0
+    fc._check_wiring()
+    fc.indices_0[0] = -1
+    with pytest.raises(ValueError, match="indices_0"):
+        fc._check_wiring()
+    # load_state_dict re-arms the checks
+    fc2 = C.LogicLayer(6, 8, implementation="python")
+    fc2._check_wiring()
+    fc2.load_state_dict(fc.state_dict())
+    with pytest.raises(ValueError):
+        fc2._check_wiring()
 
 
 # ---- model topologies -----------------------------------------------------------------------------
