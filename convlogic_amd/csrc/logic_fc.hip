@@ -7,6 +7,8 @@
 // registers; the per-sample work is one multiply and three FMAs.
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "clg_common.h"
 
 namespace {
@@ -1060,35 +1062,87 @@ extern "C" int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int6
     return 64 * k * batch * (dtype == CLG_F64 ? 8 : 4);               // at most 64 row slices
 }
 
-extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch, int64_t features, int64_t batch, int64_t k,
-                             double tau, void *stream)
+static int group_sum_impl(int dtype, const void *x, void *out, void *partial, int64_t partial_bytes, int64_t features,
+                          int64_t batch, int64_t k, double tau, void *stream, const char *name)
 {
-    CLG_REQUIRE(tau != 0.0, "clg_group_sum: tau must not be zero");
-    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_group_sum: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
-    CLG_REQUIRE(x && out && scratch, "clg_group_sum: null pointer argument");
-    CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && k <= 65535, "clg_group_sum: features, batch and k must be positive, k <= 65535");
+    CLG_REQUIRE(tau != 0.0, "%s: tau must not be zero", name);
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
+    CLG_REQUIRE(x && out && partial, "%s: null pointer argument", name);
+    CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && k <= 65535, "%s: features, batch and k must be positive, k <= 65535", name);
     CLG_REQUIRE(features % k == 0, "in_dim (%lld) has to be divisible by k (%lld) but it is not", (long long)features, (long long)k);
     const int64_t class_rows = features / k, bchunks = clg_ceil_div(batch, kWave);
-    CLG_REQUIRE(bchunks < (1ll << 31), "clg_group_sum: batch too large for one launch");
+    CLG_REQUIRE(bchunks < (1ll << 31), "%s: batch too large for one launch", name);
     // row slices until about four workgroups per CU, at least 64 rows each
     int64_t slices = clg_ceil_div(1024, bchunks * k);
     if (slices > class_rows / 64) slices = class_rows / 64;
     slices = slices < 1 ? 1 : (slices > 64 ? 64 : slices);
+    const int64_t need = slices * k * batch * (dtype == CLG_F64 ? 8 : 4);
+    CLG_REQUIRE(partial_bytes < 0 || need <= partial_bytes,
+                "%s: k * batch = %lld needs %lld bytes of partial sums, the built-in buffer holds %lld (use clg_group_sum with a "
+                "caller-provided scratch buffer for this size)", name, (long long)(k * batch), (long long)need, (long long)partial_bytes);
     hipStream_t st = clg_stream(stream);
     const dim3 grid((unsigned)bchunks, (unsigned)k, (unsigned)slices);
     if (dtype == CLG_F32) {
-        hipLaunchKernelGGL(group_sum_fm_kernel<float>, grid, dim3(256), 0, st, (const float *)x, (float *)scratch, class_rows, batch, (int)k,
+        hipLaunchKernelGGL(group_sum_fm_kernel<float>, grid, dim3(256), 0, st, (const float *)x, (float *)partial, class_rows, batch, (int)k,
                            (int)slices);
         hipLaunchKernelGGL(group_sum_finish_kernel<float>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
-                           (const float *)scratch, (float *)out, batch, (int)k, (int)slices, 1.0f / (float)tau);
+                           (const float *)partial, (float *)out, batch, (int)k, (int)slices, 1.0f / (float)tau);
     } else {
-        hipLaunchKernelGGL(group_sum_fm_kernel<double>, grid, dim3(256), 0, st, (const double *)x, (double *)scratch, class_rows, batch,
+        hipLaunchKernelGGL(group_sum_fm_kernel<double>, grid, dim3(256), 0, st, (const double *)x, (double *)partial, class_rows, batch,
                            (int)k, (int)slices);
         hipLaunchKernelGGL(group_sum_finish_kernel<double>, dim3((unsigned)clg_ceil_div(batch * k, 256)), dim3(256), 0, st,
-                           (const double *)scratch, (double *)out, batch, (int)k, (int)slices, 1.0 / tau);
+                           (const double *)partial, (double *)out, batch, (int)k, (int)slices, 1.0 / tau);
     }
-    CLG_CHECK_LAUNCH("clg_group_sum");
+    CLG_CHECK_LAUNCH(name);
     return CLG_OK;
+}
+
+extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch, int64_t features, int64_t batch, int64_t k,
+                             double tau, void *stream)
+{
+    return group_sum_impl(dtype, x, out, scratch, -1, features, batch, k, tau, stream, "clg_group_sum");
+}
+
+// ---- GroupSum for callers that cannot allocate ---------------------------------------------------
+// The partial sums of clg_group_sum live in a buffer that is part of the library image: every GPU the library runs
+// on holds its own copy of the array until the process ends.  In host code the array's name is only a stand-in for
+// the symbol; the device address is asked for once per device (with that device current) and kept.
+constexpr int64_t kStaticScratchBytes = 1 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static int static_scratch_ptr(void **out, const char *name)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptr_of[kMaxDevices];                                 // device address of `scratch` per device, nullptr = not asked yet
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        clg_set_error("%s: cannot identify the current device (%s)", name, e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return CLG_ELAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            clg_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", name, dev, hipGetErrorString(e));
+            return CLG_ELAUNCH;
+        }
+        ptr_of[dev] = p;
+    }
+    *out = ptr_of[dev];
+    return CLG_OK;
+}
+
+extern "C" int64_t clg_group_sum_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int clg_group_sum_static(int dtype, const void *x, void *out, int64_t features, int64_t batch, int64_t k, double tau,
+                                    void *stream)
+{
+    void *partial = nullptr;
+    if (int e = static_scratch_ptr(&partial, "clg_group_sum_static")) return e;
+    return group_sum_impl(dtype, x, out, partial, kStaticScratchBytes, features, batch, k, tau, stream, "clg_group_sum_static");
 }
 
 extern "C" int clg_group_sum_backward(int dtype, const void *grad_out, void *grad_x, int64_t features, int64_t batch, int64_t k,

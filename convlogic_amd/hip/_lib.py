@@ -43,6 +43,8 @@ SIGNATURES = {
     "clg_fc_backward_fused": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_group_sum_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _f64, _p]),
+    "clg_group_sum_static_max_bytes": (_i64, []),
+    "clg_group_sum_static": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_group_sum_backward": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_fc_backward_x": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_transpose_2d": (_i, [_i, _p, _p, _i64, _i64, _p]),

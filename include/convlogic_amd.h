@@ -152,6 +152,16 @@ int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int6
 int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int64_t batch, int64_t k);
 int clg_group_sum(int dtype, const void *x, void *out /*[batch,k]*/, void *scratch, int64_t features, int64_t batch,
                   int64_t k, double tau, void *stream);
+/* clg_group_sum for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no scratch argument -- the partial sums go to a buffer of
+ * clg_group_sum_static_max_bytes() bytes (1 MiB) that is part of the library image, one copy per GPU, held until the
+ * process ends.  Sizes whose partial sums (at most 64 * k * batch elements, fewer for few rows per class) do not fit are
+ * rejected with CLG_EINVAL.  The call itself allocates and frees nothing.  Every call on a GPU uses that GPU's one
+ * buffer: calls that overlap on one GPU (different streams or threads) race; calls on one stream are ordered.  Same
+ * values as clg_group_sum, bit for bit.  No counterpart in the reference. */
+int64_t clg_group_sum_static_max_bytes(void);
+int clg_group_sum_static(int dtype, const void *x /*[features,batch]*/, void *out /*[batch,k]*/, int64_t features,
+                         int64_t batch, int64_t k, double tau, void *stream);
 /* Its backward: grad_x[f][b] = grad_out[b][f / (features/k)] * (1 / tau). */
 int clg_group_sum_backward(int dtype, const void *grad_out /*[batch,k]*/, void *grad_x /*[features,batch]*/,
                            int64_t features, int64_t batch, int64_t k, double tau, void *stream);
