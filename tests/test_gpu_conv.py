@@ -491,3 +491,56 @@ def test_block_bindings_reject_mismatched_tensors():
     layer.selection[0, 0] = (7 << 16) | (1 << 8) | 1
     with pytest.raises(ValueError, match="selection names a tap outside"):
         layer(x)
+
+
+@pytest.mark.parametrize("stride,pad,kernel", [(1, 1, 3), (2, 2, 4)])
+def test_native_module_drop_in_with_the_reference_signatures(stride, pad, kernel):
+    # convlogic_cuda_compat exports the reference's nine native functions with the reference's arities
+    # (src/convlogic/cuda/convlogic.cpp:17-44).  The call sequence of the reference's FullConvLogicFunction
+    # (src/convlogic/convlogic_layer.py:51-56 forward, :76-81 backward) is restated here on top of it and checked
+    # against the oracle: y, x2, x3, indices, and both gradients.
+    import convlogic_amd.hip.convlogic_cuda_compat as convlogic_cuda
+
+    class RefShapedFunction(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, w_prob, selection, sh, sw, ph, pw, kh, kw):
+            x1 = x.contiguous()
+            y, x2, x3, indices = convlogic_cuda.full_convlogic_forward(x1, w_prob, selection, sh, sw, ph, pw, kh, kw)
+            ctx.save_for_backward(x1, x2, x3, w_prob, selection, indices)
+            ctx.stride, ctx.padding = (sh, sw), (ph, pw)
+            ctx.mark_non_differentiable(indices)
+            return y, x2, x3, indices
+
+        @staticmethod
+        def backward(ctx, grad_y, *_):
+            x1, x2, x3, w_prob, selection, indices = ctx.saved_tensors
+            grad_x1, grad_x2, grad_x3 = convlogic_cuda.full_convlogic_backward_x(grad_y.contiguous(), x1, x2, x3, w_prob, indices,
+                                                                               selection, *ctx.stride, *ctx.padding)
+            grad_w = convlogic_cuda.full_convlogic_backward_weight(grad_x2, grad_x3, grad_y.contiguous(), x1, x2, x3, indices,
+                                                                   selection, *ctx.stride, *ctx.padding)
+            return grad_x1, grad_w, None, None, None, None, None, None, None
+
+    torch.manual_seed(stride + 40)
+    layer = C.ConvLogicLayer(3, 6, stride=stride, padding=pad, kernel=kernel, complete=True, implementation="cuda").to(DEV)
+    h = 9 if stride == 1 else 12
+    while ((h + 2 * pad - kernel) // stride + 1) % 2:
+        h += 1
+    x = torch.rand(5, 3, h, h, device=DEV, requires_grad=True)
+    logits = layer.weights.detach().clone().requires_grad_(True)
+    y, x2, x3, indices = RefShapedFunction.apply(x, torch.softmax(logits, -1), layer.selection, stride, stride, pad, pad, kernel, kernel)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    routed, y_ref, idx_ref, x2_ref, x3_ref, ll, xl, x4 = block_oracle(x, logits, layer.selection, _pair(stride), _pair(pad), _pair(kernel),
+                                                                      indices)
+    assert indices.dtype == torch.int32 and indices.shape == idx_ref.shape
+    check_pool_route(indices, idx_ref, x4)
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5
+    assert (x2.detach().cpu() - x2_ref.detach()).abs().max().item() <= 1e-5
+    assert (x3.detach().cpu() - x3_ref.detach()).abs().max().item() <= 1e-5
+    routed.backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x")
+    assert_grad_close(logits.grad, ll.grad, name="grad_logits")
+    # the other six names are there with the reference's arities
+    for name in ("convlogic_forward", "convlogic_backward_x", "convlogic_backward_weight", "treelogic_forward",
+                 "treelogic_backward_x", "treelogic_backward_weight"):
+        assert callable(getattr(convlogic_cuda, name))
