@@ -688,6 +688,232 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
     block_sum_store<T, 28, 256>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 28);
 }
 
+
+// Weight gradient with the input images staged in LDS (the layout of the forward kernel): for blocks whose sample
+// images fit LDS.  A workgroup owns 16 kernels (one per wavefront, for its whole life) and a run of `rounds` groups
+// of S samples, which it stages one after the other; a wavefront walks the pooled cells of the staged samples
+// (lanes = cells), recomputes the tree at the arg-max position from LDS and keeps its kernel's 28 sums (7 gates x
+// (ab, a, b, 1)) in registers over all rounds, so the 64-lane reduction of the sums happens once per wavefront.
+// The next group's image travels through registers while the current one is evaluated (at most kStagePerThread
+// elements per thread, LDS positions computed once).  Folded coefficients and tap offsets are made by the wavefront
+// itself from w and the selection: no set-up launch, no padded copy of x, every x element is read once per 16 kernels.
+// partial [c][gridDim.x][28]; with `counter` (one zeroed int per kernel, left zero again) the wavefront that
+// finishes a kernel last adds the partial sums in block order and writes the kernel's gradient itself (no reduce launch).
+constexpr int kStagePerThread = 10;
+constexpr int kTiledWWaves = 16;
+template <typename T, int V>
+__global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_tiled_kernel(
+    const T *__restrict__ gy, const T *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ sel,
+    const uint8_t *__restrict__ argmax, T *__restrict__ partial, int *__restrict__ counter, T *__restrict__ gw,
+    const T *__restrict__ probs, Geom g, TilePlan p, int rounds)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *xs = reinterpret_cast<T *>(smem);
+    T *meet = xs + ((p.xe + 3) & ~3);                                 // [waves][28] exchange of the final sums
+    const int tid = threadIdx.x;
+    constexpr int nthreads = kTiledWWaves * kWave;
+    const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
+    // p.CT kernels per workgroup; the 16 / p.CT wavefronts of a kernel take every (16 / p.CT)-th block of cells
+    const int slices = kTiledWWaves / p.CT, slice = wave / p.CT;
+    const int c = uniform((int)blockIdx.y * p.CT + wave % p.CT);
+    const bool has_kernel = c < g.c;
+    const int cc = has_kernel ? c : g.c - 1;
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+    const int hw = g.h * g.w;
+    // this wavefront's kernel: folded coefficients and tap offsets in the LDS image
+    const Tree<T> tr = load_tree(w + (int64_t)cc * 7 * 16);
+    int to[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const Tap tp = unpack_tap(sel[(int64_t)cc * 8 + t]);
+        to[t] = uniform(tp.ch * p.chs + tp.ry * p.rs + tp.rx);
+    }
+    T acc[28];
+#pragma unroll
+    for (int k = 0; k < 28; ++k) acc[k] = T(0);
+    auto accumulate = [&](const T (&tv)[8], T gout) {
+        const TreeVals<T> v = eval_tree(tr, tv);
+        T gin[7][2], gg[7];
+        gg[6] = gout;
+        gin[6][0] = v.mid[0];
+        gin[6][1] = v.mid[1];
+        gg[4] = gout * gate_da(tr.g[6], v.mid[1]);
+        gg[5] = gout * gate_db(tr.g[6], v.mid[0]);
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            gin[4 + m][0] = v.leaf[2 * m];
+            gin[4 + m][1] = v.leaf[2 * m + 1];
+            gg[2 * m] = gg[4 + m] * gate_da(tr.g[4 + m], v.leaf[2 * m + 1]);
+            gg[2 * m + 1] = gg[4 + m] * gate_db(tr.g[4 + m], v.leaf[2 * m]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            gin[q][0] = tv[2 * q];
+            gin[q][1] = tv[2 * q + 1];
+        }
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            acc[4 * k + 0] = fma_t(gg[k], gin[k][0] * gin[k][1], acc[4 * k + 0]);
+            acc[4 * k + 1] = fma_t(gg[k], gin[k][0], acc[4 * k + 1]);
+            acc[4 * k + 2] = fma_t(gg[k], gin[k][1], acc[4 * k + 2]);
+            acc[4 * k + 3] += gg[k];
+        }
+    };
+    // rowbase[r]: LDS position of image row r = (sample, channel, iy) of a staged group (built once)
+    int *rowbase = reinterpret_cast<int *>(meet + kTiledWWaves * 28);
+    const uint32_t group_rows = (uint32_t)(p.S * g.cin * g.h), group_elems = group_rows * (uint32_t)g.w;
+    for (uint32_t r = tid; r < group_rows; r += nthreads) {
+        const uint32_t plane = fdiv(r, p.d_planes), iy = r - plane * (uint32_t)g.h;   // d_planes: division by h here
+        rowbase[r] = (int)(plane * p.chs + (iy + g.ph) * p.rs + g.pw);
+    }
+    T stage[kStagePerThread];
+    auto fetch = [&](int round) {                                     // image elements of a round's samples -> registers
+        const int n0 = ((int)blockIdx.x * rounds + round) * p.S;
+        const int s_here = n0 < g.n ? min(p.S, g.n - n0) : 0;
+        const uint32_t total = (uint32_t)(s_here * g.cin) * (uint32_t)hw;
+        const T *src = x + (int64_t)n0 * g.cin * hw;
+#pragma unroll
+        for (int k = 0; k < kStagePerThread; ++k) {
+            const uint32_t e = tid + k * nthreads;
+            stage[k] = T(0);
+            if (e < total) stage[k] = src[e];
+        }
+    };
+    // A lane takes V consecutive cells of a pooled row (V divides the row length), so one vector load brings the grad_y
+    // of V visits and one V-byte load their arg-max codes; the loads of the next group are in flight while the current
+    // one is evaluated, across round boundaries too (the kernel streams grad_y / arg-max from HBM).
+    struct Group {
+        T gout[V];
+        uint32_t codes;
+        int pos;
+    };
+    auto issue = [&](int round, int sb, Group &q) {
+        const int n0 = ((int)blockIdx.x * rounds + round) * p.S;
+        const int U = min(p.S, g.n - n0) * I;
+        const int u = (sb * kWave + lane) * V;
+        const uint32_t uu = u < U ? u : 0;
+        const uint32_t sm = fdiv(uu, p.d_slots), cl = uu - sm * (uint32_t)I;
+        const uint32_t py = fdiv(cl, p.d_wp), px = cl - py * (uint32_t)wp;
+        q.pos = (int)(sm * g.cin * p.chs + (2 * py * g.sh) * p.rs + 2 * px * g.sw);
+        q.codes = 0;
+#pragma unroll
+        for (int k = 0; k < V; ++k) q.gout[k] = T(0);
+        if (u < U) {
+            const int64_t o = ((int64_t)(n0 + sm) * g.c + c) * I + cl;
+            const T *gp = gy + o;
+            const uint8_t *ap = argmax + o;
+            if constexpr (V == 4) {
+                q.codes = *reinterpret_cast<const uint32_t *>(ap);
+                if constexpr (sizeof(T) == 4) {
+                    const float4 v = *reinterpret_cast<const float4 *>(gp);
+                    q.gout[0] = v.x, q.gout[1] = v.y, q.gout[2] = v.z, q.gout[3] = v.w;
+                } else {
+                    const double2 v0 = *reinterpret_cast<const double2 *>(gp), v1 = *reinterpret_cast<const double2 *>(gp + 2);
+                    q.gout[0] = v0.x, q.gout[1] = v0.y, q.gout[2] = v1.x, q.gout[3] = v1.y;
+                }
+            } else if constexpr (V == 2) {
+                q.codes = *reinterpret_cast<const uint16_t *>(ap);
+                if constexpr (sizeof(T) == 4) {
+                    const float2 v = *reinterpret_cast<const float2 *>(gp);
+                    q.gout[0] = v.x, q.gout[1] = v.y;
+                } else {
+                    const double2 v = *reinterpret_cast<const double2 *>(gp);
+                    q.gout[0] = v.x, q.gout[1] = v.y;
+                }
+            } else {
+                q.codes = *ap;
+                q.gout[0] = *gp;
+            }
+        }
+    };
+    Group cur, nxt;
+    bool have_cur = false;
+    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);          // halos stay zero over all rounds
+    fetch(0);
+    {
+        const int n_first = (int)blockIdx.x * rounds * p.S;           // grad_y of the first visits travels while the image is staged
+        have_cur = has_kernel && n_first < g.n && slice * kWave * V < min(p.S, g.n - n_first) * I;
+        if (have_cur) issue(0, slice, cur);
+    }
+    const int row_step = g.sh * p.rs;
+    for (int round = 0; round < rounds; ++round) {
+        const int n0 = ((int)blockIdx.x * rounds + round) * p.S;
+        if (n0 >= g.n) break;                                        // uniform over the workgroup
+        const int s_cur = min(p.S, g.n - n0);
+        __syncthreads();                                             // the previous round's reads (or the zero fill) are done
+#pragma unroll
+        for (int k = 0; k < kStagePerThread; ++k) {
+            const uint32_t e = tid + k * nthreads;
+            if (e < group_elems) {
+                const uint32_t r = fdiv(e, p.d_w);
+                xs[rowbase[r] + (int)(e - r * (uint32_t)g.w)] = stage[k];
+            }
+        }
+        __syncthreads();
+        if (round + 1 < rounds) fetch(round + 1);                    // in flight while this round is evaluated
+        if (!has_kernel) continue;
+        const int nsb = (s_cur * I + kWave * V - 1) / (kWave * V);
+        if (!have_cur && slice < nsb) issue(round, slice, cur);
+        for (int sb = slice; sb < nsb; sb += slices) {
+            // the next group of V visits: of this round, or the first one of the next round (its loads cross the barriers)
+            if (sb + slices < nsb) {
+                issue(round, sb + slices, nxt);
+            } else {
+                const int n1 = ((int)blockIdx.x * rounds + round + 1) * p.S;
+                have_cur = round + 1 < rounds && n1 < g.n && slice * kWave * V < min(p.S, g.n - n1) * I;
+                if (have_cur) issue(round + 1, slice, nxt);
+            }
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                const int code = (int)(cur.codes >> (8 * k)) & 3;
+                const int here = cur.pos + 2 * k * g.sw + (code >> 1) * row_step + (code & 1) * g.sw;
+                T tv[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) tv[t] = xs[here + to[t]];
+                accumulate(tv, cur.gout[k]);                         // lanes without a cell carry a zero gradient
+            }
+            cur = nxt;
+        }
+    }
+    if (!has_kernel) return;                                          // no workgroup barrier below
+    const int nb = gridDim.x * slices;                                // partial sums per kernel
+    T mine = T(0);                                                    // lane k < 28 ends up with total k
+#pragma unroll
+    for (int k = 0; k < 28; ++k) {
+        const T s = wave_sum(acc[k]);
+        mine = lane == k ? s : mine;
+    }
+    T *my_partial = partial + ((int64_t)c * nb + blockIdx.x * slices + slice) * 28;
+    if (lane < 28) my_partial[lane] = mine;
+    if (counter == nullptr) return;                                   // a reduce launch follows
+    // the wavefront that completes kernel c: partial sums in block order, coefficient transform, softmax backward
+    __threadfence();
+    int done = 0;
+    if (lane == 0) done = atomicAdd(counter + c, 1);
+    done = uniform(done);
+    if (done != nb - 1) return;
+    if (lane == 0) counter[c] = 0;                                    // ready for the next launch
+    __threadfence();
+    T total = T(0);
+    if (lane < 28) {
+        const T *pc = partial + (int64_t)c * nb * 28 + lane;
+        for (int b = 0; b < nb; ++b) total += __hip_atomic_load(pc + (int64_t)b * 28, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    T *mw = meet + wave * 28;                                         // private to this wavefront
+    if (lane < 28) mw[lane] = total;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int e = pass * kWave + lane;                            // output e = gate q, probability i
+        const int q = e >> 4, i = e & 15;
+        const bool ok = q < 7;
+        const T *sq = mw + (ok ? q : 0) * 4;
+        T gi = coef_transpose_row<T>(i, sq[0], sq[1], sq[2], sq[3]);
+        if (probs != nullptr) gi = softmax16_backward(gi, ok ? probs[(int64_t)c * 112 + e] : T(0));   // all lanes take part
+        if (ok) gw[(int64_t)c * 112 + e] = gi;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // plans
 // ---------------------------------------------------------------------------------------------
@@ -1030,6 +1256,90 @@ int launch_backward_w_shared(const Geom &g, const SharedPad &sh, const void *gy,
                                   "clg_convblock_backward_w(reduce)", probs);
 }
 
+// Plan of the LDS-staged weight gradient: S samples per staged group (their image elements travel through at most
+// kStagePerThread registers per thread), `rounds` groups per workgroup, nb = workgroups along the batch (= partial sums
+// per kernel, at most 64).
+struct TiledWPlan {
+    TilePlan p;
+    int rounds, nb;
+};
+bool plan_backward_w_tiled(const Geom &g, int elem, TiledWPlan *tw)
+{
+    if (const char *e = clg_knob(K_BWDW_LDS))
+        if (atoi(e) == 0) return false;
+    if (!taps_inside(g) || g.c > 65535) return false;
+    TilePlan *p = &tw->p;
+    plan_common(g, p);
+    const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
+    if (I < 1 || g.wo / 2 > 32768) return false;
+    p->slots = (int)I;
+    p->d_slots = make_fastdiv((uint32_t)I);
+    p->G = 1;
+    p->NW = kTiledWWaves;
+    const int64_t tail = g.ph * p->rs + g.pw;
+    const int64_t sample_elems = (int64_t)g.cin * g.h * g.w, sample_lds = (int64_t)g.cin * p->chs;
+    const int64_t stage_cap = (int64_t)kStagePerThread * kTiledWWaves * kWave;
+    int64_t S = stage_cap / sample_elems;                            // what the staging registers carry ...
+    const int64_t lds_cap = (96 * 1024 / elem - tail - kTiledWWaves * 28) / sample_lds;   // ... within 96 KiB of LDS
+    if (S > lds_cap) S = lds_cap;
+    if (S > g.n) S = g.n;
+    if (S > 64) S = 64;
+    if (S < 1) return false;
+    if (S * I < 48) return false;                                    // mostly empty wavefronts: the other kernels do better
+    // kernels per workgroup: 16 (one per wavefront), fewer for layers with few kernels (the wavefronts of a kernel
+    // then share its cells); rounds: at least 8 cell blocks per wavefront before its 28 reductions, at most 64 partial
+    // sums per kernel, and as many more as still leave one workgroup per CU (its 16 wavefronts fill the CU's vector
+    // registers; what a wavefront does once -- folding its kernel's coefficients, the 28 reductions -- costs as much
+    // as 7 visits, so long runs pay: 101 -> 76 us at [256,9,32,32] -> 256 from 4 to 16 rounds)
+    const int64_t groups = clg_ceil_div(g.n, S);
+    int64_t kw = kTiledWWaves;
+    while (kw > 4 && clg_ceil_div(g.c, kw) * groups < 1024) kw /= 2;
+    const int64_t slices = kTiledWWaves / kw, ktiles = clg_ceil_div(g.c, kw);
+    const int64_t blocks_per_round = clg_ceil_div(clg_ceil_div(S * I, kWave), slices);
+    int64_t R = clg_ceil_div(8, blocks_per_round);
+    while (clg_ceil_div(groups, R) * slices > 64) ++R;
+    while (R < groups && clg_ceil_div(groups, R + 1) * ktiles >= 256) ++R;
+    if (R > groups) R = groups;
+    if (clg_ceil_div(groups, R) * slices > 64) return false;
+    p->CT = (int)kw;
+    p->S = (int)S;
+    p->xe = (int)(S * sample_lds + tail);
+    p->d_planes = make_fastdiv((uint32_t)g.h);                        // image row -> (plane, iy)
+    p->lds_bytes = (size_t)(((p->xe + 3) & ~3) + kTiledWWaves * 28) * elem + (size_t)S * g.cin * g.h * 4;
+    if (p->lds_bytes > (size_t)kLdsLimit) return false;
+    tw->rounds = (int)R;
+    tw->nb = (int)clg_ceil_div(groups, R);                           // workgroups along the batch; partial sums per kernel = nb * slices
+    return S * sample_lds < (1ll << 30) && S * g.c * I < (1ll << 31) && (int64_t)g.n * g.c * I < (1ll << 62);
+}
+
+template <typename T>
+int launch_backward_w_tiled(const Geom &g, const TiledWPlan &tw, const void *gy, const void *x, const void *w, const int32_t *sel,
+                            const uint8_t *argmax, void *gw, void *scratch, int *counter, hipStream_t st, const void *probs)
+{
+    const dim3 grid((unsigned)tw.nb, (unsigned)clg_ceil_div(g.c, tw.p.CT)), block(kTiledWWaves * kWave);
+    const int nparts = tw.nb * (kTiledWWaves / tw.p.CT);
+    // cells per lane and load: 4 or 2 when they divide the pooled row length and the pointers are aligned for the vector loads
+    const int wp = g.wo / 2;
+    const uintptr_t gy_a = (uintptr_t)gy, am_a = (uintptr_t)argmax;
+    int v = 1;
+    if (wp % 4 == 0 && gy_a % (4 * sizeof(T)) == 0 && am_a % 4 == 0) v = 4;
+    else if (wp % 2 == 0 && gy_a % (2 * sizeof(T)) == 0 && am_a % 2 == 0) v = 2;
+#define CLG_BWDW_TILED(VV)                                                                                                        \
+    do {                                                                                                                          \
+        if (int e = allow_lds(convblock_backward_w_tiled_kernel<T, VV>, tw.p.lds_bytes, "clg_convblock_backward_w")) return e;    \
+        hipLaunchKernelGGL((convblock_backward_w_tiled_kernel<T, VV>), grid, block, tw.p.lds_bytes, st, (const T *)gy, (const T *)x, \
+                           (const T *)w, sel, argmax, (T *)scratch, counter, (T *)gw, (const T *)probs, g, tw.p, tw.rounds);      \
+    } while (0)
+    if (v == 4) CLG_BWDW_TILED(4);
+    else if (v == 2) CLG_BWDW_TILED(2);
+    else CLG_BWDW_TILED(1);
+#undef CLG_BWDW_TILED
+    CLG_CHECK_LAUNCH("clg_convblock_backward_w(tiled)");
+    if (counter != nullptr) return CLG_OK;
+    return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, scratch, gw, g.c, nparts, 7, st, "clg_convblock_backward_w(reduce)",
+                                  probs);
+}
+
 int elem_size(int dtype) { return dtype == CLG_F64 ? 8 : 4; }
 
 }  // namespace
@@ -1087,6 +1397,8 @@ PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void
     TilePlan pw;
     WScratch ws;
     const char *e_pad = clg_knob(K_BWDW_PADDED);
+    TiledWPlan tw;
+    if (!(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, (int)sizeof(T), &tw)) return no_pad_job<T>();   // that kernel stages x itself
     if (shared == nullptr || w_scratch == nullptr || p.bands != 1 || (e_pad && atoi(e_pad) == 0) || !plan_backward_w(g, (int)sizeof(T), &pw, &ws))
         return no_pad_job<T>();
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
@@ -1142,8 +1454,11 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
     if (clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_w_scratch_bytes")) return -1;
     TilePlan p;
     WScratch ws;
-    if (plan_backward_w(g, elem_size(dtype), &p, &ws)) return (int64_t)ws.total;
-    return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the any-shape kernel
+    TiledWPlan tw;
+    const char *e_pad = clg_knob(K_BWDW_PADDED);
+    const bool tiled = !(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, elem_size(dtype), &tw);
+    if (!tiled && plan_backward_w(g, elem_size(dtype), &p, &ws)) return (int64_t)ws.total;
+    return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the LDS-staged and the any-shape kernel
 }
 
 extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -1165,9 +1480,15 @@ static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const v
         if (dtype == CLG_F32) return launch_backward_w_shared<float>(g, *shared, grad_y, argmax, grad_w, scratch, clg_stream(stream), probs);
         return launch_backward_w_shared<double>(g, *shared, grad_y, argmax, grad_w, scratch, clg_stream(stream), probs);
     }
+    TiledWPlan tw;
+    const char *e_pad = clg_knob(K_BWDW_PADDED);
+    if (!(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, elem_size(dtype), &tw)) {     // images in LDS (CLG_BWDW_PADDED=1 forces the padded copy)
+        if (dtype == CLG_F32)
+            return launch_backward_w_tiled<float>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, nullptr, clg_stream(stream), probs);
+        return launch_backward_w_tiled<double>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, nullptr, clg_stream(stream), probs);
+    }
     TilePlan p;
     WScratch ws;
-    const char *e_pad = clg_knob(K_BWDW_PADDED);
     if ((!e_pad || atoi(e_pad) != 0) && plan_backward_w(g, elem_size(dtype), &p, &ws)) {
         if (dtype == CLG_F32)
             return launch_backward_w_padded<float>(g, p, ws, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
