@@ -77,37 +77,59 @@ class _FullConvLogicLogitsFunction(Function):
     (same values as softmax + FullConvLogicFunction up to rounding)."""
 
     @staticmethod
-    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
+    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False, plan=None):
         x1, selection, logits = x.contiguous(), selection.contiguous(), logits.contiguous()
         geo = (stride_h, stride_w, pad_h, pad_w)
         ctx.geometry, ctx.kernel = geo, (kernel_h, kernel_w)
+        ctx.plan = plan                                              # (plan bytes, signature) of the layer for this input shape, or None
         # y in memory as [C, Ho/2, Wo/2, N] where asked for and possible, handed out as the [N, C, Ho/2, Wo/2] view of it:
         # nn.Flatten and the LogicLayer behind it then work on that memory without a transposed copy, and so does the
         # way back
         fm = feature_major and convlogic_hip.feature_major_supported(x1, logits.shape[0], *geo, kernel_h, kernel_w)
+        ctx.feature_major = fm
+        if plan is not None:
+            # the forward launch also leaves the folded coefficients for the planned backward pass
+            y, argmax, w_prob, folded = convlogic_hip.full_convlogic_forward_logits(x1, logits.detach(), selection, *geo, kernel_h,
+                                                                                    kernel_w, feature_major=fm, want_folded=True,
+                                                                                    validate=False)
+            ctx.save_for_backward(x1, w_prob, selection, argmax, folded)
+            return y.permute(3, 0, 1, 2) if fm else y
+        ctx.plan = None
         y, argmax, w_prob = convlogic_hip.full_convlogic_forward_logits(x1, logits.detach(), selection, *geo, kernel_h, kernel_w,
-                                                                        feature_major=fm)
+                                                                        feature_major=fm, validate=False)
         ctx.save_for_backward(x1, w_prob, selection, argmax)
         return y.permute(3, 0, 1, 2) if fm else y
 
     @staticmethod
     def backward(ctx, grad_y):
-        x1, w_prob, selection, argmax = ctx.saved_tensors
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if ctx.plan is not None:
+            x1, w_prob, selection, argmax, folded = ctx.saved_tensors
+            if need_w:
+                ok = grad_y.dtype == x1.dtype and grad_y.device == x1.device      # everything else was validated on the way in
+                grad_fm = grad_y.permute(1, 2, 3, 0)
+                use_fm = ctx.feature_major and not grad_y.is_contiguous() and grad_fm.is_contiguous()
+                grad_x, grad_l = convlogic_hip.full_convlogic_backward_planned(grad_fm if use_fm else grad_y.contiguous(), x1, w_prob, folded,
+                                                                               argmax, selection, *ctx.plan, *ctx.geometry, need_grad_x=need_x,
+                                                                               validate=not ok, feature_major=use_fm)
+                return grad_x, grad_l, None, None, None, None, None, None, None, None, None
+            grad_x = convlogic_hip.full_convlogic_backward_x(grad_y.contiguous(), x1, w_prob, argmax, selection, *ctx.geometry) if need_x else None
+            return grad_x, None, None, None, None, None, None, None, None, None, None
+        x1, w_prob, selection, argmax = ctx.saved_tensors
         grad_x = grad_l = None
         grad_fm = grad_y.permute(1, 2, 3, 0)
         if (need_w and not grad_y.is_contiguous() and grad_fm.is_contiguous()
                 and convlogic_hip.feature_major_supported(x1, w_prob.shape[0], *ctx.geometry, *ctx.kernel)):
             grad_x, grad_l = convlogic_hip.full_convlogic_backward_fm(grad_fm, x1, w_prob, argmax, selection, *ctx.geometry,
-                                                                     need_grad_x=need_x)
-            return grad_x, grad_l, None, None, None, None, None, None, None, None
+                                                                     need_grad_x=need_x, validate=grad_y.dtype != x1.dtype or grad_y.device != x1.device)
+            return grad_x, grad_l, None, None, None, None, None, None, None, None, None
         grad_y = grad_y.contiguous()
         if need_w:
             grad_x, grad_l = convlogic_hip.full_convlogic_backward_logits(grad_y, x1, w_prob, argmax, selection, *ctx.geometry,
                                                                          need_grad_x=need_x)
         elif need_x:
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
-        return grad_x, grad_l, None, None, None, None, None, None, None, None
+        return grad_x, grad_l, None, None, None, None, None, None, None, None, None
 
 
 def _pair(v):
@@ -153,9 +175,9 @@ class ConvLogicLayer(nn.Module):
         column a tap names: a selection outside (in_channels, kernel) must raise here instead of faulting the GPU.
         Checked at construction, on the first launch and whenever the buffer was modified in place (version counter)
         or replaced; writes through `.data` bypass the counter -- call invalidate() after those."""
-        sel = self.selection
+        sel = self._buffers["selection"]                             # (not through nn.Module.__getattr__: taken on every call)
         key = (sel._version, sel.data_ptr())
-        if getattr(self, "_selection_checked", None) == key:
+        if self.__dict__.get("_selection_checked") == key:
             return
         if sel.dtype != torch.int32 or tuple(sel.shape) != (self.out_channels, 8):
             raise ValueError(f"selection must be int32 [{self.out_channels}, 8], got {sel.dtype} {tuple(sel.shape)}")
@@ -166,8 +188,25 @@ class ConvLogicLayer(nn.Module):
         self._selection_checked = key
 
     def invalidate(self):
-        """Forces the next call to check the selection buffer again (after a write through `.data`)."""
+        """Forces the next call to check the selection buffer again and to rebuild the backward plans (after a write
+        through `.data`)."""
         self._selection_checked = None
+        self._plans = {}
+
+    def _backward_plan(self, x, sel):
+        """(plan bytes, signature) of this layer's backward pass for inputs like x: the reverse map input channel ->
+        kernels and the tap offsets of the kernels' image layout, which depend only on the selection and the geometry.
+        Built on the first training step with a shape and kept (the reference's LogicLayer builds its reverse map at
+        construction, src/difflogic/difflogic.py:71-87); rebuilt when the selection buffer or the library's knobs change."""
+        from ..hip import _lib
+        key = (tuple(x.shape), x.dtype, x.device, sel._version, sel.data_ptr(), _lib.knob_generation())
+        plans = self.__dict__.setdefault("_plans", {})
+        plan = plans.get(key)
+        if plan is None:
+            if len(plans) >= 4:                                      # a few batch shapes (training, last partial batch, evaluation)
+                plans.pop(next(iter(plans)))
+            plan = plans[key] = convlogic_hip.make_backward_plan(x, self.out_channels, sel, *self.stride, *self.padding, *self.kernel)
+        return plan
 
     def _load_from_state_dict(self, *args, **kwargs):
         super()._load_from_state_dict(*args, **kwargs)
@@ -222,11 +261,14 @@ class ConvLogicLayer(nn.Module):
         if x.dim() != 4 or x.shape[1] != self.in_channels:          # the taps index channels of x without bounds checks
             raise RuntimeError(f"Expected x of shape [N, {self.in_channels}, H, W], got {tuple(x.shape)}")
         x = x.contiguous()
-        sel = self.selection.contiguous()
+        sel = self._buffers["selection"].contiguous()
+        weights = self._parameters["weights"]
         geo = (*self.stride, *self.padding, *self.kernel)
-        if (self.complete and self.training and not self.return_intermediate and not self.return_indices
-                and self.weights.dtype == x.dtype and self.weights.is_contiguous()):
-            return _FullConvLogicLogitsFunction.apply(x, self.weights, sel, *geo, getattr(self, "feature_major_output", False))
+        if (self.complete and self.training and not self.return_intermediate and not self.return_indices and x.is_cuda
+                and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64) and weights.is_contiguous()
+                and weights.device == x.device and sel.device == x.device):
+            return _FullConvLogicLogitsFunction.apply(x, weights, sel, *geo, self.__dict__.get("feature_major_output", False),
+                                                      self._backward_plan(x, sel))
         # the kernels read the probabilities in x's element type (the bindings reject any other)
         w_prob = gate_probabilities(self.weights, self.training, x.dtype).to(x.dtype).contiguous()
         if self.complete:

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
             taps[c * 16 + t] = tp.ch * chs + rel;
             taps[c * 16 + 8 + t] = rel;
         }
-        if (q < (int64_t)C * 7) {
+        if (w != nullptr && q < (int64_t)C * 7) {                    // (a plan is made without weights)
             const Coef<T> cf = fold16(w + q * 16);
             folded[q * 4 + 0] = cf.ab;
             folded[q * 4 + 1] = cf.a;
@@ -697,19 +697,19 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
 // The next group's image travels through registers while the current one is evaluated (at most kStagePerThread
 // elements per thread, LDS positions computed once).  Folded coefficients and tap offsets are made by the wavefront
 // itself from w and the selection: no set-up launch, no padded copy of x, every x element is read once per 16 kernels.
-// partial [c][gridDim.x][28]; with `counter` (one zeroed int per kernel, left zero again) the wavefront that
-// finishes a kernel last adds the partial sums in block order and writes the kernel's gradient itself (no reduce launch).
-constexpr int kStagePerThread = 10;
+// partial [c][partial sums per kernel][28], added in order by reduce_coef_partials_kernel.  (Letting the wavefront that
+// finishes a kernel last add them itself needs a device-wide release / acquire per wavefront, which on this multi-die
+// part writes the L2 back every time: 65 -> 160 us at [256,9,32,32] -> 256.)
+constexpr int kStagePerThread = 9;
 constexpr int kTiledWWaves = 16;
+constexpr int kTiledWMaxParts = 256;   // partial sums per kernel the scratch buffer holds
 template <typename T, int V>
 __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_tiled_kernel(
     const T *__restrict__ gy, const T *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ sel,
-    const uint8_t *__restrict__ argmax, T *__restrict__ partial, int *__restrict__ counter, T *__restrict__ gw,
-    const T *__restrict__ probs, Geom g, TilePlan p, int rounds)
+    const uint8_t *__restrict__ argmax, T *__restrict__ partial, Geom g, TilePlan p, int rounds)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     T *xs = reinterpret_cast<T *>(smem);
-    T *meet = xs + ((p.xe + 3) & ~3);                                 // [waves][28] exchange of the final sums
     const int tid = threadIdx.x;
     constexpr int nthreads = kTiledWWaves * kWave;
     const int lane = tid & (kWave - 1), wave = uniform(tid >> 6);
@@ -760,7 +760,7 @@ __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_til
         }
     };
     // rowbase[r]: LDS position of image row r = (sample, channel, iy) of a staged group (built once)
-    int *rowbase = reinterpret_cast<int *>(meet + kTiledWWaves * 28);
+    int *rowbase = reinterpret_cast<int *>(xs + ((p.xe + 3) & ~3));
     const uint32_t group_rows = (uint32_t)(p.S * g.cin * g.h), group_elems = group_rows * (uint32_t)g.w;
     for (uint32_t r = tid; r < group_rows; r += nthreads) {
         const uint32_t plane = fdiv(r, p.d_planes), iy = r - plane * (uint32_t)g.h;   // d_planes: division by h here
@@ -830,11 +830,6 @@ __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_til
     bool have_cur = false;
     for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);          // halos stay zero over all rounds
     fetch(0);
-    {
-        const int n_first = (int)blockIdx.x * rounds * p.S;           // grad_y of the first visits travels while the image is staged
-        have_cur = has_kernel && n_first < g.n && slice * kWave * V < min(p.S, g.n - n_first) * I;
-        if (have_cur) issue(0, slice, cur);
-    }
     const int row_step = g.sh * p.rs;
     for (int round = 0; round < rounds; ++round) {
         const int n0 = ((int)blockIdx.x * rounds + round) * p.S;
@@ -885,33 +880,6 @@ __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_til
     }
     T *my_partial = partial + ((int64_t)c * nb + blockIdx.x * slices + slice) * 28;
     if (lane < 28) my_partial[lane] = mine;
-    if (counter == nullptr) return;                                   // a reduce launch follows
-    // the wavefront that completes kernel c: partial sums in block order, coefficient transform, softmax backward
-    __threadfence();
-    int done = 0;
-    if (lane == 0) done = atomicAdd(counter + c, 1);
-    done = uniform(done);
-    if (done != nb - 1) return;
-    if (lane == 0) counter[c] = 0;                                    // ready for the next launch
-    __threadfence();
-    T total = T(0);
-    if (lane < 28) {
-        const T *pc = partial + (int64_t)c * nb * 28 + lane;
-        for (int b = 0; b < nb; ++b) total += __hip_atomic_load(pc + (int64_t)b * 28, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    T *mw = meet + wave * 28;                                         // private to this wavefront
-    if (lane < 28) mw[lane] = total;
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        const int e = pass * kWave + lane;                            // output e = gate q, probability i
-        const int q = e >> 4, i = e & 15;
-        const bool ok = q < 7;
-        const T *sq = mw + (ok ? q : 0) * 4;
-        T gi = coef_transpose_row<T>(i, sq[0], sq[1], sq[2], sq[3]);
-        if (probs != nullptr) gi = softmax16_backward(gi, ok ? probs[(int64_t)c * 112 + e] : T(0));   // all lanes take part
-        if (ok) gw[(int64_t)c * 112 + e] = gi;
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1136,16 +1104,55 @@ int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
     return CLG_OK;
 }
 
+// The tables of a per-layer plan (clg_convblock_plan): everything the gradient kernels need that depends only on the
+// selection and the geometry -- per-channel kernel lists and tap offsets -- and optionally the coefficients the forward
+// launch folded.
+struct PlanView {
+    const int32_t *count = nullptr, *hits = nullptr, *taps = nullptr;
+    const void *folded = nullptr;
+};
+// Where the gradient kernels of a call find their tables: in the call's scratch (written by the set-up launch) or in a plan.
+struct BwdTables {
+    const void *folded = nullptr;
+    const int32_t *count = nullptr, *hits = nullptr, *taps = nullptr;
+};
+// Sets a call's tables up.  Without a plan: one launch folds the coefficients, builds lists and tap offsets (and pads x
+// when `pad` names a job).  With a plan only what changes per step is left: folding (unless the forward launch did it)
+// and the padded copy -- no launch at all when neither is needed.
+template <typename T>
+int prepare_tables(const Geom &g, const BwdScratch &lay, int rs, int chs, const void *w, const int32_t *sel, void *scratch,
+                   hipStream_t st, const PadJob<T> &pad, const PlanView *pv, BwdTables *tb)
+{
+    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    if (pv == nullptr) {
+        tb->folded = base;
+        tb->count = reinterpret_cast<const int32_t *>(base + lay.count_off);
+        tb->hits = reinterpret_cast<const int32_t *>(base + lay.hits_off);
+        tb->taps = reinterpret_cast<const int32_t *>(base + lay.taps_off);
+        return launch_prepare<T>(g, lay, rs, chs, w, sel, scratch, st, pad);
+    }
+    const bool fold = pv->folded == nullptr;
+    tb->folded = fold ? (const void *)base : pv->folded;
+    tb->count = pv->count, tb->hits = pv->hits, tb->taps = pv->taps;
+    if (!fold && pad.total == 0) return CLG_OK;
+    const unsigned prep = fold ? (unsigned)clg_ceil_div((int64_t)g.c * 7, 256) : 0u;
+    hipLaunchKernelGGL((convblock_w_prepare_kernel<T, T>), dim3(prep + pad_blocks(pad)), dim3(256), 0, st, (const T *)w, sel,
+                       fold ? reinterpret_cast<T *>(base) : (T *)nullptr, (int32_t *)nullptr, g.c, 0, 0, pad, (int)prep);
+    CLG_CHECK_LAUNCH("clg_convblock_backward_planned(fold / pad)");
+    return CLG_OK;
+}
+
 template <typename T>
 int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, const void *x, const void *w, const int32_t *sel,
-                            const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, const PadJob<T> &pad)
+                            const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, const PadJob<T> &pad,
+                            const PlanView *pv = nullptr, BwdTables *tables_out = nullptr)
 {
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
-    T *folded = reinterpret_cast<T *>(scratch);
-    int32_t *count = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.count_off);
-    int32_t *hits = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.hits_off);
-    int32_t *taps = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(scratch) + lay.taps_off);
-    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, pad)) return e;
+    BwdTables tb;
+    if (int e = prepare_tables<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, pad, pv, &tb)) return e;
+    if (tables_out != nullptr) *tables_out = tb;
+    const T *folded = reinterpret_cast<const T *>(tb.folded);
+    const int32_t *count = tb.count, *hits = tb.hits, *taps = tb.taps;
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
     T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
     T *out = p.hit_split > 1 ? part : (T *)gx;
@@ -1182,26 +1189,27 @@ struct SharedPad {
 
 template <typename T>
 int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems, const void *gy, const void *x, const void *w,
-                             const int32_t *sel, const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, SharedPad *shared)
+                             const int32_t *sel, const uint8_t *argmax, void *gx, void *scratch, hipStream_t st, SharedPad *shared,
+                             const PlanView *pv = nullptr)
 {
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     T *xp = reinterpret_cast<T *>(base + bwd_x_direct_xp_off(lay));
+    BwdTables tb;
+    if (int e = prepare_tables<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems), pv, &tb))
+        return e;
     if (shared != nullptr) {
         shared->xp = xp;
-        shared->folded = base;
-        shared->taps = reinterpret_cast<const int32_t *>(base + lay.taps_off);
+        shared->folded = tb.folded;
+        shared->taps = tb.taps;
         shared->sample_elems = sample_elems;
         shared->p = p;
     }
-    if (int e = launch_prepare<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems)))
-        return e;
     if (int e = allow_lds(convblock_backward_x_direct_kernel<T>, p.lds_bytes, "clg_convblock_backward_x")) return e;
     const int64_t items = clg_ceil_div(g.n, p.G) * g.cin;
     hipLaunchKernelGGL(convblock_backward_x_direct_kernel<T>, dim3((unsigned)clg_ceil_div(items, p.NW)), dim3(p.NW * kWave),
-                       p.lds_bytes, st, (const T *)gy, (const T *)xp, reinterpret_cast<const T *>(base),
-                       reinterpret_cast<const int32_t *>(base + lay.count_off), reinterpret_cast<const int32_t *>(base + lay.hits_off),
-                       reinterpret_cast<const int32_t *>(base + lay.taps_off), argmax, (T *)gx, g, p, sample_elems);
+                       p.lds_bytes, st, (const T *)gy, (const T *)xp, reinterpret_cast<const T *>(tb.folded), tb.count, tb.hits, tb.taps,
+                       argmax, (T *)gx, g, p, sample_elems);
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(direct)");
     return CLG_OK;
 }
@@ -1257,8 +1265,8 @@ int launch_backward_w_shared(const Geom &g, const SharedPad &sh, const void *gy,
 }
 
 // Plan of the LDS-staged weight gradient: S samples per staged group (their image elements travel through at most
-// kStagePerThread registers per thread), `rounds` groups per workgroup, nb = workgroups along the batch (= partial sums
-// per kernel, at most 64).
+// kStagePerThread registers per thread), `rounds` groups per workgroup, nb = workgroups along the batch (partial sums
+// per kernel = nb x wavefronts per kernel, at most kTiledWMaxParts).
 struct TiledWPlan {
     TilePlan p;
     int rounds, nb;
@@ -1280,14 +1288,14 @@ bool plan_backward_w_tiled(const Geom &g, int elem, TiledWPlan *tw)
     const int64_t sample_elems = (int64_t)g.cin * g.h * g.w, sample_lds = (int64_t)g.cin * p->chs;
     const int64_t stage_cap = (int64_t)kStagePerThread * kTiledWWaves * kWave;
     int64_t S = stage_cap / sample_elems;                            // what the staging registers carry ...
-    const int64_t lds_cap = (96 * 1024 / elem - tail - kTiledWWaves * 28) / sample_lds;   // ... within 96 KiB of LDS
+    const int64_t lds_cap = (96 * 1024 / elem - tail) / sample_lds;   // ... within 96 KiB of LDS
     if (S > lds_cap) S = lds_cap;
     if (S > g.n) S = g.n;
     if (S > 64) S = 64;
     if (S < 1) return false;
-    if (S * I < 48) return false;                                    // mostly empty wavefronts: the other kernels do better
+    if (S * I < 2 * kWave) return false;                             // under two blocks of cells per staged group: the other kernels do better
     // kernels per workgroup: 16 (one per wavefront), fewer for layers with few kernels (the wavefronts of a kernel
-    // then share its cells); rounds: at least 8 cell blocks per wavefront before its 28 reductions, at most 64 partial
+    // then share its cells); rounds: at least 8 cell blocks per wavefront before its 28 reductions, at most 256 partial
     // sums per kernel, and as many more as still leave one workgroup per CU (its 16 wavefronts fill the CU's vector
     // registers; what a wavefront does once -- folding its kernel's coefficients, the 28 reductions -- costs as much
     // as 7 visits, so long runs pay: 101 -> 76 us at [256,9,32,32] -> 256 from 4 to 16 rounds)
@@ -1297,15 +1305,15 @@ bool plan_backward_w_tiled(const Geom &g, int elem, TiledWPlan *tw)
     const int64_t slices = kTiledWWaves / kw, ktiles = clg_ceil_div(g.c, kw);
     const int64_t blocks_per_round = clg_ceil_div(clg_ceil_div(S * I, kWave), slices);
     int64_t R = clg_ceil_div(8, blocks_per_round);
-    while (clg_ceil_div(groups, R) * slices > 64) ++R;
+    while (clg_ceil_div(groups, R) * slices > kTiledWMaxParts) ++R;
     while (R < groups && clg_ceil_div(groups, R + 1) * ktiles >= 256) ++R;
     if (R > groups) R = groups;
-    if (clg_ceil_div(groups, R) * slices > 64) return false;
+    if (clg_ceil_div(groups, R) * slices > kTiledWMaxParts) return false;
     p->CT = (int)kw;
     p->S = (int)S;
     p->xe = (int)(S * sample_lds + tail);
     p->d_planes = make_fastdiv((uint32_t)g.h);                        // image row -> (plane, iy)
-    p->lds_bytes = (size_t)(((p->xe + 3) & ~3) + kTiledWWaves * 28) * elem + (size_t)S * g.cin * g.h * 4;
+    p->lds_bytes = (size_t)((p->xe + 3) & ~3) * elem + (size_t)S * g.cin * g.h * 4;
     if (p->lds_bytes > (size_t)kLdsLimit) return false;
     tw->rounds = (int)R;
     tw->nb = (int)clg_ceil_div(groups, R);                           // workgroups along the batch; partial sums per kernel = nb * slices
@@ -1314,28 +1322,28 @@ bool plan_backward_w_tiled(const Geom &g, int elem, TiledWPlan *tw)
 
 template <typename T>
 int launch_backward_w_tiled(const Geom &g, const TiledWPlan &tw, const void *gy, const void *x, const void *w, const int32_t *sel,
-                            const uint8_t *argmax, void *gw, void *scratch, int *counter, hipStream_t st, const void *probs)
+                            const uint8_t *argmax, void *gw, void *scratch, hipStream_t st, const void *probs)
 {
     const dim3 grid((unsigned)tw.nb, (unsigned)clg_ceil_div(g.c, tw.p.CT)), block(kTiledWWaves * kWave);
     const int nparts = tw.nb * (kTiledWWaves / tw.p.CT);
     // cells per lane and load: 4 or 2 when they divide the pooled row length and the pointers are aligned for the vector loads
     const int wp = g.wo / 2;
     const uintptr_t gy_a = (uintptr_t)gy, am_a = (uintptr_t)argmax;
-    int v = 1;
-    if (wp % 4 == 0 && gy_a % (4 * sizeof(T)) == 0 && am_a % 4 == 0) v = 4;
-    else if (wp % 2 == 0 && gy_a % (2 * sizeof(T)) == 0 && am_a % 2 == 0) v = 2;
+    const int64_t group_cells = (int64_t)tw.p.S * (g.ho / 2) * wp, lanes_needed = (int64_t)kWave * (kTiledWWaves / tw.p.CT);
+    int v = 1;                                                       // (wide loads only while they leave the wavefronts of a kernel full)
+    if (wp % 4 == 0 && gy_a % (4 * sizeof(T)) == 0 && am_a % 4 == 0 && group_cells >= 4 * lanes_needed) v = 4;
+    else if (wp % 2 == 0 && gy_a % (2 * sizeof(T)) == 0 && am_a % 2 == 0 && group_cells >= 2 * lanes_needed) v = 2;
 #define CLG_BWDW_TILED(VV)                                                                                                        \
     do {                                                                                                                          \
         if (int e = allow_lds(convblock_backward_w_tiled_kernel<T, VV>, tw.p.lds_bytes, "clg_convblock_backward_w")) return e;    \
         hipLaunchKernelGGL((convblock_backward_w_tiled_kernel<T, VV>), grid, block, tw.p.lds_bytes, st, (const T *)gy, (const T *)x, \
-                           (const T *)w, sel, argmax, (T *)scratch, counter, (T *)gw, (const T *)probs, g, tw.p, tw.rounds);      \
+                           (const T *)w, sel, argmax, (T *)scratch, g, tw.p, tw.rounds);                                          \
     } while (0)
     if (v == 4) CLG_BWDW_TILED(4);
     else if (v == 2) CLG_BWDW_TILED(2);
     else CLG_BWDW_TILED(1);
 #undef CLG_BWDW_TILED
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(tiled)");
-    if (counter != nullptr) return CLG_OK;
     return clg_launch_reduce_coef(sizeof(T) == 8 ? CLG_F64 : CLG_F32, scratch, gw, g.c, nparts, 7, st, "clg_convblock_backward_w(reduce)",
                                   probs);
 }
@@ -1392,7 +1400,7 @@ extern "C" int64_t clg_convblock_backward_x_scratch_bytes(int dtype, const clg_c
 // also writes the padded copy (planes of p.chs elements, the layout its tap offsets are made for) into the weight
 // gradient's scratch, so that one neither folds nor computes tap offsets nor pads again.
 template <typename T>
-PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void *scratch, void *w_scratch, SharedPad *shared)
+PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void *w_scratch, SharedPad *shared)
 {
     TilePlan pw;
     WScratch ws;
@@ -1401,13 +1409,9 @@ PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void
     if (!(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, (int)sizeof(T), &tw)) return no_pad_job<T>();   // that kernel stages x itself
     if (shared == nullptr || w_scratch == nullptr || p.bands != 1 || (e_pad && atoi(e_pad) == 0) || !plan_backward_w(g, (int)sizeof(T), &pw, &ws))
         return no_pad_job<T>();
-    const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), p.hit_split);
-    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     const int sample_elems = g.cin * p.chs + g.ph * p.rs + g.pw;
     T *xp = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(w_scratch) + ws.xp_off);
-    shared->xp = xp;
-    shared->folded = base;
-    shared->taps = reinterpret_cast<const int32_t *>(base + lay.taps_off);
+    shared->xp = xp;                                                  // folded / taps: filled in from the call's tables
     shared->sample_elems = sample_elems;
     shared->p = pw;
     return make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems);
@@ -1415,7 +1419,7 @@ PadJob<T> share_from_tiled(const Geom &g, const TilePlan &p, const void *x, void
 
 static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
                                      const int32_t *selection, const uint8_t *argmax, void *grad_x, void *scratch, void *stream,
-                                     SharedPad *shared, void *w_scratch = nullptr)
+                                     SharedPad *shared, void *w_scratch = nullptr, const PlanView *pv = nullptr)
 {
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_backward_x")) return e;
@@ -1425,27 +1429,34 @@ static int convblock_backward_x_impl(int dtype, const clg_conv_geom *gg, const v
     const BwdXMode mode = choose_backward_x(g, elem_size(dtype), &p, &se);
     hipStream_t st = clg_stream(stream);
     if (mode == kBwdXTiled) {
+        BwdTables tb;
+        int e;
         if (dtype == CLG_F32)
-            return launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
-                                                  share_from_tiled<float>(g, p, x, scratch, w_scratch, shared));
-        return launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
-                                               share_from_tiled<double>(g, p, x, scratch, w_scratch, shared));
+            e = launch_backward_x_tiled<float>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
+                                               share_from_tiled<float>(g, p, x, w_scratch, shared), pv, &tb);
+        else
+            e = launch_backward_x_tiled<double>(g, p, grad_y, x, w, selection, argmax, grad_x, scratch, st,
+                                                share_from_tiled<double>(g, p, x, w_scratch, shared), pv, &tb);
+        if (shared != nullptr && shared->xp != nullptr) {
+            shared->folded = tb.folded;
+            shared->taps = tb.taps;
+        }
+        return e;
     }
     if (mode == kBwdXDirect) {
         if (dtype == CLG_F32)
-            return launch_backward_x_direct<float>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared);
-        return launch_backward_x_direct<double>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared);
+            return launch_backward_x_direct<float>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared, pv);
+        return launch_backward_x_direct<double>(g, p, se, grad_y, x, w, selection, argmax, grad_x, scratch, st, shared, pv);
     }
     // any other shape: per-element gather driven by the same per-channel kernel lists
     const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
-    unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
+    BwdTables tb;
     if (dtype == CLG_F32) {
-        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>())) return e;
+        if (int e = prepare_tables<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>(), pv, &tb)) return e;
     } else {
-        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>())) return e;
+        if (int e = prepare_tables<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>(), pv, &tb)) return e;
     }
-    return clg_convblock_backward_x_generic(dtype, g, grad_y, x, scratch, reinterpret_cast<const int32_t *>(base + lay.count_off),
-                                            reinterpret_cast<const int32_t *>(base + lay.hits_off), selection, argmax, grad_x, st);
+    return clg_convblock_backward_x_generic(dtype, g, grad_y, x, tb.folded, tb.count, tb.hits, selection, argmax, grad_x, st);
 }
 
 extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_conv_geom *gg)
@@ -1458,7 +1469,8 @@ extern "C" int64_t clg_convblock_backward_w_scratch_bytes(int dtype, const clg_c
     const char *e_pad = clg_knob(K_BWDW_PADDED);
     const bool tiled = !(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, elem_size(dtype), &tw);
     if (!tiled && plan_backward_w(g, elem_size(dtype), &p, &ws)) return (int64_t)ws.total;
-    return (int64_t)g.c * 64 * 28 * elem_size(dtype);              // partial sums of the LDS-staged and the any-shape kernel
+    // partial sums of the LDS-staged (at most 256 per kernel) and of the any-shape kernel (at most 64)
+    return (int64_t)g.c * (tiled ? kTiledWMaxParts : 64) * 28 * elem_size(dtype);
 }
 
 extern "C" int clg_convblock_backward_x(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
@@ -1484,8 +1496,8 @@ static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const v
     const char *e_pad = clg_knob(K_BWDW_PADDED);
     if (!(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, elem_size(dtype), &tw)) {     // images in LDS (CLG_BWDW_PADDED=1 forces the padded copy)
         if (dtype == CLG_F32)
-            return launch_backward_w_tiled<float>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, nullptr, clg_stream(stream), probs);
-        return launch_backward_w_tiled<double>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, nullptr, clg_stream(stream), probs);
+            return launch_backward_w_tiled<float>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
+        return launch_backward_w_tiled<double>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
     }
     TilePlan p;
     WScratch ws;
@@ -1515,20 +1527,20 @@ static size_t backward_4x4_tg_off(const Geom &g, int dtype) { return (bwd_scratc
 
 static int convblock_backward_4x4(int dtype, const Geom &g, const void *grad_y, const void *x, const void *w, const int32_t *selection,
                                   const uint8_t *argmax, void *grad_x, void *grad_w, void *scratch, void *stream, const void *probs,
-                                  const char *name)
+                                  const char *name, const PlanView *pv = nullptr)
 {
     CLG_REQUIRE(grad_y && x && w && selection && argmax && grad_w && scratch, "%s: null pointer argument", name);
     const BwdScratch lay = bwd_scratch_layout(g, elem_size(dtype), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     hipStream_t st = clg_stream(stream);
+    BwdTables tb;
     if (dtype == CLG_F32) {
-        if (int e = launch_prepare<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>())) return e;
+        if (int e = prepare_tables<float>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<float>(), pv, &tb)) return e;
     } else {
-        if (int e = launch_prepare<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>())) return e;
+        if (int e = prepare_tables<double>(g, lay, 0, 0, w, selection, scratch, st, no_pad_job<double>(), pv, &tb)) return e;
     }
-    return clg_convblock_backward_4x4(dtype, g, x, base, selection, grad_y, argmax, base + backward_4x4_tg_off(g, dtype), grad_w, probs,
-                                      reinterpret_cast<const int32_t *>(base + lay.count_off),
-                                      reinterpret_cast<const int32_t *>(base + lay.hits_off), grad_x, st, name);
+    return clg_convblock_backward_4x4(dtype, g, x, tb.folded, selection, grad_y, argmax, base + backward_4x4_tg_off(g, dtype), grad_w, probs,
+                                      tb.count, tb.hits, grad_x, st, name);
 }
 
 extern "C" int64_t clg_convblock_backward_scratch_bytes(int dtype, const clg_conv_geom *gg)
@@ -1604,4 +1616,100 @@ extern "C" int clg_convblock_backward_logits(int dtype, const clg_conv_geom *gg,
             return e;
     return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_logits, w_scratch, stream, w,
                                      "clg_convblock_backward_logits", &shared);
+}
+
+// ---- per-layer plan --------------------------------------------------------------------------------
+// plan = BwdScratch layout without partial images: (folded: unused) | count | cursor | hits | unsorted | taps
+namespace {
+struct PlanInfo {
+    BwdScratch lay;
+    int rs, chs;
+    size_t total;
+    int64_t signature;
+};
+PlanInfo plan_info(const Geom &g, int dtype)
+{
+    PlanInfo pi;
+    const int elem = elem_size(dtype);
+    int mode = 3, rs = 0, chs = 0;                                    // 3: one sample per lane on 4x4 images
+    if (!backward_4x4_wanted(g)) {
+        TilePlan p;
+        int se = 0;
+        mode = (int)choose_backward_x(g, elem, &p, &se);
+        if (mode != kBwdXGather) rs = p.rs, chs = p.chs;
+    }
+    pi.lay = bwd_scratch_layout(g, elem, 1);
+    pi.rs = rs, pi.chs = chs;
+    pi.total = pi.lay.part_off;
+    // what the tables were made for: a plan is rejected when geometry, element type or the path choice differ
+    const int64_t fields[] = {mode, rs, chs, pi.lay.csr, elem, g.n, g.cin, g.h, g.w, g.c, g.sh, g.sw, g.ph, g.pw, g.kh, g.kw};
+    uint64_t h = 1469598103934665603ull;
+    for (int64_t f : fields) {
+        h ^= (uint64_t)f;
+        h *= 1099511628211ull;
+    }
+    pi.signature = (int64_t)(h & 0x7fffffffffffffffull);
+    return pi;
+}
+}  // namespace
+
+extern "C" int64_t clg_convblock_plan_bytes(int dtype, const clg_conv_geom *gg)
+{
+    Geom g;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_plan_bytes")) return -1;
+    return (int64_t)plan_info(g, dtype).total;
+}
+
+extern "C" int clg_convblock_plan(int dtype, const clg_conv_geom *gg, const int32_t *selection, void *plan, int64_t *signature,
+                                  void *stream)
+{
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, "clg_convblock_plan")) return e;
+    CLG_REQUIRE(selection && plan && signature, "clg_convblock_plan: null pointer argument");
+    const PlanInfo pi = plan_info(g, dtype);
+    hipStream_t st = clg_stream(stream);
+    // lists and tap offsets by the set-up launch of the unplanned path (no weights: nothing is folded)
+    if (dtype == CLG_F32) {
+        if (int e = launch_prepare<float>(g, pi.lay, pi.rs, pi.chs, nullptr, selection, plan, st, no_pad_job<float>())) return e;
+    } else {
+        if (int e = launch_prepare<double>(g, pi.lay, pi.rs, pi.chs, nullptr, selection, plan, st, no_pad_job<double>())) return e;
+    }
+    *signature = pi.signature;
+    return CLG_OK;
+}
+
+extern "C" int clg_convblock_backward_planned(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                              const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
+                                              int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream)
+{
+    const char *name = "clg_convblock_backward_planned";
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
+    CLG_REQUIRE(grad_y && x && w && selection && argmax && plan && grad_w && scratch, "%s: null pointer argument", name);
+    CLG_REQUIRE((flags & ~(CLG_BWD_WRT_LOGITS | CLG_BWD_GY_FEATURE_MAJOR)) == 0, "%s: unknown flags 0x%x", name, flags);
+    const bool wrt_logits = (flags & CLG_BWD_WRT_LOGITS) != 0, fm = (flags & CLG_BWD_GY_FEATURE_MAJOR) != 0;
+    CLG_REQUIRE(!fm || clg_convblock_fm_supported(dtype, gg), "%s: CLG_BWD_GY_FEATURE_MAJOR needs a shape for which "
+                "clg_convblock_fm_supported() holds (4x4 images, 3x3 kernel, stride 1, padding 1, n >= 32)", name);
+    const PlanInfo pi = plan_info(g, dtype);
+    CLG_REQUIRE(signature == pi.signature, "%s: the plan was made for another geometry, element type or kernel choice (make a new one "
+                "with clg_convblock_plan; the CLG_* knobs are part of the choice)", name);
+    unsigned char *pb = reinterpret_cast<unsigned char *>(plan);
+    PlanView pv;
+    pv.count = reinterpret_cast<const int32_t *>(pb + pi.lay.count_off);
+    pv.hits = reinterpret_cast<const int32_t *>(pb + pi.lay.hits_off);
+    pv.taps = reinterpret_cast<const int32_t *>(pb + pi.lay.taps_off);
+    pv.folded = folded;
+    const void *probs = wrt_logits ? w : nullptr;
+    if (backward_4x4_wanted(g)) {
+        g.y_fm = fm ? 1 : 0;
+        return convblock_backward_4x4(dtype, g, grad_y, x, w, selection, argmax, grad_x, grad_w, scratch, stream, probs, name, &pv);
+    }
+    const int64_t a = clg_convblock_backward_x_scratch_bytes(dtype, gg);
+    if (a < 0) return CLG_EINVAL;
+    SharedPad shared;
+    void *w_scratch = reinterpret_cast<unsigned char *>(scratch) + ((a + 255) & ~255ll);
+    if (grad_x != nullptr)
+        if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared, w_scratch, &pv))
+            return e;
+    return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w, w_scratch, stream, probs, name, &shared);
 }

@@ -125,6 +125,12 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
         }
     }
     __syncthreads();
+    if constexpr (Ops::kParams == 28) {                              // float gates: the folded coefficients for the backward pass
+        if (p.folded_out != nullptr && blockIdx.x == 0) {
+            T *fo = reinterpret_cast<T *>(p.folded_out) + (int64_t)c0 * 28;
+            for (int i = tid; i < ct_cur * 28; i += nthreads) fo[i] = coef[i];
+        }
+    }
 
     const int row_step = ROWSTEP ? ROWSTEP : g.sh * p.rs;
     // lanes that pool and write: even columns, and with one position per lane even rows only
@@ -662,9 +668,11 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
     CLG_REQUIRE(x && w && selection && y && argmax, "%s: null pointer argument", name);
-    CLG_REQUIRE((flags & ~(CLG_FWD_W_LOGITS | CLG_FWD_Y_FEATURE_MAJOR)) == 0, "%s: unknown flags 0x%x", name, flags);
+    CLG_REQUIRE((flags & ~(CLG_FWD_W_LOGITS | CLG_FWD_Y_FEATURE_MAJOR | CLG_FWD_FOLDED_OUT)) == 0, "%s: unknown flags 0x%x", name, flags);
     const bool logits = (flags & CLG_FWD_W_LOGITS) != 0, fm = (flags & CLG_FWD_Y_FEATURE_MAJOR) != 0;
+    const bool want_folded = (flags & CLG_FWD_FOLDED_OUT) != 0;
     CLG_REQUIRE(!logits || probs_out, "%s: CLG_FWD_W_LOGITS needs probs_out [c_out, 7, 16]", name);
+    CLG_REQUIRE(!want_folded || probs_out, "%s: CLG_FWD_FOLDED_OUT needs probs_out with room for [c_out, 7, 16] + [c_out, 7, 4]", name);
     CLG_REQUIRE(!fm || (scratch && clg_convblock_fm_supported(dtype, gg)), "%s: CLG_FWD_Y_FEATURE_MAJOR needs scratch and a shape for "
                 "which clg_convblock_fm_supported() holds (4x4 images, 3x3 kernel, stride 1, padding 1, n >= 32)", name);
     TilePlan tp;
@@ -672,24 +680,41 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     const int elem = dtype == CLG_F64 ? 8 : 4;
     const int path = fm ? 4 : choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp);
     hipStream_t st = clg_stream(stream);
+    // the folded coefficients [c_out, 7, 4] follow the probabilities in probs_out
+    void *folded_out = want_folded ? reinterpret_cast<unsigned char *>(probs_out) + (size_t)g.c * 112 * elem : nullptr;
+    // paths whose kernels do not write them themselves: one small launch folds the probabilities (after the forward launches)
+    auto fold_after = [&](int e) {
+        if (e != CLG_OK || !want_folded) return e;
+        const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
+        const void *pr = logits ? probs_out : w;
+        if (dtype == CLG_F32)
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)pr, selection,
+                               (float *)folded_out, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
+        else
+            hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)pr, selection,
+                               (double *)folded_out, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
+        CLG_CHECK_LAUNCH(name);
+        return CLG_OK;
+    };
     if (path == 4) {
         g.y_fm = fm ? 1 : 0;
+        void *fold_to = want_folded ? folded_out : scratch;             // the 4x4 kernels read them from wherever they are
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
-                               (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
+                               (float *)fold_to, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
                                (float *)probs_out);
         else
             hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
-                               (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
+                               (double *)fold_to, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
                                (double *)probs_out);
         CLG_CHECK_LAUNCH(name);
-        return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, name);
+        return clg_convblock_forward_4x4(dtype, g, x, fold_to, selection, y, argmax, st, name);
     }
     if (path == 2) {
         if (dtype == CLG_F32)
-            return launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
-        return launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out);
+            return fold_after(launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out));
+        return fold_after(launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out));
     }
     // The staged kernels take the softmax per workgroup while they set their gate parameters up, as long as that is at
     // most two rows of 16 logits per thread (C3 graph step 66.7 -> 63.7 us against a small launch of its own; with the
@@ -711,10 +736,11 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     }
     if (staged) {
         tp.w_logits = in_kernel ? 1 : 0;
+        tp.folded_out = folded_out;                                  // written by the first sample block of every kernel tile
         if (dtype == CLG_F32) return launch_forward_tiled<FloatOps<float>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
         return launch_forward_tiled<FloatOps<double>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
     }
-    return clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, st);
+    return fold_after(clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, st));
 }
 
 // Which shapes the feature-major variants take: the one-sample-per-lane kernels for 4x4 images (conv_small.hip).

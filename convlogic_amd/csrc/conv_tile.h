@@ -37,6 +37,7 @@ struct TilePlan {
     int subset;            // forward: 1 = only the channels the kernel tile reads are staged
     int one_row;           // forward: 1 = a lane slot is one conv position (ho * wo per sample) instead of a column of two rows
     int w_logits;          // forward: 1 = the gate parameters handed to the kernel are logits (softmax taken while staging them)
+    void *folded_out = nullptr;   // forward: where the first sample block writes the folded coefficients [c, 7, 4] of its kernels (or null)
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp, d_planes;
     size_t lds_bytes;
 };

@@ -92,15 +92,17 @@ class LogicLayer(torch.nn.Module):
             assert x.is_cuda, f"x must be a CUDA tensor, got device: {x.device}"
         assert x.ndim == 2, x.ndim
         assert x.shape[1] == self.in_dim, (tuple(x.shape[::-1]), self.in_dim)
-        self._check_wiring()
-        if (self.training and self.weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
-                and self.weights.is_contiguous()):
+        key = self._wiring_key()
+        self._check_wiring(key)
+        weights, buffers = self._parameters["weights"], self._buffers
+        if (self.training and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
+                and weights.is_contiguous() and weights.device == x.device):
             # a sample-major batch is transposed inside the Function (and its gradient on the way back): one autograd
             # node per layer instead of two
             inside = _transposes_with_kernel(x)
-            return _LogicLayerLogitsFunction.apply(x if inside else _feature_major(x), self.indices_0, self.indices_1,
-                                                   self.weights, self.given_x_indices_of_y_start,
-                                                   self.given_x_indices_of_y, self._sole_consumers(), inside).transpose(0, 1)
+            return _LogicLayerLogitsFunction.apply(x if inside else _feature_major(x), buffers["indices_0"], buffers["indices_1"],
+                                                   weights, buffers["given_x_indices_of_y_start"],
+                                                   buffers["given_x_indices_of_y"], self._sole_consumers(key), inside).transpose(0, 1)
         xt = _feature_major(x)
         w = self._gate_weights(xt.dtype)
         args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
@@ -124,20 +126,31 @@ class LogicLayer(torch.nn.Module):
         return difflogic_hip.gate_argmax(self.weights.detach())
 
     def _wiring_key(self):
-        return (self.indices_0._version, self.indices_1._version, self.indices_0.data_ptr(), self.indices_1.data_ptr())
+        # (buffers and parameters straight from their dicts: nn.Module.__getattr__ costs a microsecond per lookup, and
+        # this key is taken on every call)
+        a, b = self._buffers["indices_0"], self._buffers["indices_1"]
+        return (a._version, b._version, a.data_ptr(), b.data_ptr(), self._parameters["weights"].device)
 
-    def _check_wiring(self):
+    def _check_wiring(self, key=None):
         """The kernels index x with indices_0 / indices_1 without bounds checks: an index outside [0, in_dim) must
         raise here instead of faulting the GPU.  Checked on the first launch and again whenever the buffers were
         modified in place (version counter) or replaced; writes through `.data` bypass the counter -- call
         invalidate() after those."""
-        key = self._wiring_key()
-        if getattr(self, "_wiring_checked", None) != key:
+        key = key or self._wiring_key()
+        if self.__dict__.get("_wiring_checked") != key:
             for name, idx in (("indices_0", self.indices_0), ("indices_1", self.indices_1)):
                 if idx.dtype != torch.int64 or tuple(idx.shape) != (self.out_dim,):
                     raise ValueError(f"{name} must be int64 [{self.out_dim}], got {idx.dtype} {tuple(idx.shape)}")
                 if idx.numel() and (int(idx.min()) < 0 or int(idx.max()) >= self.in_dim):
                     raise ValueError(f"{name} holds an input index outside [0, {self.in_dim})")
+            if self.implementation == "cuda":                        # the reverse map of the input gradient
+                for name, n in (("given_x_indices_of_y_start", self.in_dim + 1), ("given_x_indices_of_y", 2 * self.out_dim)):
+                    t = getattr(self, name)
+                    if t.dtype != torch.int64 or tuple(t.shape) != (n,) or t.device != self.indices_0.device or not t.is_contiguous():
+                        raise ValueError(f"{name} must be a contiguous int64 [{n}] on the device of the wiring")
+                if not (self.indices_0.is_contiguous() and self.indices_1.is_contiguous()
+                        and self.indices_0.device == self.indices_1.device == self.weights.device):
+                    raise ValueError("indices_0 / indices_1 must be contiguous and on the device of the weights")
             self._wiring_checked = key
 
     def invalidate(self):
@@ -149,14 +162,14 @@ class LogicLayer(torch.nn.Module):
         super()._load_from_state_dict(*args, **kwargs)
         self.invalidate()
 
-    def _sole_consumers(self):
+    def _sole_consumers(self, key=None):
         """True when every input feature is read by exactly one neuron operand (the halving layers of the
         reference's models, 2*out_dim == in_dim): both gradients then come from one kernel.  Rechecked when the
         wiring buffers were modified in place or moved."""
         if 2 * self.out_dim != self.in_dim:
             return False
-        key = self._wiring_key()
-        cached = getattr(self, "_sole_cache", None)
+        key = key or self._wiring_key()
+        cached = self.__dict__.get("_sole_cache")
         if cached is None or cached[0] != key:
             uses = torch.bincount(torch.cat([self.indices_0, self.indices_1]), minlength=self.in_dim)
             cached = (key, bool((uses == 1).all().item()))
@@ -301,7 +314,7 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
                 sample_major_input=False):
         if sample_major_input:                                       # x is [B, in]: its gradient goes back in that layout
             x = difflogic_hip.transpose(x)
-        y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach())
+        y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False)   # the module has checked its buffers
         ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.sole_consumers = sole_consumers
         ctx.sample_major_input = sample_major_input
@@ -313,18 +326,24 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
         grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
         grad_x = grad_l = None
         if ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]:
-            grad_x, grad_l = difflogic_hip.backward_sole(x, a, b, folded, w, grad_y)
+            grad_x, grad_l = difflogic_hip.backward_sole(x, a, b, folded, w, grad_y, validate=_needs_check(grad_y, x))
         elif (ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and grad_y.numel() <= _FUSED_BACKWARD_MAX_ELEMS
               and difflogic_hip.backward_fused_fits(x)):
-            grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, grad_y, start, flat)
+            grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, grad_y, start, flat, validate=_needs_check(grad_y, x))
         else:
             if ctx.needs_input_grad[0]:
-                grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat)
+                grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat, validate=_needs_check(grad_y, x))
             if ctx.needs_input_grad[3]:
-                grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y)
+                grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y, validate=_needs_check(grad_y, x))
         if ctx.sample_major_input and grad_x is not None:
             grad_x = difflogic_hip.transpose(grad_x)
         return grad_x, None, None, grad_l, None, None, None, None
+
+
+def _needs_check(grad_y, x):
+    """The tensors a Function saved were validated on the way in; the incoming gradient is what can still differ
+    (autograd hands over the output's shape, but a caller-made gradient may have another dtype or device)."""
+    return grad_y.dtype != x.dtype or grad_y.device != x.device
 
 
 def _contiguous_2d(t):

@@ -84,6 +84,9 @@ SIGNATURES = {
     "clg_convblock_forward_fm": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_backward_fm": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _i, _p, _p]),
     "clg_convblock_backward_scratch_bytes": (_i64, [_i, _GP]),
+    "clg_convblock_plan_bytes": (_i64, [_i, _GP]),
+    "clg_convblock_plan": (_i, [_i, _GP, _p, _p, _p, _p]),
+    "clg_convblock_backward_planned": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i, _p, _p]),
 }
 
 _lib = None
@@ -107,6 +110,21 @@ def load():
 
 def available():
     return os.path.exists(LIB_PATH)
+
+
+_knob_generation = 0
+
+
+def reload_knobs():
+    """Makes the library read its CLG_* environment knobs again (it reads them once per process) and invalidates what
+    was derived under the old values (the per-layer backward plans are keyed on knob_generation())."""
+    global _knob_generation
+    load().clg_reload_knobs()
+    _knob_generation += 1
+
+
+def knob_generation():
+    return _knob_generation
 
 
 def check(rc):

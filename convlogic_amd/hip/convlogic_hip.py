@@ -272,10 +272,11 @@ def full_convlogic_backward(grad_y, x, weight, argmax, selection, stride_h, stri
     return gx, gw
 
 
-def full_convlogic_backward_logits(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True):
+def full_convlogic_backward_logits(grad_y, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True, validate=True):
     """-> (grad_x or None, grad_logits [C,7,16]) for weight = softmax(logits): the two gradients of the block
     with the softmax backward fused into the final reduction of the weight gradient."""
-    _block_grad_args(grad_y, x, weight, argmax, selection)
+    if validate:
+        _block_grad_args(grad_y, x, weight, argmax, selection)
     g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)
@@ -311,30 +312,90 @@ def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, p
     return y, argmax
 
 
-def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False):
+def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False,
+                                  want_folded=False, validate=True):
     """full_convlogic_forward() from the LOGITS [C, 7, 16]: the softmax is taken inside the launch that sets the gate
     parameters up.  -> (y, argmax, probs); with feature_major (where feature_major_supported) y is laid out
-    [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm()."""
-    _conv_args(x, logits, selection, 7)
+    [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm().  want_folded: -> (y, argmax, probs, folded [C, 7, 4]), the
+    folded coefficients of every gate for full_convlogic_backward_planned()."""
+    if validate:
+        _conv_args(x, logits, selection, 7)
     g = _geom(x, logits.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
     ho, wo = _out_size(g)
     shape = (g.n, g.c_out, max(ho, 0) // 2, max(wo, 0) // 2)
     y = torch.empty((g.c_out, shape[2], shape[3], g.n) if feature_major else shape, dtype=x.dtype, device=x.device)
     argmax = torch.empty(shape, dtype=torch.uint8, device=x.device)
-    probs = torch.empty_like(logits)
+    c = logits.shape[0]
+    if want_folded:                                                  # one buffer: probabilities, then the folded coefficients
+        both = torch.empty((c * (112 + 28),), dtype=logits.dtype, device=logits.device)
+        probs, folded = both[:c * 112].view(c, 7, 16), both[c * 112:].view(c, 7, 4)
+    else:
+        probs, folded = torch.empty_like(logits), None
     lib = _lib.load()
     scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
     check(lib.clg_convblock_forward_ex(dtype_code(x), ctypes.byref(g), x.data_ptr(), logits.data_ptr(), selection.data_ptr(),
-                                       y.data_ptr(), argmax.data_ptr(), probs.data_ptr(), 1 | (2 if feature_major else 0),
+                                       y.data_ptr(), argmax.data_ptr(), probs.data_ptr(),
+                                       1 | (2 if feature_major else 0) | (4 if want_folded else 0),
                                        scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))
+    if want_folded:
+        return y, argmax, probs, folded
     return y, argmax, probs
 
 
+def make_backward_plan(x, c_out, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """Per-layer plan of the block's backward pass for inputs of x's shape and dtype: -> (plan bytes on the device,
+    signature).  Depends only on the selection and the geometry; built once and reused by every
+    full_convlogic_backward_planned() call of the layer (the reverse map the reference's LogicLayer builds at
+    construction, src/difflogic/difflogic.py:71-87, for the fused block)."""
+    check_input(x, "x")
+    if x.dim() != 4:
+        raise RuntimeError(f"Expected x to be 4D (N, C, H, W), but got {x.dim()}")
+    _selection_arg(x, selection, c_out)
+    g = _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    plan = _scratch(lib.clg_convblock_plan_bytes(dt, ctypes.byref(g)), x.device)
+    sig = ctypes.c_int64(0)
+    check(lib.clg_convblock_plan(dt, ctypes.byref(g), selection.data_ptr(), plan.data_ptr(), ctypes.byref(sig), stream_ptr(x)))
+    return plan, sig.value
+
+
+def full_convlogic_backward_planned(grad_y, x, weight, folded, argmax, selection, plan, signature, stride_h, stride_w, pad_h, pad_w,
+                                    need_grad_x=True, wrt_logits=True, validate=True, feature_major=False):
+    """-> (grad_x or None, grad_w [C,7,16]) with the layer's plan from make_backward_plan(): no list building, no reduce
+    launch and -- with folded [C, 7, 4] from full_convlogic_forward_logits(want_folded=True) -- no set-up launch for
+    blocks whose images fit LDS.  grad_w is the gradient w.r.t. the logits (weight = their softmax) or, with
+    wrt_logits=False, w.r.t. the probabilities; feature_major: grad_y is laid out [C, Ho/2, Wo/2, N] (as for
+    full_convlogic_backward_fm).  Same values as full_convlogic_backward(_logits / _fm)()."""
+    if feature_major:                                                # grad_y laid out [C, Ho/2, Wo/2, N]
+        g = _geom_from_out(x, grad_y.shape[0], 2 * grad_y.shape[1], 2 * grad_y.shape[2], stride_h, stride_w, pad_h, pad_w)
+    else:
+        g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    if validate:
+        _block_grad_args(grad_y, x, weight, argmax, selection, feature_major=feature_major)
+        if folded is not None:
+            check_input(folded, "folded", x.dtype, (weight.shape[0], 7, 4))
+        check_input(plan, "plan", torch.uint8)
+        if plan.numel() < lib.clg_convblock_plan_bytes(dt, ctypes.byref(g)):
+            raise RuntimeError("plan is smaller than clg_convblock_plan_bytes() for this geometry")
+    scratch = _scratch(lib.clg_convblock_backward_scratch_bytes(dt, ctypes.byref(g)), x.device)
+    gx = torch.empty_like(x) if need_grad_x else None
+    gw = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    check(lib.clg_convblock_backward_planned(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                             folded.data_ptr() if folded is not None else None, selection.data_ptr(), argmax.data_ptr(),
+                                             plan.data_ptr(), signature, gx.data_ptr() if need_grad_x else None, gw.data_ptr(),
+                                             (1 if wrt_logits else 0) | (2 if feature_major else 0), scratch.data_ptr(), stream_ptr(x)))
+    return gx, gw
+
+
 def full_convlogic_backward_fm(grad_y_fm, x, weight, argmax, selection, stride_h, stride_w, pad_h, pad_w, need_grad_x=True,
-                               wrt_logits=True):
+                               wrt_logits=True, validate=True):
     """-> (grad_x or None, grad_w [C,7,16]) from grad_y laid out [C, Ho/2, Wo/2, N]; grad_w is the gradient w.r.t. the
     logits (weight = their softmax) or, with wrt_logits=False, w.r.t. the probabilities."""
-    _block_grad_args(grad_y_fm, x, weight, argmax, selection, feature_major=True)
+    if validate:
+        _block_grad_args(grad_y_fm, x, weight, argmax, selection, feature_major=True)
     g = _geom_from_out(x, grad_y_fm.shape[0], 2 * grad_y_fm.shape[1], 2 * grad_y_fm.shape[2], stride_h, stride_w, pad_h, pad_w)
     lib = _lib.load()
     dt = dtype_code(x)

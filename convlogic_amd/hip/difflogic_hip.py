@@ -49,13 +49,15 @@ def backward_w(x, a, b, grad_y):
     return gw
 
 
-def backward_logits(x, a, b, w, grad_y):
+def backward_logits(x, a, b, w, grad_y, validate=True):
     """Gradient w.r.t. the logits [out, 16] when w = softmax(logits): backward_w and the softmax backward
     in one kernel."""
     out_dim = grad_y.shape[0] if grad_y.dim() else -1
-    in_dim, batch = _wiring(x, a, b, out_dim)
-    check_input(w, "w", x.dtype, (out_dim, 16))
-    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
+    if validate:
+        _wiring(x, a, b, out_dim)
+        check_input(w, "w", x.dtype, (out_dim, 16))
+        check_input(grad_y, "grad_y", x.dtype, (out_dim, x.shape[1]))
+    in_dim, batch = x.shape
     gl = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(),
                                              grad_y.data_ptr(), gl.data_ptr(), in_dim, out_dim, batch, stream_ptr(x)))
@@ -86,13 +88,15 @@ def forward_folded(x, a, b, folded):
     return y
 
 
-def forward_logits(x, a, b, logits):
+def forward_logits(x, a, b, logits, validate=True):
     """fold(from_logits=True) + forward_folded() in one launch -> (y [out, B], probs [out, 16], folded [out, 4])."""
-    if logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.dtype not in _lib._DTYPES:
-        raise RuntimeError(f"forward_logits expects float32/float64 logits [out, 16] of x's dtype, got {tuple(logits.shape)} {logits.dtype}")
     out_dim = logits.shape[0]
-    in_dim, batch = _wiring(x, a, b, out_dim)
-    check_input(logits, "w")
+    if validate:
+        if logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.dtype not in _lib._DTYPES:
+            raise RuntimeError(f"forward_logits expects float32/float64 logits [out, 16] of x's dtype, got {tuple(logits.shape)} {logits.dtype}")
+        _wiring(x, a, b, out_dim)
+        check_input(logits, "w")
+    in_dim, batch = x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     probs = torch.empty_like(logits)
     folded = torch.empty((out_dim, 4), dtype=x.dtype, device=x.device)
@@ -102,13 +106,15 @@ def forward_logits(x, a, b, logits):
     return y, probs, folded
 
 
-def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
+def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y, validate=True):
     """backward_x() with the folded coefficients [out, 4] of fold() in place of w."""
     out_dim = folded.shape[0] if folded.dim() else -1
-    in_dim, batch = _wiring(x, a, b, out_dim)
-    check_input(folded, "folded", x.dtype, (out_dim, 4))
-    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
-    _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
+    if validate:
+        _wiring(x, a, b, out_dim)
+        check_input(folded, "folded", x.dtype, (out_dim, 4))
+        check_input(grad_y, "grad_y", x.dtype, (out_dim, x.shape[1]))
+        _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
+    in_dim, batch = x.shape
     gx = torch.empty_like(x)
     check(_lib.load().clg_fc_backward_x_folded(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
                                                grad_y.data_ptr(), given_x_indices_of_y_start.data_ptr(),
@@ -117,15 +123,17 @@ def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given
     return gx
 
 
-def backward_sole(x, a, b, folded, probs, grad_y):
+def backward_sole(x, a, b, folded, probs, grad_y, validate=True):
     """(grad_x, grad_w) in one pass for a layer whose inputs are each read by exactly one neuron operand; grad_w is
     the gradient w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities."""
     out_dim = folded.shape[0] if folded.dim() else -1
-    in_dim, batch = _wiring(x, a, b, out_dim)
-    check_input(folded, "folded", x.dtype, (out_dim, 4))
-    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
-    if probs is not None:
-        check_input(probs, "w", x.dtype, (out_dim, 16))
+    if validate:
+        _wiring(x, a, b, out_dim)
+        check_input(folded, "folded", x.dtype, (out_dim, 4))
+        check_input(grad_y, "grad_y", x.dtype, (out_dim, x.shape[1]))
+        if probs is not None:
+            check_input(probs, "w", x.dtype, (out_dim, 16))
+    in_dim, batch = x.shape
     gx = torch.empty_like(x)
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_sole(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
@@ -139,17 +147,19 @@ def backward_fused_fits(x):
     return bool(_lib.load().clg_fc_backward_fused_fits(dtype_code(x), x.shape[1]))
 
 
-def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, given_x_indices_of_y):
+def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, given_x_indices_of_y, validate=True):
     """(grad_x, grad_w) of a layer with any wiring in one pass (see backward_fused_fits); grad_w is the gradient
     w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities.  Same values as
     backward_x_folded() + backward_w() / backward_logits()."""
     out_dim = folded.shape[0] if folded.dim() else -1
-    in_dim, batch = _wiring(x, a, b, out_dim)
-    check_input(folded, "folded", x.dtype, (out_dim, 4))
-    check_input(grad_y, "grad_y", x.dtype, (out_dim, batch))
-    _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
-    if probs is not None:
-        check_input(probs, "w", x.dtype, (out_dim, 16))
+    if validate:
+        _wiring(x, a, b, out_dim)
+        check_input(folded, "folded", x.dtype, (out_dim, 4))
+        check_input(grad_y, "grad_y", x.dtype, (out_dim, x.shape[1]))
+        _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
+        if probs is not None:
+            check_input(probs, "w", x.dtype, (out_dim, 16))
+    in_dim, batch = x.shape
     gx = torch.empty_like(x)
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
     check(_lib.load().clg_fc_backward_fused(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),

@@ -361,6 +361,9 @@ int clg_convblock_fm_supported(int dtype, const clg_conv_geom *g);
  * (src/convlogic/convlogic_layer.py:318-329).  CLG_FWD_Y_FEATURE_MAJOR: y laid out as for clg_convblock_forward_fm. */
 #define CLG_FWD_W_LOGITS 1
 #define CLG_FWD_Y_FEATURE_MAJOR 2
+#define CLG_FWD_FOLDED_OUT 4 /* probs_out holds [c_out, 7, 16] probabilities FOLLOWED BY [c_out, 7, 4] folded coefficients
+                              * (ab, a, b, 1 per gate) for clg_convblock_backward_planned; without CLG_FWD_W_LOGITS the
+                              * probability part is left untouched (w already holds them) */
 int clg_convblock_forward_ex(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection, void *y,
                              uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream);
 /* The same for packed words: y laid out [c_out, ho/2, wo/2, groups], which IS the feature-major [features, words] layout
@@ -373,6 +376,26 @@ int clg_convblock_forward_fm(int dtype, const clg_conv_geom *g, const void *x, c
 int clg_convblock_backward_fm(int dtype, const clg_conv_geom *g, const void *grad_y /*[c_out,ho/2,wo/2,n]*/, const void *x,
                               const void *w, const int32_t *selection, const uint8_t *argmax, void *grad_x, void *grad_w,
                               int wrt_logits, void *scratch, void *stream);
+
+/* Per-layer plan of the block's backward pass: everything its kernels need that depends only on `selection` and the
+ * geometry (the reverse map input channel -> kernels and taps in increasing kernel order and the tap offsets of the chosen
+ * kernels' image layout), built ONCE per layer and batch shape instead of in every
+ * backward call -- the counterpart of the reverse map that LogicLayer builds at construction
+ * (src/difflogic/difflogic.py:71-87).  plan: clg_convblock_plan_bytes() bytes of device memory that the caller keeps;
+ * *signature identifies what it was made for and is handed back to clg_convblock_backward_planned, which rejects a plan
+ * made for another geometry, element type or kernel choice (the CLG_* knobs are part of the choice).  The backward calls
+ * only read a plan. */
+int64_t clg_convblock_plan_bytes(int dtype, const clg_conv_geom *g);
+int clg_convblock_plan(int dtype, const clg_conv_geom *g, const int32_t *selection, void *plan, int64_t *signature, void *stream);
+#define CLG_BWD_WRT_LOGITS 1       /* w = softmax(logits): grad_w is the gradient w.r.t. the logits */
+#define CLG_BWD_GY_FEATURE_MAJOR 2 /* grad_y laid out [c_out, ho/2, wo/2, n] (shapes of clg_convblock_fm_supported) */
+/* clg_convblock_backward / clg_convblock_backward_logits / clg_convblock_backward_fm (chosen by flags) with a plan: no list building per call, and with folded [c_out, 7, 4] (written by clg_convblock_forward_ex with
+ * CLG_FWD_FOLDED_OUT for the same w; may be NULL) no set-up launch is left for blocks whose images fit LDS.  grad_x may
+ * be NULL.  scratch: clg_convblock_backward_scratch_bytes().  Same values as the unplanned entry points.
+ * Replaces full_convlogic_backward_x + full_convlogic_backward_weight (src/convlogic/convlogic_layer.py:71-82). */
+int clg_convblock_backward_planned(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                                   const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
+                                   int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream);
 
 /* ---------------------------------------------------------------------------------
  * input binarisation (the step in front of the first layer)

@@ -26,4 +26,4 @@ def _knobs_follow_the_environment():
     yield
     from convlogic_amd.hip import _lib
     if _lib.available():
-        _lib.load().clg_reload_knobs()
+        _lib.reload_knobs()

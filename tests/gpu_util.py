@@ -15,7 +15,7 @@ def set_knobs(monkeypatch, **knobs):
             monkeypatch.delenv(name, raising=False)
         else:
             monkeypatch.setenv(name, str(value))
-    _lib.load().clg_reload_knobs()
+    _lib.reload_knobs()
 
 
 def has_gpu():
