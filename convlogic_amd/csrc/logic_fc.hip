@@ -514,6 +514,88 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
 // (as fc_backward_w_kernel: same lanes, same order, same reduction) and writes the neuron's 16 gate gradients.
 // Saves the second pass over gy and the operand rows that a separate weight-gradient kernel makes.
 template <typename T, int VEC, int LPR>
+__device__ __forceinline__ bool fc_backward_fused_item(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                       const int64_t *__restrict__ b, const T *__restrict__ folded,
+                                                       const T *__restrict__ gy, const int64_t *__restrict__ csr_start,
+                                                       const int64_t *__restrict__ csr_list, T *__restrict__ gw, int in_dim,
+                                                       int64_t batch, const T *__restrict__ probs, int64_t it, int lane,
+                                                       Pack<T, VEC> &acc, int64_t &i)
+{
+    const int sub = lane / LPR, l = lane % LPR;
+    constexpr int ROWS = kWave / LPR;
+    const int64_t s = (int64_t)l * VEC;
+    const bool row_ok = it * ROWS + sub < in_dim;
+    i = row_ok ? it * ROWS + sub : in_dim - 1;
+    const bool live = row_ok && s < batch;                           // lanes beyond the batch add zeros to the sums
+    const int64_t beg = csr_start[i], end = row_ok ? csr_start[i + 1] : beg;
+    Pack<T, VEC> xi;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) xi.v[k] = 0;
+    if (live) xi = load_vec<T, VEC>(x + i * batch + s);
+    Pack<T, VEC> part[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
+    int64_t prev = -1;
+    for (int64_t cur = beg; cur < end; cur += 4) {                   // the lanes of a row group leave the loop together
+        int64_t j[4];
+        Pack<T, VEC> vo[4], vg[4];
+        T c_ab[4], c_lin[4];
+        bool first[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            j[u] = cur + u < end ? csr_list[cur + u] : -1;
+            first[u] = false;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) vo[u].v[k] = vg[u].v[k] = 0;
+            if (j[u] >= 0) {
+                const int64_t ia = a[j[u]], ib = b[j[u]];
+                const Coef<T> c = load_coef(folded + j[u] * 4);
+                const bool as_a = ia == i && !(ib == i && prev == j[u]);   // see fc_backward_x_folded_kernel
+                first[u] = as_a;
+                c_ab[u] = c.ab;
+                c_lin[u] = as_a ? c.a : c.b;
+                if (live) {
+                    vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
+                    vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
+                }
+            }
+            prev = j[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (j[u] < 0) continue;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
+            if (first[u]) {                                          // uniform over the row group
+                T sab = 0, sa = 0, sb = 0, s1 = 0;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    sab = fma_t(vg[u].v[k], xi.v[k] * vo[u].v[k], sab);
+                    sa = fma_t(vg[u].v[k], xi.v[k], sa);
+                    sb = fma_t(vg[u].v[k], vo[u].v[k], sb);
+                    s1 += vg[u].v[k];
+                }
+                sab = lane_group_sum<T, LPR>(sab);
+                sa = lane_group_sum<T, LPR>(sa);
+                sb = lane_group_sum<T, LPR>(sb);
+                s1 = lane_group_sum<T, LPR>(s1);
+                if (l >= LPR - 16) {
+                    const int q = lane & 15;
+                    T gi = coef_transpose_row<T>(q, sab, sa, sb, s1);
+                    if (probs != nullptr) gi = softmax16_backward(gi, probs[j[u] * 16 + q]);
+                    gw[j[u] * 16 + q] = gi;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
+    return live;
+}
+
+template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
     const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
@@ -521,80 +603,47 @@ __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
 {
     constexpr int ROWS = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-    const int sub = lane / LPR, l = lane % LPR;
     const int64_t groups = (in_dim + ROWS - 1) / ROWS;
-    const int64_t s = (int64_t)l * VEC;
+    const int64_t s = (int64_t)(lane % LPR) * VEC;
     for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < groups; it += (int64_t)gridDim.x * kWavesPerBlock) {
-        const bool row_ok = it * ROWS + sub < in_dim;
-        const int64_t i = row_ok ? it * ROWS + sub : in_dim - 1;
-        const bool live = row_ok && s < batch;                       // lanes beyond the batch add zeros to the sums
-        const int64_t beg = csr_start[i], end = row_ok ? csr_start[i + 1] : beg;
-        Pack<T, VEC> xi;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) xi.v[k] = 0;
-        if (live) xi = load_vec<T, VEC>(x + i * batch + s);
-        Pack<T, VEC> part[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
-        int64_t prev = -1;
-        for (int64_t cur = beg; cur < end; cur += 4) {               // the lanes of a row group leave the loop together
-            int64_t j[4];
-            Pack<T, VEC> vo[4], vg[4];
-            T c_ab[4], c_lin[4];
-            bool first[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                j[u] = cur + u < end ? csr_list[cur + u] : -1;
-                first[u] = false;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) vo[u].v[k] = vg[u].v[k] = 0;
-                if (j[u] >= 0) {
-                    const int64_t ia = a[j[u]], ib = b[j[u]];
-                    const Coef<T> c = load_coef(folded + j[u] * 4);
-                    const bool as_a = ia == i && !(ib == i && prev == j[u]);   // see fc_backward_x_folded_kernel
-                    first[u] = as_a;
-                    c_ab[u] = c.ab;
-                    c_lin[u] = as_a ? c.a : c.b;
-                    if (live) {
-                        vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
-                        vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
-                    }
-                }
-                prev = j[u];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (j[u] < 0) continue;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
-                if (first[u]) {                                      // uniform over the row group
-                    T sab = 0, sa = 0, sb = 0, s1 = 0;
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) {
-                        sab = fma_t(vg[u].v[k], xi.v[k] * vo[u].v[k], sab);
-                        sa = fma_t(vg[u].v[k], xi.v[k], sa);
-                        sb = fma_t(vg[u].v[k], vo[u].v[k], sb);
-                        s1 += vg[u].v[k];
-                    }
-                    sab = lane_group_sum<T, LPR>(sab);
-                    sa = lane_group_sum<T, LPR>(sa);
-                    sb = lane_group_sum<T, LPR>(sb);
-                    s1 = lane_group_sum<T, LPR>(s1);
-                    if (l >= LPR - 16) {
-                        const int q = lane & 15;
-                        T gi = coef_transpose_row<T>(q, sab, sa, sb, s1);
-                        if (probs != nullptr) gi = softmax16_backward(gi, probs[j[u] * 16 + q]);
-                        gw[j[u] * 16 + q] = gi;
-                    }
-                }
-            }
-        }
         Pack<T, VEC> acc;
+        int64_t i;
+        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i))
+            store_vec<T, VEC>(gx + i * batch + s, acc);
+    }
+}
+
+// The same pass with the input gradient written sample-major, gx [batch, in_dim]: 16 wavefronts of a workgroup own
+// F = 16 * 64/LPR consecutive inputs, park their rows in an LDS tile [F][bp] and the workgroup writes the tile out
+// transposed, F consecutive elements per sample.  Same sums in the same order as fc_backward_fused_kernel.
+constexpr int kSmOutWaves = 16;
+static inline int64_t smout_row_pitch(int64_t batch) { return ((batch + 31) & ~31ll) + 4; }   // pitch % 32 == 4: the transposed reads spread over the banks
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kSmOutWaves * kWave) void fc_backward_fused_smout_kernel(
+    const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
+    const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
+    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int batch, int bp, const T *__restrict__ probs)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *tile = reinterpret_cast<T *>(smem);
+    constexpr int ROWS = kWave / LPR, F = kSmOutWaves * ROWS;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t groups = (in_dim + ROWS - 1) / ROWS;
+    const int64_t it = (int64_t)blockIdx.x * kSmOutWaves + wave;
+    if (it < groups) {
+        Pack<T, VEC> acc;
+        int64_t i;
+        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i)) {
+            T *row = tile + (size_t)(wave * ROWS + lane / LPR) * bp + (lane % LPR) * VEC;
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
-        if (live) store_vec<T, VEC>(gx + i * batch + s, acc);
+            for (int k = 0; k < VEC; ++k) row[k] = acc.v[k];
+        }
+    }
+    __syncthreads();
+    const int64_t i0 = (int64_t)blockIdx.x * F;
+    for (int e = threadIdx.x; e < F * batch; e += kSmOutWaves * kWave) {
+        const int f = e % F, s = e / F;
+        if (i0 + f < in_dim) gx[(int64_t)s * in_dim + i0 + f] = tile[(size_t)f * bp + s];
     }
 }
 
@@ -993,22 +1042,36 @@ extern "C" int clg_fc_backward_fused_fits(int dtype, int64_t batch)
     return (dtype == CLG_F32 || dtype == CLG_F64) && batch > 0 && batch <= fused_batch_limit(dtype, batch) ? 1 : 0;
 }
 
-extern "C" int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
-                                     const void *probs, const void *grad_y, const int64_t *csr_start, const int64_t *csr_list,
-                                     void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+extern "C" int clg_fc_backward_fused_ex(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                        const void *probs, const void *grad_y, const int64_t *csr_start, const int64_t *csr_list,
+                                        void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int flags,
+                                        void *stream)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_fused")) return e;
-    CLG_REQUIRE(x && a && b && folded && grad_y && csr_start && csr_list && grad_x && grad_w,
-                "clg_fc_backward_fused: null pointer argument");
+    const char *name = "clg_fc_backward_fused";
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
+    CLG_REQUIRE(x && a && b && folded && grad_y && csr_start && csr_list && grad_x && grad_w, "%s: null pointer argument", name);
+    CLG_REQUIRE((flags & ~CLG_FC_GX_SAMPLE_MAJOR) == 0, "%s: unknown flags 0x%x", name, flags);
     CLG_REQUIRE(batch <= fused_batch_limit(dtype, batch),
-                "clg_fc_backward_fused: batch %lld exceeds what one pass covers (%lld); use clg_fc_backward_x_folded and "
-                "clg_fc_backward_logits", (long long)batch, (long long)fused_batch_limit(dtype, batch));
-    const dim3 block(kBlock);
+                "%s: batch %lld exceeds what one pass covers (%lld); use clg_fc_backward_x_folded and clg_fc_backward_logits", name,
+                (long long)batch, (long long)fused_batch_limit(dtype, batch));
     hipStream_t st = clg_stream(stream);
-#define CLG_LAUNCH_BF(T, VEC, LPR)                                                                                         \
-    hipLaunchKernelGGL((fc_backward_fused_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(in_dim, (int64_t)(kWave / LPR)))), \
-                       block, 0, st, (const T *)x, a, b, (const T *)folded, (const T *)grad_y, csr_start, csr_list,          \
-                       (T *)grad_x, (T *)grad_w, (int)in_dim, batch, (const T *)probs)
+    const bool sm_out = (flags & CLG_FC_GX_SAMPLE_MAJOR) != 0;
+    const int bp = (int)smout_row_pitch(batch);
+#define CLG_LAUNCH_BF(T, VEC, LPR)                                                                                           \
+    do {                                                                                                                    \
+        if (sm_out) {                                                                                                       \
+            constexpr int F = kSmOutWaves * (kWave / LPR);                                                                  \
+            hipLaunchKernelGGL((fc_backward_fused_smout_kernel<T, VEC, LPR>), dim3((unsigned)clg_ceil_div(in_dim, (int64_t)F)), \
+                               dim3(kSmOutWaves * kWave), (size_t)F * bp * sizeof(T), st, (const T *)x, a, b, (const T *)folded, \
+                               (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (T *)grad_w, (int)in_dim, (int)batch, bp, \
+                               (const T *)probs);                                                                           \
+        } else {                                                                                                            \
+            hipLaunchKernelGGL((fc_backward_fused_kernel<T, VEC, LPR>),                                                     \
+                               dim3(grid_for(clg_ceil_div(in_dim, (int64_t)(kWave / LPR)))), dim3(kBlock), 0, st, (const T *)x, a, b, \
+                               (const T *)folded, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (T *)grad_w, (int)in_dim, \
+                               batch, (const T *)probs);                                                                    \
+        }                                                                                                                   \
+    } while (0)
 #define CLG_LAUNCH_BF_ROWS(T, VEC)                                                                                         \
     do {                                                                                                                  \
         const int lg = lanes_per_row_log2(batch, VEC);                                                                    \
@@ -1025,8 +1088,16 @@ extern "C" int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a,
     }
 #undef CLG_LAUNCH_BF_ROWS
 #undef CLG_LAUNCH_BF
-    CLG_CHECK_LAUNCH("clg_fc_backward_fused");
+    CLG_CHECK_LAUNCH(name);
     return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                     const void *probs, const void *grad_y, const int64_t *csr_start, const int64_t *csr_list,
+                                     void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
+{
+    return clg_fc_backward_fused_ex(dtype, x, a, b, folded, probs, grad_y, csr_start, csr_list, grad_x, grad_w, in_dim, out_dim, batch, 0,
+                                    stream);
 }
 
 extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64_t rows, int64_t cols, void *stream)
