@@ -26,6 +26,18 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 
+def _traffic(workload, key):
+    """HBM bytes per launch (or per step) recorded in profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE,
+    each scaled by what the same counter reads for a plain copy of known size.  Counters need profiler runs of their own,
+    so these are recorded measurements (the file names the commit and the commands), not taken live; None when the file
+    or the entry is missing."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)["workloads"][workload][key]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def _events(n):
     import torch
     return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
@@ -110,10 +122,6 @@ def _graph_step_ms(make_leaves, run, steps):
 # config 2: packed-bit inference
 # ------------------------------------------------------------------------------------------------
 C2 = dict(width=64000, layers=3, samples=65536, bits=64)
-# HBM bytes per launch of the evaluation kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE scaled by a plain copy of known size (profiles/eval_packed_walk_c2_pmc.txt); counters
-# need their own profiler runs, so this is a recorded measurement, not taken live.
-C2_TRAFFIC_BYTES = 1143.2e6
 
 
 def bench_c2(steps, warmup, cpu=True):
@@ -174,7 +182,7 @@ def bench_c2(steps, warmup, cpu=True):
                                "(1024 words/feature), argmax gates, random 2-input wiring"},
         "gate_evals_per_s": samples * width * nl / sec,
         "roofline": {"bound": "hbm", "kernel": "eval_packed_walk_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": C2_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": alg_bytes,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": _traffic("c2", "eval_packed_walk_kernel_bytes_per_launch"), "algorithmic_bytes_per_launch": alg_bytes,
                      "avg_launch_ms": kernel_ms, **_launch_stats(pairs), "launches_timed": len(pairs),
                      "plain_copy_GBps_same_size": copy_gbs},
     }
@@ -239,9 +247,72 @@ def cpu_c2(layers, x0):
 # ------------------------------------------------------------------------------------------------
 # float workloads: forward + backward
 # ------------------------------------------------------------------------------------------------
-# HBM bytes of one training step of the block (all its kernels), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
-# a plain copy of known size in the same runs (profiles/convblock_c4_c3_hbm_traffic_pmc.txt): recorded, not taken live.
-CONV_TRAFFIC_BYTES = {"c4": 369.7e6, "c3": 36.8e6}
+
+def _cpu_reps(cpu_step, budget_s, max_reps):
+    cpu_step()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        cpu_step()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= max_reps:
+            return reps, el
+
+
+def _cpu_torch_leg(cpu_step, units_per_step, sample):
+    """cpu_baseline entry of a torch-CPU oracle step: all host threads the box grants (at most 16) for about 5 s, then
+    the same on one thread for about 3 s."""
+    import torch
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    reps, el = _cpu_reps(cpu_step, 5.0, 50)
+    torch.set_num_threads(1)
+    reps1, el1 = _cpu_reps(cpu_step, 3.0, 20)
+    torch.set_num_threads(threads)
+    return {"value": units_per_step * reps / el / 1e9, "value_one_thread": units_per_step * reps1 / el1 / 1e9, "unit": "Ggate-evals/s",
+            "cores": threads, "kind": "port", "cpu_model": _cpu_model(), "host_cores": os.cpu_count(),
+            "sample": f"{sample}: {reps} steps in {el:.1f} s on {threads} threads, {reps1} steps in {el1:.1f} s on one thread"}
+
+
+_LITERAL = {}
+
+
+def _literal_loop_block():
+    """The reference's literal python path of the block (src/convlogic/convlogic_layer.py:262-282: one indexed copy per
+    leaf gate, kernel and conv position) as restated by the oracle, forward + backward at [4,1,28,28], k=4 on one
+    thread; measured once per run.  -> (seconds per step, gate evaluations per step)"""
+    if not _LITERAL:
+        import torch
+        from oracle import convlogic_oracle as O
+        torch.manual_seed(11)
+        n, cin, h, w, k = 4, 1, 28, 28, 4
+        sel = torch.as_tensor(O.generate_selection(cin, k, (3, 3)))
+        x = torch.randint(0, 2, (n, cin, h, w)).float().requires_grad_(True)
+        logits = torch.randn(k, 7, 16, requires_grad=True)
+        gy = torch.randn(n, k, h // 2, w // 2)
+
+        def step():
+            x.grad = logits.grad = None
+            wp = torch.softmax(logits, -1)
+            x2 = O.conv4_forward_loops(x, wp[:, 0:4], sel, (1, 1), (1, 1), (3, 3))
+            x4 = O.tree_forward(O.tree_forward(x2, wp[:, 4:6]), wp[:, 6:7]).squeeze(-1)
+            torch.nn.functional.max_pool2d(x4, 2, 2).backward(gy)
+
+        threads = torch.get_num_threads()
+        torch.set_num_threads(1)
+        t0 = time.perf_counter()
+        step()
+        _LITERAL["s"] = time.perf_counter() - t0
+        _LITERAL["ge"] = n * k * h * w * 7
+        torch.set_num_threads(threads)
+    return _LITERAL["s"], _LITERAL["ge"]
+
+
+def _literal_entry(gate_evals_full):
+    sec, ge = _literal_loop_block()
+    return {"shape": "[4,1,28,28], k=4, one thread, one fwd+bwd step", "seconds_per_step": sec, "Ggate_evals_per_s": ge / sec / 1e9,
+            "extrapolated_seconds_per_step_at_this_workload": sec * gate_evals_full / ge,
+            "note": "the reference's literal 4-deep python loop, timed at the reduced shape only and scaled linearly in gate evaluations"}
 
 
 def _roof(name, alg_bytes, ms, extra=None):
@@ -302,7 +373,6 @@ def bench_c1(steps, warmup, cpu=True):
     def cpu_leg():
         from oracle import convlogic_oracle as O            # the CPU baseline is the only user of the oracle here
 
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
         xl = x.detach().cpu().requires_grad_(True)
         ll = layer.weights.detach().cpu().requires_grad_(True)
         a, b, g = layer.indices_0.cpu(), layer.indices_1.cpu(), gy.cpu()
@@ -312,14 +382,7 @@ def bench_c1(steps, warmup, cpu=True):
             ll.grad = None
             O.logic_fc_forward(xl, a, b, torch.softmax(ll, -1)).backward(g)
 
-        cpu_step()
-        reps, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < 5.0 and reps < 50:
-            cpu_step()
-            reps += 1
-        el = time.perf_counter() - t0
-        return {"value": gate_evals * reps / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(),
-                "kind": "port", "sample": f"full C1 workload, {reps} fwd+bwd steps of the torch-CPU oracle in {el:.1f} s"}
+        return _cpu_torch_leg(cpu_step, gate_evals, "full C1 workload, fwd+bwd steps of the torch-CPU oracle")
 
     if cpu:
         out["_cpu"] = cpu_leg
@@ -339,6 +402,54 @@ CONV = {
     "c3": dict(name="C3", shape=(256, 1, 28, 28), k=32),
     "c4": dict(name="C4", shape=(256, 9, 32, 32), k=256),
 }
+
+
+# fp32 lane operations of the backward pass per POOLED cell (only the arg-max position of a 2x2 window carries a gradient):
+# 21 to recompute the tree (7 gates x 3 FMA), 14 partial derivatives (2 per gate, one FMA each), 14 chain products,
+# 35 for the coefficient sums (per gate a*b, three FMAs and one add) and 8 additions into the tap gradients.
+BWD_LANE_OPS_PER_POOLED_CELL = 21 + 14 + 14 + 35 + 8
+
+
+def _block_kernels(layer, xd, gy, reps):
+    """Forward, input-gradient and weight-gradient entry points of one block timed one by one with events (each entry
+    point's launches together), with the HBM roofline of each and the fp32 lane-operation floors beside it."""
+    import torch
+    from convlogic_amd.hip import convlogic_hip
+
+    n, cin, h, w = xd.shape
+    k = layer.out_channels
+    wp = torch.softmax(layer.weights.detach(), -1).contiguous()
+    sel = layer.selection
+    geo = (1, 1, 1, 1)
+    y, am = convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
+    ev = {name: _events(reps) for name in ("fwd", "bwd_x", "bwd_w")}
+    for r in range(reps):
+        ev["fwd"][r][0].record()
+        convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
+        ev["fwd"][r][1].record()
+        ev["bwd_x"][r][0].record()
+        convlogic_hip.full_convlogic_backward_x(gy, xd, wp, am, sel, *geo)
+        ev["bwd_x"][r][1].record()
+        ev["bwd_w"][r][0].record()
+        convlogic_hip.full_convlogic_backward_weight(gy, xd, wp, am, sel, *geo)
+        ev["bwd_w"][r][1].record()
+    torch.cuda.synchronize()
+    ms = {name: _avg_ms(p) for name, p in ev.items()}
+    gate_evals = n * k * h * w * 7
+    xb, yb, pb = n * cin * h * w * 4, n * k * (h // 2) * (w // 2) * 4, k * 7 * 16 * 4 + k * 8 * 4
+    alg_f, alg_b = xb + yb + pb, yb + xb + xb + pb      # forward: x in, y out; backward: gy, x in, gx out
+    total_ms = ms["fwd"] + ms["bwd_x"] + ms["bwd_w"]
+    floor_f = gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3
+    floor_b = n * k * (h // 2) * (w // 2) * BWD_LANE_OPS_PER_POOLED_CELL / VALU_LANE_OPS_PER_S * 1e3
+    roof = _roof("convblock fwd + bwd_x + bwd_w kernels", alg_f + alg_b, total_ms,
+                 {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
+                  "backward": _roof("convblock_backward_x + convblock_backward_w", alg_b, ms["bwd_x"] + ms["bwd_w"]),
+                  # lane-operation floors: 3 FMAs per gate evaluation forward, BWD_LANE_OPS_PER_POOLED_CELL backward, non-packed fp32
+                  "valu_floor_forward_ms": floor_f, "valu_frac_forward": floor_f / ms["fwd"],
+                  "valu_floor_backward_ms": floor_b, "valu_frac_backward": floor_b / (ms["bwd_x"] + ms["bwd_w"]),
+                  "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
+                          "the lane-operation floors (39.3 T fp32 lane-ops/s) beside it"})
+    return ms, total_ms, gate_evals, roof
 
 
 def bench_conv(key, steps, warmup, cpu=True):
@@ -373,44 +484,18 @@ def bench_conv(key, steps, warmup, cpu=True):
     graph_ms = _graph_step_ms(leaves_conv, lambda lv: lv[2](lv[0]).backward(gy), max(steps, 20))
 
     # kernel-level durations: forward, input-gradient and weight-gradient launches timed one by one
-    wp = torch.softmax(layer.weights.detach(), -1).contiguous()
-    xd, sel = x.detach(), layer.selection
-    geo = (1, 1, 1, 1)
-    y, am = convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
-    reps = max(steps, 5)
-    ev = {name: _events(reps) for name in ("fwd", "bwd_x", "bwd_w")}
-    for r in range(reps):
-        ev["fwd"][r][0].record()
-        convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
-        ev["fwd"][r][1].record()
-        ev["bwd_x"][r][0].record()
-        convlogic_hip.full_convlogic_backward_x(gy, xd, wp, am, sel, *geo)
-        ev["bwd_x"][r][1].record()
-        ev["bwd_w"][r][0].record()
-        convlogic_hip.full_convlogic_backward_weight(gy, xd, wp, am, sel, *geo)
-        ev["bwd_w"][r][1].record()
-    torch.cuda.synchronize()
-    ms = {name: _avg_ms(p) for name, p in ev.items()}
-    xb, yb, pb = n * cin * h * w * 4, n * k * (h // 2) * (w // 2) * 4, k * 7 * 16 * 4 + k * 8 * 4
-    alg_f, alg_b = xb + yb + pb, yb + xb + xb + pb      # forward: x in, y out; backward: gy, x in, gx out
-    total_ms = ms["fwd"] + ms["bwd_x"] + ms["bwd_w"]
+    sel = layer.selection
+    ms, total_ms, _ge, roof = _block_kernels(layer, x.detach(), gy, max(steps, 5))
+    roof["traffic"] = _traffic(key, "step_bytes")
     out = {"workload": f"{cfg['name']}: ConvLogicLayer block [{n},{cin},{h},{w}] -> k={k}, 3x3 pad 1, depth-2 tree, 2x2 OR-pool, float32 fwd+bwd",
            "metric": "convlogic_fwd_bwd_Ggate_evals_per_s", "value": gate_evals / sec / 1e9, "unit": "Ggate-evals/s",
            "ms_per_step": sec * 1e3, "dtype": "f32", "ms_per_step_hip_graph": graph_ms,
            "value_hip_graph": (gate_evals / (graph_ms * 1e-3) / 1e9) if graph_ms else None, "kernel_ms": ms, "kernels_only_Ggate_evals_per_s": gate_evals / (total_ms * 1e-3) / 1e9,
-           "roofline": _roof("convblock fwd + bwd_x + bwd_w kernels", alg_f + alg_b, total_ms,
-                             {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
-                              # lane-operation floor of the forward: 3 FMAs per gate evaluation, non-packed fp32
-                              "valu_floor_forward_ms": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3,
-                              "valu_frac_forward": gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3 / ms["fwd"],
-                              "traffic": CONV_TRAFFIC_BYTES.get(key),
-                              "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
-                                      "the lane-operation floor (39.3 T fp32 lane-ops/s) beside it"})}
+           "roofline": roof}
     def cpu_leg():
         from oracle import convlogic_oracle as O            # the CPU baseline is the only user of the oracle here
 
         nb = 8                                              # bounded sample: 8 samples of the batch
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
         xl = x.detach()[:nb].cpu().requires_grad_(True)
         ll = layer.weights.detach().cpu().requires_grad_(True)
         selc, g = sel.cpu(), gy[:nb].cpu()
@@ -420,14 +505,9 @@ def bench_conv(key, steps, warmup, cpu=True):
             ll.grad = None
             O.conv_block_forward(xl, torch.softmax(ll, -1), selc, (1, 1), (1, 1), (3, 3)).backward(g)
 
-        cpu_step()
-        reps_c, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < 5.0 and reps_c < 20:
-            cpu_step()
-            reps_c += 1
-        el = time.perf_counter() - t0
-        return {"value": nb * k * h * w * 7 * reps_c / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(),
-                "kind": "port", "sample": f"{nb} of {n} samples, {reps_c} fwd+bwd steps of the vectorised torch-CPU oracle in {el:.1f} s"}
+        res = _cpu_torch_leg(cpu_step, nb * k * h * w * 7, f"{nb} of {n} samples, fwd+bwd steps of the vectorised torch-CPU oracle")
+        res["literal_loop_path"] = _literal_entry(gate_evals)
+        return res
 
     if cpu:
         out["_cpu"] = cpu_leg
@@ -523,6 +603,39 @@ def bench_c5(steps, warmup, cpu=True):
             b_.record()
         torch.cuda.synchronize()
     out["packed_inference"]["ms_at_256_samples_with_threshold_pack"] = _avg_ms(ev)
+    # HBM roofline of the packed network: every layer reads its input words and writes its output words once
+    # (features x 65536 / 8 bytes each), the class counts leave as int32 [65536, classes]
+    word_bytes, size, feats_in, alg_p = big // 8, 32, 9 * 32 * 32, 0
+    for m in model.network:
+        if isinstance(m, C.ConvLogicLayer):
+            size //= 2
+            feats_out = m.out_channels * size * size
+        elif isinstance(m, C.LogicLayer):
+            feats_out = m.out_dim
+        elif isinstance(m, torch.nn.Flatten):
+            continue
+        else:                                                    # GroupSum: words in, counts out
+            alg_p += feats_in * word_bytes + big * m.k * 4
+            continue
+        alg_p += (feats_in + feats_out) * word_bytes
+        feats_in = feats_out
+    out["packed_inference"]["roofline"] = _roof("packed network, all kernels (4 blocks, 3 LogicLayers, per-class counts)", alg_p, net_ms)
+    # the four blocks of the training step one by one, on the activations the network feeds them
+    model.train()
+    blocks, h_act = [], x
+    with torch.no_grad():
+        for m in model.network:
+            if isinstance(m, C.ConvLogicLayer):
+                xin = h_act.contiguous()
+                gy_b = torch.randn(xin.shape[0], m.out_channels, xin.shape[2] // 2, xin.shape[3] // 2, device=dev)
+                ms_b, total_b, ge_b, roof_b = _block_kernels(m, xin, gy_b, max(steps, 5))
+                blocks.append({"block": f"[{n},{m.in_channels},{xin.shape[2]},{xin.shape[3]}] -> k={m.out_channels}", "kernel_ms": ms_b,
+                               "kernels_only_Ggate_evals_per_s": ge_b / (total_b * 1e-3) / 1e9, "roofline": roof_b})
+                h_act = m(h_act)
+            else:
+                break
+    out["block_kernels"] = blocks
+    model.eval()
     if cpu:
         out["_cpu"] = lambda: _cpu_c5(model, x, labels, ge // n)
     return out
@@ -536,7 +649,6 @@ def _cpu_c5(model, x, labels, gate_evals_per_sample):
     from oracle import convlogic_oracle as O
 
     nb = 4
-    torch.set_num_threads(min(os.cpu_count() or 1, 16))
     xs, ys = x[:nb].cpu(), labels[:nb].cpu()
     layers = []
     for m in model.network:
@@ -560,14 +672,7 @@ def _cpu_c5(model, x, labels, gate_evals_per_sample):
                 h = O.group_sum(h, m.k, m.tau)
         torch.nn.functional.cross_entropy(h, ys).backward()
 
-    cpu_step()
-    reps, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < 5.0 and reps < 20:
-        cpu_step()
-        reps += 1
-    el = time.perf_counter() - t0
-    return {"value": nb * gate_evals_per_sample * reps / el / 1e9, "unit": "Ggate-evals/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{nb} of {x.shape[0]} samples, {reps} training steps of the vectorised torch-CPU oracle in {el:.1f} s"}
+    return _cpu_torch_leg(cpu_step, nb * gate_evals_per_sample, f"{nb} of {x.shape[0]} samples, training steps of the vectorised torch-CPU oracle")
 
 
 # ------------------------------------------------------------------------------------------------
@@ -713,7 +818,7 @@ def main():
             "roofline": primary["roofline"], "cpu_baseline": primary.get("cpu_baseline"),
             "device": torch.cuda.get_device_name(0), "host_cores": os.cpu_count(),
             "host_setting": "torch.autograd.set_multithreading_enabled(False) for the eager training steps"}
-    for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s", "kernels", "packed_inference",
+    for extra in ("gate_evals_per_s", "kernel_ms", "kernels_only_Ggate_evals_per_s", "kernels", "packed_inference", "block_kernels",
                   "ms_per_step_hip_graph", "value_hip_graph", "ms_per_step_without_optimizer", "parameters", "reference_anchor"):
         if extra in primary:
             line[extra] = primary[extra]

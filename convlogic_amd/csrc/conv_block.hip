@@ -227,7 +227,7 @@ constexpr int kChunk = 4;  // cell blocks (of 64 lanes) whose grad_y / argmax lo
 template <typename T>
 struct CellLoads {
     T gy[kChunk];
-    int code[kChunk];
+    uint32_t codes;            // the kChunk one-byte arg-max codes, block j in byte j
 };
 
 // Row band of the input image owned by one workgroup, the pooled cells whose taps can reach it and
@@ -276,8 +276,11 @@ __host__ __device__ inline Band make_band(const Geom &g, int band, int band_rows
 // p.hsw wavefronts can share one (sample group, channel) the same way: each takes every hsw-th of those
 // kernels and accumulates into its own copy of the gradient window; the copies are added in order on the
 // way out.
-template <typename T, bool BANDED, bool SHARED>
-__global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
+// FULL: every wavefront pass has all of its kChunk * 64 cells (whole images, every sample group complete): no lane is
+// ever redirected, and the per-lane liveness tests drop out of the loops.
+// (float: two workgroups of 9 wavefronts share a compute unit only with 6 wavefronts per SIMD, i.e. at most 80 registers)
+template <typename T, bool BANDED, bool SHARED, bool FULL>
+__global__ __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 6 : 4))) void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, const T *__restrict__ x,
                                                   const T *__restrict__ folded, const int32_t *__restrict__ count,
                                                   const int32_t *__restrict__ hits, const int32_t *__restrict__ taps,
                                                   const uint8_t *__restrict__ argmax, T *__restrict__ gx, Geom g, TilePlan p)
@@ -343,10 +346,16 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
             bool live[kChunk];
 #pragma unroll
             for (int j = 0; j < kChunk; ++j) {
+                if (FULL && j > 0) {                                 // whole rows of cells per block: a uniform step from block 0
+                    live[j] = true;
+                    cx[j] = cx[0] + j * (kWave / wp) * 2 * row_step;
+                    cy[j] = cy[0] + j * kWave;
+                    continue;
+                }
                 const int v = (chunk * kChunk + j) * kWave + lane;
-                live[j] = v < v_here;
+                live[j] = FULL || v < v_here;
                 uint32_t sm = 0, cl = live[j] ? v : 0;              // sample inside the group, cell inside the band
-                if (!BANDED) {
+                if (!BANDED && !FULL) {
                     sm = fdiv(cl, p.d_slots);
                     cl -= sm * (uint32_t)I;
                 }
@@ -360,15 +369,19 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
                 const int64_t crow = gbase + (int64_t)(hit[k] & 0xFFFF) * I;
                 const uint8_t *am = argmax + crow;
                 const T *gr = gy + crow;
+                uint32_t code[kChunk];
 #pragma unroll
                 for (int j = 0; j < kChunk; ++j) {
                     L.gy[j] = T(0);
-                    L.code[j] = 0;
+                    code[j] = 0;
                     if (live[j]) {
-                        L.code[j] = am[cy[j]];
+                        code[j] = am[cy[j]];
                         L.gy[j] = gr[cy[j]];
                     }
                 }
+                L.codes = code[0];
+#pragma unroll
+                for (int j = 1; j < kChunk; ++j) L.codes |= code[j] << (8 * j);
             };
             CellLoads<T> cur, nxt;
             const int hs0 = blockIdx.z + gridDim.z * slot, hsn = gridDim.z * hsw;
@@ -388,54 +401,63 @@ __global__ void convblock_backward_x_tiled_kernel(const T *__restrict__ gy, cons
                 const T *fc = folded + (int64_t)c * 28;
 #pragma unroll
                 for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
-                // phase 1: tree and tap gradients of every cell block of this chunk (registers only).
-                // No per-lane control flow: a lane without a cell recomputes cell 0 with a zero gradient.
-                int pos[kChunk];
-                T gt[kChunk][8];
+                pin_addends(tr);
+                // Two cell blocks at a time (the pinned addends serve both; the tap gradients of only two blocks are live):
+                // phase 1: tree and tap gradients of the pair (registers only).  No per-lane control flow: a lane
+                // without a cell recomputes cell 0 with a zero gradient.
+                // phase 2: read-add-write per tap.  For one tap the targets of all cells (all lanes, both blocks) are
+                // distinct elements, so the blocks of a pair go together; taps may collide with each other and are
+                // applied one after the other, and the pairs one after the other.  Only this wavefront touches the
+                // plane rows it owns.  Lanes without a cell, and (with bands) targets outside the owned rows, are
+                // redirected to a private dummy element per lane, so the whole phase is straight-line code with the
+                // LDS reads of a tap in flight together.
 #pragma unroll
-                for (int j = 0; j < kChunk; ++j) {
-                    const int code = cur.code[j];
-                    const T gout = cur.gy[j];                       // 0 for lanes without a cell
-                    pos[j] = cx[j] + (code >> 1) * row_step + (code & 1) * g.sw;
-                    T tv[8];
+                for (int jp = 0; jp < kChunk; jp += 2) {
+                    int pos[2];
+                    T gt[2][8];
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) tv[t] = xs[pos[j] + to[t]];
-                    const TreeVals<T> tvv = eval_tree(tr, tv);
-                    const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
-                    const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
+                    for (int jj = 0; jj < 2; ++jj) {
+                        const int j = jp + jj;
+                        const T gout = cur.gy[j];                   // 0 for lanes without a cell
+                        pos[jj] = cx[j] + (int)((cur.codes >> (8 * j + 1)) & 1) * row_step + (int)((cur.codes >> (8 * j)) & 1) * g.sw;
+                        T tv[8];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if ((mask >> (2 * q)) & 3) {                 // wave-uniform: a tap of this leaf is ours
-                            const int m = q >> 1;
-                            const T g_mid = m ? g_m1 : g_m0;
-                            const T g_leaf = g_mid * ((q & 1) ? gate_db(tr.g[4 + m], tvv.leaf[q ^ 1])
-                                                               : gate_da(tr.g[4 + m], tvv.leaf[q ^ 1]));
-                            gt[j][2 * q] = g_leaf * gate_da(tr.g[q], tv[2 * q + 1]);
-                            gt[j][2 * q + 1] = g_leaf * gate_db(tr.g[q], tv[2 * q]);
+                        for (int t = 0; t < 8; ++t) tv[t] = xs[pos[jj] + to[t]];
+                        const TreeVals<T> tvv = eval_tree(tr, tv);
+                        const T g_m0 = gout * gate_da(tr.g[6], tvv.mid[1]);
+                        const T g_m1 = gout * gate_db(tr.g[6], tvv.mid[0]);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            if ((mask >> (2 * q)) & 3) {             // wave-uniform: a tap of this leaf is ours
+                                const int m = q >> 1;
+                                const T g_mid = m ? g_m1 : g_m0;
+                                const T g_leaf = g_mid * ((q & 1) ? gate_db(tr.g[4 + m], tvv.leaf[q ^ 1])
+                                                                   : gate_da(tr.g[4 + m], tvv.leaf[q ^ 1]));
+                                gt[jj][2 * q] = g_leaf * gate_da(tr.g[q], tv[2 * q + 1]);
+                                gt[jj][2 * q + 1] = g_leaf * gate_db(tr.g[q], tv[2 * q]);
+                            }
                         }
                     }
-                }
-                // phase 2: read-add-write per tap.  For one tap the targets of all cells (all lanes,
-                // all blocks) are distinct elements, so the blocks of a chunk go together; taps may
-                // collide with each other and are applied one after the other.  Only this wavefront
-                // touches the plane rows it owns.  Lanes without a cell, and (with bands) targets
-                // outside the owned rows, are redirected to a private dummy element per lane, so the
-                // whole phase is straight-line code with the LDS reads of a tap in flight together.
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    if ((mask >> t) & 1) {                           // wave-uniform
-                        T old[kChunk];
-                        int at[kChunk];
+                    for (int t = 0; t < 8; ++t) {
+                        if ((mask >> t) & 1) {                       // wave-uniform
+                            T old[2];
+                            int at[2];
 #pragma unroll
-                        for (int j = 0; j < kChunk; ++j) {
-                            bool mine = live[j];
-                            if (BANDED) mine = mine && ((uint32_t)(pos[j] - img0 + tr_[t]) - own_lo) < own_len;
-                            at[j] = mine ? gw_off + pos[j] + to[t] : dummy_off;
+                            for (int jj = 0; jj < 2; ++jj) {
+                                if (FULL && !BANDED) {
+                                    at[jj] = gw_off + pos[jj] + to[t];
+                                } else {
+                                    bool mine = live[jp + jj];
+                                    if (BANDED) mine = mine && ((uint32_t)(pos[jj] - img0 + tr_[t]) - own_lo) < own_len;
+                                    at[jj] = mine ? gw_off + pos[jj] + to[t] : dummy_off;
+                                }
+                            }
+#pragma unroll
+                            for (int jj = 0; jj < 2; ++jj) old[jj] = xs[at[jj]];
+#pragma unroll
+                            for (int jj = 0; jj < 2; ++jj) xs[at[jj]] = old[jj] + gt[jj][t];
                         }
-#pragma unroll
-                        for (int j = 0; j < kChunk; ++j) old[j] = xs[at[j]];
-#pragma unroll
-                        for (int j = 0; j < kChunk; ++j) xs[at[j]] = old[j] + gt[j][t];
                     }
                 }
                 cur = nxt;
@@ -1156,17 +1178,22 @@ int launch_backward_x_tiled(const Geom &g, const TilePlan &p, const void *gy, co
     const dim3 grid((unsigned)clg_ceil_div(g.n, p.S), (unsigned)p.bands, (unsigned)p.hit_split), block(p.NW * kWave);
     T *part = reinterpret_cast<T *>(reinterpret_cast<unsigned char *>(scratch) + lay.part_off);
     T *out = p.hit_split > 1 ? part : (T *)gx;
-#define CLG_BWDX_TILED(BANDED, SHARED)                                                                                          \
+#define CLG_BWDX_TILED(BANDED, SHARED, FULL)                                                                                    \
     do {                                                                                                                        \
-        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, BANDED, SHARED>, p.lds_bytes, "clg_convblock_backward_x"))   \
+        if (int e = allow_lds(convblock_backward_x_tiled_kernel<T, BANDED, SHARED, FULL>, p.lds_bytes, "clg_convblock_backward_x")) \
             return e;                                                                                                           \
-        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, BANDED, SHARED>), grid, block, p.lds_bytes, st, (const T *)gy, \
-                           (const T *)x, (const T *)folded, (const int32_t *)count, (const int32_t *)hits, (const int32_t *)taps, \
-                           argmax, out, g, p);                                                                                  \
+        hipLaunchKernelGGL((convblock_backward_x_tiled_kernel<T, BANDED, SHARED, FULL>), grid, block, p.lds_bytes, st,          \
+                           (const T *)gy, (const T *)x, (const T *)folded, (const int32_t *)count, (const int32_t *)hits,        \
+                           (const int32_t *)taps, argmax, out, g, p);                                                           \
     } while (0)
-    if (p.bands > 1) CLG_BWDX_TILED(true, false);
-    else if (p.hsw > 1) CLG_BWDX_TILED(false, true);
-    else CLG_BWDX_TILED(false, false);
+    // whole images, one sample per wavefront pass, a multiple of kChunk * 64 cells per image and whole rows of pooled cells
+    // per block of 64: no idle lanes, and the cells of a lane are a uniform step apart
+    const bool full = p.bands == 1 && p.G == 1 && p.slots % (kChunk * kWave) == 0 && kWave % (g.wo / 2) == 0;
+    if (p.bands > 1) CLG_BWDX_TILED(true, false, false);
+    else if (p.hsw > 1 && full) CLG_BWDX_TILED(false, true, true);
+    else if (p.hsw > 1) CLG_BWDX_TILED(false, true, false);
+    else if (full) CLG_BWDX_TILED(false, false, true);
+    else CLG_BWDX_TILED(false, false, false);
 #undef CLG_BWDX_TILED
     CLG_CHECK_LAUNCH("clg_convblock_backward_x(tiled)");
     if (p.hit_split > 1) {

@@ -52,6 +52,23 @@ __device__ __forceinline__ Tree<T> load_tree(const T *__restrict__ w /* [7,16] o
     return t;
 }
 
+// A wave-uniform coefficient sits in a scalar register, and a vector instruction can read only one scalar register:
+// an FMA "scalar * vector + scalar" costs an extra move per use.  Pinning the ADDENDS (a, one) of every gate in vector
+// registers once per kernel visit leaves one scalar operand per FMA of gate() and gate_da(); the compiler cannot
+// undo the copy (it would, to save registers, and re-make it in front of every use).  float only: a double tree would
+// take 28 more registers than the kernels have.
+template <typename T>
+__device__ __forceinline__ void pin_addends(Tree<T> &t)
+{
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int k = 0; k < 7; ++k) {
+            asm volatile("" : "+v"(t.g[k].a));
+            asm volatile("" : "+v"(t.g[k].one));
+        }
+    }
+}
+
 template <typename T>
 struct TreeVals {
     T leaf[4], mid[2], root;
