@@ -858,9 +858,13 @@ __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_til
         if (n0 >= g.n) break;                                        // uniform over the workgroup
         const int s_cur = min(p.S, g.n - n0);
         __syncthreads();                                             // the previous round's reads (or the zero fill) are done
+        // (the LDS positions below are the same in every round; computed afresh so that they do not sit in -- or spill
+        // from -- nine registers while the round is evaluated)
+        uint32_t e0 = tid;
+        asm volatile("" : "+v"(e0));
 #pragma unroll
         for (int k = 0; k < kStagePerThread; ++k) {
-            const uint32_t e = tid + k * nthreads;
+            const uint32_t e = e0 + k * nthreads;
             if (e < group_elems) {
                 const uint32_t r = fdiv(e, p.d_w);
                 xs[rowbase[r] + (int)(e - r * (uint32_t)g.w)] = stage[k];
@@ -1303,6 +1307,8 @@ bool plan_backward_w_tiled(const Geom &g, int elem, TiledWPlan *tw)
     if (const char *e = clg_knob(K_BWDW_LDS))
         if (atoi(e) == 0) return false;
     if (!taps_inside(g) || g.c > 65535) return false;
+    if (elem != 4) return false;                                      // float only: the 28 sums, a tree and the staged elements of a
+                                                                     // double pass do not fit 128 registers (the padded-copy kernel serves double)
     TilePlan *p = &tw->p;
     plan_common(g, p);
     const int64_t I = (int64_t)(g.ho / 2) * (g.wo / 2);
@@ -1522,9 +1528,7 @@ static int convblock_backward_w_impl(int dtype, const clg_conv_geom *gg, const v
     TiledWPlan tw;
     const char *e_pad = clg_knob(K_BWDW_PADDED);
     if (!(e_pad && atoi(e_pad) != 0) && plan_backward_w_tiled(g, elem_size(dtype), &tw)) {     // images in LDS (CLG_BWDW_PADDED=1 forces the padded copy)
-        if (dtype == CLG_F32)
-            return launch_backward_w_tiled<float>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
-        return launch_backward_w_tiled<double>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
+        return launch_backward_w_tiled<float>(g, tw, grad_y, x, w, selection, argmax, grad_w, scratch, clg_stream(stream), probs);
     }
     TilePlan p;
     WScratch ws;
