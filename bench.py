@@ -367,7 +367,7 @@ def bench_c1(steps, warmup, cpu=True):
     alg = (2 * batch * in_dim * 4 + out_dim * 16 + out_dim * 16 * 4) + (3 * batch * in_dim * 4 + out_dim * 16 * 4 + 4 * out_dim * 8 + in_dim * 8)
     out = {"workload": "C1: LogicLayer 8000->8000, batch 256, float32, fwd+bwd (module API, incl. layout transposes)",
            "metric": "fc_fwd_bwd_Ggate_evals_per_s", "value": gate_evals / sec / 1e9, "unit": "Ggate-evals/s", "ms_per_step": sec * 1e3,
-           "dtype": "f32", "roofline": _roof("fc fwd+bwd step (all kernels)", alg, _avg_ms(pairs)),
+           "dtype": "f32", "roofline": _roof("fc fwd+bwd step (all kernels)", alg, _avg_ms(pairs), {"traffic": _traffic("c1", "step_bytes")}),
            "ms_per_step_hip_graph": graph_ms,
            "value_hip_graph": (gate_evals / (graph_ms * 1e-3) / 1e9) if graph_ms else None}
     def cpu_leg():

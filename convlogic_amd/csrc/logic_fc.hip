@@ -635,8 +635,7 @@ __global__ __launch_bounds__(kSmOutWaves * kWave) void fc_backward_fused_smout_k
         int64_t i;
         if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i)) {
             T *row = tile + (size_t)(wave * ROWS + lane / LPR) * bp + (lane % LPR) * VEC;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) row[k] = acc.v[k];
+            store_vec<T, VEC>(row, acc);                             // one wide LDS store (bp is a multiple of 4 elements)
         }
     }
     __syncthreads();

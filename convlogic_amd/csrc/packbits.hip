@@ -323,7 +323,7 @@ __global__ __launch_bounds__(FL *SG) void pack_bits_tile_kernel(const uint8_t *_
                 lo |= ((acc[o][q] >> (8 * b)) & 0xFFu) << (8 * o);
                 hi |= ((acc[4 + o][q] >> (8 * b)) & 0xFFu) << (8 * o);
             }
-            tile[fl * 16 + 4 * q + b][sg] = ((uint64_t)hi << 32) | lo;
+            tile[(4 * q + b) * FL + fl][sg] = ((uint64_t)hi << 32) | lo;   // feature-lane fastest: the lanes of a wavefront spread over the banks
         }
     }
     __syncthreads();
@@ -332,7 +332,7 @@ __global__ __launch_bounds__(FL *SG) void pack_bits_tile_kernel(const uint8_t *_
         const int row = idx / SG, w = idx % SG;
         const int64_t f = frow0 + row, byte0 = (grp0 + w) * 8;
         if (f >= features || byte0 >= row_bytes) continue;
-        const uint64_t word = tile[row][w];
+        const uint64_t word = tile[(row % 16) * FL + row / 16][w];
         uint8_t *dst = out + f * row_bytes + byte0;
         const int64_t nbytes = row_bytes - byte0 < 8 ? row_bytes - byte0 : 8;
         if (nbytes == 8 && (row_bytes & 7) == 0) {
