@@ -95,7 +95,15 @@ __global__ __launch_bounds__(256) void reduce_coef_partials_kernel(const T *__re
     const int q = (int)(gate - row * G);
     const T *p = partial + (row * nb * G + q) * 4 + (i & 3);
     T acc = 0;
-    for (int blk = i >> 2; blk < nb; blk += 4) acc += p[(int64_t)blk * G * 4];
+    int blk = i >> 2;
+    for (; blk + 28 < nb; blk += 32) {                               // eight loads in flight, added in the same order as one by one
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(int64_t)(blk + 4 * u) * G * 4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; blk < nb; blk += 4) acc += p[(int64_t)blk * G * 4];
     acc += __shfl_xor(acc, 4, 16);
     acc += __shfl_xor(acc, 8, 16);
     const T s0 = __shfl(acc, 0, 16), s1 = __shfl(acc, 1, 16), s2 = __shfl(acc, 2, 16), s3 = __shfl(acc, 3, 16);
