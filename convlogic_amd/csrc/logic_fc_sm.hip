@@ -2,7 +2,10 @@
 // API hands over at the boundary of a LogicLayer stack.  The feature-major kernels (logic_fc.hip) need a transposed copy
 // of x on the way in and of grad_y / grad_x on the way back; here a workgroup stages whole sample rows in LDS instead
 // (x[s, :] for the forward, x[s, :] and grad_y[s, :] for the input gradient), lanes run along neurons or input features,
-// gather from LDS and read / write global memory in contiguous rows.  For layers whose rows fit LDS.
+// gather from LDS and read / write global memory in contiguous rows.  For layers whose rows fit LDS.  An OPTION
+// (clg_fc_sm_preferred): on the GPU the feature-major kernels plus their transposed copies are faster at 8000 -> 8000
+// neurons and 256 samples, because summing over samples is a lane reduction there and a second pass with partial sums
+// here; these kernels need fewer microseconds of host launch work.
 //
 // Tables made once per wiring by clg_fc_sm_plan (host):
 //   ab32    int32 [out, 2]     the two inputs of every neuron
@@ -23,9 +26,9 @@ int clg_allow_lds(const void *kernel, size_t bytes, const char *name);
 
 namespace {
 
-constexpr int kSmBlock = 1024;   // 16 wavefronts per workgroup: the loops below are chains of L2 round trips, so many lanes and
+constexpr int kSmBlock = 1024;   // 16 wavefronts per workgroup and kSmUnroll independent items per lane: the loops below are
+constexpr int kSmUnroll = 4;     // chains of L2 round trips, and that is what hides them
 constexpr int kSmWNeurons = 2;   // neurons per lane of the weight-gradient kernel
-constexpr int kSmUnroll = 4;     // several independent items per lane are what hides them
 constexpr int kSmLdsBudget = 150 * 1024;    // rows a workgroup may hold
 constexpr int kSmMaxParts = 64;             // partial sums per neuron the scratch buffer holds
 
