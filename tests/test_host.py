@@ -320,3 +320,19 @@ def test_compiled_net_netlist_file_round_trip(tmp_path):
     assert len(back.stages) == 6 and back.num_classes == 10
     for s, t in zip(net.stages, back.stages):
         assert s[0] == t[0] and all(np.array_equal(np.asarray(u), np.asarray(v)) for u, v in zip(s[1:], t[1:]))
+
+
+def test_recorded_traffic_file_feeds_the_bench_line():
+    # bench.py reports `roofline.traffic` from profiles/traffic.json (recorded rocprofv3 counters): the file names the
+    # commit and method, and holds the entries bench.py asks for; a missing entry reads as None, never as a guess
+    import json
+    import bench
+    with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+        rec = json.load(f)
+    assert rec["commit"] and "rocprofv3 --pmc FETCH_SIZE" in rec["method"]
+    assert bench._traffic("c2", "eval_packed_walk_kernel_bytes_per_launch") == rec["workloads"]["c2"]["eval_packed_walk_kernel_bytes_per_launch"]
+    for wl in ("c4", "c3", "c1"):
+        got = bench._traffic(wl, "step_bytes")
+        assert got == rec["workloads"][wl]["step_bytes"] and got > 0
+        assert abs(sum(k["bytes_per_launch"] * k["launches_per_step"] for k in rec["workloads"][wl]["kernels"].values()) - got) <= len(rec["workloads"][wl]["kernels"])
+    assert bench._traffic("c9", "step_bytes") is None and bench._traffic("c4", "no_such_key") is None
