@@ -706,13 +706,23 @@ template <typename T>
 __global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t batch,
                                                              int k, int slices, T inv_tau)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;       // sample fastest: the loads of a wavefront are contiguous
     if (i >= batch * k) return;
-    const int64_t b = i / k;
-    const int g = (int)(i - b * k);
+    const int g = (int)(i / batch);
+    const int64_t b = i - (int64_t)g * batch;
+    const T *p = partial + (int64_t)g * batch + b;
+    const int64_t step = (int64_t)k * batch;
     T acc = 0;
-    for (int s = 0; s < slices; ++s) acc += partial[((int64_t)s * k + g) * batch + b];
-    out[i] = acc * inv_tau;
+    int s = 0;
+    for (; s + 8 <= slices; s += 8) {                                // eight loads in flight, added in slice order
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(s + u) * step];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; s < slices; ++s) acc += p[s * step];
+    out[b * k + g] = acc * inv_tau;
 }
 // grad_x[f][b] = grad_out[b][class of f] * (1 / tau); a workgroup writes 64 feature rows of one 64-sample column chunk
 template <typename T>
