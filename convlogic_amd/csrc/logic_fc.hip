@@ -948,6 +948,21 @@ extern "C" int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a,
     return CLG_OK;
 }
 
+extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64_t rows, int64_t cols, void *stream);
+
+extern "C" int clg_fc_forward_logits_ex(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *logits,
+                                        void *probs, void *folded, void *y, int64_t in_dim, int64_t out_dim, int64_t batch,
+                                        int flags, void *x_fm, void *stream)
+{
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_forward_logits")) return e;
+    CLG_REQUIRE((flags & ~CLG_FC_X_SAMPLE_MAJOR) == 0, "clg_fc_forward_logits: unknown flags 0x%x", flags);
+    if ((flags & CLG_FC_X_SAMPLE_MAJOR) == 0)
+        return clg_fc_forward_logits(dtype, x, a, b, logits, probs, folded, y, in_dim, out_dim, batch, stream);
+    CLG_REQUIRE(x && x_fm, "clg_fc_forward_logits: CLG_FC_X_SAMPLE_MAJOR needs x [batch, in_dim] and room for its copy [in_dim, batch]");
+    if (int e = clg_transpose_2d(dtype == CLG_F64 ? 8 : 4, x, x_fm, batch, in_dim, stream)) return e;
+    return clg_fc_forward_logits(dtype, x_fm, a, b, logits, probs, folded, y, in_dim, out_dim, batch, stream);
+}
+
 extern "C" int clg_fc_forward_logits(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *logits,
                                      void *probs, void *folded, void *y, int64_t in_dim, int64_t out_dim, int64_t batch,
                                      void *stream)
@@ -1054,12 +1069,19 @@ extern "C" int clg_fc_backward_fused_fits(int dtype, int64_t batch)
 extern "C" int clg_fc_backward_fused_ex(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
                                         const void *probs, const void *grad_y, const int64_t *csr_start, const int64_t *csr_list,
                                         void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int flags,
-                                        void *stream)
+                                        void *scratch, void *stream)
 {
     const char *name = "clg_fc_backward_fused";
     if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
     CLG_REQUIRE(x && a && b && folded && grad_y && csr_start && csr_list && grad_x && grad_w, "%s: null pointer argument", name);
-    CLG_REQUIRE((flags & ~CLG_FC_GX_SAMPLE_MAJOR) == 0, "%s: unknown flags 0x%x", name, flags);
+    CLG_REQUIRE((flags & ~(CLG_FC_GX_SAMPLE_MAJOR | CLG_FC_GY_SAMPLE_MAJOR)) == 0, "%s: unknown flags 0x%x", name, flags);
+    if (flags & CLG_FC_GY_SAMPLE_MAJOR) {                            // grad_y [batch, out_dim]: its feature-major copy goes to scratch
+        CLG_REQUIRE(scratch, "%s: CLG_FC_GY_SAMPLE_MAJOR needs scratch for out_dim * batch elements", name);
+        CLG_REQUIRE(batch <= fused_batch_limit(dtype, batch), "%s: batch %lld exceeds what one pass covers (%lld)", name, (long long)batch,
+                    (long long)fused_batch_limit(dtype, batch));
+        if (int e = clg_transpose_2d(dtype == CLG_F64 ? 8 : 4, grad_y, scratch, batch, out_dim, stream)) return e;
+        grad_y = scratch;
+    }
     CLG_REQUIRE(batch <= fused_batch_limit(dtype, batch),
                 "%s: batch %lld exceeds what one pass covers (%lld); use clg_fc_backward_x_folded and clg_fc_backward_logits", name,
                 (long long)batch, (long long)fused_batch_limit(dtype, batch));
@@ -1106,7 +1128,7 @@ extern "C" int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a,
                                      void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream)
 {
     return clg_fc_backward_fused_ex(dtype, x, a, b, folded, probs, grad_y, csr_start, csr_list, grad_x, grad_w, in_dim, out_dim, batch, 0,
-                                    stream);
+                                    nullptr, stream);
 }
 
 extern "C" int clg_transpose_2d(int elem_size, const void *src, void *dst, int64_t rows, int64_t cols, void *stream)

@@ -329,8 +329,9 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
     def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False,
                 sample_major_input=False):
         if sample_major_input:                                       # x is [B, in]: its gradient goes back in that layout
-            x = difflogic_hip.transpose(x)
-        y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False)   # the module has checked its buffers
+            y, w, folded, x = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False, sample_major_x=True)
+        else:
+            y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False)   # the module has checked its buffers
         ctx.save_for_backward(x, a, b, w, folded, given_x_indices_of_y_start, given_x_indices_of_y)
         ctx.sole_consumers = sole_consumers
         ctx.sample_major_input = sample_major_input
@@ -339,12 +340,20 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y):
         x, a, b, w, folded, start, flat = ctx.saved_tensors
+        fused = (not ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]
+                 and grad_y.numel() <= _FUSED_BACKWARD_MAX_ELEMS and difflogic_hip.backward_fused_fits(x))
+        if fused and not grad_y.is_contiguous() and grad_y.is_cuda and grad_y.dim() == 2 and grad_y.transpose(0, 1).is_contiguous():
+            # the gradient of a [B, out] consumer arrives as a transposed view: its feature-major copy is made by the call
+            # that computes both gradients
+            gy_sm = grad_y.transpose(0, 1)
+            grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, gy_sm, start, flat, validate=_needs_check(gy_sm, x),
+                                                          sample_major_grad_x=ctx.sample_major_input, sample_major_grad_y=True)
+            return grad_x, None, None, grad_l, None, None, None, None
         grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
         grad_x = grad_l = None
         if ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]:
             grad_x, grad_l = difflogic_hip.backward_sole(x, a, b, folded, w, grad_y, validate=_needs_check(grad_y, x))
-        elif (ctx.needs_input_grad[0] and ctx.needs_input_grad[3] and grad_y.numel() <= _FUSED_BACKWARD_MAX_ELEMS
-              and difflogic_hip.backward_fused_fits(x)):
+        elif fused:
             # (a sample-major input takes its gradient sample-major straight from the kernel)
             grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, grad_y, start, flat, validate=_needs_check(grad_y, x),
                                                           sample_major_grad_x=ctx.sample_major_input)

@@ -41,7 +41,8 @@ SIGNATURES = {
     "clg_fc_forward_logits": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_fused_fits": (_i, [_i, _i64]),
     "clg_fc_backward_fused": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
-    "clg_fc_backward_fused_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p]),
+    "clg_fc_backward_fused_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
+    "clg_fc_forward_logits_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
     "clg_fc_sm_fits": (_i, [_i, _i64, _i64, _i64]),
     "clg_fc_sm_preferred": (_i, [_i, _i64, _i64, _i64]),
     "clg_fc_sm_plan": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p]),

@@ -88,22 +88,38 @@ def forward_folded(x, a, b, folded):
     return y
 
 
-def forward_logits(x, a, b, logits, validate=True):
-    """fold(from_logits=True) + forward_folded() in one launch -> (y [out, B], probs [out, 16], folded [out, 4])."""
+def forward_logits(x, a, b, logits, validate=True, sample_major_x=False):
+    """fold(from_logits=True) + forward_folded() in one launch -> (y [out, B], probs [out, 16], folded [out, 4]).
+    sample_major_x: x is [B, in]; the same call makes its feature-major copy [in, B] first and returns it as a fourth
+    value (the backward functions read it)."""
     out_dim = logits.shape[0]
     if validate:
         if logits.dim() != 2 or logits.shape[1] != 16 or logits.dtype != x.dtype or x.dtype not in _lib._DTYPES:
             raise RuntimeError(f"forward_logits expects float32/float64 logits [out, 16] of x's dtype, got {tuple(logits.shape)} {logits.dtype}")
-        _wiring(x, a, b, out_dim)
+        if sample_major_x:
+            check_input(x, "x")
+            if x.dim() != 2:
+                raise RuntimeError(f"x must be 2-D, got {tuple(x.shape)}")
+            check_input(a, "a", _I64, (out_dim,))
+            check_input(b, "b", _I64, (out_dim,))
+            _lib.check_same_device(x, a, b)
+        else:
+            _wiring(x, a, b, out_dim)
         check_input(logits, "w")
-    in_dim, batch = x.shape
+    in_dim, batch = (x.shape[1], x.shape[0]) if sample_major_x else x.shape
     y = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device)
     probs = torch.empty_like(logits)
     folded = torch.empty((out_dim, 4), dtype=x.dtype, device=x.device)
-    check(_lib.load().clg_fc_forward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), logits.data_ptr(),
-                                            probs.data_ptr(), folded.data_ptr(), y.data_ptr(), in_dim, out_dim, batch,
-                                            stream_ptr(x)))
-    return y, probs, folded
+    if not sample_major_x:
+        check(_lib.load().clg_fc_forward_logits(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), logits.data_ptr(),
+                                                probs.data_ptr(), folded.data_ptr(), y.data_ptr(), in_dim, out_dim, batch,
+                                                stream_ptr(x)))
+        return y, probs, folded
+    x_fm = torch.empty((in_dim, batch), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_forward_logits_ex(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), logits.data_ptr(),
+                                               probs.data_ptr(), folded.data_ptr(), y.data_ptr(), in_dim, out_dim, batch,
+                                               1, x_fm.data_ptr(), stream_ptr(x)))
+    return y, probs, folded, x_fm
 
 
 def backward_x_folded(x, a, b, folded, grad_y, given_x_indices_of_y_start, given_x_indices_of_y, validate=True):
@@ -148,27 +164,30 @@ def backward_fused_fits(x):
 
 
 def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, given_x_indices_of_y, validate=True,
-                   sample_major_grad_x=False):
+                   sample_major_grad_x=False, sample_major_grad_y=False):
     """(grad_x, grad_w) of a layer with any wiring in one pass (see backward_fused_fits); grad_w is the gradient
     w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities.  Same values as
     backward_x_folded() + backward_w() / backward_logits().  sample_major_grad_x: grad_x comes back [B, in] instead of
-    [in, B] (the kernel writes it transposed; same values)."""
+    [in, B] (the kernel writes it transposed; same values).  sample_major_grad_y: grad_y is [B, out]; the same call makes
+    its feature-major copy first."""
     out_dim = folded.shape[0] if folded.dim() else -1
     if validate:
         _wiring(x, a, b, out_dim)
         check_input(folded, "folded", x.dtype, (out_dim, 4))
-        check_input(grad_y, "grad_y", x.dtype, (out_dim, x.shape[1]))
+        check_input(grad_y, "grad_y", x.dtype, (x.shape[1], out_dim) if sample_major_grad_y else (out_dim, x.shape[1]))
         _reverse_map(x, given_x_indices_of_y_start, given_x_indices_of_y, out_dim)
         if probs is not None:
             check_input(probs, "w", x.dtype, (out_dim, 16))
     in_dim, batch = x.shape
     gx = torch.empty((batch, in_dim) if sample_major_grad_x else (in_dim, batch), dtype=x.dtype, device=x.device)
     gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    gy_fm = torch.empty((out_dim, batch), dtype=x.dtype, device=x.device) if sample_major_grad_y else None
     check(_lib.load().clg_fc_backward_fused_ex(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
                                                probs.data_ptr() if probs is not None else None, grad_y.data_ptr(),
                                                given_x_indices_of_y_start.data_ptr(), given_x_indices_of_y.data_ptr(),
                                                gx.data_ptr(), gw.data_ptr(), in_dim, out_dim, batch,
-                                               1 if sample_major_grad_x else 0, stream_ptr(x)))
+                                               (1 if sample_major_grad_x else 0) | (2 if sample_major_grad_y else 0),
+                                               gy_fm.data_ptr() if sample_major_grad_y else None, stream_ptr(x)))
     return gx, gw
 
 

@@ -143,14 +143,24 @@ int clg_fc_backward_fused(int dtype, const void *x, const int64_t *a, const int6
                           const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, const int64_t *csr_start,
                           const int64_t *csr_list, void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch,
                           void *stream);
-/* The same with flags: CLG_FC_GX_SAMPLE_MAJOR writes grad_x sample-major, [batch, in_dim] (what autograd hands to the
- * producer of a [batch, in_dim] input), straight from the kernel -- the transposed copy of grad_x that
- * LogicLayerCudaFunction.backward makes (src/difflogic/difflogic.py:225-229) disappears; same values bit for bit. */
+/* The same with flags, for a layer called on [batch, features] tensors (src/difflogic/difflogic.py:125-147, :214-230 make a
+ * transposed copy of x, of grad_y and of grad_x there):
+ *   CLG_FC_GX_SAMPLE_MAJOR  grad_x is written sample-major, [batch, in_dim], straight from the kernel; same values bit for bit
+ *   CLG_FC_GY_SAMPLE_MAJOR  grad_y is [batch, out_dim]; its feature-major copy is made into scratch (out_dim * batch elements)
+ *                           by the same call */
 #define CLG_FC_GX_SAMPLE_MAJOR 1
+#define CLG_FC_GY_SAMPLE_MAJOR 2
 int clg_fc_backward_fused_ex(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
                              const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, const int64_t *csr_start,
                              const int64_t *csr_list, void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch,
-                             int flags, void *stream);
+                             int flags, void *scratch /*or NULL*/, void *stream);
+/* clg_fc_forward_logits with flags: CLG_FC_X_SAMPLE_MAJOR takes x as [batch, in_dim] and leaves its feature-major copy
+ * [in_dim, batch] in x_fm (what the backward entry points read) -- the x.transpose(0, 1).contiguous() of
+ * LogicLayer.forward_cuda (src/difflogic/difflogic.py:130-133) and the forward in one call. */
+#define CLG_FC_X_SAMPLE_MAJOR 1
+int clg_fc_forward_logits_ex(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *logits,
+                             void *probs /*[out_dim,16]*/, void *folded /*[out_dim,4]*/, void *y, int64_t in_dim, int64_t out_dim,
+                             int64_t batch, int flags, void *x_fm /*[in_dim,batch] or NULL*/, void *stream);
 
 /* The layer on SAMPLE-major tensors, x [batch, in_dim] -> y [batch, out_dim] (what the module API hands over at the
  * boundary of a LogicLayer stack), for layers whose sample rows fit LDS (clg_fc_sm_fits() != 0): no transposed copies

@@ -324,6 +324,10 @@ def test_fused_backward_equals_the_two_kernels(in_dim, out_dim, batch, dtype):
         # the same sums with the input gradient written [batch, in] by the kernel itself
         gx_sm, gw_sm = difflogic_hip.backward_fused(x, *tabs, folded, p_arg, gy, *csr, sample_major_grad_x=True)
         assert gx_sm.shape == (batch, in_dim) and torch.equal(gx_sm, gx_ref.t()) and torch.equal(gw_sm, gw_ref)
+        # ... and with grad_y handed over as [batch, out] (its feature-major copy made inside the call)
+        gx_io, gw_io = difflogic_hip.backward_fused(x, *tabs, folded, p_arg, gy.t().contiguous(), *csr, sample_major_grad_x=True,
+                                                    sample_major_grad_y=True)
+        assert torch.equal(gx_io, gx_sm) and torch.equal(gw_io, gw_ref)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
@@ -344,6 +348,9 @@ def test_forward_from_logits_folds_inside(in_dim, out_dim, batch, dtype):
     assert torch.equal(y, difflogic_hip.forward_folded(x, *tabs, folded))
     want = O.logic_fc_forward(x.T.cpu(), layer.indices_0.cpu(), layer.indices_1.cpu(), torch.softmax(logits.cpu(), -1))
     assert (y.T.cpu() - want).abs().max().item() <= (1e-5 if dtype == torch.float32 else 1e-12)
+    # handed a [batch, in] tensor, the same call makes the feature-major copy first: same outputs, and the copy comes back
+    y2, probs2, folded2, x_fm = difflogic_hip.forward_logits(x.t().contiguous(), *tabs, logits, sample_major_x=True)
+    assert torch.equal(x_fm, x) and torch.equal(y2, y) and torch.equal(probs2, probs) and torch.equal(folded2, folded)
     with pytest.raises(RuntimeError):
         difflogic_hip.forward_logits(x, *tabs, logits[:, :8].contiguous())
 
