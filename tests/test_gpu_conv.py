@@ -200,10 +200,11 @@ def test_block_benchmark_shapes_vs_oracle(shape):
 
 
 @pytest.mark.parametrize("shape", [(37, 24, 48, 4, 4), (5, 200, 40, 16, 16), (3, 64, 32, 32, 32), (9, 40, 24, 6, 6),
-                                   (70, 6, 12, 2, 2), (4, 1024, 2048, 4, 4)])
+                                   (70, 6, 12, 2, 2), (4, 1024, 2048, 4, 4), (2, 3, 8, 64, 64), (3, 2, 6, 32, 64), (2, 4, 5, 64, 32)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_block_deep_and_wide_shapes_vs_oracle(shape, dtype):
-    # few cells per sample (several samples share a wavefront, ragged last group) and images too large for LDS
+    # few cells per sample (several samples share a wavefront, ragged last group), images too large for LDS, and images of
+    # several passes of 256 pooled cells (rows of 32 and 16 cells: the no-idle-lane input gradient steps from block to block)
     n, cin, cout, h, w = shape
     layer, x, y, idx = _run_block(n, cin, cout, h, w, 1, 1, 3, dtype=dtype, seed=n)
     gy = torch.randn_like(y)
