@@ -566,7 +566,7 @@ def bench_c5(steps, warmup, cpu=True):
     out = {"workload": f"C5: ConvLogicCifarModel k={k}, 9 input channels, batch {n}, float32 training step (fwd + CE loss + bwd)",
            "metric": "convlogic_fwd_bwd_Ggate_evals_per_s", "value": ge / sec / 1e9, "unit": "Ggate-evals/s", "ms_per_step": sec * 1e3,
            "dtype": "f32", "ms_per_step_hip_graph": graph_ms, "value_hip_graph": (ge / (graph_ms * 1e-3) / 1e9) if graph_ms else None,
-           "roofline": _roof("whole training step (all kernels)", alg, graph_ms if graph_ms else sec * 1e3)}
+           "roofline": _roof("whole training step (all kernels)", alg, graph_ms if graph_ms else sec * 1e3, {"traffic": _traffic("c5", "step_bytes")})}
 
     # packed inference of the same network: thresholds + packing fused, 65536 samples
     model.eval()

@@ -324,14 +324,14 @@ def test_compiled_net_netlist_file_round_trip(tmp_path):
 
 def test_recorded_traffic_file_feeds_the_bench_line():
     # bench.py reports `roofline.traffic` from profiles/traffic.json (recorded rocprofv3 counters): the file names the
-    # commit and method, and holds the entries bench.py asks for; a missing entry reads as None, never as a guess
+    # commit of every measurement and the method, and holds the entries bench.py asks for; a missing entry reads as None, never as a guess
     import json
     import bench
     with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
         rec = json.load(f)
-    assert rec["commit"] and "rocprofv3 --pmc FETCH_SIZE" in rec["method"]
+    assert "rocprofv3 --pmc FETCH_SIZE" in rec["method"] and all(w["commit"] for w in rec["workloads"].values())
     assert bench._traffic("c2", "eval_packed_walk_kernel_bytes_per_launch") == rec["workloads"]["c2"]["eval_packed_walk_kernel_bytes_per_launch"]
-    for wl in ("c4", "c3", "c1"):
+    for wl in ("c4", "c3", "c1", "c5"):
         got = bench._traffic(wl, "step_bytes")
         assert got == rec["workloads"][wl]["step_bytes"] and got > 0
         assert abs(sum(k["bytes_per_launch"] * k["launches_per_step"] for k in rec["workloads"][wl]["kernels"].values()) - got) <= len(rec["workloads"][wl]["kernels"])
