@@ -498,7 +498,9 @@ __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const 
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = uniform((int)(threadIdx.x >> 6));
     const int groups = (g.n + p.G - 1) / p.G;
-    const int item = uniform((int)blockIdx.x * p.NW + wave);           // channel fastest: a workgroup shares its samples
+    // channel fastest: a workgroup shares its samples, and so do its neighbours on the same XCD (they read the same
+    // padded images through one L2)
+    const int item = uniform((int)xcd_contiguous_block(blockIdx.x, gridDim.x) * p.NW + wave);
     if (item >= groups * g.cin) return;
     const int grp = item / g.cin, ch = item - grp * g.cin;
     const int n0 = grp * p.G, g_here = min(p.G, g.n - n0);
@@ -630,7 +632,12 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
                                                                         T *__restrict__ partial, Geom g, TilePlan p,
                                                                         FastDiv d_cells, int sample_elems, int tap_stride)
 {
-    const int c = blockIdx.y, nb = gridDim.x;
+    // Workgroups that read the same samples (one sample block, every kernel) take consecutive logical numbers, so they run
+    // on one XCD and share its L2 (the hardware deals workgroups to the 8 XCDs round-robin over x + gridDim.x * y).
+    const int nb = gridDim.x;
+    const unsigned logical = xcd_contiguous_block(blockIdx.x + (unsigned)nb * blockIdx.y, (unsigned)nb * gridDim.y);
+    const int c = uniform((int)(logical % gridDim.y));
+    const uint32_t bx = uniform((int)(logical / gridDim.y));        // sample block
     const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
     const uint32_t items = (uint32_t)g.n * I;
     Tree<T> tr;
@@ -652,7 +659,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
     const uint32_t f_py = fdiv(f_cell, p.d_wp), f_px = f_cell - f_py * (uint32_t)wp;
     const uint32_t f_pos = (2 * f_py) * row_step + (2 * f_px) * g.sw;
     const uint32_t f_out = (uint32_t)(kernel_row + f_cell);
-    const uint32_t f_n0 = blockIdx.x * per_block + threadIdx.x / (uint32_t)I, f_step = (uint32_t)nb * per_block;
+    const uint32_t f_n0 = bx * per_block + threadIdx.x / (uint32_t)I, f_step = (uint32_t)nb * per_block;
     // tree, upstream gradients and the 28 sums of one pooled cell
     auto accumulate = [&](const T (&tv)[8], T gout) {
         const TreeVals<T> v = eval_tree(tr, tv);
@@ -694,7 +701,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
             accumulate(tv, gout);
         }
     } else {
-        for (uint32_t it = blockIdx.x * 256 + threadIdx.x; it < items; it += (uint32_t)nb * 256) {
+        for (uint32_t it = bx * 256 + threadIdx.x; it < items; it += (uint32_t)nb * 256) {
             const uint32_t n = fdiv(it, d_cells), cell = it - n * (uint32_t)I;
             const uint32_t py = fdiv(cell, p.d_wp), px = cell - py * (uint32_t)wp;
             const int64_t o = (int64_t)n * sample_cells + kernel_row + cell;
@@ -707,7 +714,7 @@ __global__ __launch_bounds__(256) void convblock_backward_w_padded_kernel(const 
             accumulate(tv, gout);
         }
     }
-    block_sum_store<T, 28, 256>(acc, partial + ((int64_t)c * nb + blockIdx.x) * 28);
+    block_sum_store<T, 28, 256>(acc, partial + ((int64_t)c * nb + bx) * 28);
 }
 
 

@@ -99,6 +99,16 @@ __device__ __forceinline__ T to_sgpr(T v)
     }
 }
 
+// Workgroup `bid` of a 1-D grid of `nb` runs on XCD bid % 8 (each XCD has its own L2).  Returns the logical block it
+// should take so that every XCD works on a CONTIGUOUS range of logical blocks: neighbours that read the same rows then
+// share one L2 instead of fetching them once per XCD.  A bijection of 0..nb-1 for any nb.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned bid, unsigned nb)
+{
+    constexpr unsigned kXcds = 8;
+    const unsigned q = nb / kXcds, r = nb % kXcds, xcd = bid % kXcds, idx = bid / kXcds;
+    return xcd < r ? xcd * (q + 1) + idx : r * (q + 1) + (xcd - r) * q + idx;
+}
+
 // ---- plan helpers (host) ---------------------------------------------------------------------
 static inline void plan_common(const Geom &g, TilePlan *p)
 {
