@@ -132,6 +132,30 @@ class _FullConvLogicLogitsFunction(Function):
         return grad_x, grad_l, None, None, None, None, None, None, None, None, None
 
 
+class _FullConvLogicBinaryFunction(Function):
+    """The complete block on an input that holds only 0 and 1 (the thresholded image in front of the first block,
+    src/convlogic/data.py:46-50): forward through one 256-entry table per kernel, backward from the saved tap bytes
+    alone.  w: the logits (is_logits, training path) or the probabilities.  Same y and pool routing as
+    FullConvLogicFunction bit for bit; gradients equal up to float rounding."""
+
+    @staticmethod
+    def forward(ctx, x, w, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, is_logits, flag):
+        x1, w1, selection = x.contiguous(), w.detach().contiguous(), selection.contiguous()
+        geo = (stride_h, stride_w, pad_h, pad_w)
+        y, taps, bctx = convlogic_hip.bin_forward(x1, w1, selection, *geo, kernel_h, kernel_w, flag, logits=is_logits)
+        ctx.save_for_backward(taps, bctx)                            # x itself is not needed again
+        ctx.geometry, ctx.x_shape, ctx.is_logits = geo, tuple(x1.shape), is_logits
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        taps, bctx = ctx.saved_tensors
+        grad_x, grad_w = convlogic_hip.bin_backward(grad_y.contiguous(), taps, bctx, ctx.x_shape, *ctx.geometry,
+                                                    need_grad_x=ctx.needs_input_grad[0], need_grad_w=ctx.needs_input_grad[1],
+                                                    wrt_logits=ctx.is_logits)
+        return grad_x, grad_w, None, None, None, None, None, None, None, None, None
+
+
 def _pair(v):
     return (v, v) if isinstance(v, int) else tuple(v)
 
@@ -152,6 +176,10 @@ class ConvLogicLayer(nn.Module):
         self.return_intermediate, self.return_indices = return_intermediate, return_indices
         self.input_bits = 8
         self.implementation = implementation
+        # A promise of the caller (the model topologies set it on their first block): every input element is 0 or 1.
+        # The "cuda" path then runs the binary-input kernels where they apply; the kernels verify the promise and
+        # check_binary_input() / the next forward call raise when it was broken.
+        self.binary_input = False
         if implementation == "cuda" and not torch.cuda.is_available():
             raise RuntimeError("CUDA implementation requested, but CUDA is not available.")
 
@@ -264,6 +292,17 @@ class ConvLogicLayer(nn.Module):
         sel = self._buffers["selection"].contiguous()
         weights = self._parameters["weights"]
         geo = (*self.stride, *self.padding, *self.kernel)
+        if (self.__dict__.get("binary_input") and self.complete and not self.return_intermediate and not self.return_indices
+                and x.is_cuda and x.dtype == torch.float32 and weights.dtype == torch.float32 and weights.device == x.device
+                and sel.device == x.device and convlogic_hip.bin_supported(x, self.out_channels, *geo)):
+            flag = self._binary_flag()
+            if flag.raised():
+                flag.clear()
+                raise RuntimeError("ConvLogicLayer(binary_input=True) was given an input with elements other than 0 and 1")
+            if self.training and weights.is_contiguous():
+                return _FullConvLogicBinaryFunction.apply(x, weights, sel, *geo, True, flag)
+            w_prob = gate_probabilities(self.weights, self.training, x.dtype).to(x.dtype).contiguous()
+            return _FullConvLogicBinaryFunction.apply(x, w_prob, sel, *geo, False, flag)
         if (self.complete and self.training and not self.return_intermediate and not self.return_indices and x.is_cuda
                 and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64) and weights.is_contiguous()
                 and weights.device == x.device and sel.device == x.device):
@@ -274,6 +313,24 @@ class ConvLogicLayer(nn.Module):
         if self.complete:
             return FullConvLogicFunction.apply(x, w_prob, sel, *geo, self.return_intermediate, self.return_indices)
         return ConvLogicFunction.apply(x, w_prob, sel, *geo)
+
+    def _binary_flag(self):
+        flag = self.__dict__.get("_bin_flag")
+        if flag is None:
+            flag = self.__dict__["_bin_flag"] = convlogic_hip.BinaryFlag()
+        return flag
+
+    def check_binary_input(self):
+        """Waits for the device and raises if a forward call since the last check saw an input element other than 0 or 1
+        although binary_input was set (without this call the violation is reported by the next forward call that runs
+        after the offending launch has finished)."""
+        flag = self.__dict__.get("_bin_flag")
+        if flag is None:
+            return
+        torch.cuda.synchronize()
+        if flag.raised():
+            flag.clear()
+            raise RuntimeError("ConvLogicLayer(binary_input=True) was given an input with elements other than 0 and 1")
 
     def forward_cuda_eval(self, x: PackBitsTensor):
         """Packed-bit inference of the complete block on a group-major image batch: replaces x.t by the

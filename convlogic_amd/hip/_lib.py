@@ -96,6 +96,12 @@ SIGNATURES = {
     "clg_convblock_plan_bytes": (_i64, [_i, _GP]),
     "clg_convblock_plan": (_i, [_i, _GP, _p, _p, _p, _p]),
     "clg_convblock_backward_planned": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i, _p, _p]),
+    "clg_convblock_bin_supported": (_i, [_i, _GP]),
+    "clg_convblock_bin_ctx_bytes": (_i64, [_i, _GP]),
+    "clg_convblock_bin_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _i, _p, _p]),
+    "clg_convblock_bin_backward_scratch_bytes": (_i64, [_i, _GP]),
+    "clg_convblock_bin_backward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _i, _p, _p]),
+    "clg_host_flag_device_pointer": (_i, [_p, _p]),
 }
 
 _lib = None

@@ -439,3 +439,73 @@ def threshold_pack_images(x, thresholds):
         check(_lib.load().clg_threshold_pack_images(x.data_ptr(), thresholds.data_ptr(), out.data_ptr(), n, c0, h * w, levels,
                                                     stream_ptr(x)))
     return out, groups * 64 - n
+
+
+# ---- fused block on binary inputs ---------------------------------------------------------------
+def bin_supported(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w):
+    """True when the binary-input kernels take a block on x (float32, stride 1, at most 32 columns, at most 256 pooled
+    cells per plane)."""
+    if not (x.is_cuda and x.dim() == 4 and x.dtype == torch.float32):
+        return False
+    g = _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    return bool(_lib.load().clg_convblock_bin_supported(dtype_code(x), ctypes.byref(g)))
+
+
+class BinaryFlag:
+    """One int32 in pinned host memory that the kernels set when an input promised to be binary is not: the host reads
+    it without a copy or a synchronisation (a violation therefore shows at the next check after the launch has run)."""
+
+    def __init__(self):
+        self.host = torch.zeros(1, dtype=torch.int32).pin_memory()
+        dev = ctypes.c_void_p(0)
+        check(_lib.load().clg_host_flag_device_pointer(self.host.data_ptr(), ctypes.byref(dev)))
+        self.device_ptr = dev.value
+
+    def raised(self):
+        return bool(self.host[0].item())
+
+    def clear(self):
+        self.host.zero_()
+
+
+def bin_forward(x, w, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, flag, logits=False, validate=True):
+    """Fused block on binary x (every element 0 or 1) -> (y [N,C,Ho/2,Wo/2], taps uint16 [N,C,Ho/2,Wo/2] = arg-max code
+    << 8 | tap byte, ctx: the buffer the backward call needs).  w: probabilities, or the logits with logits=True.
+    y and the arg-max equal full_convlogic_forward() bit for bit.  flag: a BinaryFlag, set when x is not binary."""
+    if validate:
+        _conv_args(x, w, selection, 7)
+    g = _geom(x, w.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
+    lib = _lib.load()
+    dt = dtype_code(x)
+    ctx = _scratch(lib.clg_convblock_bin_ctx_bytes(dt, ctypes.byref(g)), x.device)
+    ho, wo = _out_size(g)
+    shape = (g.n, g.c_out, ho // 2, wo // 2)
+    y = torch.empty(shape, dtype=x.dtype, device=x.device)
+    taps = torch.empty(shape, dtype=torch.int16, device=x.device)
+    check(lib.clg_convblock_bin_forward(dt, ctypes.byref(g), x.data_ptr(), w.data_ptr(), selection.data_ptr(), y.data_ptr(),
+                                        taps.data_ptr(), ctx.data_ptr(), 1 if logits else 0, flag.device_ptr, stream_ptr(x)))
+    return y, taps, ctx
+
+
+def bin_backward(grad_y, taps, ctx, x_shape, stride_h, stride_w, pad_h, pad_w, need_grad_x=True, need_grad_w=True, wrt_logits=False):
+    """-> (grad_x or None, grad_w [C,7,16] or None) of bin_forward() from grad_y [N,C,Ho/2,Wo/2], the saved taps and ctx.
+    grad_w is the gradient w.r.t. the logits with wrt_logits=True (the forward was given logits), else w.r.t. the
+    probabilities."""
+    check_input(grad_y, "grad_y", torch.float32, tuple(taps.shape))
+    check_input(taps, "taps", torch.int16)
+    check_input(ctx, "ctx", torch.uint8)
+    n, c_in, h, w = x_shape
+    c, hp, wp = grad_y.shape[1], grad_y.shape[2], grad_y.shape[3]
+    g = ConvGeom(n, c_in, h, w, c, stride_h, stride_w, pad_h, pad_w, h + 2 * pad_h - (2 * hp - 1) * stride_h, w + 2 * pad_w - (2 * wp - 1) * stride_w)
+    lib = _lib.load()
+    dt = dtype_code(grad_y)
+    if ctx.numel() < lib.clg_convblock_bin_ctx_bytes(dt, ctypes.byref(g)):
+        raise RuntimeError("ctx is smaller than clg_convblock_bin_ctx_bytes() for this geometry")
+    gx = torch.empty(x_shape, dtype=grad_y.dtype, device=grad_y.device) if need_grad_x else None
+    gw = torch.empty((c, 7, 16), dtype=grad_y.dtype, device=grad_y.device) if need_grad_w else None
+    scratch = _scratch(lib.clg_convblock_bin_backward_scratch_bytes(dt, ctypes.byref(g)), grad_y.device) if need_grad_w else None
+    if need_grad_x or need_grad_w:
+        check(lib.clg_convblock_bin_backward(dt, ctypes.byref(g), grad_y.data_ptr(), taps.data_ptr(), ctx.data_ptr(),
+                                             gx.data_ptr() if need_grad_x else None, gw.data_ptr() if need_grad_w else None,
+                                             1 if wrt_logits else 0, scratch.data_ptr() if need_grad_w else None, stream_ptr(grad_y)))
+    return gx, gw

@@ -442,6 +442,34 @@ int clg_convblock_backward_planned(int dtype, const clg_conv_geom *g, const void
                                    const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
                                    int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream);
 
+/* The fused block on BINARY inputs (every x is 0 or 1: the first block of a network, behind the threshold transform of
+ * src/convlogic/data.py:46-50).  float32, stride 1, images at most 32 columns wide, at most 256 pooled cells (a multiple
+ * of 4) per plane: clg_convblock_bin_supported.  A kernel's tree is then a 256-entry table over its 8 tap bits, made with
+ * the same gate arithmetic as clg_convblock_forward, so y and the pooled position are bit-identical to that entry point.
+ *   forward   y [n,c_out,ho/2,wo/2]; taps uint16 [n,c_out,ho/2,wo/2] = (dy*2+dx of the first maximum) << 8 | tap byte
+ *             (bit i = tap i of the kernel at that position); ctx: clg_convblock_bin_ctx_bytes() bytes that the caller
+ *             keeps for the backward call (bit rows of x, tables, folded coefficients, probabilities, per-channel
+ *             kernel lists).  flags: CLG_FWD_W_LOGITS as for clg_convblock_forward_ex.  *not_binary (device-writable
+ *             int32, e.g. pinned host memory) is set to 1 when some x is neither 0 nor 1 -- y is then undefined; it is
+ *             never cleared.
+ *   backward  from grad_y, taps and ctx alone (x is not read): grad_x [n,c_in,h,w] and / or grad_w [c_out,7,16]
+ *             (either may be NULL); flags: CLG_BWD_WRT_LOGITS.  scratch: clg_convblock_bin_backward_scratch_bytes().
+ *             Deterministic; equal to clg_convblock_backward(_logits) up to float rounding.
+ * Replaces full_convlogic_forward / full_convlogic_backward_x / full_convlogic_backward_weight
+ * (src/convlogic/cuda/convlogic.cpp:39-43; src/convlogic/cuda/full_convlogic_kernel.cu:10-145,233-363,463-701) for
+ * binary inputs. */
+int clg_convblock_bin_supported(int dtype, const clg_conv_geom *g);
+/* Device address of a flag word in PINNED host memory (hipHostMalloc), for `not_binary`: the host can then read the flag
+ * without a copy or a synchronisation.  CLG_EINVAL when `host` is not pinned memory mapped for the current device.  No
+ * counterpart in the reference (its kernels do not check their inputs). */
+int clg_host_flag_device_pointer(void *host, void **device);
+int64_t clg_convblock_bin_ctx_bytes(int dtype, const clg_conv_geom *g);
+int clg_convblock_bin_forward(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection, void *y,
+                              uint16_t *taps, void *ctx, int flags, int32_t *not_binary, void *stream);
+int64_t clg_convblock_bin_backward_scratch_bytes(int dtype, const clg_conv_geom *g);
+int clg_convblock_bin_backward(int dtype, const clg_conv_geom *g, const void *grad_y, const uint16_t *taps, const void *ctx,
+                               void *grad_x, void *grad_w, int flags, void *scratch, void *stream);
+
 /* ---------------------------------------------------------------------------------
  * input binarisation (the step in front of the first layer)
  * --------------------------------------------------------------------------------- */
