@@ -412,7 +412,9 @@ BWD_LANE_OPS_PER_POOLED_CELL = 21 + 14 + 14 + 35 + 8
 
 def _block_kernels(layer, xd, gy, reps):
     """Forward, input-gradient and weight-gradient entry points of one block timed one by one with events (each entry
-    point's launches together), with the HBM roofline of each and the fp32 lane-operation floors beside it."""
+    point's launches together), with the HBM roofline of each and the fp32 lane-operation floors beside it.  A block
+    whose input is declared binary (layer.binary_input) is timed through the binary-input entry points it runs, and the
+    any-input entry points are timed beside them (`generic_kernel_ms`)."""
     import torch
     from convlogic_amd.hip import convlogic_hip
 
@@ -421,34 +423,74 @@ def _block_kernels(layer, xd, gy, reps):
     wp = torch.softmax(layer.weights.detach(), -1).contiguous()
     sel = layer.selection
     geo = (1, 1, 1, 1)
+
+    def timed(calls):
+        """per entry point: `inner` consecutive calls captured into one HIP graph (so that the host's per-call cost --
+        allocations, ctypes -- does not leave the GPU idle between the launches of a call), replayed `reps` times between
+        two events on the launch stream; eager calls between events when capture is not possible"""
+        inner, out = 8, {}
+        for name, fn in calls.items():
+            try:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    fn()
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(inner):
+                        fn()
+                graph.replay()
+                ev = _events(reps)
+                for a_, b_ in ev:
+                    a_.record()
+                    graph.replay()
+                    b_.record()
+                torch.cuda.synchronize()
+                out[name] = _avg_ms(ev) / inner
+            except Exception as exc:  # noqa: BLE001
+                print(f"bench.py: entry point {name} timed eagerly ({exc})", file=sys.stderr)
+                ev = _events(reps)
+                for a_, b_ in ev:
+                    a_.record()
+                    fn()
+                    b_.record()
+                torch.cuda.synchronize()
+                out[name] = _avg_ms(ev)
+        return out
+
     y, am = convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
-    ev = {name: _events(reps) for name in ("fwd", "bwd_x", "bwd_w")}
-    for r in range(reps):
-        ev["fwd"][r][0].record()
-        convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3)
-        ev["fwd"][r][1].record()
-        ev["bwd_x"][r][0].record()
-        convlogic_hip.full_convlogic_backward_x(gy, xd, wp, am, sel, *geo)
-        ev["bwd_x"][r][1].record()
-        ev["bwd_w"][r][0].record()
-        convlogic_hip.full_convlogic_backward_weight(gy, xd, wp, am, sel, *geo)
-        ev["bwd_w"][r][1].record()
-    torch.cuda.synchronize()
-    ms = {name: _avg_ms(p) for name, p in ev.items()}
+    generic = timed({"fwd": lambda: convlogic_hip.full_convlogic_forward(xd, wp, sel, *geo, 3, 3),
+                     "bwd_x": lambda: convlogic_hip.full_convlogic_backward_x(gy, xd, wp, am, sel, *geo),
+                     "bwd_w": lambda: convlogic_hip.full_convlogic_backward_weight(gy, xd, wp, am, sel, *geo)})
+    binary = bool(getattr(layer, "binary_input", False)) and convlogic_hip.bin_supported(xd, k, *geo, 3, 3)
+    ms = generic
+    if binary:
+        flag = convlogic_hip.BinaryFlag()
+        _, taps, bctx = convlogic_hip.bin_forward(xd, wp, sel, *geo, 3, 3, flag)
+        ms = timed({"fwd": lambda: convlogic_hip.bin_forward(xd, wp, sel, *geo, 3, 3, flag),
+                    "bwd_x": lambda: convlogic_hip.bin_backward(gy, taps, bctx, tuple(xd.shape), *geo, need_grad_w=False),
+                    "bwd_w": lambda: convlogic_hip.bin_backward(gy, taps, bctx, tuple(xd.shape), *geo, need_grad_x=False)})
     gate_evals = n * k * h * w * 7
     xb, yb, pb = n * cin * h * w * 4, n * k * (h // 2) * (w // 2) * 4, k * 7 * 16 * 4 + k * 8 * 4
     alg_f, alg_b = xb + yb + pb, yb + xb + xb + pb      # forward: x in, y out; backward: gy, x in, gx out
     total_ms = ms["fwd"] + ms["bwd_x"] + ms["bwd_w"]
     floor_f = gate_evals * 3 / VALU_LANE_OPS_PER_S * 1e3
     floor_b = n * k * (h // 2) * (w // 2) * BWD_LANE_OPS_PER_POOLED_CELL / VALU_LANE_OPS_PER_S * 1e3
+    note = ("binary-input kernels (table lookups on bit rows, histogram weight gradient): the lane-operation floors are those of "
+            "evaluating the 7 gates per position and do not bound this path" if binary else
+            "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
+            "the lane-operation floors (39.3 T fp32 lane-ops/s) beside it")
     roof = _roof("convblock fwd + bwd_x + bwd_w kernels", alg_f + alg_b, total_ms,
                  {"forward": _roof("convblock_forward", alg_f, ms["fwd"]),
                   "backward": _roof("convblock_backward_x + convblock_backward_w", alg_b, ms["bwd_x"] + ms["bwd_w"]),
                   # lane-operation floors: 3 FMAs per gate evaluation forward, BWD_LANE_OPS_PER_POOLED_CELL backward, non-packed fp32
                   "valu_floor_forward_ms": floor_f, "valu_frac_forward": floor_f / ms["fwd"],
                   "valu_floor_backward_ms": floor_b, "valu_frac_backward": floor_b / (ms["bwd_x"] + ms["bwd_w"]),
-                  "note": "float block is VALU-bound once fused (about 0.34 B per gate-eval); HBM fraction reported as asked, "
-                          "the lane-operation floors (39.3 T fp32 lane-ops/s) beside it"})
+                  "path": "binary-input" if binary else "any-input", "note": note})
+    if binary:
+        roof["generic_kernel_ms"] = generic
     return ms, total_ms, gate_evals, roof
 
 
@@ -464,6 +506,7 @@ def bench_conv(key, steps, warmup, cpu=True):
     k = cfg["k"]
     torch.manual_seed(2)
     layer = C.ConvLogicLayer(cin, k, kernel=3, padding=1, complete=True, implementation="cuda").to(dev)
+    layer.binary_input = True                                # configs 3 and 4 feed {0,1} images (BASELINE.json)
     x = _conv_inputs(cfg, dev).requires_grad_(True)
     gy = torch.randn(n, k, h // 2, w // 2, device=dev)
 

@@ -38,6 +38,8 @@ class ConvLogicCifarModel(nn.Module):
         # the last block feeds nn.Flatten and a LogicLayer, which reads feature-major memory: when the block's kernels
         # can write that layout (4x4 images on the GPU) its output is the [N, C, 2, 2] view of a [C, 2, 2, N] tensor
         blocks[-1].feature_major_output = implementation == "cuda"
+        # the network's input is the thresholded image (src/convlogic/data.py:46-50): every element is 0 or 1
+        blocks[0].binary_input = implementation == "cuda"
         self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
 
     def forward(self, x):
@@ -55,6 +57,7 @@ class ConvLogicMnistModel(nn.Module):
         blocks = [_block(input_channels, k, implementation, kernel=5, padding=0),
                   _block(k, 3 * k, implementation, kernel=3, padding=1),
                   _block(3 * k, 9 * k, implementation, kernel=3, padding=1)]
+        blocks[0].binary_input = implementation == "cuda"          # binarised digits, as in the CIFAR topology
         self.network = nn.Sequential(*blocks, *_head([81 * k, 1280 * k, 640 * k, 320 * k], tau, implementation))
 
     def forward(self, x):

@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void convblock_bin_prepare_kernel(PrepArgs a, 
             tp.ch = min(tp.ch, g.cin - 1), tp.ry = min(tp.ry, g.kh - 1), tp.rx = min(tp.rx, g.kw - 1);   // a bad selection must not fault
             const int sh = tp.rx - g.pw;                              // tap word = row word >> sh (<< -sh)
             a.tapinfo[c * 8 + t] = ((tp.ch * a.RP + tp.ry) << 16) | ((sh < 0 ? -sh : 0) << 8) | (sh > 0 ? sh : 0);
-            a.xtap[c * 8 + t] = tp.ry * a.prs + tp.rx;
+            a.xtap[c * 8 + t] = tp.ry * a.prs + tp.rx;                 // offset of the tap in a gradient plane
         }
         __syncthreads();
         Tree<float> tr;
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void convblock_bin_prepare_kernel(PrepArgs a, 
             int mask = 0;
             if (c < g.c) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) mask |= (((a.sel[c * 8 + t] >> 16) & 0xFFFF) == ch) << t;
+                for (int t = 0; t < 8; ++t) mask |= (min((a.sel[c * 8 + t] >> 16) & 0xFFFF, g.cin - 1) == ch) << t;
             }
             const uint64_t vote = __ballot(mask != 0);
             if (mask) {
@@ -197,7 +197,8 @@ __global__ __launch_bounds__(256) void convblock_bin_prepare_kernel(PrepArgs a, 
 // ---- forward --------------------------------------------------------------------------------------------------------
 struct BinFwd {
     int S, LB, CT, ktiles, RP, hp, wp;
-    FastDiv d_hp, d_ktiles, d_lb;
+    int tr_words;       // 32-bit words of a wavefront's buffer for the ordered write-out
+    FastDiv d_hp, d_ktiles, d_lb, d_npc;
 };
 
 // 8 words of 32 columns -> per column one byte: afterwards byte g of word j holds bit (8 g + j) of the 8 input words
@@ -225,8 +226,33 @@ __device__ __forceinline__ void transpose_bits8(uint32_t (&t)[8])
 
 typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x2u __attribute__((ext_vector_type(2), aligned(4)));
+typedef float f32x2u __attribute__((ext_vector_type(2), aligned(4)));
 
-// grid: (sample tiles x kernel tiles) flat.  LDS: tables of the CT kernels [CT][256], bit planes of the S samples.
+// A piece of PC pooled cells of one row as it travels through the write-out buffer: PC floats of y, PC uint16 of taps.
+template <int PC>
+struct Piece;
+template <>
+struct Piece<4> {
+    using Y = float4;
+    using A = uint2;
+    static __device__ __forceinline__ Y y(const float *v) { return make_float4(v[0], v[1], v[2], v[3]); }
+    static __device__ __forceinline__ A a(const uint32_t *t) { return make_uint2(t[0] | (t[1] << 16), t[2] | (t[3] << 16)); }
+    static __device__ __forceinline__ void store_y(float *dst, const Y &v) { *reinterpret_cast<f32x4u *>(dst) = f32x4u{v.x, v.y, v.z, v.w}; }
+    static __device__ __forceinline__ void store_a(uint16_t *dst, const A &v) { *reinterpret_cast<u32x2u *>(dst) = u32x2u{v.x, v.y}; }
+};
+template <>
+struct Piece<2> {
+    using Y = float2;
+    using A = uint32_t;
+    static __device__ __forceinline__ Y y(const float *v) { return make_float2(v[0], v[1]); }
+    static __device__ __forceinline__ A a(const uint32_t *t) { return t[0] | (t[1] << 16); }
+    static __device__ __forceinline__ void store_y(float *dst, const Y &v) { *reinterpret_cast<f32x2u *>(dst) = f32x2u{v.x, v.y}; }
+    static __device__ __forceinline__ void store_a(uint16_t *dst, const A &v) { *reinterpret_cast<uint32_t *>(dst) = v; }
+};
+
+// grid: (sample tiles x kernel tiles) flat.  LDS: tables of the CT kernels [CT][256], bit planes of the S samples and, with
+// PC > 0 (rows of a multiple of PC = 4 or 2 cells), one write-out buffer per wavefront; PC = 0 writes rows directly.
+template <int PC>
 __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32_t *__restrict__ bits, const float *__restrict__ lut,
                                                                   const int32_t *__restrict__ tapinfo, float *__restrict__ y,
                                                                   uint16_t *__restrict__ aux, Geom g, BinFwd p)
@@ -234,6 +260,7 @@ __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32
     extern __shared__ __align__(16) uint32_t smem_u[];
     float *lut_s = reinterpret_cast<float *>(smem_u);
     uint32_t *img = smem_u + p.CT * 256;
+    uint32_t *trbuf = img + ((p.S * g.cin * p.RP + 3) & ~3);
     const int tid = threadIdx.x, nthreads = blockDim.x;
     const int lane = tid & (kWave - 1), wave = uniform(tid >> 6), nw = nthreads >> 6;
     const uint32_t b = xcd_contiguous_block(blockIdx.x, gridDim.x);
@@ -249,7 +276,7 @@ __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32
         for (int i = tid; i < words; i += nthreads) img[i] = bsrc[i];
     }
     __syncthreads();
-    const int slots = s_cur * p.hp;
+    const int slots = s_cur * p.hp, P = p.hp * p.wp;
     const int units = p.LB * ct_cur;
     for (int u = wave; u < units; u += nw) {
         const int ct = (int)fdiv((uint32_t)u, p.d_lb), lb = u - ct * p.LB;     // wave-uniform
@@ -271,14 +298,10 @@ __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32
         transpose_bits8(ta);
         transpose_bits8(tb);
         const float *L = lut_s + ct * 256;
-        const int64_t cell0 = (((int64_t)(n0 + (int)s) * g.c + c) * p.hp + rp) * p.wp;
-        float *yr = y + cell0;
-        uint16_t *ar = aux + cell0;
+        float yv[16];
+        uint32_t ax[16];
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
-            if (4 * gq >= p.wp) break;                                // wave-uniform
-            float yv[4];
-            uint32_t ax[4];
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
                 const uint32_t i0 = (ta[2 * m] >> (8 * gq)) & 255u, i1 = (ta[2 * m + 1] >> (8 * gq)) & 255u;
@@ -289,26 +312,66 @@ __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32
                 if (v1 > best) best = v1, t = i1 | 0x100u;
                 if (v2 > best) best = v2, t = i2 | 0x200u;
                 if (v3 > best) best = v3, t = i3 | 0x300u;
-                yv[m] = best;
-                ax[m] = t;
+                yv[4 * gq + m] = best;
+                ax[4 * gq + m] = t;
             }
-            if (live) {
-                if (4 * gq + 4 <= p.wp) {
-                    *reinterpret_cast<f32x4u *>(yr + 4 * gq) = f32x4u{yv[0], yv[1], yv[2], yv[3]};
-                    if ((p.wp & 1) == 0) {
-                        *reinterpret_cast<u32x2u *>(ar + 4 * gq) = u32x2u{ax[0] | (ax[1] << 16), ax[2] | (ax[3] << 16)};
-                    } else {
+            if (4 * gq + 4 >= p.wp) break;                            // wave-uniform
+        }
+        if constexpr (PC > 0) {
+            // The lane holds one row of wp cells; rows of consecutive lanes are consecutive in memory.  Through a buffer of
+            // the wavefront's own in LDS the rows go out as pieces of PC cells in lane order: every store instruction
+            // writes one contiguous run per sample.
+            using YP = typename Piece<PC>::Y;
+            using AP = typename Piece<PC>::A;
+            float *tb_y = reinterpret_cast<float *>(trbuf) + wave * p.tr_words;
+            const int ys = p.wp + 4, npc = p.wp / PC;                 // padded row stride (floats); pieces per row
+            constexpr int K = 16 / PC;
 #pragma unroll
-                        for (int m = 0; m < 4; ++m) ar[4 * gq + m] = (uint16_t)ax[m];
-                    }
-                } else {
+            for (int k = 0; k < K; ++k)
+                if (k < npc) *reinterpret_cast<YP *>(tb_y + lane * ys + PC * k) = Piece<PC>::y(yv + PC * k);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t base = (uint32_t)((n0 * g.c + c) * P), sstep = (uint32_t)((g.c - 1) * P);
+            // piece i of the wavefront = (row r, piece q of the row); its cell index in y / taps
+            auto place = [&](int k, uint32_t &r, uint32_t &q, uint32_t &cell) {
+                const uint32_t i = (uint32_t)(k * kWave + lane);
+                r = fdiv(i, p.d_npc), q = i - r * (uint32_t)npc;
+                const uint32_t vr = (uint32_t)(lb * kWave) + r;
+                const bool ok = k < npc && (int)vr < slots;
+                const uint32_t vs = ok ? vr : 0u;
+                cell = base + vs * (uint32_t)p.wp + fdiv(vs, p.d_hp) * sstep + (uint32_t)PC * q;
+                return ok;
+            };
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) {
-                        if (4 * gq + m < p.wp) {
-                            yr[4 * gq + m] = yv[m];
-                            ar[4 * gq + m] = (uint16_t)ax[m];
-                        }
-                    }
+            for (int k = 0; k < K; ++k) {
+                uint32_t r, q, cell;
+                if (place(k, r, q, cell)) Piece<PC>::store_y(y + cell, *reinterpret_cast<const YP *>(tb_y + r * ys + PC * q));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            uint32_t *tb_a = reinterpret_cast<uint32_t *>(tb_y);
+            const int as = (p.wp >> 1) + 2;                            // padded row stride (dwords)
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (k < npc) *reinterpret_cast<AP *>(tb_a + lane * as + (PC / 2) * k) = Piece<PC>::a(ax + PC * k);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                uint32_t r, q, cell;
+                if (place(k, r, q, cell)) Piece<PC>::store_a(aux + cell, *reinterpret_cast<const AP *>(tb_a + r * as + (PC / 2) * q));
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        } else if (live) {
+            const int64_t cell0 = (((int64_t)(n0 + (int)s) * g.c + c) * p.hp + rp) * p.wp;
+            float *yr = y + cell0;
+            uint16_t *ar = aux + cell0;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                if (e < p.wp) {
+                    yr[e] = yv[e];
+                    ar[e] = (uint16_t)ax[e];
                 }
             }
         }
@@ -323,7 +386,7 @@ struct BinHist {
     int C, P, Q, n, parts, per_part;      // Q = P / 4 quads per (sample, kernel) plane
     FastDiv d_q;
 };
-constexpr int kHistDepth = 4;           // steps whose loads are in flight together
+constexpr int kHistDepth = 8;           // steps whose loads are in flight together
 
 __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const float *__restrict__ gy, const uint16_t *__restrict__ aux,
                                                                       float *__restrict__ hpart, BinHist p)
@@ -344,25 +407,20 @@ __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const fl
     const uint16_t *axc = aux + ((int64_t)s0 * p.C + c) * p.P;
     float *mine = bins + lane;
 
-    float4 G[2][kHistDepth];
-    uint2 A[2][kHistDepth];
-    auto issue = [&](int step0, float4 (&Gd)[kHistDepth], uint2 (&Ad)[kHistDepth]) {
-#pragma unroll
-        for (int d = 0; d < kHistDepth; ++d) {
-            const int e = (step0 + d) * kHistLanes + lane;
-            Gd[d] = make_float4(0.f, 0.f, 0.f, 0.f);
-            Ad[d] = make_uint2(0u, 0u);
-            if (e < items) {
-                const uint32_t smp = fdiv((uint32_t)e, p.d_q), quad = (uint32_t)e - smp * (uint32_t)p.Q;
-                const int64_t at = smp * plane_stride + quad * 4;
-                Gd[d] = *reinterpret_cast<const float4 *>(gyc + at);
-                Ad[d] = *reinterpret_cast<const uint2 *>(axc + at);
-            }
-        }
+    // loads never depend on a branch (an index past the end is clamped), so the compiler can count them and let a
+    // whole group of steps stay in flight while the previous group is applied
+    auto load = [&](int step, float4 &g4, uint2 &a2) {
+        int e = step * kHistLanes + lane;
+        e = e < items ? e : items - 1;
+        const uint32_t smp = fdiv((uint32_t)e, p.d_q), quad = (uint32_t)e - smp * (uint32_t)p.Q;
+        const int64_t at = smp * plane_stride + quad * 4;
+        g4 = *reinterpret_cast<const float4 *>(gyc + at);
+        a2 = *reinterpret_cast<const uint2 *>(axc + at);
     };
     auto apply = [&](const float4 &g4, const uint2 &a2) {
         const uint32_t t0 = a2.x & 255u, t1 = (a2.x >> 16) & 255u, t2 = a2.y & 255u, t3 = (a2.y >> 16) & 255u;
-        const float r0 = mine[t0 * kHistLanes], r1 = mine[t1 * kHistLanes], r2 = mine[t2 * kHistLanes], r3 = mine[t3 * kHistLanes];
+        float r0 = mine[t0 * kHistLanes], r1 = mine[t1 * kHistLanes], r2 = mine[t2 * kHistLanes], r3 = mine[t3 * kHistLanes];
+        asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));   // all four reads in flight together
         const float v0 = r0 + g4.x;
         const float v1 = (t1 == t0 ? v0 : r1) + g4.y;
         const float v2 = (t2 == t1 ? v1 : (t2 == t0 ? v0 : r2)) + g4.z;
@@ -373,14 +431,34 @@ __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const fl
         mine[t3 * kHistLanes] = v3;
     };
     const int steps = (items + kHistLanes - 1) / kHistLanes;
-    issue(0, G[0], A[0]);
-    for (int st = 0; st < steps; st += 2 * kHistDepth) {
-        issue(st + kHistDepth, G[1], A[1]);
+    if (steps > 0) {
+        float4 G[2][kHistDepth];
+        uint2 A[2][kHistDepth];
+        // a group of kHistDepth steps; in a group that reaches past the end the lanes without a quad add 0
+        auto apply_group = [&](int s0, const float4 (&Gd)[kHistDepth], const uint2 (&Ad)[kHistDepth]) {
+            if (s0 >= steps) return;                                  // wave-uniform
+            if ((s0 + kHistDepth) * kHistLanes <= items) {
 #pragma unroll
-        for (int d = 0; d < kHistDepth; ++d) apply(G[0][d], A[0][d]);     // lanes past the end add 0 to bin 0
-        issue(st + 2 * kHistDepth, G[0], A[0]);
+                for (int d = 0; d < kHistDepth; ++d) apply(Gd[d], Ad[d]);
+            } else {
 #pragma unroll
-        for (int d = 0; d < kHistDepth; ++d) apply(G[1][d], A[1][d]);
+                for (int d = 0; d < kHistDepth; ++d) {
+                    float4 g4 = Gd[d];
+                    if ((s0 + d) * kHistLanes + lane >= items) g4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    apply(g4, Ad[d]);
+                }
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < kHistDepth; ++d) load(d, G[0][d], A[0][d]);
+        for (int st = 0; st < steps; st += 2 * kHistDepth) {
+#pragma unroll
+            for (int d = 0; d < kHistDepth; ++d) load(st + kHistDepth + d, G[1][d], A[1][d]);     // (clamped past the end; unused then)
+            apply_group(st, G[0], A[0]);
+#pragma unroll
+            for (int d = 0; d < kHistDepth; ++d) load(st + 2 * kHistDepth + d, G[0][d], A[0][d]);
+            apply_group(st + kHistDepth, G[1], A[1]);
+        }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -409,7 +487,16 @@ __global__ __launch_bounds__(256) void convblock_bin_wgrad_finish_kernel(const f
     __shared__ float sums[28];
     const int c = blockIdx.x, t = threadIdx.x;
     float H = 0.f;
-    for (int k = 0; k < parts; ++k) H += hpart[((int64_t)c * parts + k) * 256 + t];
+    const float *hp = hpart + (int64_t)c * parts * 256 + t;
+    int k = 0;
+    for (; k + 8 <= parts; k += 8) {                                  // eight loads in flight, added in the order of one by one
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = hp[(k + u) * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) H += v[u];
+    }
+    for (; k < parts; ++k) H += hp[k * 256];
     Tree<float> tr;
     const float *fc = folded + (int64_t)c * 28;
 #pragma unroll
@@ -652,6 +739,7 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
         if (lanes * 100 >= blocks * 64 * 85) break;
     }
     const size_t img_per_sample = (size_t)g.cin * cx.RP * 4;
+    if (const char *e = clg_knob(K_BIN_S)) S = std::min(64, std::max(1, atoi(e)));
     while (S > 1 && S * img_per_sample > 64 * 1024) S /= 2;
     CLG_REQUIRE(S * img_per_sample <= 96 * 1024, "%s: the bit planes of one sample (%zu bytes) do not fit LDS", name, img_per_sample);
     if (S > g.n) S = g.n;
@@ -660,6 +748,7 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
     const int stiles = (int)clg_ceil_div(g.n, S);
     int CT = 64;
     while (CT > 8 && (int64_t)stiles * clg_ceil_div(g.c, CT) < 512) CT /= 2;
+    if (const char *e = clg_knob(K_BIN_CT)) CT = std::min(64, std::max(1, atoi(e)));
     if (CT > g.c) CT = g.c;
     p.CT = CT;
     p.ktiles = (int)clg_ceil_div(g.c, CT);
@@ -668,10 +757,22 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
     p.d_lb = make_fastdiv((uint32_t)p.LB);
     int nw = p.LB * CT;
     nw = nw > 8 ? 8 : nw;
-    const size_t lds = (size_t)CT * 1024 + S * img_per_sample;
-    if (int e = allow_lds(convblock_bin_forward_kernel, lds, name)) return e;
-    hipLaunchKernelGGL(convblock_bin_forward_kernel, dim3((unsigned)(stiles * p.ktiles)), dim3(nw * kWave), lds, st,
-                       (const uint32_t *)a.bits, (const float *)a.lut, (const int32_t *)a.tapinfo, (float *)y, taps, g, p);
+    if (const char *e = clg_knob(K_BIN_NW)) nw = std::min(8, std::max(1, atoi(e)));
+    int pc = p.wp % 4 == 0 ? 4 : (p.wp % 2 == 0 ? 2 : 0);
+    if (const char *e = clg_knob(K_BIN_DBG)) pc = atoi(e) == 1 ? 0 : pc;
+    p.tr_words = pc ? kWave * (p.wp + 4) : 0;
+    p.d_npc = make_fastdiv((uint32_t)std::max(1, pc ? p.wp / pc : 1));
+    const size_t lds = (size_t)CT * 1024 + (((size_t)S * g.cin * cx.RP + 3) & ~(size_t)3) * 4 + (size_t)nw * p.tr_words * 4;
+#define CLG_BIN_FWD(PC)                                                                                                          \
+    do {                                                                                                                         \
+        if (int e = allow_lds(convblock_bin_forward_kernel<PC>, lds, name)) return e;                                            \
+        hipLaunchKernelGGL(convblock_bin_forward_kernel<PC>, dim3((unsigned)(stiles * p.ktiles)), dim3(nw * kWave), lds, st,     \
+                           (const uint32_t *)a.bits, (const float *)a.lut, (const int32_t *)a.tapinfo, (float *)y, taps, g, p);  \
+    } while (0)
+    if (pc == 4) CLG_BIN_FWD(4);
+    else if (pc == 2) CLG_BIN_FWD(2);
+    else CLG_BIN_FWD(0);
+#undef CLG_BIN_FWD
     CLG_CHECK_LAUNCH(name);
     return CLG_OK;
 }
@@ -681,6 +782,7 @@ int hist_parts(const Geom &g)
 {
     int parts = 512 / g.c;
     if (parts < 1) parts = 1;
+    if (const char *e = clg_knob(K_BIN_PARTS)) parts = std::max(1, atoi(e));
     if (parts > g.n) parts = g.n;
     return parts;
 }
@@ -720,7 +822,8 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
         // wavefronts per plane: enough of them to give every SIMD a few, bounded by the shortest useful list
         int hsw = 1;
         const int64_t avg_hits = std::max<int64_t>(1, (int64_t)g.c * 2 / g.cin);
-        while (hsw < 16 && p.items * hsw * 2 <= 6144 && hsw * 2 * 4 <= avg_hits) hsw *= 2;
+        while (hsw < 16 && p.items * hsw * 2 <= 10240 && hsw * 2 * 4 <= avg_hits) hsw *= 2;
+        if (const char *e = clg_knob(K_BIN_HSW)) hsw = std::min(16, std::max(1, atoi(e)));
         p.hsw = hsw;
         int per_wg = std::max(1, 4 / hsw);
         while (per_wg > 1 && (size_t)per_wg * hsw * p.plane_pad * 4 > 64 * 1024) per_wg /= 2;

@@ -461,6 +461,12 @@ class BinaryFlag:
         check(_lib.load().clg_host_flag_device_pointer(self.host.data_ptr(), ctypes.byref(dev)))
         self.device_ptr = dev.value
 
+    def __deepcopy__(self, memo):                                    # a copied layer gets a flag of its own
+        return BinaryFlag()
+
+    def __reduce__(self):
+        return (BinaryFlag, ())
+
     def raised(self):
         return bool(self.host[0].item())
 
