@@ -187,11 +187,24 @@ __device__ __forceinline__ T softmax16_backward(T g, T p) { return p * (g - row1
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// A wiring / reverse-map entry as the kernels use it: forced into 0..n-1, so that a corrupted index buffer (the host checks
+// are cached and a write through `.data` goes past them) reads a wrong row instead of faulting the GPU.
+__device__ __forceinline__ int64_t clamp_index(int64_t i, int64_t n) { return i < 0 ? 0 : (i < n ? i : n - 1); }
+
 // selection tap: ch << 16 | row << 8 | col
 struct Tap {
     int ch, ry, rx;
 };
-__device__ __forceinline__ Tap unpack_tap(int32_t s) { return Tap{(s >> 16) & 0xFFFF, (s >> 8) & 0xFF, s & 0xFF}; }
+// Decoded and forced into the layer's ranges (channel < cin, row < kh, column < kw): the kernels turn taps into addresses
+// without bounds checks, so a selection buffer that was corrupted behind the cached host check must not reach them raw.
+struct TapLimit {
+    int cin, kh, kw;
+};
+__device__ __forceinline__ int tap_channel(int32_t s, int cin) { return min((s >> 16) & 0xFFFF, cin - 1); }
+__device__ __forceinline__ Tap unpack_tap(int32_t s, const TapLimit &lim)
+{
+    return Tap{tap_channel(s, lim.cin), min((s >> 8) & 0xFF, lim.kh - 1), min(s & 0xFF, lim.kw - 1)};
+}
 
 // ---- bitwise gates on packed samples ---------------------------------------------------------
 struct Masks {

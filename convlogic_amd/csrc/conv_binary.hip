@@ -102,8 +102,7 @@ __global__ __launch_bounds__(256) void convblock_bin_prepare_kernel(PrepArgs a, 
         }
         if (tid >= 64 && tid < 72) {
             const int t = tid - 64;
-            Tap tp = unpack_tap(a.sel[(int64_t)c * 8 + t]);
-            tp.ch = min(tp.ch, g.cin - 1), tp.ry = min(tp.ry, g.kh - 1), tp.rx = min(tp.rx, g.kw - 1);   // a bad selection must not fault
+            const Tap tp = unpack_tap(a.sel[(int64_t)c * 8 + t], tap_limit(g));   // (forced into the layer's ranges)
             const int sh = tp.rx - g.pw;                              // tap word = row word >> sh (<< -sh)
             a.tapinfo[c * 8 + t] = ((tp.ch * a.RP + tp.ry) << 16) | ((sh < 0 ? -sh : 0) << 8) | (sh > 0 ? sh : 0);
             a.xtap[c * 8 + t] = tp.ry * a.prs + tp.rx;                 // offset of the tap in a gradient plane
@@ -155,7 +154,7 @@ __global__ __launch_bounds__(256) void convblock_bin_prepare_kernel(PrepArgs a, 
             int mask = 0;
             if (c < g.c) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) mask |= (min((a.sel[c * 8 + t] >> 16) & 0xFFFF, g.cin - 1) == ch) << t;
+                for (int t = 0; t < 8; ++t) mask |= (tap_channel(a.sel[c * 8 + t], g.cin) == ch) << t;
             }
             const uint64_t vote = __ballot(mask != 0);
             if (mask) {

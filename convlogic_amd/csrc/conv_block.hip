@@ -87,7 +87,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restrict__ w, const int32_t *__restrict__ sel,
                                                               T *__restrict__ folded, int32_t *__restrict__ count,
                                                               int32_t *__restrict__ hits, int32_t *__restrict__ taps, int C,
-                                                              int cin, int fold_blocks, int rs, int chs, PadJob<T> pad, int pad_block0)
+                                                              int cin, int fold_blocks, int rs, int chs, PadJob<T> pad, int pad_block0,
+                                                              TapLimit lim)
 {
     if ((int)blockIdx.x >= pad_block0) {                            // tail of the launch: the padded copy of x
         pad_image_elem(pad, (int64_t)(blockIdx.x - pad_block0) * 256 + threadIdx.x);
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
     if ((int)blockIdx.x < fold_blocks) {
         const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
         if (q < (int64_t)C * 8) {                                   // tap offsets of the LDS window layout
-            const Tap tp = unpack_tap(sel[q]);
+            const Tap tp = unpack_tap(sel[q], lim);
             const int rel = tp.ry * rs + tp.rx;
             const int64_t c = q >> 3, t = q & 7;
             taps[c * 16 + t] = tp.ch * chs + rel;
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
         int mask = 0;
         if (c < C) {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) mask |= (((sel[c * 8 + t] >> 16) & 0xFFFF) == ch) << t;
+            for (int t = 0; t < 8; ++t) mask |= (tap_channel(sel[c * 8 + t], cin) == ch) << t;
         }
         const uint64_t vote = __ballot(mask != 0);
         if (mask) {
@@ -138,12 +139,12 @@ __global__ __launch_bounds__(256) void convblock_prepare_kernel(const T *__restr
 
 // ---- compressed lists ------------------------------------------------------------------------
 // tap mask of kernel c for the channel of its tap t, or 0 when an earlier tap names the same channel
-__device__ __forceinline__ int first_use_mask(const int32_t *__restrict__ sq, int t)
+__device__ __forceinline__ int first_use_mask(const int32_t *__restrict__ sq, int t, int cin)
 {
-    const int ch = (sq[t] >> 16) & 0xFFFF;
+    const int ch = tap_channel(sq[t], cin);
     int mask = 0;
     for (int u = 0; u < 8; ++u) {
-        if (((sq[u] >> 16) & 0xFFFF) == ch) {
+        if (tap_channel(sq[u], cin) == ch) {
             if (u < t) return 0;
             mask |= 1 << u;
         }
@@ -158,13 +159,13 @@ __global__ __launch_bounds__(256) void hits_zero_kernel(int32_t *__restrict__ co
     count[2 * ch + 1] = 0;
     cursor[ch] = 0;
 }
-__global__ __launch_bounds__(256) void hits_count_kernel(const int32_t *__restrict__ sel, int32_t *__restrict__ count, int C)
+__global__ __launch_bounds__(256) void hits_count_kernel(const int32_t *__restrict__ sel, int32_t *__restrict__ count, int C, int cin)
 {
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     const int32_t *sq = sel + (int64_t)c * 8;
     for (int t = 0; t < 8; ++t)
-        if (first_use_mask(sq, t)) atomicAdd(count + 2 * ((sq[t] >> 16) & 0xFFFF), 1);
+        if (first_use_mask(sq, t, cin)) atomicAdd(count + 2 * tap_channel(sq[t], cin), 1);
 }
 // exclusive prefix sum of the counts into the offsets, one workgroup
 __global__ __launch_bounds__(1024) void hits_scan_kernel(int32_t *__restrict__ count, int cin)
@@ -190,15 +191,15 @@ __global__ __launch_bounds__(1024) void hits_scan_kernel(int32_t *__restrict__ c
     }
 }
 __global__ __launch_bounds__(256) void hits_fill_kernel(const int32_t *__restrict__ sel, const int32_t *__restrict__ count,
-                                                      int32_t *__restrict__ cursor, int32_t *__restrict__ unsorted, int C)
+                                                      int32_t *__restrict__ cursor, int32_t *__restrict__ unsorted, int C, int cin)
 {
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     const int32_t *sq = sel + (int64_t)c * 8;
     for (int t = 0; t < 8; ++t) {
-        const int mask = first_use_mask(sq, t);
+        const int mask = first_use_mask(sq, t, cin);
         if (mask) {
-            const int ch = (sq[t] >> 16) & 0xFFFF;
+            const int ch = tap_channel(sq[t], cin);
             unsorted[count[2 * ch + 1] + atomicAdd(cursor + ch, 1)] = c | (mask << 16);
         }
     }
@@ -754,7 +755,7 @@ __global__ __launch_bounds__(kTiledWWaves * kWave) void convblock_backward_w_til
     int to[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        const Tap tp = unpack_tap(sel[(int64_t)cc * 8 + t]);
+        const Tap tp = unpack_tap(sel[(int64_t)cc * 8 + t], tap_limit(g));
         to[t] = uniform(tp.ch * p.chs + tp.ry * p.rs + tp.rx);
     }
     T acc[28];
@@ -1122,14 +1123,15 @@ int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
     const int fold_blocks = (int)clg_ceil_div((int64_t)g.c * 8, 256), list_blocks = lay.csr ? 0 : (int)clg_ceil_div(g.cin, 4);
     hipLaunchKernelGGL(convblock_prepare_kernel<T>, dim3((unsigned)(fold_blocks + list_blocks) + pad_blocks(pad)), dim3(256), 0, st,
                        (const T *)w, sel, reinterpret_cast<T *>(base), count, lay.csr ? nullptr : hits,
-                       reinterpret_cast<int32_t *>(base + lay.taps_off), g.c, g.cin, fold_blocks, rs, chs, pad, fold_blocks + list_blocks);
+                       reinterpret_cast<int32_t *>(base + lay.taps_off), g.c, g.cin, fold_blocks, rs, chs, pad, fold_blocks + list_blocks,
+                       host_tap_limit(g));
     if (lay.csr) {
         int32_t *cursor = reinterpret_cast<int32_t *>(base + lay.cursor_off), *unsorted = reinterpret_cast<int32_t *>(base + lay.unsorted_off);
         const unsigned cb = (unsigned)clg_ceil_div(g.c, 256);
         hipLaunchKernelGGL(hits_zero_kernel, dim3((unsigned)clg_ceil_div(g.cin, 256)), dim3(256), 0, st, count, cursor, g.cin);
-        hipLaunchKernelGGL(hits_count_kernel, dim3(cb), dim3(256), 0, st, sel, count, g.c);
+        hipLaunchKernelGGL(hits_count_kernel, dim3(cb), dim3(256), 0, st, sel, count, g.c, g.cin);
         hipLaunchKernelGGL(hits_scan_kernel, dim3(1), dim3(1024), 0, st, count, g.cin);
-        hipLaunchKernelGGL(hits_fill_kernel, dim3(cb), dim3(256), 0, st, sel, (const int32_t *)count, cursor, unsorted, g.c);
+        hipLaunchKernelGGL(hits_fill_kernel, dim3(cb), dim3(256), 0, st, sel, (const int32_t *)count, cursor, unsorted, g.c, g.cin);
         hipLaunchKernelGGL(hits_sort_kernel, dim3((unsigned)clg_ceil_div(g.cin, 4)), dim3(256), 0, st, (const int32_t *)count,
                            (const int32_t *)unsorted, hits, g.cin);
     }
@@ -1170,7 +1172,7 @@ int prepare_tables(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
     if (!fold && pad.total == 0) return CLG_OK;
     const unsigned prep = fold ? (unsigned)clg_ceil_div((int64_t)g.c * 7, 256) : 0u;
     hipLaunchKernelGGL((convblock_w_prepare_kernel<T, T>), dim3(prep + pad_blocks(pad)), dim3(256), 0, st, (const T *)w, sel,
-                       fold ? reinterpret_cast<T *>(base) : (T *)nullptr, (int32_t *)nullptr, g.c, 0, 0, pad, (int)prep);
+                       fold ? reinterpret_cast<T *>(base) : (T *)nullptr, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), pad, (int)prep);
     CLG_CHECK_LAUNCH("clg_convblock_backward_planned(fold / pad)");
     return CLG_OK;
 }
@@ -1264,7 +1266,7 @@ int launch_backward_w_padded(const Geom &g, const TilePlan &p, const WScratch &w
     const PadJob<T> job = make_pad_job((const T *)x, xp, g, p.rs, p.chs, ws.sample_elems);
     const unsigned prep = (unsigned)clg_ceil_div((int64_t)g.c * 8, 256);
     hipLaunchKernelGGL((convblock_w_prepare_kernel<T, T>), dim3(prep + pad_blocks(job)), dim3(256), 0, st, (const T *)w, sel, folded, taps,
-                       g.c, p.rs, p.chs, job, (int)prep);
+                       g.c, p.rs, p.chs, host_tap_limit(g), job, (int)prep);
     CLG_CHECK_LAUNCH("clg_convblock_backward_w(prepare)");
     const int I = (g.ho / 2) * (g.wo / 2);
     if (fixed_cells(g, (int)sizeof(T)))

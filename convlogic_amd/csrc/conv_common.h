@@ -29,6 +29,8 @@ static inline int clg_make_geom(const clg_conv_geom *g, Geom *out, const char *n
 
 #if defined(__HIPCC__)
 
+__device__ __forceinline__ TapLimit tap_limit(const Geom &g) { return TapLimit{g.cin, g.kh, g.kw}; }
+
 // Tap value of one sample (xn = x + n*cin*h*w) for conv output position (oy, ox); 0 outside.
 template <typename T>
 __device__ __forceinline__ T read_tap(const T *__restrict__ xn, const Geom &g, const Tap &t, int oy, int ox)

@@ -62,7 +62,7 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     Ops::stage_params(coef, params, c0, ct_cur, tid, nthreads, p.w_logits != 0, blockIdx.x == 0 ? probs_out : nullptr);
     if (!SUBSET) {
         for (int q = tid; q < ct_cur * 8; q += nthreads) {
-            const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q]);
+            const Tap t = unpack_tap(sel[(int64_t)c0 * 8 + q], tap_limit(g));
             toff[q] = t.ch * p.chs + t.ry * p.rs + t.rx;
         }
     } else {
@@ -70,11 +70,11 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
             int ch_a = 0, ch_b = 0, wd = 0;
             if (q < ct_cur) {
                 const int32_t *sq = sel + ((int64_t)c0 + q) * 8;
-                ch_a = ch_b = unpack_tap(sq[0]).ch;
+                ch_a = ch_b = unpack_tap(sq[0], tap_limit(g)).ch;
                 for (int t = 7; t >= 1; --t)
-                    if (unpack_tap(sq[t]).ch != ch_a) ch_b = unpack_tap(sq[t]).ch;   // ends on the first other channel
+                    if (unpack_tap(sq[t], tap_limit(g)).ch != ch_a) ch_b = unpack_tap(sq[t], tap_limit(g)).ch;   // ends on the first other channel
                 for (int t = 0; t < 8; ++t) {
-                    const Tap tp = unpack_tap(sq[t]);
+                    const Tap tp = unpack_tap(sq[t], tap_limit(g));
                     int pl = 2 * q;
                     if (tp.ch == ch_b) pl = 2 * q + 1;
                     if (tp.ch == ch_a) pl = 2 * q;
@@ -225,11 +225,11 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
                 const T *xn = x + (int64_t)(n0 + s) * g.cin * hw;
                 const int32_t *sq = sel + ((int64_t)c0 + lc) * 8;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)oy, (int)ox);
+                for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t], tap_limit(g)), (int)oy, (int)ox);
                 r0 = Ops::root(pr, v);
                 if (!ONE_ROW) {
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t]), (int)(oy + 1), (int)ox);
+                    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sq[t], tap_limit(g)), (int)(oy + 1), (int)ox);
                     r1 = Ops::root(pr, v);
                 }
             }
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256) void convblock_packed_generic_kernel(const uin
     for (int q = 0; q < 4; ++q) {
         uint64_t v[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t]), 2 * py + (q >> 1), 2 * px + (q & 1));
+        for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t], tap_limit(g)), 2 * py + (q >> 1), 2 * px + (q & 1));
         acc |= BitOps::root_true(pr, v);
     }
     y[((int64_t)n * g.c + c) * I + cell] = acc;
@@ -504,7 +504,7 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
     const unsigned prep = (unsigned)clg_ceil_div((int64_t)g.c * 8, 256);
     hipLaunchKernelGGL((convblock_w_prepare_kernel<P, T>), dim3(prep + pad_blocks(job)), dim3(256), 0, st,
                        fold ? (const P *)params : (const P *)nullptr, sel, fold ? reinterpret_cast<P *>(base) : (P *)nullptr, taps, g.c,
-                       d.p.rs, d.p.chs, job, (int)prep, fold && from_logits ? 1 : 0, reinterpret_cast<P *>(probs_out));
+                       d.p.rs, d.p.chs, host_tap_limit(g), job, (int)prep, fold && from_logits ? 1 : 0, reinterpret_cast<P *>(probs_out));
     CLG_CHECK_LAUNCH(name);
     const int64_t sets = clg_ceil_div(g.n, d.p.G) * d.nblk;
     hipLaunchKernelGGL(convblock_forward_direct_kernel<Ops>, dim3((unsigned)clg_ceil_div(sets, 4), (unsigned)clg_ceil_div(g.c, d.p.CT)),
@@ -633,10 +633,10 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
-                               (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
+                               (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<float>(), (int)pgrid.x);
         else
             hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
-                               (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
+                               (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x);
         CLG_CHECK_LAUNCH("clg_convblock_forward_ws");
         return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_ws");
     }
@@ -689,10 +689,10 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
         const void *pr = logits ? probs_out : w;
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)pr, selection,
-                               (float *)folded_out, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
+                               (float *)folded_out, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<float>(), (int)pgrid.x);
         else
             hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)pr, selection,
-                               (double *)folded_out, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
+                               (double *)folded_out, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x);
         CLG_CHECK_LAUNCH(name);
         return CLG_OK;
     };
@@ -702,11 +702,11 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
-                               (float *)fold_to, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
+                               (float *)fold_to, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
                                (float *)probs_out);
         else
             hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
-                               (double *)fold_to, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
+                               (double *)fold_to, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
                                (double *)probs_out);
         CLG_CHECK_LAUNCH(name);
         return clg_convblock_forward_4x4(dtype, g, x, fold_to, selection, y, argmax, st, name);
@@ -767,10 +767,10 @@ extern "C" int clg_convblock_forward_fm(int dtype, const clg_conv_geom *gg, cons
     const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
     if (dtype == CLG_F32)
         hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
-                           (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<float>(), (int)pgrid.x);
+                           (float *)scratch, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<float>(), (int)pgrid.x);
     else
         hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
-                           (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, no_pad_job<double>(), (int)pgrid.x);
+                           (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x);
     CLG_CHECK_LAUNCH("clg_convblock_forward_fm");
     return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_fm");
 }

@@ -41,8 +41,8 @@ __global__ __launch_bounds__(kBlk) void conv4_forward_kernel(const T *__restrict
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
-        const T a = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p]), oy, ox);
-        const T b = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p + 1]), oy, ox);
+        const T a = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p], tap_limit(g)), oy, ox);
+        const T b = read_tap(xn, g, unpack_tap(sel[c * 8 + 2 * p + 1], tap_limit(g)), oy, ox);
         out.v[p] = gate(cf, a, b);
     }
     reinterpret_cast<Quad<T> *>(y)[((int64_t)n * g.c + c) * P + pos] = out;
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kBlk) void conv4_backward_w_kernel(const T *__restr
     const int64_t items = (int64_t)g.n * P;
     Tap tap[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t], tap_limit(g));
     T acc[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) acc[k] = 0;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *_
     T acc = 0;
     for (int c = 0; c < g.c; ++c) {
         for (int t = 0; t < 8; ++t) {
-            const Tap tp = unpack_tap(sel[c * 8 + t]);
+            const Tap tp = unpack_tap(sel[c * 8 + t], tap_limit(g));
             if (tp.ch != ch) continue;
             const int ny = iy + g.ph - tp.ry, nx = ix + g.pw - tp.rx;
             if (ny < 0 || nx < 0 || ny % g.sh != 0 || nx % g.sw != 0) continue;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(kBlk) void conv_backward_x_gather_kernel(const T *_
             const int p = t >> 1;
             const T gl = gy[(((int64_t)n * g.c + c) * P + oy * g.wo + ox) * 4 + p];
             const Coef<T> cf = fold16(w + (c * 4 + p) * 16);
-            const T other = read_tap(xn, g, unpack_tap(sel[c * 8 + (t ^ 1)]), oy, ox);
+            const T other = read_tap(xn, g, unpack_tap(sel[c * 8 + (t ^ 1)], tap_limit(g)), oy, ox);
             acc += gl * ((t & 1) ? gate_db(cf, other) : gate_da(cf, other));
         }
     }
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(kBlk) void convblock_backward_x_hits_kernel(const T
         const int c = ent & 0xFFFF, mask = (ent >> 16) & 0xFF;
         for (int t = 0; t < 8; ++t) {
             if (!((mask >> t) & 1)) continue;
-            const Tap tp = unpack_tap(sel[c * 8 + t]);
+            const Tap tp = unpack_tap(sel[c * 8 + t], tap_limit(g));
             const int ny = iy + g.ph - tp.ry, nx = ix + g.pw - tp.rx;
             if (ny < 0 || nx < 0 || ny % g.sh != 0 || nx % g.sw != 0) continue;
             const int oy = ny / g.sh, ox = nx / g.sw;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kBlk) void convblock_backward_x_hits_kernel(const T
             for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
             T tap[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) tap[q] = read_tap(xn, g, unpack_tap(sel[c * 8 + q]), oy, ox);
+            for (int q = 0; q < 8; ++q) tap[q] = read_tap(xn, g, unpack_tap(sel[c * 8 + q], tap_limit(g)), oy, ox);
             const TreeVals<T> v = eval_tree(tr, tap);
             const int p = t >> 1, m = p >> 1;
             const T g_mid = gy[cell] * (m ? gate_db(tr.g[6], v.mid[0]) : gate_da(tr.g[6], v.mid[1]));
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(kBlk) void convblock_forward_generic_kernel(const T
     const Tree<T> tr = load_tree(w + c * 7 * 16);
     Tap tap[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t], tap_limit(g));
     T best = -INFINITY;
     int code = 0;
 #pragma unroll
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kBlk) void convblock_intermediates_kernel(const T *
     const Tree<T> tr = load_tree(w + c * 7 * 16);
     T v[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t]), oy, ox);
+    for (int t = 0; t < 8; ++t) v[t] = read_tap(xn, g, unpack_tap(sel[c * 8 + t], tap_limit(g)), oy, ox);
     const TreeVals<T> tv = eval_tree(tr, v);
     const int64_t o = ((int64_t)n * g.c + c) * P + pos;
     if (x2) {
@@ -337,7 +337,7 @@ __global__ __launch_bounds__(kBlk) void convblock_backward_w_generic_kernel(cons
     const Tree<T> tr = load_tree(w + c * 7 * 16);
     Tap tap[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t]);
+    for (int t = 0; t < 8; ++t) tap[t] = unpack_tap(sel[c * 8 + t], tap_limit(g));
     T acc[28];
 #pragma unroll
     for (int k = 0; k < 28; ++k) acc[k] = 0;

@@ -25,12 +25,12 @@ struct LaneTaps {
     int ch0, ch1;
     bool wide;
 };
-__device__ __forceinline__ LaneTaps lane_taps(const int32_t *__restrict__ sel, int c)
+__device__ __forceinline__ LaneTaps lane_taps(const int32_t *__restrict__ sel, int c, const TapLimit &lim)
 {
     LaneTaps t;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        const Tap tp = unpack_tap(sel[c * 8 + k]);
+        const Tap tp = unpack_tap(sel[c * 8 + k], lim);
         t.ch[k] = tp.ch, t.ry[k] = tp.ry, t.rx[k] = tp.rx;
     }
     t.ch0 = t.ch[0];
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
     const int c0 = blockIdx.y * ct, c1 = min(g.c, c0 + ct);
     int c = c0 + wave;
     if (c >= c1) return;
-    LaneTaps tp = lane_taps(sel, c);
+    LaneTaps tp = lane_taps(sel, c, tap_limit(g));
     Planes<T> pl;
     fetch_planes(pl, tp, xn, live);
     while (true) {
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_forward_4x4_kernel(
         const int cn = c + kLsWaves;
         const bool more = cn < c1;
         if (more) {                                                   // in flight while this kernel is evaluated
-            tp = lane_taps(sel, cn);
+            tp = lane_taps(sel, cn, tap_limit(g));
             fetch_planes(pl, tp, xn, live);
         }
         const T *ta[8];
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
     // scalar registers are scarce next to 28 gate masks).  Both planes are always fetched and written, also when a
     // kernel reads one channel only: one code path, so the registers of `pl` need no copies where paths meet.
     auto fetch = [&](int kernel) {
-        const LaneTaps t = lane_taps(sel, kernel);
+        const LaneTaps t = lane_taps(sel, kernel, tap_limit(g));
         if (t.wide) return;
 #pragma unroll
         for (int j = 0; j < 8; ++j) pl.raw[0][j] = *reinterpret_cast<const u32x4 *>(xw + j * group_step + t.ch0 * 16);
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kLsWaves *kWave, 2) void convblock_eval_packed_4x4_
     fetch(c);
     while (true) {
         const BitOps::Params pr = BitOps::load_global(gates, c);
-        const LaneTaps cur = lane_taps(sel, c);
+        const LaneTaps cur = lane_taps(sel, c, tap_limit(g));
         const int cn = c + kLsWaves;
         const bool more = cn < c1;
         const uint32_t *ta[8];
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_backward_4x4_kernel
     const int sblocks = (g.n + kWave - 1) / kWave;
     const int c0 = blockIdx.x * ct, c1 = min(g.c, c0 + ct);
     for (int c = c0; c < c1; ++c) {
-        const LaneTaps tp = lane_taps(sel, c);
+        const LaneTaps tp = lane_taps(sel, c, tap_limit(g));
         Tree<T> tr;
         const T *fc = folded + (int64_t)c * 28;
 #pragma unroll
@@ -501,7 +501,7 @@ __global__ __launch_bounds__(kLsWaves *kWave) void convblock_backward_x_4x4_kern
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             if ((mask >> t) & 1) {                                    // wave-uniform: tap t of kernel c reads this channel
-                const Tap tp = unpack_tap(sel[c * 8 + t]);
+                const Tap tp = unpack_tap(sel[c * 8 + t], tap_limit(g));
                 const int off = tp.ry * 6 + tp.rx;
                 T old[4];
                 // the four cells' targets of one tap are distinct elements; taps are applied one after the other

@@ -110,6 +110,7 @@ __device__ __forceinline__ unsigned xcd_contiguous_block(unsigned bid, unsigned 
 }
 
 // ---- plan helpers (host) ---------------------------------------------------------------------
+static inline TapLimit host_tap_limit(const Geom &g) { return TapLimit{g.cin, g.kh, g.kw}; }
 static inline void plan_common(const Geom &g, TilePlan *p)
 {
     p->rs = g.w + g.pw;
@@ -194,7 +195,7 @@ static inline unsigned pad_blocks(const PadJob<T> &j) { return (unsigned)clg_cei
 template <typename P, typename T>
 __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const P *__restrict__ w, const int32_t *__restrict__ sel,
                                                                 P *__restrict__ folded, int32_t *__restrict__ taps, int C, int rs,
-                                                                int chs, PadJob<T> pad, int pad_block0, int from_logits = 0,
+                                                                int chs, TapLimit lim, PadJob<T> pad, int pad_block0, int from_logits = 0,
                                                                 P *__restrict__ probs_out = nullptr)
 {
     if ((int)blockIdx.x >= pad_block0) {
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void convblock_w_prepare_kernel(const P *__res
     }
     const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (taps != nullptr && q < (int64_t)C * 8) {
-        const Tap tp = unpack_tap(sel[q]);
+        const Tap tp = unpack_tap(sel[q], lim);
         taps[q] = tp.ch * chs + tp.ry * rs + tp.rx;
     }
     if (folded != nullptr && q < (int64_t)C * 7) {

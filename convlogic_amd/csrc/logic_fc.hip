@@ -127,14 +127,14 @@ __device__ __forceinline__ Coef<T> load_coef(const T *__restrict__ f)
 template <typename S, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_forward_kernel(const S *__restrict__ x, const int64_t *__restrict__ a,
                                                           const int64_t *__restrict__ b, const S *__restrict__ w,
-                                                          S *__restrict__ y, int out_dim, int64_t batch)
+                                                          S *__restrict__ y, int out_dim, int64_t batch, int in_dim)
 {
     using T = typename ComputeOf<S>::type;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
     for (int j = blockIdx.x * kWavesPerBlock + wave; j < out_dim; j += gridDim.x * kWavesPerBlock) {
-        const S *xa = x + a[j] * batch;
-        const S *xb = x + b[j] * batch;
+        const S *xa = x + clamp_index(a[j], in_dim) * batch;
+        const S *xb = x + clamp_index(b[j], in_dim) * batch;
         S *yj = y + (int64_t)j * batch;
         const Coef<T> c = fold16_stored(w + (int64_t)j * 16);
         for (int64_t s = (int64_t)lane * VEC; s < batch; s += kWave * VEC) {
@@ -166,7 +166,7 @@ template <typename S, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const S *__restrict__ x, const int64_t *__restrict__ a,
                                                              const int64_t *__restrict__ b,
                                                              const S *__restrict__ gy, S *__restrict__ gw, int out_dim,
-                                                             int64_t batch, const S *__restrict__ probs)
+                                                             int64_t batch, const S *__restrict__ probs, int in_dim)
 {
     using T = typename ComputeOf<S>::type;
     constexpr int ROWS = kWave / LPR;
@@ -176,8 +176,8 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const S *__restri
          j0 += (int64_t)gridDim.x * kWavesPerBlock * ROWS) {
         const bool valid = j0 + sub < out_dim;
         const int64_t j = valid ? j0 + sub : out_dim - 1;           // every lane takes part in the reductions
-        const S *xa = x + a[j] * batch;
-        const S *xb = x + b[j] * batch;
+        const S *xa = x + clamp_index(a[j], in_dim) * batch;
+        const S *xb = x + clamp_index(b[j], in_dim) * batch;
         const S *gj = gy + j * batch;
         T sab = 0, sa = 0, sb = 0, s1 = 0;
         for (int64_t s = (int64_t)l * VEC; s < batch; s += LPR * VEC) {
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__res
          j0 += (int64_t)gridDim.x * kWavesPerBlock * ROWS) {
         const bool valid = j0 + sub < out_dim;
         const int64_t j = valid ? j0 + sub : out_dim - 1;           // every lane takes part in the reductions
-        const int64_t ia = a[j], ib = b[j];
+        const int64_t ia = clamp_index(a[j], 2 * (int64_t)out_dim), ib = clamp_index(b[j], 2 * (int64_t)out_dim);   // in_dim = 2 out_dim here
         const Coef<T> c = load_coef(folded + j * 4);
         const T *xa = x + ia * batch;
         const T *xb = x + ib * batch;
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const S *__restri
                                                              const int64_t *__restrict__ csr_start,
                                                              const int64_t *__restrict__ csr_list,
                                                              S *__restrict__ gx, int in_dim, int64_t batch,
-                                                             int batch_chunks)
+                                                             int batch_chunks, int out_dim)
 {
     using T = typename ComputeOf<S>::type;
     const int lane = threadIdx.x & (kWave - 1);
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const S *__restri
         const int i = (int)(it / batch_chunks);
         const int64_t s = ((it % batch_chunks) * kWave + lane) * VEC;
         const bool live = s < batch;
-        const int64_t beg = csr_start[i], end = csr_start[i + 1];
+        const int64_t beg = clamp_index(csr_start[i], 2 * (int64_t)out_dim + 1), end = clamp_index(csr_start[i + 1], 2 * (int64_t)out_dim + 1);
         // consumers in groups of four, one partial sum per position in the group (as fc_backward_x_folded_kernel,
         // whose results this kernel matches bit for bit)
         Pack<T, VEC> part[4];
@@ -291,9 +291,9 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_kernel(const S *__restri
             T c_ab[4], c_lin[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                j[u] = cur + u < end ? csr_list[cur + u] : -1;
+                j[u] = cur + u < end ? clamp_index(csr_list[cur + u], out_dim) : -1;
                 if (j[u] >= 0) {
-                    const int64_t ia = a[j[u]], ib = b[j[u]];
+                    const int64_t ia = clamp_index(a[j[u]], in_dim), ib = clamp_index(b[j[u]], in_dim);
                     const Coef<T> c = fold16_stored(w + j[u] * 16);
                     // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
                     // feature twice appears twice in the list and takes the B derivative the second time.
@@ -370,7 +370,7 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_forward_folded_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                                  const int64_t *__restrict__ b,
                                                                  const T *__restrict__ folded, T *__restrict__ y,
-                                                                 int out_dim, int64_t batch, int lpr_log2)
+                                                                 int out_dim, int64_t batch, int lpr_log2, int in_dim)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
@@ -380,8 +380,8 @@ __global__ __launch_bounds__(kBlock) void fc_forward_folded_kernel(const T *__re
         const int64_t j = j0 + sub;
         if (j >= out_dim) continue;
         const Coef<T> c = load_coef(folded + j * 4);
-        const T *xa = x + a[j] * batch;
-        const T *xb = x + b[j] * batch;
+        const T *xa = x + clamp_index(a[j], in_dim) * batch;
+        const T *xb = x + clamp_index(b[j], in_dim) * batch;
         T *yj = y + j * batch;
         for (int64_t s = (int64_t)l * VEC; s < batch; s += pass) {
             const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(kBlock) void fc_forward_logits_kernel(const T *__re
                                                                  const int64_t *__restrict__ b,
                                                                  const T *__restrict__ logits, T *__restrict__ probs,
                                                                  T *__restrict__ folded, T *__restrict__ y, int out_dim,
-                                                                 int64_t batch, int lpr_log2)
+                                                                 int64_t batch, int lpr_log2, int in_dim)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
@@ -437,8 +437,8 @@ __global__ __launch_bounds__(kBlock) void fc_forward_logits_kernel(const T *__re
             if (q < 4) folded[j * 4 + q] = q == 0 ? c.ab : (q == 1 ? c.a : (q == 2 ? c.b : c.one));
         }
         if (!valid) continue;
-        const T *xa = x + a[j] * batch;
-        const T *xb = x + b[j] * batch;
+        const T *xa = x + clamp_index(a[j], in_dim) * batch;
+        const T *xb = x + clamp_index(b[j], in_dim) * batch;
         T *yj = y + j * batch;
         for (int64_t s = (int64_t)l * VEC; s < batch; s += pass) {
             const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
@@ -454,7 +454,7 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
     const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
-    T *__restrict__ gx, int in_dim, int64_t batch, int batch_chunks, int lpr_log2)
+    T *__restrict__ gx, int in_dim, int64_t batch, int batch_chunks, int lpr_log2, int out_dim)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int rows = kWave >> lpr_log2, sub = lane >> lpr_log2, l = lane & ((1 << lpr_log2) - 1);
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
         const int64_t i = (it / batch_chunks) * rows + sub;
         const int64_t s = (((it % batch_chunks) << lpr_log2) + l) * VEC;
         if (i >= in_dim || s >= batch) continue;
-        const int64_t beg = csr_start[i], end = csr_start[i + 1];
+        const int64_t beg = clamp_index(csr_start[i], 2 * (int64_t)out_dim + 1), end = clamp_index(csr_start[i + 1], 2 * (int64_t)out_dim + 1);
         // Consumers in groups of four with one partial sum per position in the group, so that the rows of four
         // consumers are in flight together; the partial sums are added as (0 + 1) + (2 + 3).
         Pack<T, VEC> part[4];
@@ -478,9 +478,9 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
             T c_ab[4], c_lin[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                j[u] = cur + u < end ? csr_list[cur + u] : -1;
+                j[u] = cur + u < end ? clamp_index(csr_list[cur + u], out_dim) : -1;
                 if (j[u] >= 0) {
-                    const int64_t ia = a[j[u]], ib = b[j[u]];
+                    const int64_t ia = clamp_index(a[j[u]], in_dim), ib = clamp_index(b[j[u]], in_dim);
                     const Coef<T> c = load_coef(folded + j[u] * 4);
                     // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
                     // feature twice appears twice in the list and takes the B derivative the second time.
@@ -519,7 +519,7 @@ __device__ __forceinline__ bool fc_backward_fused_item(const T *__restrict__ x, 
                                                        const T *__restrict__ gy, const int64_t *__restrict__ csr_start,
                                                        const int64_t *__restrict__ csr_list, T *__restrict__ gw, int in_dim,
                                                        int64_t batch, const T *__restrict__ probs, int64_t it, int lane,
-                                                       Pack<T, VEC> &acc, int64_t &i)
+                                                       Pack<T, VEC> &acc, int64_t &i, int out_dim)
 {
     const int sub = lane / LPR, l = lane % LPR;
     constexpr int ROWS = kWave / LPR;
@@ -527,7 +527,7 @@ __device__ __forceinline__ bool fc_backward_fused_item(const T *__restrict__ x, 
     const bool row_ok = it * ROWS + sub < in_dim;
     i = row_ok ? it * ROWS + sub : in_dim - 1;
     const bool live = row_ok && s < batch;                           // lanes beyond the batch add zeros to the sums
-    const int64_t beg = csr_start[i], end = row_ok ? csr_start[i + 1] : beg;
+    const int64_t beg = clamp_index(csr_start[i], 2 * (int64_t)out_dim + 1), end = row_ok ? clamp_index(csr_start[i + 1], 2 * (int64_t)out_dim + 1) : beg;
     Pack<T, VEC> xi;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) xi.v[k] = 0;
@@ -545,12 +545,12 @@ __device__ __forceinline__ bool fc_backward_fused_item(const T *__restrict__ x, 
         bool first[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            j[u] = cur + u < end ? csr_list[cur + u] : -1;
+            j[u] = cur + u < end ? clamp_index(csr_list[cur + u], out_dim) : -1;
             first[u] = false;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) vo[u].v[k] = vg[u].v[k] = 0;
             if (j[u] >= 0) {
-                const int64_t ia = a[j[u]], ib = b[j[u]];
+                const int64_t ia = clamp_index(a[j[u]], in_dim), ib = clamp_index(b[j[u]], in_dim);
                 const Coef<T> c = load_coef(folded + j[u] * 4);
                 const bool as_a = ia == i && !(ib == i && prev == j[u]);   // see fc_backward_x_folded_kernel
                 first[u] = as_a;
@@ -599,7 +599,7 @@ template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
     const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
-    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int64_t batch, const T *__restrict__ probs)
+    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int64_t batch, const T *__restrict__ probs, int out_dim)
 {
     constexpr int ROWS = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
@@ -608,7 +608,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
     for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < groups; it += (int64_t)gridDim.x * kWavesPerBlock) {
         Pack<T, VEC> acc;
         int64_t i;
-        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i))
+        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i, out_dim))
             store_vec<T, VEC>(gx + i * batch + s, acc);
     }
 }
@@ -622,7 +622,7 @@ template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kSmOutWaves * kWave) void fc_backward_fused_smout_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
     const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
-    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int batch, int bp, const T *__restrict__ probs)
+    T *__restrict__ gx, T *__restrict__ gw, int in_dim, int batch, int bp, const T *__restrict__ probs, int out_dim)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     T *tile = reinterpret_cast<T *>(smem);
@@ -633,7 +633,7 @@ __global__ __launch_bounds__(kSmOutWaves * kWave) void fc_backward_fused_smout_k
     if (it < groups) {
         Pack<T, VEC> acc;
         int64_t i;
-        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i)) {
+        if (fc_backward_fused_item<T, VEC, LPR>(x, a, b, folded, gy, csr_start, csr_list, gw, in_dim, batch, probs, it, lane, acc, i, out_dim)) {
             T *row = tile + (size_t)(wave * ROWS + lane / LPR) * bp + (lane % LPR) * VEC;
             store_vec<T, VEC>(row, acc);                             // one wide LDS store (bp is a multiple of 4 elements)
         }
@@ -811,7 +811,7 @@ extern "C" int clg_fc_forward(int dtype, const void *x, const int64_t *a, const 
     const dim3 grid(grid_for(out_dim)), block(kBlock);
     hipStream_t st = clg_stream(stream);
 #define CLG_LAUNCH_F(S, VEC) \
-    hipLaunchKernelGGL((fc_forward_kernel<S, VEC>), grid, block, 0, st, (const S *)x, a, b, (const S *)w, (S *)y, (int)out_dim, batch)
+    hipLaunchKernelGGL((fc_forward_kernel<S, VEC>), grid, block, 0, st, (const S *)x, a, b, (const S *)w, (S *)y, (int)out_dim, batch, (int)in_dim)
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_F(float, 4);
         else CLG_LAUNCH_F(float, 1);
@@ -837,7 +837,7 @@ static int fc_backward_w_impl(int dtype, const void *x, const int64_t *a, const 
 #define CLG_LAUNCH_BW(T, VEC, LPR)                                                                                      \
     hipLaunchKernelGGL((fc_backward_w_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave / LPR)))), \
                        block, 0, st, (const T *)x, a, b, (const T *)grad_y, (T *)grad_w, (int)out_dim, batch,              \
-                       (const T *)probs)
+                       (const T *)probs, (int)in_dim)
 #define CLG_LAUNCH_BW_ROWS(T, VEC)                                                                                      \
     do {                                                                                                               \
         const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
@@ -888,7 +888,7 @@ extern "C" int clg_fc_backward_x(int dtype, const void *x, const int64_t *a, con
         const int chunks = (int)clg_ceil_div(batch, (int64_t)kWave * VEC);                                             \
         hipLaunchKernelGGL((fc_backward_x_kernel<T, VEC>), dim3(grid_for(in_dim * chunks)), block, 0, st, (const T *)x, \
                            a, b, (const T *)w, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (int)in_dim, batch,  \
-                           chunks);                                                                                    \
+                           chunks, (int)out_dim);                                                                                 \
     } while (0)
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_BX(float, 4);
@@ -934,7 +934,7 @@ extern "C" int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a,
     do {                                                                                                               \
         const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
         hipLaunchKernelGGL((fc_forward_folded_kernel<T, VEC>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave >> lg)))), \
-                           block, 0, st, (const T *)x, a, b, (const T *)folded, (T *)y, (int)out_dim, batch, lg);          \
+                           block, 0, st, (const T *)x, a, b, (const T *)folded, (T *)y, (int)out_dim, batch, lg, (int)in_dim);       \
     } while (0)
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_FF(float, 4);
@@ -976,7 +976,7 @@ extern "C" int clg_fc_forward_logits(int dtype, const void *x, const int64_t *a,
         const int lg = lanes_per_row_log2(batch, VEC);                                                                 \
         hipLaunchKernelGGL((fc_forward_logits_kernel<T, VEC>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave >> lg)))), \
                            block, 0, st, (const T *)x, a, b, (const T *)logits, (T *)probs, (T *)folded, (T *)y,           \
-                           (int)out_dim, batch, lg);                                                                   \
+                           (int)out_dim, batch, lg, (int)in_dim);                                                              \
     } while (0)
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_FL(float, 4);
@@ -1006,7 +1006,7 @@ extern "C" int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t 
         const int64_t items = clg_ceil_div(in_dim, (int64_t)(kWave >> lg)) * chunks;                                   \
         hipLaunchKernelGGL((fc_backward_x_folded_kernel<T, VEC>), dim3(grid_for(items)), block, 0, st, (const T *)x, a, b, \
                            (const T *)folded, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (int)in_dim, batch,     \
-                           chunks, lg);                                                                                \
+                           chunks, lg, (int)out_dim);                                                                        \
     } while (0)
     if (dtype == CLG_F32) {
         if (batch % 4 == 0) CLG_LAUNCH_BXF(float, 4);
@@ -1095,12 +1095,12 @@ extern "C" int clg_fc_backward_fused_ex(int dtype, const void *x, const int64_t 
             hipLaunchKernelGGL((fc_backward_fused_smout_kernel<T, VEC, LPR>), dim3((unsigned)clg_ceil_div(in_dim, (int64_t)F)), \
                                dim3(kSmOutWaves * kWave), (size_t)F * bp * sizeof(T), st, (const T *)x, a, b, (const T *)folded, \
                                (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (T *)grad_w, (int)in_dim, (int)batch, bp, \
-                               (const T *)probs);                                                                           \
+                               (const T *)probs, (int)out_dim);                                                                      \
         } else {                                                                                                            \
             hipLaunchKernelGGL((fc_backward_fused_kernel<T, VEC, LPR>),                                                     \
                                dim3(grid_for(clg_ceil_div(in_dim, (int64_t)(kWave / LPR)))), dim3(kBlock), 0, st, (const T *)x, a, b, \
                                (const T *)folded, (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (T *)grad_w, (int)in_dim, \
-                               batch, (const T *)probs);                                                                    \
+                               batch, (const T *)probs, (int)out_dim);                                                              \
         }                                                                                                                   \
     } while (0)
 #define CLG_LAUNCH_BF_ROWS(T, VEC)                                                                                         \

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_kernel(const V *__rest
                                                                const int64_t *__restrict__ b,
                                                                const uint8_t *__restrict__ gate, V *__restrict__ y,
                                                                int out_dim, int64_t row_vecs, int chunk_vecs,
-                                                               int groups_per_chunk, int neurons_per_wave)
+                                                               int groups_per_chunk, int neurons_per_wave, int64_t in_dim)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
@@ -36,8 +36,8 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_kernel(const V *__rest
     for (int jj = 0; jj < neurons_per_wave; ++jj) {
         const int j = j0 + jj;
         if (j >= out_dim) break;
-        const V *xa = x + a[j] * row_vecs;
-        const V *xb = x + b[j] * row_vecs;
+        const V *xa = x + clamp_index(a[j], in_dim) * row_vecs;    // (a bad index reads a wrong row; it never leaves x)
+        const V *xb = x + clamp_index(b[j], in_dim) * row_vecs;
         V *yj = y + (int64_t)j * row_vecs;
         const Masks m = gate_masks(gate[j]);
         for (int64_t v = v0 + lane; v < v1; v += (int64_t)kWave * UNROLL) {
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x
                                                                     const int64_t *__restrict__ b,
                                                                     const uint8_t *__restrict__ gate,
                                                                     const int32_t *__restrict__ plan, u32x4 *__restrict__ y,
-                                                                    int steps, int seg_len, int64_t row_vecs)
+                                                                    int steps, int seg_len, int64_t row_vecs, int64_t in_dim)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
@@ -87,10 +87,10 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x
     for (int r = 0; r < R; ++r) carry[r] = (u32x4)0u;
     for (int k = k0; k < k1; ++k) {
         const int p = plan[k];
-        const int j = p & 0x0FFFFFFF, keep = (p >> 30) & 1;
+        const int j = min(p & 0x0FFFFFFF, steps - 1), keep = (p >> 30) & 1;   // one plan entry per neuron
         const int use = k == k0 ? 0 : (p >> 28) & 3;
-        const u32x4 *xa = x + a[j] * row_vecs + col0;
-        const u32x4 *xb = x + b[j] * row_vecs + col0;
+        const u32x4 *xa = x + clamp_index(a[j], in_dim) * row_vecs + col0;
+        const u32x4 *xb = x + clamp_index(b[j], in_dim) * row_vecs + col0;
         if (use != 1 && use != 3) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
@@ -120,13 +120,13 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x
 // bytewise tail / odd row sizes: one thread per byte of the output
 __global__ void eval_packed_bytes_kernel(const uint8_t *__restrict__ x, const int64_t *__restrict__ a,
                                          const int64_t *__restrict__ b, const uint8_t *__restrict__ gate,
-                                         uint8_t *__restrict__ y, int64_t out_dim, int64_t row_bytes)
+                                         uint8_t *__restrict__ y, int64_t out_dim, int64_t row_bytes, int64_t in_dim)
 {
     const int64_t total = out_dim * row_bytes;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t j = i / row_bytes, c = i % row_bytes;
         const Masks m = gate_masks(gate[j]);
-        y[i] = (uint8_t)gate_bits(m, x[a[j] * row_bytes + c], x[b[j] * row_bytes + c]);
+        y[i] = (uint8_t)gate_bits(m, x[clamp_index(a[j], in_dim) * row_bytes + c], x[clamp_index(b[j], in_dim) * row_bytes + c]);
     }
 }
 
@@ -509,7 +509,7 @@ int small_grid(int64_t items, int block)
 
 template <typename V>
 void launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate, void *y, int64_t out_dim,
-                 int64_t row_bytes, hipStream_t st)
+                 int64_t row_bytes, hipStream_t st, int64_t in_dim)
 {
     const int64_t row_vecs = row_bytes / (int64_t)sizeof(V);
     // column chunks of at most 4 KiB per row: both uses of a row segment fall inside one chunk pass,
@@ -522,7 +522,7 @@ void launch_eval(const void *x, const int64_t *a, const int64_t *b, const uint8_
     const int neurons_per_wave = e_npw ? atoi(e_npw) : 1;
     const int groups = (int)clg_ceil_div(out_dim, (int64_t)kEvalWaves * neurons_per_wave);
     hipLaunchKernelGGL((eval_packed_kernel<V, 2>), dim3((unsigned)(chunks * groups)), dim3(kEvalBlock), 0, st, (const V *)x, a,
-                       b, gate, (V *)y, (int)out_dim, row_vecs, chunk_vecs, groups, neurons_per_wave);
+                       b, gate, (V *)y, (int)out_dim, row_vecs, chunk_vecs, groups, neurons_per_wave, in_dim);
 }
 
 bool valid_elem(int e) { return e == 1 || e == 2 || e == 4 || e == 8; }
@@ -544,12 +544,12 @@ extern "C" int clg_fc_eval_packed(int elem_size, const void *x, const int64_t *a
     if (blocks_needed >= (1ll << 31)) {
         CLG_REQUIRE(false, "clg_fc_eval_packed: problem too large for one launch (%lld blocks)", (long long)blocks_needed);
     }
-    if ((align & 15) == 0) launch_eval<u32x4>(x, a, b, gate, y, out_dim, row_bytes, st);
-    else if ((align & 7) == 0) launch_eval<u32x2>(x, a, b, gate, y, out_dim, row_bytes, st);
-    else if ((align & 3) == 0) launch_eval<uint32_t>(x, a, b, gate, y, out_dim, row_bytes, st);
+    if ((align & 15) == 0) launch_eval<u32x4>(x, a, b, gate, y, out_dim, row_bytes, st, in_dim);
+    else if ((align & 7) == 0) launch_eval<u32x2>(x, a, b, gate, y, out_dim, row_bytes, st, in_dim);
+    else if ((align & 3) == 0) launch_eval<uint32_t>(x, a, b, gate, y, out_dim, row_bytes, st, in_dim);
     else
         hipLaunchKernelGGL(eval_packed_bytes_kernel, dim3(small_grid(out_dim * row_bytes, 256)), dim3(256), 0, st,
-                           (const uint8_t *)x, a, b, gate, (uint8_t *)y, out_dim, row_bytes);
+                           (const uint8_t *)x, a, b, gate, (uint8_t *)y, out_dim, row_bytes, in_dim);
     CLG_CHECK_LAUNCH("clg_fc_eval_packed");
     return CLG_OK;
 }
@@ -735,7 +735,7 @@ extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const in
     hipStream_t st = clg_stream(stream);
 #define CLG_WALK(RR)                                                                                                          \
     hipLaunchKernelGGL(eval_packed_walk_kernel<RR>, grid, block, 0, st, (const u32x4 *)x, a, b, gate, plan, (u32x4 *)y, (int)out_dim, \
-                       seg, row_vecs)
+                       seg, row_vecs, in_dim)
     switch (R) {
     case 1: CLG_WALK(1); break;
     case 2: CLG_WALK(2); break;

@@ -56,6 +56,7 @@ class LogicLayer(torch.nn.Module):
             start, flat = _reverse_wiring(self.indices_0.cpu().numpy(), self.indices_1.cpu().numpy(), in_dim)
             self.register_buffer("given_x_indices_of_y_start", start)
             self.register_buffer("given_x_indices_of_y", flat)
+            self._reverse_built = (self.indices_0._version, self.indices_1._version)
 
         self.num_neurons = out_dim
         self.num_weights = out_dim
@@ -155,6 +156,16 @@ class LogicLayer(torch.nn.Module):
                 if not (self.indices_0.is_contiguous() and self.indices_1.is_contiguous()
                         and self.indices_0.device == self.indices_1.device == self.weights.device):
                     raise ValueError("indices_0 / indices_1 must be contiguous and on the device of the weights")
+                # The reverse map belongs to the wiring it was built from: after an in-place rewiring or a state_dict
+                # that replaced the indices it is rebuilt here (into the same buffers), so the input gradient never walks
+                # the lists of an older wiring.  (The reference builds it once, src/difflogic/difflogic.py:71-87.)
+                built = (self.indices_0._version, self.indices_1._version)
+                if self.__dict__.get("_reverse_built") != built:
+                    start, flat = _reverse_wiring(self.indices_0.cpu().numpy(), self.indices_1.cpu().numpy(), self.in_dim)
+                    with torch.no_grad():
+                        self.given_x_indices_of_y_start.copy_(start)
+                        self.given_x_indices_of_y.copy_(flat)
+                    self._reverse_built = built
             self._wiring_checked = key
 
     def _sm_tables(self, key=None):
@@ -172,7 +183,7 @@ class LogicLayer(torch.nn.Module):
         """Drops everything derived from the wiring buffers (range check, consumer analysis, packed walk plan, tables of
         the sample-major kernels).  Needed only after writing indices_0 / indices_1 through `.data`, which the version
         counters do not see."""
-        self._wiring_checked = self._sole_cache = self._plan_cache = self._sm_cache = None
+        self._wiring_checked = self._sole_cache = self._plan_cache = self._sm_cache = self._reverse_built = None
 
     def _load_from_state_dict(self, *args, **kwargs):
         super()._load_from_state_dict(*args, **kwargs)

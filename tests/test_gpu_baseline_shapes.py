@@ -86,30 +86,47 @@ def test_config3_block_256x1x28x28_forward_and_gradients_vs_oracle():
 
 @pytest.mark.timeout(600)
 def test_config4_block_256x9x32x32_forward_and_gradients_vs_oracle():
-    layer, xg, gy = _block_full_size(256, 9, 256, 32, _c4_input(256, 4), seed=44, chunk=32)
-    # the reference-shaped pair of calls (probabilities from torch.softmax in, gradient w.r.t. the probabilities out)
-    # on the same data: its probabilities differ from the in-kernel softmax in the last bit, so a pooled cell whose two
-    # best positions tie to rounding may route its gradient to the other one -- agreement up to those cells
+    _block_full_size(256, 9, 256, 32, _c4_input(256, 4), seed=44, chunk=32)
+
+
+@pytest.mark.timeout(600)
+def test_config4_reference_shaped_function_vs_oracle_along_its_own_route():
+    # the reference-shaped pair of calls (probabilities from torch.softmax in, gradient w.r.t. the probabilities out) at
+    # full C4: forward and both gradients against the float64 oracle evaluated along the route THIS call pooled
+    torch.manual_seed(45)
+    n, cin, cout, size, chunk = 256, 9, 256, 32, 32
+    layer = C.ConvLogicLayer(cin, cout, complete=True, implementation="cuda").to(DEV)
     w = torch.softmax(layer.weights.detach(), -1).requires_grad_(True)
-    x2 = xg.detach().clone().requires_grad_(True)
-    y2 = C.FullConvLogicFunction.apply(x2, w, layer.selection, 1, 1, 1, 1, 3, 3)
-    y2.backward(gy)
-    p = torch.softmax(layer.weights.detach().double(), -1)
-    gw = w.grad.double()
-    gl = p * (gw - (p * gw).sum(-1, keepdim=True))
-    for got, ref, name in ((gl, layer.weights.grad.double(), "grad_logits"), (x2.grad.double(), xg.grad.double(), "grad_x")):
-        assert ((got - ref).norm() / ref.norm()).item() <= 1e-2, name
-        assert (got - ref).abs().max().item() <= 5e-2 * ref.abs().max().item(), name
+    x = _c4_input(n, 4).to(DEV).requires_grad_(True)
+    y, idx = C.FullConvLogicFunction.apply(x, w, layer.selection, 1, 1, 1, 1, 3, 3, False, True)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    gw_ref = torch.zeros(cout, 7, 16, dtype=torch.float64)
+    flips = 0
+    for s0 in range(0, n, chunk):
+        sl = slice(s0, s0 + chunk)
+        xl = x.detach()[sl].cpu().double().requires_grad_(True)
+        wl = w.detach().cpu().double().requires_grad_(True)
+        y_ref, _, x3, idx_ref = O.conv_block_forward(xl, wl, layer.selection.cpu(), (1, 1), (1, 1), (3, 3), return_all=True)
+        x4 = O.tree_forward(x3, wl[:, 6:7]).squeeze(-1)
+        flips += check_pool_route(idx[sl], idx_ref, x4)
+        routed = x4.flatten(2).gather(2, idx[sl].cpu().long()).view_as(y_ref)
+        assert (y.detach()[sl].cpu().double() - routed.detach()).abs().max().item() <= 1e-5, s0
+        routed.backward(gy[sl].cpu().double())
+        assert_grad_close(x.grad[sl], xl.grad, name=f"grad_x[{s0}:]")
+        gw_ref += wl.grad
+    assert flips <= 1e-4 * idx.numel(), flips
+    assert_grad_close(w.grad, gw_ref, name="grad_w")
 
 
-@pytest.mark.timeout(900)
-def test_config5_network_batch256_float32_vs_oracle():
-    # the k = 32 CIFAR topology (4 blocks, flatten, 3 LogicLayers, GroupSum(10, 6.5)) with random-init logits, one
-    # cross-entropy training step in float32 at batch 256: scores, loss and every layer's logit gradient against the
-    # float64 oracle routed through the pooling choices of the GPU
+def _config5_network_step(residual_init, binary_first_block):
+    """the k = 32 CIFAR topology (4 blocks, flatten, 3 LogicLayers, GroupSum(10, 6.5)), one cross-entropy training step in
+    float32 at batch 256: scores, loss and every layer's logit gradient against the float64 oracle routed through the
+    pooling choices of the GPU.  -> (pool-route flips per block, pooled cells per block, check(rel_elem))"""
     from tests.test_gpu_model import build
     torch.manual_seed(55)
-    model = build().to(DEV)
+    model = build(residual_init=residual_init).to(DEV)
+    model[0].binary_input = binary_first_block
     n = 256
     x = _c4_input(n, 5)
     labels = torch.randint(0, 10, (n,), generator=torch.Generator().manual_seed(6))
@@ -161,13 +178,45 @@ def test_config5_network_batch256_float32_vs_oracle():
     # into a random-init network the activations of neighbouring positions agree to float32 rounding in a sizeable
     # share of the windows (measured: several percent), which is why the oracle follows the GPU's route.
     print("pool route flips per block:", flips, "of", cells)
-    assert flips[0] <= 1e-4 * cells[0], (flips, cells)
     # scores are sums of 1024 gate outputs / 6.5: 1e-5 per value allows 1.6e-3; measured differences are ~1e-5
     assert (scores.detach().cpu().double() - torch.cat(ref_scores)).abs().max().item() <= 1e-4
     assert abs(loss.item() - ref_loss) <= 1e-5
-    # global and max-scaled bounds at 1e-4; the per-element bound against the MEAN magnitude at 5e-4: the gradients of
-    # the early layers (~1e-11) have passed through up to seven float32 layers, each within 1e-4 on its own
-    # (measured worst element: 1.4e-4 in the second block)
-    for i, (m, leaf) in enumerate(zip(params, leaves)):
-        assert_grad_close(m.weights.grad, leaf.grad, name=f"layer {i} grad_logits", rel_elem=5e-4)
-    assert_grad_close(xg.grad, torch.cat(ref_gx), name="grad_x", rel_elem=5e-4)
+
+    def check(rel_elem):
+        worst = []
+        for i, (m, leaf) in enumerate(zip(params, leaves)):
+            got, ref = m.weights.grad.detach().double().cpu(), leaf.grad
+            worst.append(((got - ref).abs() / (ref.abs() + ref.abs().mean() + 1e-30)).max().item())
+        print("worst per-element relative error of grad_logits per layer:", ["%.2e" % w for w in worst])
+        for i, (m, leaf) in enumerate(zip(params, leaves)):
+            assert_grad_close(m.weights.grad, leaf.grad, name=f"layer {i} grad_logits", rel_elem=rel_elem)
+        assert_grad_close(xg.grad, torch.cat(ref_gx), name="grad_x", rel_elem=rel_elem)
+
+    return flips, cells, check
+
+
+@pytest.mark.timeout(900)
+def test_config5_network_batch256_float32_vs_oracle():
+    # random-init logits (BASELINE config 5).  Deep into a random-init network the activations of neighbouring positions
+    # agree to float32 rounding in a sizeable share of the windows, so only the first block's route is bounded; the
+    # per-element bound against the MEAN magnitude is 5e-4: the gradients of the early layers (~1e-11) have passed
+    # through up to seven float32 layers, each within 1e-4 on its own (measured worst element: 1.4e-4 in the second block)
+    flips, cells, check = _config5_network_step(residual_init=False, binary_first_block=False)
+    assert flips[0] <= 1e-4 * cells[0], (flips, cells)
+    check(5e-4)
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("binary_first_block", [True, False])
+def test_config5_network_residual_init_vs_oracle(binary_first_block):
+    # the reference's own initialisation (residual_init=True, src/convlogic/model.py:36,55), the first block on the
+    # binary-input kernels as in the model topologies.  Every kernel starts as (almost) the pass-through gate A, so the
+    # activations take few distinct levels and the four positions of a pooling window are often EQUAL up to rounding: which
+    # of them wins is then decided by the last bit, in float32 here and in float64 in the oracle (measured: 8 %, 22 % and
+    # 33 % of the windows of blocks 2-4 pick another position, every one of them within the 1e-5 value gap that
+    # check_pool_route asserts; block 1, on binary inputs, has none).  The per-element bound against the mean magnitude is
+    # 5e-4 as for the random-init network: measured worst element 2.4e-4 (first block) with the binary-input kernels and
+    # with the any-input kernels alike -- float32 rounding through seven layers, not a property of either path.
+    flips, cells, check = _config5_network_step(residual_init=True, binary_first_block=binary_first_block)
+    assert flips[0] <= 1e-4 * cells[0], (flips, cells)
+    check(5e-4)

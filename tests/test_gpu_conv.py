@@ -545,3 +545,33 @@ def test_native_module_drop_in_with_the_reference_signatures(stride, pad, kernel
     for name in ("convlogic_forward", "convlogic_backward_x", "convlogic_backward_weight", "treelogic_forward",
                  "treelogic_backward_x", "treelogic_backward_weight"):
         assert callable(getattr(convlogic_cuda, name))
+
+
+def test_selection_corrupted_behind_the_host_check_is_clamped_not_faulting():
+    # a selection written through `.data` after the (cached) host check names a channel, row and column outside the
+    # layer: every kernel decodes taps through the layer's limits, so the calls return instead of faulting the GPU
+    torch.manual_seed(41)
+    for binary in (False, True):
+        layer = C.ConvLogicLayer(3, 6, complete=True, implementation="cuda").to(DEV)
+        layer.binary_input = binary
+        x = torch.randint(0, 2, (4, 3, 8, 8), device=DEV).float().requires_grad_(True)
+        layer(x).sum().backward()
+        bad = layer.selection.data.clone()
+        bad[2, 1] = (200 << 16) | (9 << 8) | 7
+        bad[4, 6] = (3 << 16) | (3 << 8) | 3
+        layer.selection.data.copy_(bad)
+        layer._plans = {}                                            # (plans are keyed on the version counter, which .data bypasses)
+        y = layer(x)
+        y.sum().backward()
+        torch.cuda.synchronize()
+        assert torch.isfinite(y).all() and torch.isfinite(x.grad).all() and torch.isfinite(layer.weights.grad).all()
+        # the result is that of the selection forced into range
+        fixed = layer.selection.clone()
+        ch, ry, rx = (fixed >> 16) & 0xFFFF, (fixed >> 8) & 0xFF, fixed & 0xFF
+        fixed = (ch.clamp(max=2) << 16) | (ry.clamp(max=2) << 8) | rx.clamp(max=2)
+        ref = C.ConvLogicLayer(3, 6, complete=True, implementation="cuda", selection=fixed.to(torch.int32)).to(DEV)
+        ref.weights.data.copy_(layer.weights.data)
+        assert torch.equal(y, ref(x.detach()))
+        layer.invalidate()
+        with pytest.raises(ValueError, match="selection"):
+            layer(x)

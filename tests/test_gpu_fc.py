@@ -520,6 +520,55 @@ def test_fc_rewired_out_of_range_raises_instead_of_launching():
         layer(C.PackBitsTensor(x > 0.5, 64))
 
 
+def test_fc_rewired_in_range_rebuilds_the_reverse_map():
+    # an in-place rewiring (version counter) must reach the input gradient: the reverse map is rebuilt from the indices
+    torch.manual_seed(31)
+    layer = C.LogicLayer(20, 30, implementation="cuda").to(DEV)
+    x = torch.rand(8, 20, device=DEV, requires_grad=True)
+    layer(x).sum().backward()
+    layer.indices_0[7] = 3
+    layer.indices_1[11] = 19
+    x.grad = None
+    gy = torch.randn(8, 30, device=DEV)
+    layer(x).backward(gy)
+    xl = x.detach().cpu().requires_grad_(True)
+    O.logic_fc_forward(xl, layer.indices_0.cpu(), layer.indices_1.cpu(), torch.softmax(layer.weights.detach().cpu(), -1)).backward(gy.cpu())
+    assert_grad_close(x.grad, xl.grad, name="grad_x after rewiring")
+
+
+def test_fc_index_corrupted_behind_the_host_check_is_clamped_not_faulting():
+    # a write through `.data` is invisible to the cached host check: the kernels force every index into range, so the
+    # call returns (reading a wrong row) instead of faulting the GPU -- forward, both gradients and the packed path
+    torch.manual_seed(32)
+    layer = C.LogicLayer(16, 24, implementation="cuda").to(DEV)
+    x = torch.rand(8, 16, device=DEV, requires_grad=True)
+    layer(x).sum().backward()                                        # host checks are now cached
+    layer.eval()
+    layer(C.PackBitsTensor(x.detach() > 0.5, 64))                    # ... and so is the walk plan of the packed path
+    layer.train()
+    layer.indices_0.data[5] = 1 << 40
+    layer.indices_1.data[6] = -3
+    y = layer(x)
+    y.sum().backward()
+    torch.cuda.synchronize()
+    clamped = layer.indices_0.clamp(0, 15), layer.indices_1.clamp(0, 15)
+    want = O.logic_fc_forward(x.detach().cpu(), clamped[0].cpu(), clamped[1].cpu(), torch.softmax(layer.weights.detach().cpu(), -1))
+    assert (y.detach().cpu() - want).abs().max().item() <= 1e-5
+    assert torch.isfinite(x.grad).all() and torch.isfinite(layer.weights.grad).all()
+    layer.eval()
+    bits = x.detach() > 0.5
+    out = layer(C.PackBitsTensor(bits, 64)).t                        # packed path on the cached plan: clamped as well
+    torch.cuda.synchronize()
+    import numpy as np
+    words, _ = O.pack_bits(bits.cpu().numpy().T, 64)
+    want_words = O.eval_packed(words, clamped[0].cpu().numpy(), clamped[1].cpu().numpy(), layer.weights.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(out.cpu().numpy(), want_words)
+    # invalidate() brings the host check back
+    layer.invalidate()
+    with pytest.raises(ValueError, match="indices_0"):
+        layer(x)
+
+
 def test_packed_gates_follow_in_place_weight_updates():
     # the arg-max gates of the packed path are taken from the logits on every call: an update through `.data`
     # (EMA swap, legacy optimiser), which no version counter sees, must change the evaluated network

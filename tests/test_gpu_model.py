@@ -13,13 +13,14 @@ from tests.gpu_util import DEV, assert_grad_close
 pytestmark = pytest.mark.gpu
 
 
-def build(k=32, cin=9, size=32, tau=6.5):
+def build(k=32, cin=9, size=32, tau=6.5, residual_init=False):
     chans = [cin, k, 4 * k, 16 * k, 32 * k]
-    layers = [C.ConvLogicLayer(a, b, padding=1, complete=True, implementation="cuda") for a, b in zip(chans[:-1], chans[1:])]
+    layers = [C.ConvLogicLayer(a, b, padding=1, complete=True, implementation="cuda", residual_init=residual_init)
+              for a, b in zip(chans[:-1], chans[1:])]
     flat = chans[-1] * (size // 16) ** 2
     dims = [flat, flat * 10, flat * 5, (flat * 10) // 4]
     layers.append(torch.nn.Flatten())
-    layers += [C.LogicLayer(a, b, implementation="cuda") for a, b in zip(dims[:-1], dims[1:])]
+    layers += [C.LogicLayer(a, b, implementation="cuda", residual_init=residual_init) for a, b in zip(dims[:-1], dims[1:])]
     layers.append(C.GroupSum(10, tau))
     return torch.nn.Sequential(*layers)
 

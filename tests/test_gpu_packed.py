@@ -190,3 +190,42 @@ def test_eval_plan_follows_in_place_rewiring():
     want = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(),
                          layer.weights.argmax(-1).cpu().numpy().astype(np.uint8))
     assert np.array_equal(y2.cpu().numpy(), want) and not torch.equal(y1, y2)
+
+
+@pytest.mark.timeout(600)
+def test_eval_packed_config2_full_size_vs_c_oracle():
+    # BASELINE config 2 at full size against the CPU oracle, word for word: 3 layers of 64000 neurons on 65536 samples in
+    # 1024 int64 words per feature through the module path, every layer's output compared with oracle/packed_oracle.c
+    # (OpenMP, about 25 ms per layer on the host cores), then the per-class counts against numpy on the oracle's words.
+    import ctypes
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "libpacked_oracle.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/libpacked_oracle.so not built (make -C oracle)")
+    lib = ctypes.CDLL(path)
+    width, words, k = 64000, 1024, 10
+    rng = np.random.default_rng(22)
+    x = rng.integers(-2**63, 2**63 - 1, (width, words), dtype=np.int64, endpoint=True)
+    torch.manual_seed(22)
+    layers = [C.LogicLayer(width, width, implementation="cuda").to(DEV).eval() for _ in range(3)]
+    packed = C.PackBitsTensor.__new__(C.PackBitsTensor)
+    packed.bit_count, packed.pad_len, packed.image, packed.t = 64, 0, False, torch.from_numpy(x).to(DEV)
+    ref = x
+    vp = ctypes.c_void_p
+    with torch.no_grad():
+        for i, layer in enumerate(layers):
+            packed = layer(packed)
+            a = layer.indices_0.cpu().numpy().astype(np.int64)
+            b = layer.indices_1.cpu().numpy().astype(np.int64)
+            gate = layer.weights.argmax(-1).cpu().numpy().astype(np.uint8)
+            out = np.empty_like(ref)
+            lib.oracle_eval_packed(ref.ctypes.data_as(vp), a.ctypes.data_as(vp), b.ctypes.data_as(vp), gate.ctypes.data_as(vp),
+                                   out.ctypes.data_as(vp), ctypes.c_int64(width), ctypes.c_int64(words * 8))
+            assert np.array_equal(packed.t.cpu().numpy(), out), f"layer {i}"
+            ref = out
+        counts = packed.group_sum(k).cpu().numpy()
+    assert counts.shape == (65536, k) and counts.dtype == np.int32
+    per = width // k
+    for g in range(k):                                               # class g: rows g*per .. (g+1)*per, sample s = bit s%8 of byte s/8
+        bits = np.unpackbits(ref[g * per:(g + 1) * per].view(np.uint8), axis=1, bitorder="little")
+        assert np.array_equal(counts[:, g], bits.sum(axis=0, dtype=np.int32)), f"class {g}"

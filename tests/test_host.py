@@ -336,3 +336,16 @@ def test_recorded_traffic_file_feeds_the_bench_line():
         assert got == rec["workloads"][wl]["step_bytes"] and got > 0
         assert abs(sum(k["bytes_per_launch"] * k["launches_per_step"] for k in rec["workloads"][wl]["kernels"].values()) - got) <= len(rec["workloads"][wl]["kernels"])
     assert bench._traffic("c9", "step_bytes") is None and bench._traffic("c4", "no_such_key") is None
+
+
+def test_python_path_rejects_an_index_rewired_out_of_range_through_data():
+    # the torch-op backend indexes with the wiring on every call (as the reference does, src/difflogic/difflogic.py:149-164):
+    # an index written through `.data` past the version counter raises there; the HIP kernels force it into range instead
+    # (tests/test_gpu_fc.py::test_fc_index_corrupted_behind_the_host_check_is_clamped_not_faulting)
+    import pytest
+    layer = C.LogicLayer(8, 12, implementation="python")
+    x = torch.rand(4, 8)
+    layer(x)
+    layer.indices_0.data[3] = 8
+    with pytest.raises((IndexError, RuntimeError)):
+        layer(x)
