@@ -9,7 +9,7 @@ import sys
 
 PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
-SOURCES = ["clg_api.hip", "conv_binary.hip", "logic_fc.hip", "logic_fc_sm.hip", "packbits.hip", "binarize.hip", "conv_generic.hip", "conv_forward.hip", "conv_small.hip", "conv_block.hip"]
+SOURCES = ["clg_api.hip", "conv_binary.hip", "logic_fc.hip", "packbits.hip", "binarize.hip", "conv_generic.hip", "conv_forward.hip", "conv_small.hip", "conv_block.hip"]
 LIB = os.path.join(PKG, "libconvlogic_amd.so")
 
 

@@ -1239,6 +1239,15 @@ static int static_scratch_ptr(void **out, const char *name)
 
 extern "C" int64_t clg_group_sum_static_max_bytes(void) { return kStaticScratchBytes; }
 
+// Looks the buffer's device address up for the current device (a runtime query, not a stream operation): callers that
+// capture clg_group_sum_static into a HIP graph call this once per device BEFORE the capture starts; after it the entry
+// point makes no runtime call besides its two launches.
+extern "C" int clg_group_sum_static_init(void)
+{
+    void *p = nullptr;
+    return static_scratch_ptr(&p, "clg_group_sum_static_init");
+}
+
 extern "C" int clg_group_sum_static(int dtype, const void *x, void *out, int64_t features, int64_t batch, int64_t k, double tau,
                                     void *stream)
 {

@@ -98,10 +98,6 @@ class LogicLayer(torch.nn.Module):
         weights, buffers = self._parameters["weights"], self._buffers
         if (self.training and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
                 and weights.is_contiguous() and weights.device == x.device):
-            if x.is_contiguous() and difflogic_hip.sm_preferred(x, self.out_dim):
-                # asked for with CLG_FC_SAMPLE_MAJOR=1, on a sample-major batch whose rows fit LDS: kernels that work in
-                # that layout, no transposed copies on either side
-                return _LogicLayerSampleMajorFunction.apply(x, weights, *self._sm_tables(key))
             # a sample-major batch is transposed inside the Function (and its gradient on the way back): one autograd
             # node per layer instead of two
             inside = _transposes_with_kernel(x)
@@ -168,22 +164,10 @@ class LogicLayer(torch.nn.Module):
                     self._reverse_built = built
             self._wiring_checked = key
 
-    def _sm_tables(self, key=None):
-        """Tables of the sample-major kernels (32-bit wiring, reverse map with the other operand of every consumer), made
-        once per wiring on the host."""
-        key = key or self._wiring_key()
-        cached = self.__dict__.get("_sm_cache")
-        if cached is None or cached[0] != key:
-            cached = (key, difflogic_hip.sm_plan(self.indices_0, self.indices_1, self.given_x_indices_of_y_start,
-                                                 self.given_x_indices_of_y, self.in_dim))
-            self._sm_cache = cached
-        return cached[1]
-
     def invalidate(self):
-        """Drops everything derived from the wiring buffers (range check, consumer analysis, packed walk plan, tables of
-        the sample-major kernels).  Needed only after writing indices_0 / indices_1 through `.data`, which the version
+        """Drops everything derived from the wiring buffers (range check, consumer analysis, packed walk plan, reverse map).  Needed only after writing indices_0 / indices_1 through `.data`, which the version
         counters do not see."""
-        self._wiring_checked = self._sole_cache = self._plan_cache = self._sm_cache = self._reverse_built = None
+        self._wiring_checked = self._sole_cache = self._plan_cache = self._reverse_built = None
 
     def _load_from_state_dict(self, *args, **kwargs):
         super()._load_from_state_dict(*args, **kwargs)
@@ -377,25 +361,6 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
         if ctx.sample_major_input and grad_x is not None:
             grad_x = difflogic_hip.transpose(grad_x)
         return grad_x, None, None, grad_l, None, None, None, None
-
-
-class _LogicLayerSampleMajorFunction(torch.autograd.Function):
-    """Training path of the module on a sample-major batch: y [B, out] = layer(x [B, in]) as a function of the LOGITS,
-    on kernels that stage sample rows in LDS -- no transposed copies of x, grad_y or grad_x.  Same values as the
-    feature-major path up to the order of float additions."""
-
-    @staticmethod
-    def forward(ctx, x, logits, ab32, start32, entry):
-        probs, folded, coef_e = difflogic_hip.fold_sm(logits.detach(), entry)
-        ctx.save_for_backward(x, probs, coef_e, ab32, start32, entry)
-        return difflogic_hip.forward_sm(x, ab32, folded)
-
-    @staticmethod
-    def backward(ctx, grad_y):
-        x, probs, coef_e, ab32, start32, entry = ctx.saved_tensors
-        grad_x, grad_l = difflogic_hip.backward_sm(x, grad_y.contiguous(), ab32, start32, entry, coef_e, probs,
-                                                   need_grad_x=ctx.needs_input_grad[0], need_grad_w=ctx.needs_input_grad[1])
-        return grad_x, grad_l, None, None, None
 
 
 def _needs_check(grad_y, x):

@@ -43,16 +43,10 @@ SIGNATURES = {
     "clg_fc_backward_fused": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_fused_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
     "clg_fc_forward_logits_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
-    "clg_fc_sm_fits": (_i, [_i, _i64, _i64, _i64]),
-    "clg_fc_sm_preferred": (_i, [_i, _i64, _i64, _i64]),
-    "clg_fc_sm_plan": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p]),
-    "clg_fc_fold_sm": (_i, [_i, _p, _p, _p, _p, _p, _i64, _p]),
-    "clg_fc_forward_sm": (_i, [_i, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
-    "clg_fc_backward_sm_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
-    "clg_fc_backward_sm": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_group_sum_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_group_sum_static_max_bytes": (_i64, []),
+    "clg_group_sum_static_init": (_i, []),
     "clg_group_sum_static": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_group_sum_backward": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_fc_backward_x": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),

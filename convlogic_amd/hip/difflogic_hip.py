@@ -191,96 +191,6 @@ def backward_fused(x, a, b, folded, probs, grad_y, given_x_indices_of_y_start, g
     return gx, gw
 
 
-# ---- sample-major kernels (x [B, in] -> y [B, out]) -------------------------------------------------
-def sm_fits(x, out_dim):
-    """True when the sample-major kernels take a layer on x [B, in] with out_dim neurons (float32 / float64, sample rows
-    of x and of grad_y within LDS)."""
-    if x.dtype not in _lib._DTYPES or x.dim() != 2 or not x.is_cuda:
-        return False
-    return bool(_lib.load().clg_fc_sm_fits(dtype_code(x), x.shape[1], out_dim, x.shape[0]))
-
-
-def sm_preferred(x, out_dim):
-    """sm_fits() and CLG_FC_SAMPLE_MAJOR=1: the module's rule.  (Measured at 8000 -> 8000, batch 256: fewer microseconds of
-    launch work per step than the feature-major kernels with their transposed copies, more microseconds of GPU time.)"""
-    if x.dtype not in _lib._DTYPES or x.dim() != 2 or not x.is_cuda:
-        return False
-    return bool(_lib.load().clg_fc_sm_preferred(dtype_code(x), x.shape[1], out_dim, x.shape[0]))
-
-
-def sm_plan(a, b, given_x_indices_of_y_start, given_x_indices_of_y, in_dim):
-    """Tables of the sample-major kernels for a wiring (host computation, once per wiring):
-    -> (ab32 int32 [out, 2], start32 int32 [in + 1], entry int32 [2 out, 2]) on the device of `a`."""
-    host = [t.detach().to("cpu", torch.int64).contiguous() for t in (a, b, given_x_indices_of_y_start, given_x_indices_of_y)]
-    out_dim = host[0].shape[0]
-    if host[1].shape[0] != out_dim or host[2].shape[0] != in_dim + 1 or host[3].shape[0] != 2 * out_dim:
-        raise RuntimeError("sm_plan: wiring and reverse map do not belong together")
-    ab32 = torch.empty((out_dim, 2), dtype=torch.int32)
-    start32 = torch.empty((in_dim + 1,), dtype=torch.int32)
-    entry = torch.empty((2 * out_dim, 2), dtype=torch.int32)
-    check(_lib.load().clg_fc_sm_plan(host[0].data_ptr(), host[1].data_ptr(), host[2].data_ptr(), host[3].data_ptr(), in_dim, out_dim,
-                                     ab32.data_ptr(), start32.data_ptr(), entry.data_ptr()))
-    return ab32.to(a.device), start32.to(a.device), entry.to(a.device)
-
-
-def fold_sm(logits, entry):
-    """logits [out, 16] -> (probs [out, 16], folded [out, 4], coef_e [2 out, 2]) in one launch."""
-    check_input(logits, "w")
-    out_dim = logits.shape[0]
-    check_input(entry, "entry", torch.int32, (2 * out_dim, 2))
-    if logits.dim() != 2 or logits.shape[1] != 16:
-        raise RuntimeError(f"w must have shape [out_dim, 16], got {tuple(logits.shape)}")
-    probs = torch.empty_like(logits)
-    folded = torch.empty((out_dim, 4), dtype=logits.dtype, device=logits.device)
-    coef_e = torch.empty((2 * out_dim, 2), dtype=logits.dtype, device=logits.device)
-    check(_lib.load().clg_fc_fold_sm(dtype_code(logits), logits.data_ptr(), entry.data_ptr(), probs.data_ptr(), folded.data_ptr(),
-                                     coef_e.data_ptr(), out_dim, stream_ptr(logits)))
-    return probs, folded, coef_e
-
-
-def forward_sm(x, ab32, folded):
-    """y [B, out] from sample-major x [B, in] (contiguous)."""
-    check_input(x, "x")
-    out_dim = folded.shape[0]
-    check_input(ab32, "ab32", torch.int32, (out_dim, 2))
-    check_input(folded, "folded", x.dtype, (out_dim, 4))
-    batch, in_dim = x.shape
-    y = torch.empty((batch, out_dim), dtype=x.dtype, device=x.device)
-    check(_lib.load().clg_fc_forward_sm(dtype_code(x), x.data_ptr(), ab32.data_ptr(), folded.data_ptr(), y.data_ptr(), in_dim, out_dim,
-                                        batch, stream_ptr(x)))
-    return y
-
-
-def backward_sm(x, grad_y, ab32, start32, entry, coef_e, probs, need_grad_x=True, need_grad_w=True):
-    """-> (grad_x [B, in] or None, grad_w [out, 16] or None) from sample-major x and grad_y [B, out]; grad_w is the
-    gradient w.r.t. the logits when probs = softmax(logits) is given, else w.r.t. the probabilities."""
-    check_input(x, "x")
-    batch, in_dim = x.shape
-    out_dim = ab32.shape[0]
-    check_input(grad_y, "grad_y", x.dtype, (batch, out_dim))
-    check_input(ab32, "ab32", torch.int32, (out_dim, 2))
-    check_input(start32, "start32", torch.int32, (in_dim + 1,))
-    check_input(entry, "entry", torch.int32, (2 * out_dim, 2))
-    check_input(coef_e, "coef_e", x.dtype, (2 * out_dim, 2))
-    if probs is not None:
-        check_input(probs, "w", x.dtype, (out_dim, 16))
-    lib = _lib.load()
-    dt = dtype_code(x)
-    gx = torch.empty_like(x) if need_grad_x else None
-    gw = scratch = None
-    if need_grad_w:
-        nbytes = lib.clg_fc_backward_sm_scratch_bytes(dt, in_dim, out_dim, batch)
-        if nbytes < 0:
-            raise RuntimeError("backward_sm: the layer does not fit the sample-major kernels (sm_fits)")
-        scratch = torch.empty((max(int(nbytes), 8),), dtype=torch.uint8, device=x.device)
-        gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
-    check(lib.clg_fc_backward_sm(dt, x.data_ptr(), grad_y.data_ptr(), ab32.data_ptr(), start32.data_ptr(), entry.data_ptr(),
-                                 coef_e.data_ptr(), probs.data_ptr() if probs is not None else None,
-                                 gx.data_ptr() if need_grad_x else None, gw.data_ptr() if need_grad_w else None,
-                                 scratch.data_ptr() if need_grad_w else None, in_dim, out_dim, batch, stream_ptr(x)))
-    return gx, gw
-
-
 def group_sum(x_fm, k, tau=1.0):
     """Feature-major activations [F, B] -> per-class sums [B, k] divided by tau, fixed summation order."""
     check_input(x_fm, "x")

@@ -162,33 +162,6 @@ int clg_fc_forward_logits_ex(int dtype, const void *x, const int64_t *a, const i
                              void *probs /*[out_dim,16]*/, void *folded /*[out_dim,4]*/, void *y, int64_t in_dim, int64_t out_dim,
                              int64_t batch, int flags, void *x_fm /*[in_dim,batch] or NULL*/, void *stream);
 
-/* The layer on SAMPLE-major tensors, x [batch, in_dim] -> y [batch, out_dim] (what the module API hands over at the
- * boundary of a LogicLayer stack), for layers whose sample rows fit LDS (clg_fc_sm_fits() != 0): no transposed copies
- * of x, grad_y and grad_x around the kernels.  Replaces x.transpose(0, 1).contiguous() + difflogic_cuda.forward /
- * backward_x / backward_w + the transposes back (src/difflogic/difflogic.py:125-147, :214-230).
- *   clg_fc_sm_plan      HOST function (host pointers): tables made once per wiring from a, b and the reverse map of
- *                       src/difflogic/difflogic.py:71-87 -- ab32 int32 [out, 2], start32 int32 [in + 1], entry int32
- *                       [2 out, 2] = (consumer neuron | first-operand flag << 31, that neuron's other input)
- *   clg_fc_fold_sm      per step: logits [out, 16] -> probs [out, 16] (their softmax), folded [out, 4] and, per reverse-
- *                       map entry, coef_e [2 out, 2] = the two coefficients of that consumer's derivative
- *   clg_fc_forward_sm   y[s][j] from x[s][:] staged in LDS
- *   clg_fc_backward_sm  grad_x [batch, in] (NULL: skipped) by a deterministic gather over the reverse map, and grad_w
- *                       [out, 16] (NULL: skipped) -- w.r.t. the logits when probs is given, else w.r.t. the
- *                       probabilities; scratch: clg_fc_backward_sm_scratch_bytes() (partial sums of the weight gradient)
- * Same values as the feature-major entry points up to the order of the float additions. */
-int clg_fc_sm_fits(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch);
-int clg_fc_sm_preferred(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch);   /* fits, and CLG_FC_SAMPLE_MAJOR=1 asks for them */
-int clg_fc_sm_plan(const int64_t *a_host, const int64_t *b_host, const int64_t *csr_start_host, const int64_t *csr_list_host,
-                   int64_t in_dim, int64_t out_dim, int32_t *ab32_host, int32_t *start32_host, int32_t *entry_host);
-int clg_fc_fold_sm(int dtype, const void *logits, const int32_t *entry, void *probs, void *folded, void *coef_e, int64_t out_dim,
-                   void *stream);
-int clg_fc_forward_sm(int dtype, const void *x /*[batch,in_dim]*/, const int32_t *ab32, const void *folded, void *y /*[batch,out_dim]*/,
-                      int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
-int64_t clg_fc_backward_sm_scratch_bytes(int dtype, int64_t in_dim, int64_t out_dim, int64_t batch);
-int clg_fc_backward_sm(int dtype, const void *x, const void *grad_y /*[batch,out_dim]*/, const int32_t *ab32, const int32_t *start32,
-                       const int32_t *entry, const void *coef_e, const void *probs, void *grad_x, void *grad_w, void *scratch,
-                       int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
-
 /* GroupSum on feature-major activations x [features, batch] (what the last LogicLayer produces): out[b][g] =
  * (sum of the features/k rows of class g) * (1 / tau), the reciprocal rounded to dtype as torch's division of a
  * device tensor by a scalar does; fixed summation order (reproducible).
@@ -203,8 +176,12 @@ int clg_group_sum(int dtype, const void *x, void *out /*[batch,k]*/, void *scrat
  * process ends.  Sizes whose partial sums (at most 64 * k * batch elements, fewer for few rows per class) do not fit are
  * rejected with CLG_EINVAL.  The call itself allocates and frees nothing.  Every call on a GPU uses that GPU's one
  * buffer: calls that overlap on one GPU (different streams or threads) race; calls on one stream are ordered.  Same
- * values as clg_group_sum, bit for bit.  No counterpart in the reference. */
+ * values as clg_group_sum, bit for bit.  The first call on a device asks the runtime for the buffer's address
+ * (hipGetSymbolAddress, not a stream operation): before CAPTURING the entry point into a HIP graph, call
+ * clg_group_sum_static_init() -- or the entry point itself -- once on that device outside the capture.  No counterpart in
+ * the reference. */
 int64_t clg_group_sum_static_max_bytes(void);
+int clg_group_sum_static_init(void);
 int clg_group_sum_static(int dtype, const void *x /*[features,batch]*/, void *out /*[batch,k]*/, int64_t features,
                          int64_t batch, int64_t k, double tau, void *stream);
 /* Its backward: grad_x[f][b] = grad_out[b][f / (features/k)] * (1 / tau). */

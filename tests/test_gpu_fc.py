@@ -6,7 +6,7 @@ import torch
 import convlogic_amd as C
 from convlogic_amd.hip import difflogic_hip
 from oracle import convlogic_oracle as O
-from tests.gpu_util import DEV, assert_grad_close, set_knobs
+from tests.gpu_util import DEV, assert_grad_close
 
 pytestmark = pytest.mark.gpu
 
@@ -31,13 +31,9 @@ def _oracle_grads(x, logits, idx0, idx1, gy):
     return y.detach(), xl.grad, ll.grad
 
 
-@pytest.mark.parametrize("layout", ["sample_major", "feature_major"])
 @pytest.mark.parametrize("in_dim,out_dim,batch", [(8, 8, 32), (12, 16, 5), (100, 64, 256), (33, 40, 257), (1, 1, 1)])
-def test_fc_module_forward_backward(in_dim, out_dim, batch, layout, monkeypatch):
-    # the feature-major kernels with transposed copies of x and grad_y (grad_x leaves its kernel sample-major); with
-    # CLG_FC_SAMPLE_MAJOR=1 a contiguous [batch, in] input takes the kernels that work on sample-major tensors instead
-    if layout == "sample_major":
-        set_knobs(monkeypatch, CLG_FC_SAMPLE_MAJOR="1")
+def test_fc_module_forward_backward(in_dim, out_dim, batch):
+    # the feature-major kernels with transposed copies of x and grad_y (grad_x leaves its kernel sample-major)
     torch.manual_seed(in_dim * 1000 + batch)
     layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV)
     x = torch.rand(batch, in_dim, device=DEV, requires_grad=True)
@@ -46,73 +42,10 @@ def test_fc_module_forward_backward(in_dim, out_dim, batch, layout, monkeypatch)
     y.backward(gy)
     y_ref, gx_ref, gl_ref = _oracle_grads(x, layer.weights, layer.indices_0, layer.indices_1, gy)
     assert y.shape == (batch, out_dim)
-    assert y.is_contiguous() == (layout == "sample_major") or batch == 1 or out_dim == 1
     assert (y.detach().cpu() - y_ref).abs().max().item() <= 1e-5
     assert x.grad.is_contiguous()
     assert_grad_close(x.grad, gx_ref, name="grad_x")
     assert_grad_close(layer.weights.grad, gl_ref, name="grad_logits")
-
-
-def test_fc_sample_major_entry_points():
-    # the tables of clg_fc_sm_plan against the wiring, a neuron wired twice to one feature, the gradient w.r.t. the
-    # probabilities (probs = None), single gradients, float64, and the size limits of clg_fc_sm_fits
-    import numpy as np
-    from convlogic_amd.difflogic.difflogic import _reverse_wiring
-    torch.manual_seed(31)
-    in_dim, out_dim, batch = 37, 50, 70
-    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda")
-    idx0, idx1 = layer.indices_0.clone(), layer.indices_1.clone()
-    idx1[4] = idx0[4]                                                # self-paired neuron: d/da + d/db
-    start, flat = _reverse_wiring(idx0.numpy(), idx1.numpy(), in_dim)
-    a, b, start, flat = idx0.to(DEV), idx1.to(DEV), start.to(DEV), flat.to(DEV)
-    ab32, start32, entry = difflogic_hip.sm_plan(a, b, start, flat, in_dim)
-    assert torch.equal(ab32[:, 0].long(), a) and torch.equal(ab32[:, 1].long(), b) and torch.equal(start32.long(), start)
-    en = entry.cpu().numpy()
-    j, first, other = en[:, 0] & 0x7fffffff, en[:, 0] < 0, en[:, 1]
-    assert np.array_equal(j, flat.cpu().numpy())
-    owner = np.repeat(np.arange(in_dim), np.diff(start.cpu().numpy()))
-    a_n, b_n = idx0.numpy(), idx1.numpy()
-    assert np.all(np.where(first, a_n[j], b_n[j]) == owner) and np.all(np.where(first, b_n[j], a_n[j]) == other)
-    assert first[(j == 4)].sum() == 1                                # the self-paired neuron: once as A, once as B
-    for dtype in (torch.float32, torch.float64):
-        x = torch.rand(batch, in_dim, device=DEV, dtype=dtype)
-        logits = torch.randn(out_dim, 16, device=DEV, dtype=dtype)
-        gy = torch.randn(batch, out_dim, device=DEV, dtype=dtype)
-        assert difflogic_hip.sm_fits(x, out_dim)
-        probs, folded, coef_e = difflogic_hip.fold_sm(logits, entry)
-        assert (probs - torch.softmax(logits, -1)).abs().max().item() <= (1e-6 if dtype == torch.float32 else 1e-14)
-        y = difflogic_hip.forward_sm(x, ab32, folded)
-        xl = x.cpu().requires_grad_(True)
-        pl = probs.cpu().requires_grad_(True)
-        want = O.logic_fc_forward(xl, idx0, idx1, pl)
-        want.backward(gy.cpu())
-        tol = 1e-5 if dtype == torch.float32 else 1e-12
-        assert (y.cpu() - want.detach()).abs().max().item() <= tol
-        gx, gw = difflogic_hip.backward_sm(x, gy, ab32, start32, entry, coef_e, None)      # w.r.t. the probabilities
-        assert_grad_close(gx, xl.grad, name="grad_x")
-        assert_grad_close(gw, pl.grad, name="grad_w")
-        assert torch.all(gw[:, 0] == 0)
-        gx2, none = difflogic_hip.backward_sm(x, gy, ab32, start32, entry, coef_e, probs, need_grad_w=False)
-        none2, gl = difflogic_hip.backward_sm(x, gy, ab32, start32, entry, coef_e, probs, need_grad_x=False)
-        assert none is None and none2 is None and torch.equal(gx2, gx)
-        p64 = probs.double().cpu()
-        gl_ref = p64 * (pl.grad.double() - (p64 * pl.grad.double()).sum(-1, keepdim=True))
-        assert_grad_close(gl, gl_ref, name="grad_logits")
-    # rows that do not fit LDS stay with the feature-major kernels
-    assert not difflogic_hip.sm_fits(torch.empty(8, 30000, device=DEV), 30000)
-    assert difflogic_hip.sm_fits(torch.empty(4096, 8000, device=DEV), 8000)
-    assert not difflogic_hip.sm_preferred(torch.empty(256, 8000, device=DEV), 8000)         # an option, off unless asked for
-    assert difflogic_hip.sm_fits(torch.empty(256, 8000, device=DEV), 8000)
-
-
-def test_fc_sample_major_gradcheck_float64():
-    torch.manual_seed(12)
-    layer = C.LogicLayer(12, 16, implementation="cuda").double().to(DEV)
-    x = torch.sigmoid(torch.randn(9, 12, dtype=torch.double, device=DEV)).requires_grad_(True)
-    from convlogic_amd.difflogic.difflogic import _LogicLayerSampleMajorFunction
-    tables = layer._sm_tables()
-    logits = layer.weights.clone().detach().requires_grad_(True)
-    assert torch.autograd.gradcheck(lambda inp, lg: _LogicLayerSampleMajorFunction.apply(inp, lg, *tables), (x, logits), eps=1e-6, atol=1e-4)
 
 
 def test_fc_self_paired_neuron_follows_python_derivative():

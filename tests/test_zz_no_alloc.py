@@ -47,3 +47,35 @@ def test_group_sum_static_rejects_what_does_not_fit():
     assert rc != 0 and b"built-in buffer" in lib.clg_last_error()
     rc = lib.clg_group_sum_static(0, x.data_ptr(), out.data_ptr(), 640, 65536, 7, 1.0, _lib.stream_ptr(x))
     assert rc != 0 and b"divisible" in lib.clg_last_error()
+
+
+def test_group_sum_static_captured_in_a_hip_graph_replays_like_eager():
+    # the documented order: address look-up once outside the capture (clg_group_sum_static_init), then the entry point
+    # captured into a HIP graph (no allocation inside the capture) and replayed on new contents of the same input buffer,
+    # with eager work and synchronisations between the replays; every replay equals clg_group_sum on that input
+    lib = _lib.load()
+    _lib.check(lib.clg_group_sum_static_init())
+    torch.manual_seed(9)
+    features, batch, k, tau = 2560, 128, 10, 6.5
+    x = torch.rand(features, batch, device=DEV)
+    out = torch.zeros(batch, k, device=DEV)
+    dt = _lib.dtype_code(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _lib.check(lib.clg_group_sum_static(dt, x.data_ptr(), out.data_ptr(), features, batch, k, tau, _lib.stream_ptr(x)))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.clg_group_sum_static(dt, x.data_ptr(), out.data_ptr(), features, batch, k, tau, _lib.stream_ptr(x)))
+    scratch = torch.empty(lib.clg_group_sum_scratch_bytes(dt, features, batch, k), dtype=torch.uint8, device=DEV)
+    for r in range(3):
+        x.copy_(torch.rand(features, batch, device=DEV))
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = torch.empty(batch, k, device=DEV)
+        _lib.check(lib.clg_group_sum(dt, x.data_ptr(), want.data_ptr(), scratch.data_ptr(), features, batch, k, tau, _lib.stream_ptr(x)))
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), r
