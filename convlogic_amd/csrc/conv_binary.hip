@@ -27,7 +27,6 @@ int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char 
 namespace {
 
 constexpr int kFtab = 160;          // per kernel: F1[2][16], F2[8][16]
-constexpr int kHistLanes = 64;
 
 // ---- context: what the forward leaves for the backward pass (one device buffer) --------------------------------
 struct BinCtx {
@@ -378,7 +377,10 @@ __global__ __launch_bounds__(512) void convblock_bin_forward_kernel(const uint32
 }
 
 // ---- weight gradient: histogram of grad_y over the tap byte ---------------------------------------------------------
-// One wavefront per (kernel, part of the batch); lane-private bins bins[t][lane] (bank = lane: no conflicts, no atomics).
+// One wavefront of HL active lanes per (kernel, part of the batch); lane-private bins bins[t][lane] (bank = lane: no
+// conflicts, no atomics).  A wavefront's steps are a serial chain (tap bytes -> LDS reads -> adds -> LDS writes) and a CU
+// holds 160 KiB / (256 * HL * 4 bytes) wavefronts; more wavefronts of fewer lanes do not pay (the chain per step stays as
+// long), so HL = 64 is the default and the narrower instantiations are for measurement (CLG_BIN_HL).
 // A lane takes 4 consecutive cells per step; equal tap bytes among them are chained in registers, the four stores then
 // go out in order, so the bin holds the sum in program order.
 struct BinHist {
@@ -387,16 +389,17 @@ struct BinHist {
 };
 constexpr int kHistDepth = 8;           // steps whose loads are in flight together
 
-__global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const float *__restrict__ gy, const uint16_t *__restrict__ aux,
+template <int HL>
+__global__ __launch_bounds__(HL) void convblock_bin_hist_kernel(const float *__restrict__ gy, const uint16_t *__restrict__ aux,
                                                                       float *__restrict__ hpart, BinHist p)
 {
-    extern __shared__ __align__(16) float bins[];                     // [256][64]
+    extern __shared__ __align__(16) float bins[];                     // [256][HL]
     const int lane = threadIdx.x;
     const int c = blockIdx.x / p.parts, part = blockIdx.x - c * p.parts;
     const int s0 = part * p.per_part, s1 = min(p.n, s0 + p.per_part);
     {
         float4 *z = reinterpret_cast<float4 *>(bins);
-        for (int i = lane; i < 256 * kHistLanes / 4; i += kHistLanes) z[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = lane; i < 256 * HL / 4; i += HL) z[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -409,7 +412,7 @@ __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const fl
     // loads never depend on a branch (an index past the end is clamped), so the compiler can count them and let a
     // whole group of steps stay in flight while the previous group is applied
     auto load = [&](int step, float4 &g4, uint2 &a2) {
-        int e = step * kHistLanes + lane;
+        int e = step * HL + lane;
         e = e < items ? e : items - 1;
         const uint32_t smp = fdiv((uint32_t)e, p.d_q), quad = (uint32_t)e - smp * (uint32_t)p.Q;
         const int64_t at = smp * plane_stride + quad * 4;
@@ -418,32 +421,32 @@ __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const fl
     };
     auto apply = [&](const float4 &g4, const uint2 &a2) {
         const uint32_t t0 = a2.x & 255u, t1 = (a2.x >> 16) & 255u, t2 = a2.y & 255u, t3 = (a2.y >> 16) & 255u;
-        float r0 = mine[t0 * kHistLanes], r1 = mine[t1 * kHistLanes], r2 = mine[t2 * kHistLanes], r3 = mine[t3 * kHistLanes];
+        float r0 = mine[t0 * HL], r1 = mine[t1 * HL], r2 = mine[t2 * HL], r3 = mine[t3 * HL];
         asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));   // all four reads in flight together
         const float v0 = r0 + g4.x;
         const float v1 = (t1 == t0 ? v0 : r1) + g4.y;
         const float v2 = (t2 == t1 ? v1 : (t2 == t0 ? v0 : r2)) + g4.z;
         const float v3 = (t3 == t2 ? v2 : (t3 == t1 ? v1 : (t3 == t0 ? v0 : r3))) + g4.w;
-        mine[t0 * kHistLanes] = v0;
-        mine[t1 * kHistLanes] = v1;
-        mine[t2 * kHistLanes] = v2;
-        mine[t3 * kHistLanes] = v3;
+        mine[t0 * HL] = v0;
+        mine[t1 * HL] = v1;
+        mine[t2 * HL] = v2;
+        mine[t3 * HL] = v3;
     };
-    const int steps = (items + kHistLanes - 1) / kHistLanes;
+    const int steps = (items + HL - 1) / HL;
     if (steps > 0) {
         float4 G[2][kHistDepth];
         uint2 A[2][kHistDepth];
         // a group of kHistDepth steps; in a group that reaches past the end the lanes without a quad add 0
         auto apply_group = [&](int s0, const float4 (&Gd)[kHistDepth], const uint2 (&Ad)[kHistDepth]) {
             if (s0 >= steps) return;                                  // wave-uniform
-            if ((s0 + kHistDepth) * kHistLanes <= items) {
+            if ((s0 + kHistDepth) * HL <= items) {
 #pragma unroll
                 for (int d = 0; d < kHistDepth; ++d) apply(Gd[d], Ad[d]);
             } else {
 #pragma unroll
                 for (int d = 0; d < kHistDepth; ++d) {
                     float4 g4 = Gd[d];
-                    if ((s0 + d) * kHistLanes + lane >= items) g4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if ((s0 + d) * HL + lane >= items) g4 = make_float4(0.f, 0.f, 0.f, 0.f);
                     apply(g4, Ad[d]);
                 }
             }
@@ -464,17 +467,17 @@ __global__ __launch_bounds__(kHistLanes) void convblock_bin_hist_kernel(const fl
     // lane l sums bins l, l+64, l+128, l+192 over the 64 lane copies, starting at its own column (conflict-free, fixed order)
     float *out = hpart + ((int64_t)c * p.parts + part) * 256;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const float *row = bins + (q * 64 + lane) * kHistLanes;
+    for (int q = 0; q < 256 / HL; ++q) {
+        const float *row = bins + (q * HL + lane) * HL;
         float acc = 0.f;
-        for (int k0 = 0; k0 < kHistLanes; k0 += 8) {
+        for (int k0 = 0; k0 < HL; k0 += 8) {
             float v[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = row[(lane + k0 + k) & (kHistLanes - 1)];
+            for (int k = 0; k < 8; ++k) v[k] = row[(lane + k0 + k) & (HL - 1)];
 #pragma unroll
             for (int k = 0; k < 8; ++k) acc += v[k];
         }
-        out[q * 64 + lane] = acc;
+        out[q * HL + lane] = acc;
     }
 }
 
@@ -758,7 +761,7 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
     nw = nw > 8 ? 8 : nw;
     if (const char *e = clg_knob(K_BIN_NW)) nw = std::min(8, std::max(1, atoi(e)));
     int pc = p.wp % 4 == 0 ? 4 : (p.wp % 2 == 0 ? 2 : 0);
-    if (const char *e = clg_knob(K_BIN_DBG)) pc = atoi(e) == 1 ? 0 : pc;
+    if (const char *e = clg_knob(K_BIN_PIECE)) pc = atoi(e) == 0 ? 0 : (atoi(e) == 2 && pc ? 2 : pc);   // narrower pieces / rows written directly
     p.tr_words = pc ? kWave * (p.wp + 4) : 0;
     p.d_npc = make_fastdiv((uint32_t)std::max(1, pc ? p.wp / pc : 1));
     const size_t lds = (size_t)CT * 1024 + (((size_t)S * g.cin * cx.RP + 3) & ~(size_t)3) * 4 + (size_t)nw * p.tr_words * 4;
@@ -777,9 +780,17 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
 }
 
 namespace {
+int hist_lanes()
+{
+    if (const char *e = clg_knob(K_BIN_HL)) {
+        const int v = atoi(e);
+        if (v == 64 || v == 32 || v == 16) return v;
+    }
+    return 64;                                                       // measured at [256,9,32,32] -> 256: 28.7 us with 64 lanes, 33.3 with 32, 42.4 with 16
+}
 int hist_parts(const Geom &g)
 {
-    int parts = 512 / g.c;
+    int parts = 512 * (64 / hist_lanes()) / g.c;
     if (parts < 1) parts = 1;
     if (const char *e = clg_knob(K_BIN_PARTS)) parts = std::max(1, atoi(e));
     if (parts > g.n) parts = g.n;
@@ -849,15 +860,23 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
         BinHist h;
         h.C = g.c, h.P = P, h.n = g.n;
         h.parts = hist_parts(g);
+        const int hl = hist_lanes();
         h.per_part = (int)clg_ceil_div(g.n, h.parts);
         CLG_REQUIRE(P % 4 == 0, "%s: the pooled plane must hold a multiple of 4 cells", name);
         h.Q = P / 4;
         h.d_q = make_fastdiv((uint32_t)h.Q);
         CLG_REQUIRE((int64_t)h.per_part * h.Q < (1ll << 31) - 4096, "%s: batch too large", name);
-        const size_t lds = 256 * kHistLanes * 4;
-        if (int e = allow_lds(convblock_bin_hist_kernel, lds, name)) return e;
-        hipLaunchKernelGGL(convblock_bin_hist_kernel, dim3((unsigned)(g.c * h.parts)), dim3(kHistLanes), lds, st, (const float *)grad_y, taps,
-                           (float *)scratch, h);
+        const size_t lds = (size_t)256 * hl * 4;
+#define CLG_BIN_HIST(HL)                                                                                                         \
+    do {                                                                                                                         \
+        if (int e = allow_lds(convblock_bin_hist_kernel<HL>, lds, name)) return e;                                               \
+        hipLaunchKernelGGL(convblock_bin_hist_kernel<HL>, dim3((unsigned)(g.c * h.parts)), dim3(HL), lds, st, (const float *)grad_y, \
+                           taps, (float *)scratch, h);                                                                           \
+    } while (0)
+        if (hl == 64) CLG_BIN_HIST(64);
+        else if (hl == 32) CLG_BIN_HIST(32);
+        else CLG_BIN_HIST(16);
+#undef CLG_BIN_HIST
         CLG_CHECK_LAUNCH("clg_convblock_bin_backward(histogram)");
         hipLaunchKernelGGL(convblock_bin_wgrad_finish_kernel, dim3((unsigned)g.c), dim3(256), 0, st, (const float *)scratch,
                            reinterpret_cast<const float *>(base + cx.folded_off),

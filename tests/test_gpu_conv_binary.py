@@ -36,6 +36,7 @@ SHAPES = [
     (3, 4, 10, 18, 9, 0, 3),
     (2, 3, 16, 16, 6, 2, 5),
     (70, 2, 8, 8, 3, 1, 3),
+    (3, 2, 8, 6, 5, 1, 3),                                           # rows of 3 pooled cells: written without the ordered write-out
 ]
 
 
@@ -162,6 +163,20 @@ def test_bin_unsupported_shapes_fall_back():
     assert torch.equal(layer(x), layer2(x))
     assert not convlogic_hip.bin_supported(_binary(2, 2, 30, 30, seed=1), 4, 1, 1, 1, 1, 3, 3)    # 225 pooled cells: not a multiple of 4
     assert not convlogic_hip.bin_supported(_binary(2, 2, 16, 16, seed=1), 4, 2, 2, 1, 1, 3, 3)    # stride 2
+
+
+@pytest.mark.parametrize("piece", ["0", "2"])
+def test_bin_forward_write_out_variants(piece, monkeypatch):
+    # the write-out of y / taps in pieces of 4 cells (default where rows allow), 2 cells and row by row gives the same bytes
+    from tests.gpu_util import set_knobs
+    torch.manual_seed(12)
+    layer = C.ConvLogicLayer(3, 10, complete=True, implementation="cuda").to(DEV)
+    x = _binary(9, 3, 16, 16, seed=8)
+    flag = convlogic_hip.BinaryFlag()
+    y0, t0, _ = convlogic_hip.bin_forward(x, layer.weights.detach(), layer.selection, 1, 1, 1, 1, 3, 3, flag, logits=True)
+    set_knobs(monkeypatch, CLG_BIN_PIECE=piece)
+    y1, t1, _ = convlogic_hip.bin_forward(x, layer.weights.detach(), layer.selection, 1, 1, 1, 1, 3, 3, flag, logits=True)
+    assert torch.equal(y0, y1) and torch.equal(t0, t1)
 
 
 def test_bin_deterministic():
