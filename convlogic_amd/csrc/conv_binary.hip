@@ -540,15 +540,15 @@ struct BinBwdX {
     int64_t items;      // n * cin
     FastDiv d_wp, d_cin;
 };
-constexpr int kXBlocks = 4;             // cell blocks of 64 lanes per (sample, kernel) plane: at most 256 pooled cells
 
 __device__ __forceinline__ float lane_read(float v, int byte_addr)
 {
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
 }
 
-// FULL: every plane has exactly 256 pooled cells (no idle lanes, no sink element).
-template <bool FULL>
+// NB: blocks of 64 lanes that a plane's pooled cells (at most 256) fill.  FULL: they fill the last block too (no idle
+// lanes, no sink element).
+template <int NB, bool FULL>
 __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const float *__restrict__ gy, const uint16_t *__restrict__ aux,
                                                                       const float *__restrict__ ftab, const int32_t *__restrict__ xtap,
                                                                       const int32_t *__restrict__ count, const int32_t *__restrict__ hits,
@@ -557,7 +557,9 @@ __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const fl
     extern __shared__ __align__(16) float planes[];                   // [waves][plane_pad]
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = uniform(tid >> 6);
     const int slot = wave % p.hsw, local = wave / p.hsw;
-    const int64_t item = (int64_t)blockIdx.x * p.items_per_wg + local;
+    // planes in sample-major order, every XCD on a contiguous range of them: the channel planes of one sample read the
+    // same gradient rows and then find them in one L2
+    const int64_t item = (int64_t)xcd_contiguous_block(blockIdx.x, gridDim.x) * p.items_per_wg + local;
     const bool have = item < p.items;
     float *pl = planes + wave * p.plane_pad;
     for (int i = lane; i < p.plane_pad; i += kWave) pl[i] = 0.f;
@@ -567,10 +569,10 @@ __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const fl
     if (have) {
         n = fdiv((uint32_t)item, p.d_cin);
         ch = (uint32_t)item - n * (uint32_t)g.cin;
-        int cellbase[kXBlocks];
-        bool live[kXBlocks];
+        int cellbase[NB];
+        bool live[NB];
 #pragma unroll
-        for (int j = 0; j < kXBlocks; ++j) {
+        for (int j = 0; j < NB; ++j) {
             const int cell = j * kWave + lane;
             live[j] = FULL || cell < p.P;
             const uint32_t cl = live[j] ? (uint32_t)cell : 0u;
@@ -582,15 +584,15 @@ __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const fl
         const int32_t *hit = hits + count[2 * ch + 1];
         const int64_t nbase = (int64_t)n * g.c * p.P;
         struct Loads {
-            float gyv[kXBlocks];
-            uint32_t ax[kXBlocks];
+            float gyv[NB];
+            uint32_t ax[NB];
             float tab[3];
         };
         auto issue = [&](int k, Loads &L) {
             const int c = hit[k] & 0xFFFF;
             const int64_t row = nbase + (int64_t)c * p.P;
 #pragma unroll
-            for (int j = 0; j < kXBlocks; ++j) {
+            for (int j = 0; j < NB; ++j) {
                 L.gyv[j] = 0.f;
                 L.ax[j] = 0;
                 if (live[j]) {
@@ -605,6 +607,9 @@ __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const fl
         };
         Loads cur, nxt;
         if (slot < nhits) issue(slot, cur);
+        // the kernel's derivative tables in the wavefront's own LDS slot: a lookup is a read at nibble + constant, and
+        // two lookups with one nibble are one ds_read2_b32
+        float *tabw = planes + (int)(blockDim.x >> 6) * p.plane_pad + wave * kFtab;
         for (int k = slot; k < nhits; k += p.hsw) {
             if (k + p.hsw < nhits) issue(k + p.hsw, nxt);
             const int ent = hit[k];
@@ -612,49 +617,76 @@ __global__ __launch_bounds__(1024) void convblock_bin_backward_x_kernel(const fl
             int to[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t) to[t] = xtap[c * 8 + t];
-            int pos[kXBlocks], lo4[kXBlocks], hi4[kXBlocks];
-            float u0[kXBlocks], u1[kXBlocks];
+            tabw[lane] = cur.tab[0];
+            tabw[64 + lane] = cur.tab[1];
+            if (lane < 32) tabw[128 + lane] = cur.tab[2];
+            int pos[NB];
+            const float *tl[NB], *th[NB];
+            float u0[NB], u1[NB];
 #pragma unroll
-            for (int j = 0; j < kXBlocks; ++j) {
+            for (int j = 0; j < NB; ++j) {
                 const uint32_t a = cur.ax[j];
-                pos[j] = cellbase[j] + (int)((a >> 9) & 1) * p.prs + (int)((a >> 8) & 1);
-                lo4[j] = (int)(a & 15u) << 2;
-                hi4[j] = (int)((a >> 4) & 15u) << 2;
-                if (mask & 0x0F) u0[j] = cur.gyv[j] * lane_read(cur.tab[0], hi4[j]);           // F1[0][hi]
-                if (mask & 0xF0) u1[j] = cur.gyv[j] * lane_read(cur.tab[0], 64 + lo4[j]);      // F1[1][lo]
+                pos[j] = FULL || live[j] ? cellbase[j] + (int)((a >> 9) & 1) * p.prs + (int)((a >> 8) & 1) : sink;
+                tl[j] = tabw + (a & 15u);
+                th[j] = tabw + ((a >> 4) & 15u);
             }
+            if (mask & 0x0F) {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                if ((mask >> t) & 1) {                               // wave-uniform
-                    float val[kXBlocks], old[kXBlocks];
-                    int at[kXBlocks];
+                for (int j = 0; j < NB; ++j) u0[j] = cur.gyv[j] * th[j][0];                     // F1[0][hi]
+            }
+            if (mask & 0xF0) {
 #pragma unroll
-                    for (int j = 0; j < kXBlocks; ++j) {
-                        // F2[t][own nibble]: entry 32 + 16 t + nibble of the table
-                        const int e = (32 + 16 * t) & 63;
-                        const float f2 = lane_read(t < 2 ? cur.tab[0] : (t < 6 ? cur.tab[1] : cur.tab[2]), e * 4 + (t < 4 ? lo4[j] : hi4[j]));
-                        val[j] = (t < 4 ? u0[j] : u1[j]) * f2;
-                        at[j] = FULL || live[j] ? pos[j] + to[t] : sink;
+                for (int j = 0; j < NB; ++j) u1[j] = cur.gyv[j] * tl[j][16];                    // F1[1][lo]
+            }
+            // read-add-write of one tap for all cell blocks: reads first, so that they are in flight together
+            auto add_tap = [&](int off, const float (&val)[NB]) {
+                float old[NB];
+#pragma unroll
+                for (int j = 0; j < NB; ++j) old[j] = pl[pos[j] + off];
+#pragma unroll
+                for (int j = 0; j < NB; ++j) pl[pos[j] + off] = old[j] + val[j];
+            };
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {                          // taps 2 pr and 2 pr + 1 share their nibble
+                const int ta = 2 * pr, tb = ta + 1;
+                const int both = (mask >> ta) & 3;                    // wave-uniform
+                if (both == 0) continue;
+                // F2[t][own nibble]: entry 32 + 16 t + nibble of the table
+                float va[NB], vb[NB];
+                if (both == 3) {
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) {
+                        const float *q = pr < 2 ? tl[j] : th[j];
+                        const float fa = q[32 + 16 * ta], fb = q[32 + 16 * tb];
+                        const float u = pr < 2 ? u0[j] : u1[j];
+                        va[j] = u * fa, vb[j] = u * fb;
                     }
+                    add_tap(to[ta], va);
+                    add_tap(to[tb], vb);
+                } else {
+                    const int t = both == 1 ? ta : tb;
 #pragma unroll
-                    for (int j = 0; j < kXBlocks; ++j) old[j] = pl[at[j]];
-#pragma unroll
-                    for (int j = 0; j < kXBlocks; ++j) pl[at[j]] = old[j] + val[j];
+                    for (int j = 0; j < NB; ++j) {
+                        const float *q = pr < 2 ? tl[j] : th[j];
+                        va[j] = (pr < 2 ? u0[j] : u1[j]) * q[32 + 16 * t];
+                    }
+                    add_tap(both == 1 ? to[ta] : to[tb], va);
                 }
             }
             cur = nxt;
         }
     }
     __syncthreads();
-    // the first wavefront of every plane adds the copies in order and writes the image rows out
-    if (have && slot == 0) {
+    // the wavefronts of a plane share its pixels; each adds the copies in order and writes its image elements out
+    if (have) {
         float *dst = gx + ((int64_t)n * g.cin + ch) * g.h * g.w;
+        const float *first = planes + (wave - slot) * p.plane_pad;
         const int total = g.h * g.w;
-        for (int e = lane; e < total; e += kWave) {
+        for (int e = slot * kWave + lane; e < total; e += p.hsw * kWave) {
             const int iy = e / g.w, ix = e - iy * g.w;
             const int at = (iy + g.ph) * p.prs + ix + g.pw;
-            float v = pl[at];
-            for (int k = 1; k < p.hsw; ++k) v += pl[k * p.plane_pad + at];
+            float v = first[at];
+            for (int k = 1; k < p.hsw; ++k) v += first[k * p.plane_pad + at];
             dst[e] = v;
         }
     }
@@ -827,7 +859,9 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
     if (grad_x != nullptr) {
         BinBwdX p;
         p.P = P, p.wp = wp, p.prs = cx.prs, p.plane = cx.plane;
-        p.plane_pad = (cx.plane + 64 + 3) & ~3;
+        // behind the plane: one element per lane for the lanes without a cell, which add their zeros there at the tap's
+        // offset like every other lane
+        p.plane_pad = (cx.plane + 64 + (g.kh - 1) * cx.prs + g.kw + 3) & ~3;
         p.items = (int64_t)g.n * g.cin;
         // wavefronts per plane: enough of them to give every SIMD a few, bounded by the shortest useful list
         int hsw = 1;
@@ -836,23 +870,33 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
         if (const char *e = clg_knob(K_BIN_HSW)) hsw = std::min(16, std::max(1, atoi(e)));
         p.hsw = hsw;
         int per_wg = std::max(1, 4 / hsw);
-        while (per_wg > 1 && (size_t)per_wg * hsw * p.plane_pad * 4 > 64 * 1024) per_wg /= 2;
+        while (per_wg > 1 && (size_t)per_wg * hsw * (p.plane_pad + kFtab) * 4 > 64 * 1024) per_wg /= 2;
         p.items_per_wg = per_wg;
         p.d_wp = make_fastdiv((uint32_t)wp);
         p.d_cin = make_fastdiv((uint32_t)g.cin);
-        const size_t lds = (size_t)per_wg * hsw * p.plane_pad * 4;
+        const size_t lds = (size_t)per_wg * hsw * (p.plane_pad + kFtab) * 4;   // gradient planes, then a table slot per wavefront
         CLG_REQUIRE(lds <= (size_t)kLdsLimit, "%s: gradient planes of %zu bytes do not fit LDS", name, lds);
         const dim3 grid((unsigned)clg_ceil_div(p.items, per_wg)), block(per_wg * hsw * kWave);
-#define CLG_BIN_BWDX(FULL)                                                                                                       \
+#define CLG_BIN_BWDX(NB, FULL)                                                                                                   \
     do {                                                                                                                         \
-        if (int e = allow_lds(convblock_bin_backward_x_kernel<FULL>, lds, name)) return e;                                       \
-        hipLaunchKernelGGL(convblock_bin_backward_x_kernel<FULL>, grid, block, lds, st, (const float *)grad_y, taps,             \
+        if (int e = allow_lds(convblock_bin_backward_x_kernel<NB, FULL>, lds, name)) return e;                                   \
+        hipLaunchKernelGGL((convblock_bin_backward_x_kernel<NB, FULL>), grid, block, lds, st, (const float *)grad_y, taps,       \
                            reinterpret_cast<const float *>(base + cx.ftab_off), reinterpret_cast<const int32_t *>(base + cx.xtap_off), \
                            reinterpret_cast<const int32_t *>(base + cx.count_off), reinterpret_cast<const int32_t *>(base + cx.hits_off), \
                            (float *)grad_x, g, p);                                                                               \
     } while (0)
-        if (P == 256) CLG_BIN_BWDX(true);
-        else CLG_BIN_BWDX(false);
+#define CLG_BIN_BWDX_NB(NB)                                                                                                      \
+    do {                                                                                                                         \
+        if (P == NB * kWave) CLG_BIN_BWDX(NB, true);                                                                             \
+        else CLG_BIN_BWDX(NB, false);                                                                                            \
+    } while (0)
+        switch ((P + kWave - 1) / kWave) {
+        case 1: CLG_BIN_BWDX_NB(1); break;
+        case 2: CLG_BIN_BWDX_NB(2); break;
+        case 3: CLG_BIN_BWDX_NB(3); break;
+        default: CLG_BIN_BWDX_NB(4); break;
+        }
+#undef CLG_BIN_BWDX_NB
 #undef CLG_BIN_BWDX
         CLG_CHECK_LAUNCH("clg_convblock_bin_backward(input gradient)");
     }
