@@ -782,6 +782,7 @@ extern "C" int clg_convblock_bin_forward(int dtype, const clg_conv_geom *gg, con
     const int stiles = (int)clg_ceil_div(g.n, S);
     int CT = 64;
     while (CT > 8 && (int64_t)stiles * clg_ceil_div(g.c, CT) < 512) CT /= 2;
+    while (CT > 2 && (int64_t)stiles * clg_ceil_div(g.c, CT) < 256) CT /= 2;   // few kernels: a workgroup per CU first
     if (const char *e = clg_knob(K_BIN_CT)) CT = std::min(64, std::max(1, atoi(e)));
     if (CT > g.c) CT = g.c;
     p.CT = CT;
