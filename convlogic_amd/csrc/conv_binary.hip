@@ -13,7 +13,8 @@
 //   input gradient   the walk of the generic kernels (one owner wavefront per (sample, input channel) plane, kernels of
 //                    the channel in increasing order, read-add-write into an LDS plane nobody else touches), with the
 //                    tap derivative as a product of two 16-entry table reads, d tree / d tap_i = F1[other nibble] *
-//                    F2_i[own nibble], taken from registers with ds_bpermute instead of 8 tap reads and 49 FMAs.
+//                    F2_i[own nibble], from a 640-byte LDS slot per wavefront (two taps of one nibble in one ds_read2_b32)
+//                    instead of 8 tap reads and 49 FMAs.
 // Replaces, for such inputs, src/convlogic/cuda/full_convlogic_kernel.cu:10-145 (forward), :233-363 (input gradient),
 // :463-701 (weight gradient).
 #include <stdlib.h>
@@ -540,11 +541,6 @@ struct BinBwdX {
     int64_t items;      // n * cin
     FastDiv d_wp, d_cin;
 };
-
-__device__ __forceinline__ float lane_read(float v, int byte_addr)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
-}
 
 // NB: blocks of 64 lanes that a plane's pooled cells (at most 256) fill.  FULL: they fill the last block too (no idle
 // lanes, no sink element).
