@@ -37,6 +37,8 @@ SHAPES = [
     (2, 3, 16, 16, 6, 2, 5),
     (70, 2, 8, 8, 3, 1, 3),
     (3, 2, 8, 6, 5, 1, 3),                                           # rows of 3 pooled cells: written without the ordered write-out
+    (2, 93, 32, 32, 48, 1, 3),                                       # the thresholded channels of the large CIFAR topology
+    (3, 5, 32, 32, 600, 1, 3),                                       # more kernels than histogram parts, not a multiple of 64
 ]
 
 
