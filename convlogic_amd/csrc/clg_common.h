@@ -129,6 +129,11 @@ __device__ __forceinline__ float dpp_zero(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
 }
 template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_zero(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xF, false);
+}
+template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ double dpp_zero(double v)
 {
     const uint64_t u = __builtin_bit_cast(uint64_t, v);

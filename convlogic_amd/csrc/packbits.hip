@@ -69,10 +69,36 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_kernel(const V *__rest
 // plan[k] = neuron | use << 28 | keep << 30
 //   use : 0 nothing carried, 1 carried row is input a, 2 carried row is input b, 3 it is both
 //   keep: row carried to the next step, 0 = input a, 1 = input b
-template <int R>
+// Index of the first maximum of 16 float32 logits, a NaN counting as the maximum (the rule of gate_argmax_kernel and of
+// torch.argmax), computed by the whole wavefront: lane l holds logit l % 16 (`v`) as an order-preserving integer key (-0
+// and +0 equal, NaN on top), the row maximum comes over DPP, the first lane that holds it names the gate.  Wave-uniform.
+__device__ __forceinline__ int argmax16_uniform(float v)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, v + 0.0f);
+    const uint32_t key = v != v ? 0xFFFFFFFFu : (u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u));
+    const uint32_t top = row16_max(key);
+    const uint32_t first = (uint32_t)__ballot(key == top) & 0xFFFFu;
+    return uniform(__builtin_ctz(first));
+}
+
+// gate[j] for a wave-uniform j through the scalar cache: the aligned 32-bit word that holds it (a byte load would be a
+// vector load, and the wait for it would also wait for the row loads in flight).  The last word is read bytewise when
+// it reaches past the table; the table starts at a 4-byte boundary or is read bytewise altogether.
+__device__ __forceinline__ int gate_id_uniform(const uint8_t *__restrict__ gate, int j, int n)
+{
+    if ((reinterpret_cast<uintptr_t>(gate) & 3) == 0 && (j | 3) < n) {
+        const uint32_t w = reinterpret_cast<const uint32_t *>(gate)[j >> 2];
+        return (int)((w >> ((j & 3) * 8)) & 0xFFu);
+    }
+    return gate[j];
+}
+
+// LOGITS: `gate` points to float32 logits [out_dim, 16] and the wavefront takes their arg-max itself (the layer's eval
+// call then needs no launch of its own for the gate ids); else to uint8 gate ids [out_dim].
+template <int R, bool LOGITS>
 __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x4 *__restrict__ x, const int64_t *__restrict__ a,
                                                                     const int64_t *__restrict__ b,
-                                                                    const uint8_t *__restrict__ gate,
+                                                                    const void *__restrict__ gate,
                                                                     const int32_t *__restrict__ plan, u32x4 *__restrict__ y,
                                                                     int steps, int seg_len, int64_t row_vecs, int64_t in_dim)
 {
@@ -91,6 +117,8 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x
         const int use = k == k0 ? 0 : (p >> 28) & 3;
         const u32x4 *xa = x + clamp_index(a[j], in_dim) * row_vecs + col0;
         const u32x4 *xb = x + clamp_index(b[j], in_dim) * row_vecs + col0;
+        float logit = 0.f;                                            // requested ahead of the rows: vector loads return in order
+        if constexpr (LOGITS) logit = reinterpret_cast<const float *>(gate)[(int64_t)j * 16 + (lane & 15)];
         if (use != 1 && use != 3) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
@@ -107,7 +135,10 @@ __global__ __launch_bounds__(kEvalBlock) void eval_packed_walk_kernel(const u32x
 #pragma unroll
             for (int r = 0; r < R; ++r) rb[r] = carry[r];
         }
-        const Masks m = gate_masks(gate[j]);
+        int id;
+        if constexpr (LOGITS) id = argmax16_uniform(logit);
+        else id = gate_id_uniform(reinterpret_cast<const uint8_t *>(gate), j, steps);
+        const Masks m = gate_masks(id);
         u32x4 *yj = y + (int64_t)j * row_vecs + col0;
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -711,31 +742,32 @@ extern "C" int clg_fc_eval_plan(const int64_t *a, const int64_t *b, int64_t in_d
     return CLG_OK;
 }
 
-extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate,
-                                          const int32_t *plan, void *y, int64_t in_dim, int64_t out_dim, int64_t words,
-                                          void *stream)
+namespace {
+// rows the walk kernel takes: whole 16-byte vectors at 16-byte aligned addresses, at least 1 KiB long (shorter rows gain
+// nothing from carrying a row in registers)
+bool walk_fits(int elem_size, const void *x, const void *y, int64_t words)
 {
-    CLG_REQUIRE(valid_elem(elem_size), "clg_fc_eval_packed_planned: elem_size must be 1, 2, 4 or 8, got %d", elem_size);
-    CLG_REQUIRE(x && a && b && gate && plan && y, "clg_fc_eval_packed_planned: null pointer argument");
-    CLG_REQUIRE(x != y, "clg_fc_eval_packed_planned: x and y must not overlap");
-    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && words > 0, "clg_fc_eval_packed_planned: in_dim, out_dim and words must be positive");
-    CLG_REQUIRE(out_dim < (1ll << 28), "clg_fc_eval_packed_planned: out_dim above 2^28-1 is not supported");
     const int64_t row_bytes = words * elem_size;
     const uintptr_t align = (uintptr_t)x | (uintptr_t)y | (uintptr_t)row_bytes;
-    // short or unaligned rows gain nothing from carrying a row in registers
-    if ((align & 15) != 0 || row_bytes < 1024) return clg_fc_eval_packed(elem_size, x, a, b, gate, y, in_dim, out_dim, words, stream);
-    const int64_t row_vecs = row_bytes / 16;
+    return (align & 15) == 0 && row_bytes >= 1024;
+}
+
+template <bool LOGITS>
+int launch_walk(const char *name, int elem_size, const void *x, const int64_t *a, const int64_t *b, const void *gate, const int32_t *plan,
+                void *y, int64_t in_dim, int64_t out_dim, int64_t words, void *stream)
+{
+    const int64_t row_vecs = words * elem_size / 16;
     const char *e_r = clg_knob(K_EVAL_WALK_R), *e_l = clg_knob(K_EVAL_WALK_SEG);
     int R = e_r ? atoi(e_r) : 4;
     while (R > 1 && (int64_t)kWave * (R / 2) >= row_vecs) R /= 2;
     const int seg = e_l ? atoi(e_l) : 8;
     const int64_t col_chunks = clg_ceil_div(row_vecs, (int64_t)kWave * R);
-    CLG_REQUIRE(col_chunks <= 65535, "clg_fc_eval_packed_planned: rows above %lld bytes are not supported", 65535ll * kWave * R * 16);
+    CLG_REQUIRE(col_chunks <= 65535, "%s: rows above %lld bytes are not supported", name, 65535ll * kWave * R * 16);
     const dim3 grid((unsigned)clg_ceil_div(out_dim, (int64_t)kEvalWaves * seg), (unsigned)col_chunks), block(kEvalBlock);
     hipStream_t st = clg_stream(stream);
 #define CLG_WALK(RR)                                                                                                          \
-    hipLaunchKernelGGL(eval_packed_walk_kernel<RR>, grid, block, 0, st, (const u32x4 *)x, a, b, gate, plan, (u32x4 *)y, (int)out_dim, \
-                       seg, row_vecs, in_dim)
+    hipLaunchKernelGGL((eval_packed_walk_kernel<RR, LOGITS>), grid, block, 0, st, (const u32x4 *)x, a, b, gate, plan, (u32x4 *)y, \
+                       (int)out_dim, seg, row_vecs, in_dim)
     switch (R) {
     case 1: CLG_WALK(1); break;
     case 2: CLG_WALK(2); break;
@@ -743,6 +775,41 @@ extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const in
     default: CLG_WALK(8); break;
     }
 #undef CLG_WALK
-    CLG_CHECK_LAUNCH("clg_fc_eval_packed_planned");
+    CLG_CHECK_LAUNCH(name);
     return CLG_OK;
+}
+}  // namespace
+
+extern "C" int clg_fc_eval_packed_planned(int elem_size, const void *x, const int64_t *a, const int64_t *b, const uint8_t *gate,
+                                          const int32_t *plan, void *y, int64_t in_dim, int64_t out_dim, int64_t words,
+                                          void *stream)
+{
+    const char *name = "clg_fc_eval_packed_planned";
+    CLG_REQUIRE(valid_elem(elem_size), "%s: elem_size must be 1, 2, 4 or 8, got %d", name, elem_size);
+    CLG_REQUIRE(x && a && b && gate && plan && y, "%s: null pointer argument", name);
+    CLG_REQUIRE(x != y, "%s: x and y must not overlap", name);
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && words > 0, "%s: in_dim, out_dim and words must be positive", name);
+    CLG_REQUIRE(out_dim < (1ll << 28), "%s: out_dim above 2^28-1 is not supported", name);
+    if (!walk_fits(elem_size, x, y, words)) return clg_fc_eval_packed(elem_size, x, a, b, gate, y, in_dim, out_dim, words, stream);
+    return launch_walk<false>(name, elem_size, x, a, b, gate, plan, y, in_dim, out_dim, words, stream);
+}
+
+extern "C" int clg_fc_eval_walk_fits(int elem_size, const void *x, const void *y, int64_t words)
+{
+    return valid_elem(elem_size) && x && y && words > 0 && walk_fits(elem_size, x, y, words) ? 1 : 0;
+}
+
+extern "C" int clg_fc_eval_packed_planned_logits(int elem_size, const void *x, const int64_t *a, const int64_t *b, const float *logits,
+                                                 const int32_t *plan, void *y, int64_t in_dim, int64_t out_dim, int64_t words,
+                                                 void *stream)
+{
+    const char *name = "clg_fc_eval_packed_planned_logits";
+    CLG_REQUIRE(valid_elem(elem_size), "%s: elem_size must be 1, 2, 4 or 8, got %d", name, elem_size);
+    CLG_REQUIRE(x && a && b && logits && plan && y, "%s: null pointer argument", name);
+    CLG_REQUIRE(x != y, "%s: x and y must not overlap", name);
+    CLG_REQUIRE(in_dim > 0 && out_dim > 0 && words > 0, "%s: in_dim, out_dim and words must be positive", name);
+    CLG_REQUIRE(out_dim < (1ll << 28), "%s: out_dim above 2^28-1 is not supported", name);
+    CLG_REQUIRE(walk_fits(elem_size, x, y, words), "%s: rows must be whole 16-byte vectors of at least 1 KiB at 16-byte aligned addresses "
+                "(clg_fc_eval_walk_fits); use clg_gate_argmax + clg_fc_eval_packed_planned otherwise", name);
+    return launch_walk<true>(name, elem_size, x, a, b, logits, plan, y, in_dim, out_dim, words, stream);
 }

@@ -117,14 +117,11 @@ class LogicLayer(torch.nn.Module):
         assert not self.training
         assert isinstance(x, PackBitsTensor)
         assert x.t.shape[0] == self.in_dim, (x.t.shape, self.in_dim)
-        x.t = difflogic_hip.eval_planned(x.t, self.indices_0, self.indices_1, self._eval_gates(), self._eval_plan())
+        # gate ids = arg-max of the logits, taken on every call as the reference does (src/difflogic/difflogic.py:161): no
+        # cache that an in-place update of `weights.data` (EMA swaps, legacy optimisers) could leave stale.  Where the row
+        # layout allows, the evaluation kernel takes the arg-max itself and the call is one launch.
+        x.t = difflogic_hip.eval_planned_logits(x.t, self.indices_0, self.indices_1, self.weights.detach(), self._eval_plan())
         return x
-
-    def _eval_gates(self):
-        """uint8 arg-max gate id per neuron, taken from the logits on every call as the reference does
-        (src/difflogic/difflogic.py:161): one small launch, and no cache that an in-place update of
-        `weights.data` (EMA swaps, legacy optimisers) could leave stale."""
-        return difflogic_hip.gate_argmax(self.weights.detach())
 
     def _wiring_key(self):
         # (buffers and parameters straight from their dicts: nn.Module.__getattr__ costs a microsecond per lookup, and

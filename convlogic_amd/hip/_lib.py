@@ -56,6 +56,8 @@ SIGNATURES = {
     "clg_fc_eval_packed": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_eval_plan": (_i, [_p, _p, _i64, _i64, _p]),
     "clg_fc_eval_packed_planned": (_i, [_i, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_fc_eval_walk_fits": (_i, [_i, _p, _p, _i64]),
+    "clg_fc_eval_packed_planned_logits": (_i, [_i, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_group_bit_sum": (_i, [_i, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "clg_conv4_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p]),
     "clg_conv4_backward_x": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p]),

@@ -299,6 +299,27 @@ def eval_planned(x, a, b, w, plan):
     return y
 
 
+def eval_planned_logits(x, a, b, logits, plan):
+    """eval_planned(x, a, b, gate_argmax(logits), plan) -- in one launch where the rows are whole 16-byte vectors of at
+    least 1 KiB and the logits float32 (the kernel takes the arg-max itself), in two launches otherwise.
+    LogicLayer.forward_cuda_eval (src/difflogic/difflogic.py:149-164)."""
+    if x.dtype not in _WORD_DTYPE.values() or plan.dtype != torch.int32 or logits.dim() != 2 or logits.shape[1] != 16:
+        raise RuntimeError("eval_planned_logits expects int8/16/32/64 words, logits [out, 16] and an int32 plan")
+    out_dim = logits.shape[0]
+    in_dim, words = _wiring(x, a, b, out_dim)
+    check_input(logits, "weights")
+    check_input(plan, "plan")
+    if tuple(plan.shape) != (out_dim,):
+        raise RuntimeError("plan does not match the number of neurons")
+    lib = _lib.load()
+    y = torch.empty((out_dim, words), dtype=x.dtype, device=x.device)
+    if logits.dtype != torch.float32 or not lib.clg_fc_eval_walk_fits(x.element_size(), x.data_ptr(), y.data_ptr(), words):
+        return eval_planned(x, a, b, gate_argmax(logits), plan)
+    check(lib.clg_fc_eval_packed_planned_logits(x.element_size(), x.data_ptr(), a.data_ptr(), b.data_ptr(), logits.data_ptr(),
+                                                plan.data_ptr(), y.data_ptr(), in_dim, out_dim, words, stream_ptr(x)))
+    return y
+
+
 def _alloc_words(features, batch, bit_count, device):
     if bit_count not in _WORD_DTYPE:
         raise ValueError("`bit_count` has to be in { 8, 16, 32, 64 }")

@@ -240,6 +240,17 @@ int clg_fc_eval_packed_planned(int elem_size, const void *x /*[in_dim,words]*/, 
                                const uint8_t *gate /*[out_dim]*/, const int32_t *plan /*[out_dim]*/,
                                void *y /*[out_dim,words]*/, int64_t in_dim, int64_t out_dim, int64_t words, void *stream);
 
+/* clg_gate_argmax + clg_fc_eval_packed_planned in ONE launch: the kernel takes the arg-max of the 16 float32 logits of a
+ * neuron itself (first maximum, a NaN counts as the maximum: the same gate ids, tested), so a packed layer call is a
+ * single launch.  Needs rows the walk kernel takes -- clg_fc_eval_walk_fits(): whole 16-byte vectors, at least 1 KiB, x
+ * and y 16-byte aligned -- and is rejected with CLG_EINVAL otherwise (use the two calls then).
+ * Replaces `self.weights.argmax(-1).to(torch.uint8)` + difflogic_cuda.eval of LogicLayer.forward_cuda_eval
+ * (src/difflogic/difflogic.py:149-164; src/difflogic/cuda/difflogic_kernel.cu:295-330). */
+int clg_fc_eval_walk_fits(int elem_size, const void *x, const void *y, int64_t words);
+int clg_fc_eval_packed_planned_logits(int elem_size, const void *x /*[in_dim,words]*/, const int64_t *a, const int64_t *b,
+                                      const float *logits /*[out_dim,16]*/, const int32_t *plan /*[out_dim]*/,
+                                      void *y /*[out_dim,words]*/, int64_t in_dim, int64_t out_dim, int64_t words, void *stream);
+
 /* out[s][g] = number of features of class g (features/k consecutive rows) whose sample-s bit is set,
  * for s < words*8*elem_size - pad_len.  features must be divisible by k.
  * Replaces difflogic_cuda.groupbitsum -- src/difflogic/cuda/difflogic.cpp:22-33,

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import convlogic_amd as C
-from convlogic_amd.hip import difflogic_hip
+from convlogic_amd.hip import _lib, difflogic_hip
 from oracle import convlogic_oracle as O
 from tests.gpu_util import DEV
 
@@ -177,6 +177,51 @@ def test_eval_planned_equals_unplanned(in_dim, out_dim, words, bits):
     got = difflogic_hip.eval_planned(xd, a, b, g, plan)
     assert torch.equal(got, difflogic_hip.eval(xd, a, b, g))
     assert np.array_equal(got.cpu().numpy(), O.eval_packed(x, idx0.numpy(), idx1.numpy(), gate.numpy()))
+
+
+@pytest.mark.parametrize("in_dim,out_dim,words,bits", [(64, 96, 1024, 64), (37, 53, 128, 64), (16, 40, 512, 32), (9, 30, 64, 64)])
+def test_eval_planned_from_logits_takes_the_gates_torch_argmax_takes(in_dim, out_dim, words, bits):
+    # arg-max inside the evaluation kernel (rows of at least 1 KiB) or by the separate launch (the 512-byte rows of the
+    # last case): in both cases the gate ids of torch.argmax -- first maximum on ties, -0 == +0, a NaN beats everything,
+    # the first NaN wins -- and the bits of the oracle
+    rng = np.random.default_rng(in_dim * 7 + words)
+    torch.manual_seed(in_dim * 7 + words)
+    info = np.iinfo(O.NP_WORD[bits])
+    x = rng.integers(info.min, info.max, (in_dim, words), dtype=O.NP_WORD[bits])
+    idx0, idx1 = torch.randint(0, in_dim, (out_dim,)), torch.randint(0, in_dim, (out_dim,))
+    logits = torch.randn(out_dim, 16)
+    logits[0] = 0.0                                                  # all equal: gate 0
+    logits[1, 3] = logits[1, 9] = 7.0                                # tie: the first
+    logits[2] = -1.0
+    logits[2, 5], logits[2, 11] = -0.0, 0.0                          # -0 and +0 tie: the first
+    logits[3, 2], logits[3, 6] = float("inf"), float("nan")         # NaN above +inf
+    logits[4, 10], logits[4, 12] = float("nan"), float("nan")       # the first NaN
+    logits[5] = float("-inf")
+    logits[6, 15] = 100.0
+    logits[7] = -torch.arange(16.0) * 1e-30                          # denormal steps downwards: gate 0
+    want = logits.argmax(-1)
+    assert want[:8].tolist() == [0, 3, 5, 6, 10, 0, 15, 0]
+    xd, a, b, lg = torch.from_numpy(x).to(DEV), idx0.to(DEV), idx1.to(DEV), logits.to(DEV)
+    plan = difflogic_hip.eval_plan(a, b, in_dim)
+    got = difflogic_hip.eval_planned_logits(xd, a, b, lg, plan)
+    assert torch.equal(got, difflogic_hip.eval_planned(xd, a, b, difflogic_hip.gate_argmax(lg), plan))
+    assert np.array_equal(got.cpu().numpy(), O.eval_packed(x, idx0.numpy(), idx1.numpy(), want.numpy().astype(np.uint8)))
+    # float64 logits: the two-launch route, same result
+    assert torch.equal(got, difflogic_hip.eval_planned_logits(xd, a, b, lg.double(), plan))
+
+
+def test_eval_planned_logits_entry_point_rejects_rows_the_walk_kernel_does_not_take():
+    lib = _lib.load()
+    x = torch.zeros(8, 16, dtype=torch.int64, device=DEV)            # 128-byte rows
+    y = torch.empty(8, 16, dtype=torch.int64, device=DEV)
+    a = torch.zeros(8, dtype=torch.int64, device=DEV)
+    lg = torch.zeros(8, 16, device=DEV)
+    plan = torch.arange(8, dtype=torch.int32, device=DEV)
+    assert lib.clg_fc_eval_walk_fits(8, x.data_ptr(), y.data_ptr(), 16) == 0
+    assert lib.clg_fc_eval_walk_fits(8, x.data_ptr(), y.data_ptr(), 128) == 1
+    rc = lib.clg_fc_eval_packed_planned_logits(8, x.data_ptr(), a.data_ptr(), a.data_ptr(), lg.data_ptr(), plan.data_ptr(), y.data_ptr(),
+                                               8, 8, 16, 0)
+    assert rc != 0 and b"clg_fc_eval_walk_fits" in lib.clg_last_error()
 
 
 def test_eval_plan_follows_in_place_rewiring():
