@@ -190,6 +190,8 @@ def bench_c2(steps, warmup, cpu=True):
 
     sec = _timed(step, steps, warmup)
     kernel_ms = _avg_ms(pairs)
+    # the same pass as a HIP-graph replay (three launches and their output tensors captured once)
+    graph_ms = _graph_step_ms(lambda: [], lambda leaves: step(None), steps)
     row_bytes = words * 8
     # algorithmic bytes of one layer: every input row read once, every output row written once,
     # wiring (2 x int64) and gate id (uint8) per neuron
@@ -200,6 +202,8 @@ def bench_c2(steps, warmup, cpu=True):
         "value": samples / sec,
         "unit": "samples/s",
         "ms_per_step": sec * 1e3,
+        "ms_per_step_hip_graph": graph_ms,
+        "value_hip_graph": samples / (graph_ms * 1e-3) if graph_ms else None,
         "dtype": "int64",
         "config": {"workload": "C2: 3 x LogicLayer 64000->64000 as packed bits, 65536 samples in int64 words "
                                "(1024 words/feature), argmax gates, random 2-input wiring"},
