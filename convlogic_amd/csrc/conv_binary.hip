@@ -864,6 +864,8 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
         int hsw = 1;
         const int64_t avg_hits = std::max<int64_t>(1, (int64_t)g.c * 2 / g.cin);
         while (hsw < 16 && p.items * hsw * 2 <= 10240 && hsw * 2 * 4 <= avg_hits) hsw *= 2;
+        // one round of the launch when three quarters of that fit the 256 x 32 wavefront slots and the power of two does not
+        if (hsw >= 4 && p.items * hsw > 8192 && p.items * (hsw / 4 * 3) <= 8192) hsw = hsw / 4 * 3;
         if (const char *e = clg_knob(K_BIN_HSW)) hsw = std::min(16, std::max(1, atoi(e)));
         p.hsw = hsw;
         int per_wg = std::max(1, 4 / hsw);
