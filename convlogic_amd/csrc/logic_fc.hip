@@ -734,7 +734,18 @@ __global__ __launch_bounds__(256) void group_sum_backward_fm_kernel(const T *__r
     const int64_t b = bc * kWave + lane;
     if (b >= batch) return;
     const int64_t f0 = fb * 64, features = class_rows * k;
-    for (int64_t f = f0 + wave; f < f0 + 64 && f < features; f += 4) grad_x[f * batch + b] = grad_out[b * k + f / class_rows] * inv_tau;
+    const int64_t f_end = f0 + 64 < features ? f0 + 64 : features;
+    // the class of a row changes at most a few times along the 64 rows: the value is loaded when it does (wave-uniform)
+    int64_t next = 0;
+    T v = T(0);
+    for (int64_t f = f0 + wave; f < f_end; f += 4) {
+        if (f >= next) {
+            const int64_t cls = f / class_rows;
+            next = (cls + 1) * class_rows;
+            v = grad_out[b * k + cls] * inv_tau;
+        }
+        grad_x[f * batch + b] = v;
+    }
 }
 
 // gate[r] = index of the first maximum of the 16 logits of row r (a NaN counts as the maximum, as in torch.argmax)
