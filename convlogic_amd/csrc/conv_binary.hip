@@ -390,7 +390,9 @@ struct BinHist {
 };
 constexpr int kHistDepth = 8;           // steps whose loads are in flight together
 
-template <int HL>
+// PLANE: a (sample, kernel) plane is exactly one step of the wavefront (P = 4 HL cells): the step index is the sample, so a
+// step's addresses are a wave-uniform base plus a constant per lane and cost no vector arithmetic.
+template <int HL, bool PLANE>
 __global__ __launch_bounds__(HL) void convblock_bin_hist_kernel(const float *__restrict__ gy, const uint16_t *__restrict__ aux,
                                                                       float *__restrict__ hpart, BinHist p)
 {
@@ -413,12 +415,20 @@ __global__ __launch_bounds__(HL) void convblock_bin_hist_kernel(const float *__r
     // loads never depend on a branch (an index past the end is clamped), so the compiler can count them and let a
     // whole group of steps stay in flight while the previous group is applied
     auto load = [&](int step, float4 &g4, uint2 &a2) {
-        int e = step * HL + lane;
-        e = e < items ? e : items - 1;
-        const uint32_t smp = fdiv((uint32_t)e, p.d_q), quad = (uint32_t)e - smp * (uint32_t)p.Q;
-        const int64_t at = smp * plane_stride + quad * 4;
-        g4 = *reinterpret_cast<const float4 *>(gyc + at);
-        a2 = *reinterpret_cast<const uint2 *>(axc + at);
+        if constexpr (PLANE) {
+            const int smp = min(step, s1 - s0 - 1);                   // wave-uniform (items = samples * HL)
+            const float *gs = gyc + (int64_t)smp * plane_stride;
+            const uint16_t *as = axc + (int64_t)smp * plane_stride;
+            g4 = reinterpret_cast<const float4 *>(gs)[lane];
+            a2 = reinterpret_cast<const uint2 *>(as)[lane];
+        } else {
+            int e = step * HL + lane;
+            e = e < items ? e : items - 1;
+            const uint32_t smp = fdiv((uint32_t)e, p.d_q), quad = (uint32_t)e - smp * (uint32_t)p.Q;
+            const int64_t at = smp * plane_stride + quad * 4;
+            g4 = *reinterpret_cast<const float4 *>(gyc + at);
+            a2 = *reinterpret_cast<const uint2 *>(axc + at);
+        }
     };
     auto apply = [&](const float4 &g4, const uint2 &a2) {
         const uint32_t t0 = a2.x & 255u, t1 = (a2.x >> 16) & 255u, t2 = a2.y & 255u, t3 = (a2.y >> 16) & 255u;
@@ -912,9 +922,9 @@ extern "C" int clg_convblock_bin_backward(int dtype, const clg_conv_geom *gg, co
         const size_t lds = (size_t)256 * hl * 4;
 #define CLG_BIN_HIST(HL)                                                                                                         \
     do {                                                                                                                         \
-        if (int e = allow_lds(convblock_bin_hist_kernel<HL>, lds, name)) return e;                                               \
-        hipLaunchKernelGGL(convblock_bin_hist_kernel<HL>, dim3((unsigned)(g.c * h.parts)), dim3(HL), lds, st, (const float *)grad_y, \
-                           taps, (float *)scratch, h);                                                                           \
+        auto kern = h.Q == HL ? convblock_bin_hist_kernel<HL, true> : convblock_bin_hist_kernel<HL, false>;                      \
+        if (int e = allow_lds(kern, lds, name)) return e;                                                                        \
+        hipLaunchKernelGGL(kern, dim3((unsigned)(g.c * h.parts)), dim3(HL), lds, st, (const float *)grad_y, taps, (float *)scratch, h); \
     } while (0)
         if (hl == 64) CLG_BIN_HIST(64);
         else if (hl == 32) CLG_BIN_HIST(32);
