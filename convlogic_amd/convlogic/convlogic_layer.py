@@ -88,11 +88,13 @@ class _FullConvLogicLogitsFunction(Function):
         fm = feature_major and convlogic_hip.feature_major_supported(x1, logits.shape[0], *geo, kernel_h, kernel_w)
         ctx.feature_major = fm
         if plan is not None:
-            # the forward launch also leaves the folded coefficients for the planned backward pass
-            y, argmax, w_prob, folded = convlogic_hip.full_convlogic_forward_logits(x1, logits.detach(), selection, *geo, kernel_h,
-                                                                                    kernel_w, feature_major=fm, want_folded=True,
-                                                                                    validate=False)
-            ctx.save_for_backward(x1, w_prob, selection, argmax, folded)
+            # the forward launch also leaves the folded coefficients for the planned backward pass and -- when the input
+            # needs a gradient and the kernels of this shape read one -- the zero-padded copy of x it staged
+            y, argmax, w_prob, folded, *rest = convlogic_hip.full_convlogic_forward_logits(
+                x1, logits.detach(), selection, *geo, kernel_h, kernel_w, feature_major=fm, want_folded=True, validate=False,
+                want_padded=ctx.needs_input_grad[0])
+            padded = rest[0] if rest else None
+            ctx.save_for_backward(x1, w_prob, selection, argmax, folded, *(() if padded is None else (padded,)))
             return y.permute(3, 0, 1, 2) if fm else y
         ctx.plan = None
         y, argmax, w_prob = convlogic_hip.full_convlogic_forward_logits(x1, logits.detach(), selection, *geo, kernel_h, kernel_w,
@@ -104,14 +106,16 @@ class _FullConvLogicLogitsFunction(Function):
     def backward(ctx, grad_y):
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if ctx.plan is not None:
-            x1, w_prob, selection, argmax, folded = ctx.saved_tensors
+            x1, w_prob, selection, argmax, folded, *rest = ctx.saved_tensors
+            padded = rest[0] if rest else None
             if need_w:
                 ok = grad_y.dtype == x1.dtype and grad_y.device == x1.device      # everything else was validated on the way in
                 grad_fm = grad_y.permute(1, 2, 3, 0)
                 use_fm = ctx.feature_major and not grad_y.is_contiguous() and grad_fm.is_contiguous()
                 grad_x, grad_l = convlogic_hip.full_convlogic_backward_planned(grad_fm if use_fm else grad_y.contiguous(), x1, w_prob, folded,
                                                                                argmax, selection, *ctx.plan, *ctx.geometry, need_grad_x=need_x,
-                                                                               validate=not ok, feature_major=use_fm)
+                                                                               validate=not ok, feature_major=use_fm,
+                                                                               padded=None if use_fm else padded)
                 return grad_x, grad_l, None, None, None, None, None, None, None, None, None
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y.contiguous(), x1, w_prob, argmax, selection, *ctx.geometry) if need_x else None
             return grad_x, None, None, None, None, None, None, None, None, None, None

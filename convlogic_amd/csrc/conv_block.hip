@@ -1145,6 +1145,7 @@ int launch_prepare(const Geom &g, const BwdScratch &lay, int rs, int chs, const 
 struct PlanView {
     const int32_t *count = nullptr, *hits = nullptr, *taps = nullptr;
     const void *folded = nullptr;
+    const void *padded = nullptr;   // the zero-padded copy of x the forward call left (clg_convblock_forward_padded), or null
 };
 // Where the gradient kernels of a call find their tables: in the call's scratch (written by the set-up launch) or in a plan.
 struct BwdTables {
@@ -1234,9 +1235,11 @@ int launch_backward_x_direct(const Geom &g, const TilePlan &p, int sample_elems,
 {
     const BwdScratch lay = bwd_scratch_layout(g, (int)sizeof(T), 1);
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
-    T *xp = reinterpret_cast<T *>(base + bwd_x_direct_xp_off(lay));
+    const bool have_copy = pv != nullptr && pv->padded != nullptr;   // made by the forward call: nothing to pad here
+    T *xp = have_copy ? const_cast<T *>(reinterpret_cast<const T *>(pv->padded)) : reinterpret_cast<T *>(base + bwd_x_direct_xp_off(lay));
     BwdTables tb;
-    if (int e = prepare_tables<T>(g, lay, p.rs, p.chs, w, sel, scratch, st, make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems), pv, &tb))
+    if (int e = prepare_tables<T>(g, lay, p.rs, p.chs, w, sel, scratch, st,
+                                  have_copy ? no_pad_job<T>() : make_pad_job((const T *)x, xp, g, p.rs, p.chs, sample_elems), pv, &tb))
         return e;
     if (shared != nullptr) {
         shared->xp = xp;
@@ -1718,11 +1721,19 @@ extern "C" int clg_convblock_plan(int dtype, const clg_conv_geom *gg, const int3
     return CLG_OK;
 }
 
-extern "C" int clg_convblock_backward_planned(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
-                                              const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
-                                              int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream)
+// One sample of the padded copy the planned backward pass reads when its input gradient is the direct kernel, else 0.
+int64_t clg_convblock_backward_padded_sample_elems(int dtype, const Geom &g)
 {
-    const char *name = "clg_convblock_backward_planned";
+    if (backward_4x4_wanted(g)) return 0;
+    TilePlan p;
+    int se = 0;
+    return choose_backward_x(g, elem_size(dtype), &p, &se) == kBwdXDirect ? se : 0;
+}
+
+static int backward_planned_impl(const char *name, int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                 const void *folded, const void *padded, const int32_t *selection, const uint8_t *argmax, void *plan,
+                                 int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream)
+{
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
     CLG_REQUIRE(grad_y && x && w && selection && argmax && plan && grad_w && scratch, "%s: null pointer argument", name);
@@ -1739,6 +1750,7 @@ extern "C" int clg_convblock_backward_planned(int dtype, const clg_conv_geom *gg
     pv.hits = reinterpret_cast<const int32_t *>(pb + pi.lay.hits_off);
     pv.taps = reinterpret_cast<const int32_t *>(pb + pi.lay.taps_off);
     pv.folded = folded;
+    pv.padded = padded;
     const void *probs = wrt_logits ? w : nullptr;
     if (backward_4x4_wanted(g)) {
         g.y_fm = fm ? 1 : 0;
@@ -1752,4 +1764,26 @@ extern "C" int clg_convblock_backward_planned(int dtype, const clg_conv_geom *gg
         if (int e = convblock_backward_x_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_x, scratch, stream, &shared, w_scratch, &pv))
             return e;
     return convblock_backward_w_impl(dtype, gg, grad_y, x, w, selection, argmax, grad_w, w_scratch, stream, probs, name, &shared);
+}
+
+extern "C" int clg_convblock_backward_planned(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                              const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
+                                              int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream)
+{
+    return backward_planned_impl("clg_convblock_backward_planned", dtype, gg, grad_y, x, w, folded, nullptr, selection, argmax, plan, signature,
+                                 grad_x, grad_w, flags, scratch, stream);
+}
+
+extern "C" int clg_convblock_backward_planned_padded(int dtype, const clg_conv_geom *gg, const void *grad_y, const void *x, const void *w,
+                                                     const void *folded, const void *padded, const int32_t *selection,
+                                                     const uint8_t *argmax, void *plan, int64_t signature, void *grad_x, void *grad_w,
+                                                     int flags, void *scratch, void *stream)
+{
+    const char *name = "clg_convblock_backward_planned_padded";
+    Geom g;
+    if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
+    CLG_REQUIRE(padded == nullptr || (grad_x != nullptr && clg_convblock_backward_padded_sample_elems(dtype, g) > 0),
+                "%s: a padded copy is only taken with grad_x and where clg_convblock_padded_elems() is not 0", name);
+    return backward_planned_impl(name, dtype, gg, grad_y, x, w, folded, padded, selection, argmax, plan, signature, grad_x, grad_w, flags,
+                                 scratch, stream);
 }

@@ -125,6 +125,21 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
         }
     }
     __syncthreads();
+    if constexpr (!SUBSET) {
+        // The staged image IS the zero-padded copy of x that the direct input gradient and the padded weight gradient read
+        // (same row and plane strides): the first kernel tile of every sample block leaves it in global memory, and the
+        // backward call needs no launch to make it.  A sample's tail (the halo behind its last plane) reads as zeros here:
+        // it is the top halo of the next sample's first plane, or the image's own tail.
+        if (p.padded_out != nullptr && blockIdx.y == 0) {
+            T *po = reinterpret_cast<T *>(p.padded_out);
+            const int se = p.padded_sample_elems;
+            for (int s = 0; s < s_cur; ++s) {
+                T *dst = po + (int64_t)(n0 + s) * se;
+                const T *img = xs + s * p.planes * p.chs;
+                for (int e = tid; e < se; e += nthreads) dst[e] = img[e];
+            }
+        }
+    }
     if constexpr (Ops::kParams == 28) {                              // float gates: the folded coefficients for the backward pass
         if (p.folded_out != nullptr && blockIdx.x == 0) {
             T *fo = reinterpret_cast<T *>(p.folded_out) + (int64_t)c0 * 28;
@@ -491,12 +506,13 @@ int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scr
 template <typename Ops, typename P>
 int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, const void *params, const int32_t *sel, void *y,
                           uint8_t *argmax, void *scratch, hipStream_t st, const char *name, bool from_logits = false,
-                          void *probs_out = nullptr)
+                          void *probs_out = nullptr, void *padded_out = nullptr)
 {
     using T = typename Ops::Elem;
     unsigned char *base = reinterpret_cast<unsigned char *>(scratch);
     int32_t *taps = reinterpret_cast<int32_t *>(base + d.taps_off);
-    T *xp = reinterpret_cast<T *>(base + d.xp_off);
+    // the padded copy this path reads: in the scratch, or where the caller keeps it for the backward call
+    T *xp = padded_out != nullptr ? reinterpret_cast<T *>(padded_out) : reinterpret_cast<T *>(base + d.xp_off);
     // one launch: folded coefficients (float gates only), tap offsets and the padded copy
     const bool fold = Ops::kParams > 1;
     const void *kernel_params = fold ? (const void *)base : params;
@@ -661,10 +677,11 @@ __global__ __launch_bounds__(256) void softmax16_rows_kernel(const T *__restrict
 }  // namespace
 
 // Forward of the complete block with options (flags: CLG_FWD_W_LOGITS, CLG_FWD_Y_FEATURE_MAJOR).
-extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
-                                        void *y, uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream)
+int64_t clg_convblock_backward_padded_sample_elems(int dtype, const Geom &g);
+
+static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                           void *y, uint8_t *argmax, void *probs_out, int flags, void *scratch, void *padded_out, void *stream)
 {
-    const char *name = "clg_convblock_forward_ex";
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
     CLG_REQUIRE(x && w && selection && y && argmax, "%s: null pointer argument", name);
@@ -713,8 +730,10 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     }
     if (path == 2) {
         if (dtype == CLG_F32)
-            return fold_after(launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out));
-        return fold_after(launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out));
+            return fold_after(launch_forward_direct<FloatOps<float>, float>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out,
+                                                                            padded_out));
+        return fold_after(launch_forward_direct<FloatOps<double>, double>(g, dp, x, w, selection, y, argmax, scratch, st, name, logits, probs_out,
+                                                                          padded_out));
     }
     // The staged kernels take the softmax per workgroup while they set their gate parameters up, as long as that is at
     // most two rows of 16 logits per thread (C3 graph step 66.7 -> 63.7 us against a small launch of its own; with the
@@ -737,10 +756,49 @@ extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, cons
     if (staged) {
         tp.w_logits = in_kernel ? 1 : 0;
         tp.folded_out = folded_out;                                  // written by the first sample block of every kernel tile
+        if (padded_out != nullptr) {
+            tp.padded_out = padded_out;                              // written by the first kernel tile of every sample block
+            tp.padded_sample_elems = g.cin * tp.chs + g.ph * tp.rs + g.pw;
+        }
         if (dtype == CLG_F32) return launch_forward_tiled<FloatOps<float>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
         return launch_forward_tiled<FloatOps<double>>(g, tp, x, w, selection, y, argmax, st, name, probs_out);
     }
     return fold_after(clg_convblock_forward_generic(dtype, g, x, w, selection, y, argmax, st));
+}
+
+extern "C" int clg_convblock_forward_ex(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                        void *y, uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream)
+{
+    return forward_ex_impl("clg_convblock_forward_ex", dtype, gg, x, w, selection, y, argmax, probs_out, flags, scratch, nullptr, stream);
+}
+
+// Elements of the padded copy of x that clg_convblock_forward_padded leaves for clg_convblock_backward_planned_padded, or 0
+// when the pair has no use for one at this shape: the forward must stage or read the copy anyway (all channels in LDS, or
+// the direct kernel) and the backward must be the one that reads its taps from such a copy.
+extern "C" int64_t clg_convblock_padded_elems(int dtype, const clg_conv_geom *gg, int have_scratch)
+{
+    Geom g;
+    if (clg_convblock_check(gg, &g, dtype, "clg_convblock_padded_elems")) return -1;
+    TilePlan tp;
+    DirectPlan dp;
+    const int elem = dtype == CLG_F64 ? 8 : 4;
+    const int path = choose_forward(g, elem, 28, have_scratch != 0, &tp, &dp);
+    if (path != 0 && path != 2) return 0;
+    const int64_t se = clg_convblock_backward_padded_sample_elems(dtype, g);
+    if (se <= 0) return 0;
+    const int64_t mine = path == 2 ? dp.sample_elems : (int64_t)g.cin * tp.chs + g.ph * tp.rs + g.pw;
+    return se == mine ? se * g.n : 0;
+}
+
+extern "C" int clg_convblock_forward_padded(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
+                                            void *y, uint8_t *argmax, void *probs_out, int flags, void *scratch, void *padded_out,
+                                            void *stream)
+{
+    const char *name = "clg_convblock_forward_padded";
+    CLG_REQUIRE(padded_out, "%s: null pointer argument", name);
+    CLG_REQUIRE((flags & CLG_FWD_Y_FEATURE_MAJOR) == 0 && clg_convblock_padded_elems(dtype, gg, scratch != nullptr) > 0,
+                "%s: no padded copy at this shape (clg_convblock_padded_elems)", name);
+    return forward_ex_impl(name, dtype, gg, x, w, selection, y, argmax, probs_out, flags, scratch, padded_out, stream);
 }
 
 // Which shapes the feature-major variants take: the one-sample-per-lane kernels for 4x4 images (conv_small.hip).

@@ -38,6 +38,8 @@ struct TilePlan {
     int one_row;           // forward: 1 = a lane slot is one conv position (ho * wo per sample) instead of a column of two rows
     int w_logits;          // forward: 1 = the gate parameters handed to the kernel are logits (softmax taken while staging them)
     void *folded_out = nullptr;   // forward: where the first sample block writes the folded coefficients [c, 7, 4] of its kernels (or null)
+    void *padded_out = nullptr;   // forward: where the first kernel tile writes its staged, zero-padded image: [n][sample_elems] (or null)
+    int padded_sample_elems = 0;  // cin * chs + ph * rs + pw: one sample of that copy
     FastDiv d_hw, d_w, d_slots, d_wo, d_wp, d_planes;
     size_t lds_bytes;
 };

@@ -84,6 +84,8 @@ SIGNATURES = {
     "clg_convblock_backward_logits": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "clg_convblock_fm_supported": (_i, [_i, _GP]),
     "clg_convblock_forward_ex": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _i, _p, _p]),
+    "clg_convblock_padded_elems": (_i64, [_i, _GP, _i]),
+    "clg_convblock_forward_padded": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _i, _p, _p, _p]),
     "clg_convblock_eval_packed_fm_supported": (_i, [_GP]),
     "clg_convblock_eval_packed_fm": (_i, [_GP, _p, _p, _p, _p, _p]),
     "clg_convblock_forward_fm": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p]),
@@ -92,6 +94,7 @@ SIGNATURES = {
     "clg_convblock_plan_bytes": (_i64, [_i, _GP]),
     "clg_convblock_plan": (_i, [_i, _GP, _p, _p, _p, _p]),
     "clg_convblock_backward_planned": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i, _p, _p]),
+    "clg_convblock_backward_planned_padded": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i, _p, _p]),
     "clg_convblock_bin_supported": (_i, [_i, _GP]),
     "clg_convblock_bin_ctx_bytes": (_i64, [_i, _GP]),
     "clg_convblock_bin_forward": (_i, [_i, _GP, _p, _p, _p, _p, _p, _p, _i, _p, _p]),

@@ -313,11 +313,13 @@ def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, p
 
 
 def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False,
-                                  want_folded=False, validate=True):
+                                  want_folded=False, validate=True, want_padded=False):
     """full_convlogic_forward() from the LOGITS [C, 7, 16]: the softmax is taken inside the launch that sets the gate
     parameters up.  -> (y, argmax, probs); with feature_major (where feature_major_supported) y is laid out
     [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm().  want_folded: -> (y, argmax, probs, folded [C, 7, 4]), the
-    folded coefficients of every gate for full_convlogic_backward_planned()."""
+    folded coefficients of every gate for full_convlogic_backward_planned().  want_padded (with want_folded): a fifth
+    result, the zero-padded copy of x that the forward kernels stage anyway and the planned backward pass would otherwise
+    make in a launch of its own -- or None where the pair of kernels at this shape has no use for one."""
     if validate:
         _conv_args(x, logits, selection, 7)
     g = _geom(x, logits.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
@@ -333,10 +335,22 @@ def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_
         probs, folded = torch.empty_like(logits), None
     lib = _lib.load()
     scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
-    check(lib.clg_convblock_forward_ex(dtype_code(x), ctypes.byref(g), x.data_ptr(), logits.data_ptr(), selection.data_ptr(),
-                                       y.data_ptr(), argmax.data_ptr(), probs.data_ptr(),
-                                       1 | (2 if feature_major else 0) | (4 if want_folded else 0),
-                                       scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))
+    flags = 1 | (2 if feature_major else 0) | (4 if want_folded else 0)
+    padded = None
+    if want_padded and want_folded and not feature_major:
+        elems = lib.clg_convblock_padded_elems(dtype_code(x), ctypes.byref(g), 1 if scratch is not None else 0)
+        if elems > 0:
+            padded = torch.empty((elems,), dtype=x.dtype, device=x.device)
+    if padded is not None:
+        check(lib.clg_convblock_forward_padded(dtype_code(x), ctypes.byref(g), x.data_ptr(), logits.data_ptr(), selection.data_ptr(),
+                                               y.data_ptr(), argmax.data_ptr(), probs.data_ptr(), flags,
+                                               scratch.data_ptr() if scratch is not None else None, padded.data_ptr(), stream_ptr(x)))
+    else:
+        check(lib.clg_convblock_forward_ex(dtype_code(x), ctypes.byref(g), x.data_ptr(), logits.data_ptr(), selection.data_ptr(),
+                                           y.data_ptr(), argmax.data_ptr(), probs.data_ptr(), flags,
+                                           scratch.data_ptr() if scratch is not None else None, stream_ptr(x)))
+    if want_padded:
+        return y, argmax, probs, folded, padded
     if want_folded:
         return y, argmax, probs, folded
     return y, argmax, probs
@@ -361,7 +375,7 @@ def make_backward_plan(x, c_out, selection, stride_h, stride_w, pad_h, pad_w, ke
 
 
 def full_convlogic_backward_planned(grad_y, x, weight, folded, argmax, selection, plan, signature, stride_h, stride_w, pad_h, pad_w,
-                                    need_grad_x=True, wrt_logits=True, validate=True, feature_major=False):
+                                    need_grad_x=True, wrt_logits=True, validate=True, feature_major=False, padded=None):
     """-> (grad_x or None, grad_w [C,7,16]) with the layer's plan from make_backward_plan(): no list building, no reduce
     launch and -- with folded [C, 7, 4] from full_convlogic_forward_logits(want_folded=True) -- no set-up launch for
     blocks whose images fit LDS.  grad_w is the gradient w.r.t. the logits (weight = their softmax) or, with
@@ -383,10 +397,20 @@ def full_convlogic_backward_planned(grad_y, x, weight, folded, argmax, selection
     scratch = _scratch(lib.clg_convblock_backward_scratch_bytes(dt, ctypes.byref(g)), x.device)
     gx = torch.empty_like(x) if need_grad_x else None
     gw = torch.empty((g.c_out, 7, 16), dtype=x.dtype, device=x.device)
+    flags = (1 if wrt_logits else 0) | (2 if feature_major else 0)
+    if padded is not None and need_grad_x:
+        # the padded copy of x that full_convlogic_forward_logits(want_padded=True) left: no launch to make one
+        if validate:
+            check_input(padded, "padded", x.dtype, (lib.clg_convblock_padded_elems(dt, ctypes.byref(g), 1),))
+        check(lib.clg_convblock_backward_planned_padded(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                                        folded.data_ptr() if folded is not None else None, padded.data_ptr(),
+                                                        selection.data_ptr(), argmax.data_ptr(), plan.data_ptr(), signature, gx.data_ptr(),
+                                                        gw.data_ptr(), flags, scratch.data_ptr(), stream_ptr(x)))
+        return gx, gw
     check(lib.clg_convblock_backward_planned(dt, ctypes.byref(g), grad_y.data_ptr(), x.data_ptr(), weight.data_ptr(),
                                              folded.data_ptr() if folded is not None else None, selection.data_ptr(), argmax.data_ptr(),
                                              plan.data_ptr(), signature, gx.data_ptr() if need_grad_x else None, gw.data_ptr(),
-                                             (1 if wrt_logits else 0) | (2 if feature_major else 0), scratch.data_ptr(), stream_ptr(x)))
+                                             flags, scratch.data_ptr(), stream_ptr(x)))
     return gx, gw
 
 

@@ -430,6 +430,23 @@ int clg_convblock_backward_planned(int dtype, const clg_conv_geom *g, const void
                                    const void *folded, const int32_t *selection, const uint8_t *argmax, void *plan,
                                    int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch, void *stream);
 
+/* The padded hand-off.  The forward kernels of most shapes stage a zero-padded copy of x (in LDS, or in their scratch), and
+ * the input gradient of layers with many channels reads its taps from exactly such a copy, which the backward call
+ * otherwise makes in a launch of its own.  clg_convblock_padded_elems(): elements of that copy (n samples of
+ * c_in * (h + ph) * (w + pw) + ph * (w + pw) + pw) when both sides have use for it at this shape, else 0.
+ * clg_convblock_forward_padded = clg_convblock_forward_ex that also leaves the copy in padded_out;
+ * clg_convblock_backward_planned_padded = clg_convblock_backward_planned that reads it (`padded` may be NULL: the plain
+ * call) -- same values.  The reference pads x once per weight-gradient call (torch::constant_pad_nd,
+ * src/convlogic/cuda/full_convlogic_kernel.cu:635) and bounds-checks every tap elsewhere (:16-33, :241-257); here one
+ * padded copy per step serves the forward and both gradients. */
+int64_t clg_convblock_padded_elems(int dtype, const clg_conv_geom *g, int have_scratch);
+int clg_convblock_forward_padded(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection, void *y,
+                                 uint8_t *argmax, void *probs_out, int flags, void *scratch, void *padded_out, void *stream);
+int clg_convblock_backward_planned_padded(int dtype, const clg_conv_geom *g, const void *grad_y, const void *x, const void *w,
+                                          const void *folded, const void *padded, const int32_t *selection, const uint8_t *argmax,
+                                          void *plan, int64_t signature, void *grad_x, void *grad_w, int flags, void *scratch,
+                                          void *stream);
+
 /* The fused block on BINARY inputs (every x is 0 or 1: the first block of a network, behind the threshold transform of
  * src/convlogic/data.py:46-50).  float32, stride 1, images at most 32 columns wide, at most 256 pooled cells (a multiple
  * of 4) per plane: clg_convblock_bin_supported.  A kernel's tree is then a 256-entry table over its 8 tap bits, made with

@@ -575,3 +575,37 @@ def test_selection_corrupted_behind_the_host_check_is_clamped_not_faulting():
         layer.invalidate()
         with pytest.raises(ValueError, match="selection"):
             layer(x)
+
+
+@pytest.mark.parametrize("n,cin,h,w,cout", [(130, 32, 16, 16, 24), (20, 128, 8, 8, 40), (6, 1100, 16, 16, 48), (9, 3, 12, 12, 5)])
+def test_padded_copy_left_by_the_forward_gives_the_planned_backward_its_taps(n, cin, h, w, cout):
+    # the forward leaves the zero-padded copy of x it staged (all channels in LDS: the first two shapes; the direct
+    # kernel's copy: the third) and the planned backward reads it instead of making one: bit-identical gradients; shapes
+    # without such a pair of kernels (the last) report 0 elements and take the plain route
+    torch.manual_seed(n + cin)
+    x = torch.rand(n, cin, h, w, device=DEV)
+    layer = C.ConvLogicLayer(cin, cout, complete=True, implementation="cuda").to(DEV)
+    logits, sel = layer.weights.detach(), layer.selection
+    geo = (1, 1, 1, 1)
+    plan, sig = convlogic_hip.make_backward_plan(x, cout, sel, *geo, 3, 3)
+    y, am, probs, folded, padded = convlogic_hip.full_convlogic_forward_logits(x, logits, sel, *geo, 3, 3, want_folded=True, want_padded=True)
+    y0, am0, probs0, folded0 = convlogic_hip.full_convlogic_forward_logits(x, logits, sel, *geo, 3, 3, want_folded=True)
+    assert torch.equal(y, y0) and torch.equal(am, am0) and torch.equal(folded, folded0)
+    gy = torch.randn_like(y)
+    gx0, gw0 = convlogic_hip.full_convlogic_backward_planned(gy, x, probs0, folded0, am0, sel, plan, sig, *geo)
+    if cin == 3:
+        assert padded is None
+        return
+    assert padded is not None
+    # the copy itself: x inside, zeros in every halo
+    rs, rows = w + 1, h + 1
+    se = cin * rows * rs + rs + 1
+    img = padded.view(n, se)[:, :cin * rows * rs].view(n, cin, rows, rs)
+    assert torch.equal(img[:, :, 1:, 1:], x)
+    assert not img[:, :, 0, :].any() and not img[:, :, :, 0].any() and not padded.view(n, se)[:, cin * rows * rs:].any()
+    gx, gw = convlogic_hip.full_convlogic_backward_planned(gy, x, probs, folded, am, sel, plan, sig, *geo, padded=padded)
+    assert torch.equal(gx, gx0) and torch.equal(gw, gw0)
+    # and through the module: same gradients as the oracle route checks elsewhere, here against the plain call
+    xg = x.clone().requires_grad_(True)
+    layer(xg).backward(gy)
+    assert torch.equal(xg.grad, gx0)
