@@ -127,16 +127,16 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     __syncthreads();
     if constexpr (!SUBSET) {
         // The staged image IS the zero-padded copy of x that the direct input gradient and the padded weight gradient read
-        // (same row and plane strides): the first kernel tile of every sample block leaves it in global memory, and the
-        // backward call needs no launch to make it.  A sample's tail (the halo behind its last plane) reads as zeros here:
-        // it is the top halo of the next sample's first plane, or the image's own tail.
-        if (p.padded_out != nullptr && blockIdx.y == 0) {
+        // (same row and plane strides): the kernel tiles of a sample block, which all hold it, each leave their share of it
+        // in global memory, and the backward call needs no launch to make it.  A sample's tail (the halo behind its last
+        // plane) reads as zeros here: it is the top halo of the next sample's first plane, or the image's own tail.
+        if (p.padded_out != nullptr) {
             T *po = reinterpret_cast<T *>(p.padded_out);
             const int se = p.padded_sample_elems;
             for (int s = 0; s < s_cur; ++s) {
                 T *dst = po + (int64_t)(n0 + s) * se;
                 const T *img = xs + s * p.planes * p.chs;
-                for (int e = tid; e < se; e += nthreads) dst[e] = img[e];
+                for (int e = (int)blockIdx.y * nthreads + tid; e < se; e += nthreads * (int)gridDim.y) dst[e] = img[e];
             }
         }
     }
