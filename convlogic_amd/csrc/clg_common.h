@@ -35,7 +35,7 @@ void clg_set_error(const char *fmt, ...);
     X(BWDW_CELLS) X(BWDW_PADDED) X(BWDX_BANDS) X(BWDX_CSR) X(BWDX_DIRECT) X(BWDX_HSW) X(BWDX_SPLIT) X(BWD_4X4)         \
     X(EVAL_CHUNK_BYTES) X(EVAL_NPW) X(EVAL_WALK_R) X(EVAL_WALK_SEG) X(FWD_4X4) X(FWD_CT) X(FWD_DIRECT) X(FWD_NW)       \
     X(FWD_ONE_ROW) X(FWD_S) X(FWD_SOFTMAX_IN_KERNEL) X(FWD_SUBSET) X(GSUM_SLICES) X(PACKED_4X4_HALVES) X(PACK_TILE)    \
-    X(BWDW_LDS) X(BIN_CT) X(BIN_S) X(BIN_NW) X(BIN_HSW) X(BIN_PARTS) X(BIN_PIECE) X(BIN_HL)
+    X(BWDW_LDS) X(BIN_CT) X(BIN_S) X(BIN_NW) X(BIN_HSW) X(BIN_PARTS) X(BIN_PIECE) X(BIN_HL) X(FWD_KPL)
 enum ClgKnob {
 #define CLG_KNOB_ENUM(name) K_##name,
     CLG_KNOBS(CLG_KNOB_ENUM)

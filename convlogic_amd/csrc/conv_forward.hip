@@ -17,6 +17,8 @@
 // parameters and tap offsets sit in scalar registers.
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include "conv_ops.h"
 
 int clg_convblock_check(const clg_conv_geom *gg, Geom *g, int dtype, const char *name);
@@ -275,6 +277,112 @@ __global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restr
     }
 }
 
+// Forward with one KERNEL per lane: for deep blocks on small images -- hundreds of kernels, at most 16 pooled cells per
+// sample, all input planes of a sample in LDS.  With lanes along positions (the kernel above) every wavefront fetches a
+// kernel's 28 coefficients and 8 tap offsets from LDS for ONE block of 64 positions: 9 of its 17 LDS instructions per
+// kernel.  Here a lane keeps its kernel's coefficients and tap offsets in registers for the whole sample and walks the
+// conv positions cell by cell: 8 LDS gathers per position and nothing else, the 2x2 pool is a running maximum in
+// registers (first maximum wins, in window order), and a lane's pooled values leave as whole 16-byte vectors.
+// folded = [c][7][4] coefficients made by convblock_w_prepare_kernel.  Same values bit for bit: the same gate().
+constexpr int kKplMaxCells = 16;
+template <typename T>
+__global__ __launch_bounds__(512) void convblock_forward_kpl_kernel(const T *__restrict__ x, const T *__restrict__ folded,
+                                                                  const int32_t *__restrict__ sel, T *__restrict__ y,
+                                                                  uint8_t *__restrict__ argmax, Geom g, TilePlan p, int kernels_per_wg)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *xs = reinterpret_cast<T *>(smem);
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int n = blockIdx.x, c0 = blockIdx.y * kernels_per_wg;
+    const int hw = g.h * g.w;
+    for (int i = tid; i < p.xe; i += nthreads) xs[i] = T(0);
+    __syncthreads();
+    {
+        const T *src = x + (int64_t)n * g.cin * hw;
+        const uint32_t total = (uint32_t)g.cin * (uint32_t)hw;
+        for (uint32_t e0 = tid; e0 < total; e0 += 4 * nthreads) {
+            T v[4];
+            int at[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t e = e0 + k * nthreads;
+                at[k] = -1;
+                if (e < total) {
+                    const uint32_t plane = fdiv(e, p.d_hw), rem = e - plane * (uint32_t)hw;
+                    const uint32_t iy = fdiv(rem, p.d_w), ix = rem - iy * (uint32_t)g.w;
+                    at[k] = (int)(plane * p.chs + (iy + g.ph) * p.rs + ix + g.pw);
+                    v[k] = src[e];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (at[k] >= 0) xs[at[k]] = v[k];
+        }
+    }
+    __syncthreads();
+    if (p.padded_out != nullptr) {                                    // the staged image = the padded copy for the backward pass
+        T *dst = reinterpret_cast<T *>(p.padded_out) + (int64_t)n * p.padded_sample_elems;
+        for (int e = (int)blockIdx.y * nthreads + tid; e < p.padded_sample_elems; e += nthreads * (int)gridDim.y) dst[e] = xs[e];
+    }
+    const int k = c0 + tid;
+    if (tid >= kernels_per_wg || k >= g.c) return;
+    Tree<T> tr;
+    const T *fc = folded + (int64_t)k * 28;
+#pragma unroll
+    for (int q = 0; q < 7; ++q) tr.g[q] = Coef<T>{fc[4 * q], fc[4 * q + 1], fc[4 * q + 2], fc[4 * q + 3]};
+    int to[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const Tap tp = unpack_tap(sel[(int64_t)k * 8 + t], tap_limit(g));
+        to[t] = tp.ch * p.chs + tp.ry * p.rs + tp.rx;
+    }
+    const int wp = g.wo >> 1, I = (g.ho >> 1) * wp;
+    T best[kKplMaxCells];
+    uint32_t codes = 0;
+#pragma unroll
+    for (int cell = 0; cell < kKplMaxCells; ++cell) {
+        best[cell] = T(0);
+        if (cell < I) {                                               // wave-uniform
+            const int cy = cell / wp, cx = cell - cy * wp;
+            int code = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int off = ((2 * cy + (q >> 1)) * g.sh) * p.rs + (2 * cx + (q & 1)) * g.sw;
+                T v[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = xs[to[t] + off];
+                const T r = eval_tree(tr, v).root;
+                if (q == 0) {
+                    best[cell] = r;
+                } else if (r > best[cell]) {
+                    best[cell] = r;
+                    code = q;
+                }
+            }
+            codes |= (uint32_t)code << (2 * cell);
+        }
+    }
+    const int64_t o = ((int64_t)n * g.c + k) * I;
+    if (I == kKplMaxCells && sizeof(T) == 4) {
+        float4 *yo = reinterpret_cast<float4 *>(y + o);
+        uint32_t packed[4];
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+            yo[v4] = make_float4((float)best[4 * v4], (float)best[4 * v4 + 1], (float)best[4 * v4 + 2], (float)best[4 * v4 + 3]);
+            const uint32_t c8 = (codes >> (8 * v4)) & 0xFFu;      // four 2-bit codes -> four bytes
+            packed[v4] = (c8 & 3u) | ((c8 & 12u) << 6) | ((c8 & 48u) << 12) | ((c8 & 192u) << 18);
+        }
+        *reinterpret_cast<uint4 *>(argmax + o) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    } else {
+#pragma unroll
+        for (int cell = 0; cell < kKplMaxCells; ++cell)
+            if (cell < I) {
+                y[o + cell] = best[cell];
+                argmax[o + cell] = (uint8_t)((codes >> (2 * cell)) & 3u);
+            }
+    }
+}
+
 // Forward without LDS: for layers whose input channels do not fit LDS or whose images leave lanes idle.
 // Taps come from a zero-padded global copy of x (shared-halo layout, served by L1/L2), so there is no
 // staging, no barrier and no bounds check.  A wavefront keeps one set of 64 lane slots (sample, conv row
@@ -485,13 +593,22 @@ bool plan_forward_direct(const Geom &g, int elem, bool needs_folded, DirectPlan 
 
 // Which forward path a shape takes: 0 = tiled (all channels in LDS), 1 = tiled with channel subsets,
 // 2 = direct from a padded copy (needs scratch), 3 = any-shape kernel, 4 = one sample per lane on 4x4 images
-// (float gates; needs scratch for the folded coefficients).
+// (float gates; needs scratch for the folded coefficients), 5 = one kernel per lane (float gates, at most 16 pooled
+// cells, all planes of a sample in LDS, at least 256 kernels; needs scratch for the folded coefficients).
 int choose_forward(const Geom &g, int elem, int params_per_kernel, bool have_scratch, TilePlan *tp, DirectPlan *dp)
 {
     bool lane_sample = have_scratch && params_per_kernel > 1 && clg_convblock_is_4x4(g);
     if (const char *e = clg_knob(K_FWD_4X4)) lane_sample = lane_sample && atoi(e) != 0;
     if (lane_sample) return 4;
     const bool tiled = plan_forward(g, elem, params_per_kernel, tp);
+    {
+        // one kernel per lane: 40.4 -> 21.2 us (+ 3.9 us for the launch that folds the coefficients) at [256,128,8,8] -> 512
+        const int I = (g.ho / 2) * (g.wo / 2);
+        bool kpl = have_scratch && params_per_kernel > 1 && tiled && !tp->subset && tp->one_row && tp->S == 1 && I <= kKplMaxCells && g.c >= 256 &&
+                   g.ho % 2 == 0 && g.wo % 2 == 0;
+        if (const char *e = clg_knob(K_FWD_KPL)) kpl = kpl && atoi(e) != 0;
+        if (kpl) return 5;
+    }
     const bool direct = have_scratch && plan_forward_direct(g, elem, params_per_kernel > 1, dp);
     // 4-byte elements: direct beats the channel-subset staging (354 -> 163 us at [256,256,16,16] -> 1024); 8-byte
     // elements load twice the bytes per tap and stay on the staged kernels (200 vs 329 us at [256,4096,4,4] -> 8192)
@@ -531,6 +648,24 @@ int launch_forward_direct(const Geom &g, const DirectPlan &d, const void *x, con
 }
 
 // ---- launch ------------------------------------------------------------------------------------
+// one kernel per lane (path 5): tp = the tiled plan of the shape (strides and size of the LDS image of one sample)
+template <typename T>
+int launch_forward_kpl(const Geom &g, TilePlan tp, const void *x, const void *folded, const int32_t *sel, void *y, uint8_t *argmax,
+                       void *padded_out, hipStream_t st, const char *name)
+{
+    int per_wg = 512;
+    if (const char *e = clg_knob(K_FWD_CT)) per_wg = std::min(512, std::max(64, atoi(e) / 64 * 64));
+    per_wg = std::min(per_wg, (int)clg_ceil_div(g.c, 64) * 64);
+    tp.padded_out = padded_out;
+    tp.padded_sample_elems = g.cin * tp.chs + g.ph * tp.rs + g.pw;
+    const size_t lds = (size_t)tp.xe * sizeof(T);
+    if (int e = allow_lds(convblock_forward_kpl_kernel<T>, lds, name)) return e;
+    hipLaunchKernelGGL(convblock_forward_kpl_kernel<T>, dim3((unsigned)g.n, (unsigned)clg_ceil_div(g.c, per_wg)), dim3(per_wg), lds, st,
+                       (const T *)x, (const T *)folded, sel, (T *)y, argmax, g, tp, per_wg);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
+}
+
 template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW = false>
 int launch_forward_one(const Geom &g, const TilePlan &p, const void *x, const void *params, const int32_t *sel, void *y,
                        uint8_t *argmax, hipStream_t st, const char *name, void *probs_out = nullptr)
@@ -631,7 +766,7 @@ extern "C" int64_t clg_convblock_forward_scratch_bytes(int dtype, const clg_conv
     DirectPlan dp;
     const int elem = dtype == CLG_F64 ? 8 : 4;
     const int path = choose_forward(g, elem, 28, true, &tp, &dp);
-    return path == 2 ? (int64_t)dp.total : (path == 4 ? (int64_t)g.c * 28 * elem : 0);
+    return path == 2 ? (int64_t)dp.total : (path == 4 || path == 5 ? (int64_t)g.c * 28 * elem : 0);
 }
 
 extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, const void *x, const void *w, const int32_t *selection,
@@ -645,7 +780,7 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
     const int elem = dtype == CLG_F64 ? 8 : 4;
     const int path = choose_forward(g, elem, 28, scratch != nullptr, &tp, &dp);
     hipStream_t st = clg_stream(stream);
-    if (path == 4) {
+    if (path == 4 || path == 5) {
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
@@ -654,6 +789,11 @@ extern "C" int clg_convblock_forward_ws(int dtype, const clg_conv_geom *gg, cons
             hipLaunchKernelGGL((convblock_w_prepare_kernel<double, double>), pgrid, dim3(256), 0, st, (const double *)w, selection,
                                (double *)scratch, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x);
         CLG_CHECK_LAUNCH("clg_convblock_forward_ws");
+        if (path == 5) {
+            if (dtype == CLG_F32)
+                return launch_forward_kpl<float>(g, tp, x, scratch, selection, y, argmax, nullptr, st, "clg_convblock_forward_ws");
+            return launch_forward_kpl<double>(g, tp, x, scratch, selection, y, argmax, nullptr, st, "clg_convblock_forward_ws");
+        }
         return clg_convblock_forward_4x4(dtype, g, x, scratch, selection, y, argmax, st, "clg_convblock_forward_ws");
     }
     if (path != 2) return clg_convblock_forward(dtype, gg, x, w, selection, y, argmax, stream);
@@ -713,9 +853,9 @@ static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg,
         CLG_CHECK_LAUNCH(name);
         return CLG_OK;
     };
-    if (path == 4) {
+    if (path == 4 || path == 5) {
         g.y_fm = fm ? 1 : 0;
-        void *fold_to = want_folded ? folded_out : scratch;             // the 4x4 kernels read them from wherever they are
+        void *fold_to = want_folded ? folded_out : scratch;             // the kernels read them from wherever they are
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
         if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
@@ -726,6 +866,10 @@ static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg,
                                (double *)fold_to, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<double>(), (int)pgrid.x, logits ? 1 : 0,
                                (double *)probs_out);
         CLG_CHECK_LAUNCH(name);
+        if (path == 5) {
+            if (dtype == CLG_F32) return launch_forward_kpl<float>(g, tp, x, fold_to, selection, y, argmax, padded_out, st, name);
+            return launch_forward_kpl<double>(g, tp, x, fold_to, selection, y, argmax, padded_out, st, name);
+        }
         return clg_convblock_forward_4x4(dtype, g, x, fold_to, selection, y, argmax, st, name);
     }
     if (path == 2) {
@@ -783,7 +927,7 @@ extern "C" int64_t clg_convblock_padded_elems(int dtype, const clg_conv_geom *gg
     DirectPlan dp;
     const int elem = dtype == CLG_F64 ? 8 : 4;
     const int path = choose_forward(g, elem, 28, have_scratch != 0, &tp, &dp);
-    if (path != 0 && path != 2) return 0;
+    if (path != 0 && path != 2 && path != 5) return 0;
     const int64_t se = clg_convblock_backward_padded_sample_elems(dtype, g);
     if (se <= 0) return 0;
     const int64_t mine = path == 2 ? dp.sample_elems : (int64_t)g.cin * tp.chs + g.ph * tp.rs + g.pw;

@@ -609,3 +609,27 @@ def test_padded_copy_left_by_the_forward_gives_the_planned_backward_its_taps(n, 
     xg = x.clone().requires_grad_(True)
     layer(xg).backward(gy)
     assert torch.equal(xg.grad, gx0)
+
+
+@pytest.mark.parametrize("n,cin,h,w,cout,dtype", [(5, 128, 8, 8, 512, torch.float32), (3, 16, 8, 8, 300, torch.float32),
+                                                  (4, 24, 6, 6, 256, torch.float32), (2, 32, 8, 8, 256, torch.float64),
+                                                  (3, 8, 8, 4, 260, torch.float32)])
+def test_forward_with_one_kernel_per_lane_equals_the_position_major_kernel(n, cin, h, w, cout, dtype, monkeypatch):
+    # deep blocks on small images (at least 256 kernels, at most 16 pooled cells): a lane keeps its kernel and walks the
+    # positions; the same gate arithmetic, so y and the pooled positions equal those of the kernel with lanes along
+    # positions bit for bit, and the oracle's to rounding
+    torch.manual_seed(cin + cout)
+    x = torch.rand(n, cin, h, w, device=DEV, dtype=dtype)
+    layer = C.ConvLogicLayer(cin, cout, complete=True, implementation="cuda").to(DEV).to(dtype)
+    w_prob = torch.softmax(layer.weights.detach(), -1)
+    geo = (1, 1, 1, 1, 3, 3)
+    set_knobs(monkeypatch, CLG_FWD_KPL=0)
+    y0, am0 = convlogic_hip.full_convlogic_forward(x, w_prob, layer.selection, *geo)
+    set_knobs(monkeypatch, CLG_FWD_KPL=None)
+    y1, am1 = convlogic_hip.full_convlogic_forward(x, w_prob, layer.selection, *geo)
+    assert torch.equal(y0, y1) and torch.equal(am0, am1)
+    ref = O.conv_block_forward(x.cpu(), w_prob.cpu(), layer.selection.cpu(), (1, 1), (1, 1), (3, 3))
+    assert (y1.cpu() - ref).abs().max().item() <= (1e-5 if dtype == torch.float32 else 1e-12)
+    # from the logits, with the folded coefficients and the padded copy left for the backward pass
+    res = convlogic_hip.full_convlogic_forward_logits(x, layer.weights.detach(), layer.selection, *geo, want_folded=True, want_padded=True)
+    assert (res[0] - y1).abs().max().item() <= (2e-6 if dtype == torch.float32 else 1e-14)
