@@ -450,6 +450,134 @@ __global__ __launch_bounds__(kBlock) void fc_forward_logits_kernel(const T *__re
     }
 }
 
+// The walk of input i over its consumers, shared by the kernels below: returns the input gradient of the lane's VEC
+// samples from s on, sum over the consumers j of gy[j] * d gate_j / d x_i, taken in groups of four with one partial
+// sum per position in the group and added as (0 + 1) + (2 + 3).  Input i is operand A of neuron j unless only B
+// matches; a neuron wired to the same feature twice appears twice in the list and takes the B derivative the second
+// time.  With LPR != 0 (a row of the batch = LPR lanes x VEC samples, xi = the lane's samples of x[i]) the visit that
+// reaches a neuron through its first operand also writes the neuron's 16 gate gradients.
+template <typename T, int VEC, int LPR>
+__device__ __forceinline__ Pack<T, VEC> fc_walk_consumers(const T *__restrict__ x, const int64_t *__restrict__ a,
+                                                          const int64_t *__restrict__ b, const T *__restrict__ folded,
+                                                          const T *__restrict__ gy, const int64_t *__restrict__ csr_list,
+                                                          T *__restrict__ gw, const T *__restrict__ probs, int in_dim, int out_dim,
+                                                          int64_t batch, int64_t i, int64_t beg, int64_t end, int64_t s, bool live,
+                                                          const Pack<T, VEC> &xi, int lane)
+{
+    Pack<T, VEC> part[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
+    // A group of four consumers needs three dependent fetches (list entry -> wiring, coefficients, probabilities -> rows).
+    // They are staggered over the groups: while the rows of group g are fetched and used, the wiring of group g + 1 and
+    // the list entries of group g + 2 are already on their way, so a group waits for ONE fetch, not three.  Every load
+    // is issued unconditionally from a clamped, always valid address and its value discarded afterwards where it does
+    // not count: a load under a per-lane condition makes the compiler wait for ALL outstanding loads at the end of its
+    // branch, which turned the 4 x 3 fetches of a group into twelve round trips in a row.
+    struct Meta {
+        int32_t j[4], io[4];                                         // consumer (-1: none), row of its other operand
+        T c_ab[4], c_lin[4], pr[4];
+        bool first[4];
+    };
+    const int64_t list_last = 2 * (int64_t)out_dim - 1;
+    auto list_entries = [&](int64_t cur, int32_t (&j)[4]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t at = cur + u;
+            const int32_t v = (int32_t)clamp_index(csr_list[at < list_last ? at : list_last], out_dim);
+            j[u] = at < end ? v : -1;
+        }
+    };
+    const int q16 = lane & 15;
+    auto wiring = [&](const int32_t (&j)[4], int32_t prev_j, Meta &m) {
+        int64_t ia[4], ib[4];
+        Coef<T> c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int32_t jj = j[u] < 0 ? 0 : j[u];
+            ia[u] = a[jj];
+            ib[u] = b[jj];
+            c[u] = load_coef(folded + (int64_t)jj * 4);
+            m.pr[u] = T(0);
+        }
+        if (probs != nullptr) {                                      // uniform over the launch
+#pragma unroll
+            for (int u = 0; u < 4; ++u) m.pr[u] = probs[(int64_t)(j[u] < 0 ? 0 : j[u]) * 16 + q16];
+        }
+        int32_t prev = prev_j;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t ja = clamp_index(ia[u], in_dim), jb = clamp_index(ib[u], in_dim);
+            const bool have = j[u] >= 0;
+            const bool as_a = ja == i && !(jb == i && prev == j[u]);
+            m.j[u] = j[u];
+            m.first[u] = have && as_a;
+            m.io[u] = (int32_t)(as_a ? jb : ja);
+            m.c_ab[u] = have ? c[u].ab : T(0);
+            m.c_lin[u] = have ? (as_a ? c[u].a : c[u].b) : T(0);
+            prev = j[u];
+        }
+    };
+    int32_t j_next[4], j_after[4];
+    Meta cur_m, next_m;
+    list_entries(beg, j_next);
+    wiring(j_next, -1, cur_m);
+    list_entries(beg + 4, j_next);
+    const int64_t s_at = live ? s : 0;                               // lanes beyond the batch read the row's start and drop it
+    for (int64_t cur = beg; cur < end; cur += 4) {                   // the lanes of a row group leave the loop together
+        Pack<T, VEC> vo[4], vg[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            vo[u] = load_vec<T, VEC>(x + (int64_t)cur_m.io[u] * batch + s_at);
+            vg[u] = load_vec<T, VEC>(gy + (int64_t)(cur_m.j[u] < 0 ? 0 : cur_m.j[u]) * batch + s_at);
+        }
+        wiring(j_next, cur_m.j[3], next_m);
+        list_entries(cur + 8, j_after);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool use = cur_m.j[u] >= 0 && live;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                vo[u].v[k] = use ? vo[u].v[k] : T(0);
+                vg[u].v[k] = use ? vg[u].v[k] : T(0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (cur_m.j[u] < 0) continue;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(cur_m.c_ab[u], vo[u].v[k], cur_m.c_lin[u]), vg[u].v[k], part[u].v[k]);
+            if constexpr (LPR != 0) if (cur_m.first[u]) {                    // uniform over the row group
+                T sab = 0, sa = 0, sb = 0, s1 = 0;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    sab = fma_t(vg[u].v[k], xi.v[k] * vo[u].v[k], sab);
+                    sa = fma_t(vg[u].v[k], xi.v[k], sa);
+                    sb = fma_t(vg[u].v[k], vo[u].v[k], sb);
+                    s1 += vg[u].v[k];
+                }
+                sab = lane_group_sum<T, LPR>(sab);
+                sa = lane_group_sum<T, LPR>(sa);
+                sb = lane_group_sum<T, LPR>(sb);
+                s1 = lane_group_sum<T, LPR>(s1);
+                if (lane % LPR >= LPR - 16) {
+                    T gi = coef_transpose_row<T>(q16, sab, sa, sb, s1);
+                    if (probs != nullptr) gi = softmax16_backward(gi, cur_m.pr[u]);
+                    gw[(int64_t)cur_m.j[u] * 16 + q16] = gi;
+                }
+            }
+        }
+        cur_m = next_m;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) j_next[u] = j_after[u];
+    }
+    Pack<T, VEC> acc;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
+    return acc;
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
@@ -464,51 +592,15 @@ __global__ __launch_bounds__(kBlock) void fc_backward_x_folded_kernel(
         const int64_t s = (((it % batch_chunks) << lpr_log2) + l) * VEC;
         if (i >= in_dim || s >= batch) continue;
         const int64_t beg = clamp_index(csr_start[i], 2 * (int64_t)out_dim + 1), end = clamp_index(csr_start[i + 1], 2 * (int64_t)out_dim + 1);
-        // Consumers in groups of four with one partial sum per position in the group, so that the rows of four
-        // consumers are in flight together; the partial sums are added as (0 + 1) + (2 + 3).
-        Pack<T, VEC> part[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
-        int64_t prev = -1;
-        for (int64_t cur = beg; cur < end; cur += 4) {
-            int64_t j[4];
-            Pack<T, VEC> vo[4], vg[4];
-            T c_ab[4], c_lin[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                j[u] = cur + u < end ? clamp_index(csr_list[cur + u], out_dim) : -1;
-                if (j[u] >= 0) {
-                    const int64_t ia = clamp_index(a[j[u]], in_dim), ib = clamp_index(b[j[u]], in_dim);
-                    const Coef<T> c = load_coef(folded + j[u] * 4);
-                    // Input i is operand A of neuron j unless only B matches; a neuron wired to the same
-                    // feature twice appears twice in the list and takes the B derivative the second time.
-                    const bool as_a = ia == i && !(ib == i && prev == j[u]);
-                    c_ab[u] = c.ab;
-                    c_lin[u] = as_a ? c.a : c.b;
-                    vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
-                    vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
-                }
-                prev = j[u];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (j[u] >= 0) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
-                }
-            }
-        }
-        Pack<T, VEC> acc;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
+        const Pack<T, VEC> none{};
+        const Pack<T, VEC> acc = fc_walk_consumers<T, VEC, 0>(x, a, b, folded, gy, csr_list, (T *)nullptr, (const T *)nullptr, in_dim, out_dim,
+                                                              batch, i, beg, end, s, true, none, lane);
         store_vec<T, VEC>(gx + i * batch + s, acc);
     }
 }
 
 // Both gradients in one pass for any wiring, as long as one pass of LPR lanes x VEC samples covers the batch: the
-// wavefront that owns input i walks its consumers (as fc_backward_x_folded_kernel) and, on the visit that reaches a
+// wavefront that owns input i walks its consumers (fc_walk_consumers) and, on the visit that reaches a
 // consumer through its FIRST operand -- which happens exactly once per neuron, and has the neuron's gy row, its first
 // operand row (x[i]) and its second operand row in registers -- also forms the four sums of the weight gradient
 // (as fc_backward_w_kernel: same lanes, same order, same reduction) and writes the neuron's 16 gate gradients.
@@ -532,66 +624,7 @@ __device__ __forceinline__ bool fc_backward_fused_item(const T *__restrict__ x, 
 #pragma unroll
     for (int k = 0; k < VEC; ++k) xi.v[k] = 0;
     if (live) xi = load_vec<T, VEC>(x + i * batch + s);
-    Pack<T, VEC> part[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) part[u].v[k] = 0;
-    int64_t prev = -1;
-    for (int64_t cur = beg; cur < end; cur += 4) {                   // the lanes of a row group leave the loop together
-        int64_t j[4];
-        Pack<T, VEC> vo[4], vg[4];
-        T c_ab[4], c_lin[4];
-        bool first[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            j[u] = cur + u < end ? clamp_index(csr_list[cur + u], out_dim) : -1;
-            first[u] = false;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) vo[u].v[k] = vg[u].v[k] = 0;
-            if (j[u] >= 0) {
-                const int64_t ia = clamp_index(a[j[u]], in_dim), ib = clamp_index(b[j[u]], in_dim);
-                const Coef<T> c = load_coef(folded + j[u] * 4);
-                const bool as_a = ia == i && !(ib == i && prev == j[u]);   // see fc_backward_x_folded_kernel
-                first[u] = as_a;
-                c_ab[u] = c.ab;
-                c_lin[u] = as_a ? c.a : c.b;
-                if (live) {
-                    vo[u] = load_vec<T, VEC>(x + (as_a ? ib : ia) * batch + s);
-                    vg[u] = load_vec<T, VEC>(gy + j[u] * batch + s);
-                }
-            }
-            prev = j[u];
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if (j[u] < 0) continue;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) part[u].v[k] = fma_t(fma_t(c_ab[u], vo[u].v[k], c_lin[u]), vg[u].v[k], part[u].v[k]);
-            if (first[u]) {                                          // uniform over the row group
-                T sab = 0, sa = 0, sb = 0, s1 = 0;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    sab = fma_t(vg[u].v[k], xi.v[k] * vo[u].v[k], sab);
-                    sa = fma_t(vg[u].v[k], xi.v[k], sa);
-                    sb = fma_t(vg[u].v[k], vo[u].v[k], sb);
-                    s1 += vg[u].v[k];
-                }
-                sab = lane_group_sum<T, LPR>(sab);
-                sa = lane_group_sum<T, LPR>(sa);
-                sb = lane_group_sum<T, LPR>(sb);
-                s1 = lane_group_sum<T, LPR>(s1);
-                if (l >= LPR - 16) {
-                    const int q = lane & 15;
-                    T gi = coef_transpose_row<T>(q, sab, sa, sb, s1);
-                    if (probs != nullptr) gi = softmax16_backward(gi, probs[j[u] * 16 + q]);
-                    gw[j[u] * 16 + q] = gi;
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) acc.v[k] = (part[0].v[k] + part[1].v[k]) + (part[2].v[k] + part[3].v[k]);
+    acc = fc_walk_consumers<T, VEC, LPR>(x, a, b, folded, gy, csr_list, gw, probs, in_dim, out_dim, batch, i, beg, end, s, live, xi, lane);
     return live;
 }
 
@@ -602,7 +635,7 @@ __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
     T *__restrict__ gx, T *__restrict__ gw, int in_dim, int64_t batch, const T *__restrict__ probs, int out_dim)
 {
     constexpr int ROWS = kWave / LPR;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform(threadIdx.x >> 6);   // with one row per wavefront the whole index walk is scalar
     const int64_t groups = (in_dim + ROWS - 1) / ROWS;
     const int64_t s = (int64_t)(lane % LPR) * VEC;
     for (int64_t it = (int64_t)blockIdx.x * kWavesPerBlock + wave; it < groups; it += (int64_t)gridDim.x * kWavesPerBlock) {
@@ -613,21 +646,23 @@ __global__ __launch_bounds__(kBlock) void fc_backward_fused_kernel(
     }
 }
 
-// The same pass with the input gradient written sample-major, gx [batch, in_dim]: 16 wavefronts of a workgroup own
-// F = 16 * 64/LPR consecutive inputs, park their rows in an LDS tile [F][bp] and the workgroup writes the tile out
+// The same pass with the input gradient written sample-major, gx [batch, in_dim]: the wavefronts of a workgroup own
+// F = waves * 64/LPR consecutive inputs, park their rows in an LDS tile [F][bp] and the workgroup writes the tile out
 // transposed, F consecutive elements per sample.  Same sums in the same order as fc_backward_fused_kernel.
-constexpr int kSmOutWaves = 16;
+// 16 wavefronts when a wavefront owns one input (F = 16), 8 when it owns two or four (F = 16 or 32): the walk of several
+// rows at once needs more than the 128 registers a workgroup of 1024 lanes leaves a lane.
+template <int LPR> constexpr int smout_waves() { return LPR == kWave ? 16 : 8; }
 static inline int64_t smout_row_pitch(int64_t batch) { return ((batch + 31) & ~31ll) + 4; }   // pitch % 32 == 4: the transposed reads spread over the banks
 template <typename T, int VEC, int LPR>
-__global__ __launch_bounds__(kSmOutWaves * kWave) void fc_backward_fused_smout_kernel(
+__global__ __launch_bounds__(smout_waves<LPR>() * kWave) void fc_backward_fused_smout_kernel(
     const T *__restrict__ x, const int64_t *__restrict__ a, const int64_t *__restrict__ b, const T *__restrict__ folded,
     const T *__restrict__ gy, const int64_t *__restrict__ csr_start, const int64_t *__restrict__ csr_list,
     T *__restrict__ gx, T *__restrict__ gw, int in_dim, int batch, int bp, const T *__restrict__ probs, int out_dim)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     T *tile = reinterpret_cast<T *>(smem);
-    constexpr int ROWS = kWave / LPR, F = kSmOutWaves * ROWS;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    constexpr int kSmOutWaves = smout_waves<LPR>(), ROWS = kWave / LPR, F = kSmOutWaves * ROWS;
+    const int lane = threadIdx.x & (kWave - 1), wave = uniform(threadIdx.x >> 6);   // with one row per wavefront the whole index walk is scalar
     const int64_t groups = (in_dim + ROWS - 1) / ROWS;
     const int64_t it = (int64_t)blockIdx.x * kSmOutWaves + wave;
     if (it < groups) {
@@ -1102,7 +1137,7 @@ extern "C" int clg_fc_backward_fused_ex(int dtype, const void *x, const int64_t 
 #define CLG_LAUNCH_BF(T, VEC, LPR)                                                                                           \
     do {                                                                                                                    \
         if (sm_out) {                                                                                                       \
-            constexpr int F = kSmOutWaves * (kWave / LPR);                                                                  \
+            constexpr int kSmOutWaves = smout_waves<LPR>(), F = kSmOutWaves * (kWave / LPR);                                \
             hipLaunchKernelGGL((fc_backward_fused_smout_kernel<T, VEC, LPR>), dim3((unsigned)clg_ceil_div(in_dim, (int64_t)F)), \
                                dim3(kSmOutWaves * kWave), (size_t)F * bp * sizeof(T), st, (const T *)x, a, b, (const T *)folded, \
                                (const T *)grad_y, csr_start, csr_list, (T *)grad_x, (T *)grad_w, (int)in_dim, (int)batch, bp, \

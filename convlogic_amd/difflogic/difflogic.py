@@ -306,10 +306,9 @@ class LogicLayerCudaFunction(torch.autograd.Function):
         return grad_x, None, None, grad_w, None, None, None
 
 
-# One walk for both gradients pays while the layer is small enough for launches and latency to count (C1: 16 -> 12 us,
-# first LogicLayer of the k=32 CIFAR net: 41 -> 37 us); at 1.3 M neurons x 128 samples the two throughput-bound
-# kernels are 4 % faster (1553 vs 1614 us), so large layers keep them.
-_FUSED_BACKWARD_MAX_ELEMS = 1 << 25
+# One walk over the consumer lists gives both gradients whenever a row of the batch fits one pass of a wavefront
+# (backward_fused_fits): C1 16 -> 12 us, first LogicLayer of the k=32 CIFAR net 41 -> 30 us, 131072 -> 1.31 M neurons
+# x 128 samples 1554 -> 1131 us against the input-gradient and weight-gradient kernels run one after the other.
 
 
 class _LogicLayerLogitsFunction(torch.autograd.Function):
@@ -333,7 +332,7 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
     def backward(ctx, grad_y):
         x, a, b, w, folded, start, flat = ctx.saved_tensors
         fused = (not ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]
-                 and grad_y.numel() <= _FUSED_BACKWARD_MAX_ELEMS and difflogic_hip.backward_fused_fits(x))
+                 and difflogic_hip.backward_fused_fits(x))
         if fused and not grad_y.is_contiguous() and grad_y.is_cuda and grad_y.dim() == 2 and grad_y.transpose(0, 1).is_contiguous():
             # the gradient of a [B, out] consumer arrives as a transposed view: its feature-major copy is made by the call
             # that computes both gradients
