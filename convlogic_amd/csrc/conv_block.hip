@@ -487,6 +487,13 @@ __global__ __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 6 : 4))) void con
 // LDS (same shared-halo layout, private to the wavefront, so the kernel has no barriers) and reads the
 // taps from a zero-padded copy of x in global memory, which the L2 serves.  Same walk as the tiled
 // kernel: kernels that read the channel in increasing order, taps in order, read-add-write per tap.
+// What a launch of 8192 owners costs (wall-clock stamps per wavefront at [256,128,8,8] -> 512 and [256,32,16,16] -> 128):
+// 106 scalar registers leave 6 wavefronts per SIMD, so 6144 owners start at once and the last 2048 between 12 and 18 us;
+// a hit takes 1.2-1.8 us of a wavefront's life (about 620 clocks issuing the ten gathers of the hits ahead, 520 waiting,
+// 1240 in the tree and the read-add-write rounds, with five or six wavefronts sharing the SIMD), a list 4 to 16 hits.
+// Measured without gain on that: hit records through LDS instead of the scalar cache, the owner's own channel from an
+// LDS copy (half the gathers), five hits in flight instead of three, register budgets for 7 and 8 wavefronts per SIMD,
+// wavefront priority by list length, longest lists first.
 template <typename T>
 __global__ __launch_bounds__(256) void convblock_backward_x_direct_kernel(const T *__restrict__ gy, const T *__restrict__ xp,
                                                                         const T *__restrict__ folded,

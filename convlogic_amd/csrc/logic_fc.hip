@@ -519,11 +519,11 @@ __device__ __forceinline__ Pack<T, VEC> fc_walk_consumers(const T *__restrict__ 
             prev = j[u];
         }
     };
-    int32_t j_next[4], j_after[4];
+    int32_t j_next[4] = {-1, -1, -1, -1}, j_after[4] = {-1, -1, -1, -1};
     Meta cur_m, next_m;
     list_entries(beg, j_next);
     wiring(j_next, -1, cur_m);
-    list_entries(beg + 4, j_next);
+    if (beg + 4 < end) list_entries(beg + 4, j_next);               // (uniform over the row group, like the loop's tests)
     const int64_t s_at = live ? s : 0;                               // lanes beyond the batch read the row's start and drop it
     for (int64_t cur = beg; cur < end; cur += 4) {                   // the lanes of a row group leave the loop together
         Pack<T, VEC> vo[4], vg[4];
@@ -532,8 +532,10 @@ __device__ __forceinline__ Pack<T, VEC> fc_walk_consumers(const T *__restrict__ 
             vo[u] = load_vec<T, VEC>(x + (int64_t)cur_m.io[u] * batch + s_at);
             vg[u] = load_vec<T, VEC>(gy + (int64_t)(cur_m.j[u] < 0 ? 0 : cur_m.j[u]) * batch + s_at);
         }
-        wiring(j_next, cur_m.j[3], next_m);
-        list_entries(cur + 8, j_after);
+        if (cur + 4 < end) {                                         // a list of up to four consumers fetches nothing ahead
+            wiring(j_next, cur_m.j[3], next_m);
+            if (cur + 8 < end) list_entries(cur + 8, j_after);
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const bool use = cur_m.j[u] >= 0 && live;
