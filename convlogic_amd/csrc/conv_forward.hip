@@ -38,8 +38,11 @@ namespace {
 // SUBSET: stage two planes per kernel of the tile instead of all input channels.
 // ONE_ROW: a lane slot is one conv position instead of a column of two rows (plan.one_row; compile-time so that the
 // two-row loop carries nothing of it); ROWSTEP is then wo if that is 8 or 4 (and all channels are staged), else 0.
+// At most 80 scalar registers: with the 83 the compiler takes by itself a SIMD holds 7 wavefronts, not 8, and the last
+// eighth of a launch of 8192 waits for the first to end (the launch stalled on scalar registers; [256,32,16,16] -> 128:
+// 25.2 -> 23.2 us).
 template <typename Ops, int ROWSTEP, bool SUBSET, bool ONE_ROW>
-__global__ void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
+__global__ __attribute__((amdgpu_num_sgpr(80))) void convblock_forward_tiled_kernel(const typename Ops::Elem *__restrict__ x, const void *__restrict__ params,
                                                const int32_t *__restrict__ sel, typename Ops::Elem *__restrict__ y,
                                                uint8_t *__restrict__ argmax, Geom g, TilePlan p, void *__restrict__ probs_out)
 {
