@@ -523,7 +523,10 @@ __device__ __forceinline__ Pack<T, VEC> fc_walk_consumers(const T *__restrict__ 
     Meta cur_m, next_m;
     list_entries(beg, j_next);
     wiring(j_next, -1, cur_m);
-    if (beg + 4 < end) list_entries(beg + 4, j_next);               // (uniform over the row group, like the loop's tests)
+    // With one row per wavefront the tests below are scalar branches and a list of up to four consumers fetches nothing
+    // ahead; with several rows they would diverge, and fetching ahead regardless is the faster code.
+    constexpr bool kAlwaysAhead = LPR != 0 && LPR != kWave;
+    if (kAlwaysAhead || beg + 4 < end) list_entries(beg + 4, j_next);
     const int64_t s_at = live ? s : 0;                               // lanes beyond the batch read the row's start and drop it
     for (int64_t cur = beg; cur < end; cur += 4) {                   // the lanes of a row group leave the loop together
         Pack<T, VEC> vo[4], vg[4];
@@ -532,9 +535,9 @@ __device__ __forceinline__ Pack<T, VEC> fc_walk_consumers(const T *__restrict__ 
             vo[u] = load_vec<T, VEC>(x + (int64_t)cur_m.io[u] * batch + s_at);
             vg[u] = load_vec<T, VEC>(gy + (int64_t)(cur_m.j[u] < 0 ? 0 : cur_m.j[u]) * batch + s_at);
         }
-        if (cur + 4 < end) {                                         // a list of up to four consumers fetches nothing ahead
+        if (kAlwaysAhead || cur + 4 < end) {
             wiring(j_next, cur_m.j[3], next_m);
-            if (cur + 8 < end) list_entries(cur + 8, j_after);
+            if (kAlwaysAhead || cur + 8 < end) list_entries(cur + 8, j_after);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
