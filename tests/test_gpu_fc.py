@@ -31,7 +31,10 @@ def _oracle_grads(x, logits, idx0, idx1, gy):
     return y.detach(), xl.grad, ll.grad
 
 
-@pytest.mark.parametrize("in_dim,out_dim,batch", [(8, 8, 32), (12, 16, 5), (100, 64, 256), (33, 40, 257), (1, 1, 1)])
+@pytest.mark.parametrize("in_dim,out_dim,batch", [(8, 8, 32), (12, 16, 5), (100, 64, 256), (33, 40, 257), (1, 1, 1),
+                                                  # 20 to 43 consumers per input (several groups of four in flight in the
+                                                  # backward walk) at 16, 32 and 64 lanes per row and beyond one pass
+                                                  (6, 60, 12), (10, 100, 100), (7, 150, 256), (6, 61, 300), (5, 43, 64)])
 def test_fc_module_forward_backward(in_dim, out_dim, batch):
     # the feature-major kernels with transposed copies of x and grad_y (grad_x leaves its kernel sample-major)
     torch.manual_seed(in_dim * 1000 + batch)
@@ -229,7 +232,8 @@ def test_folded_kernels_equal_probability_kernels(in_dim, out_dim, batch, dtype)
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("in_dim,out_dim,batch", [(24, 50, 8), (24, 50, 60), (40, 97, 100), (64, 131, 128), (30, 75, 256),
-                                                  (70, 40, 64), (7, 9, 33), (3, 5, 1), (8000, 8000, 256), (16, 8, 12)])
+                                                  (70, 40, 64), (7, 9, 33), (3, 5, 1), (8000, 8000, 256), (16, 8, 12),
+                                                  (6, 60, 12), (10, 100, 100), (7, 150, 256)])   # lists of 20 to 43 consumers
 def test_fused_backward_equals_the_two_kernels(in_dim, out_dim, batch, dtype):
     # one walk over the consumer lists gives both gradients: bit for bit what the input-gradient kernel and the
     # weight-gradient kernel give separately (w.r.t. the probabilities and w.r.t. the logits), for 16 / 32 / 64 lanes
