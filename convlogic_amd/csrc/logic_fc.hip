@@ -764,6 +764,45 @@ __global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restri
     for (; s < slices; ++s) acc += p[s * step];
     out[b * k + g] = acc * inv_tau;
 }
+// GroupSum in ONE launch for classes of a few thousand rows: a workgroup of 16 wavefronts owns one class and 16
+// samples; a lane keeps sample lane % 16 and takes rows 64 t + 4 wave + lane / 16 (sixteen loads in flight); the four row
+// phases of a wavefront are added through lane shuffles, the 16 wavefronts in LDS, pairwise -- a fixed order.
+constexpr int kGroupSumOnceWaves = 16;
+constexpr int64_t kGroupSumOnceMaxRows = 4096;
+template <typename T>
+__global__ __launch_bounds__(kGroupSumOnceWaves * kWave) void group_sum_once_kernel(const T *__restrict__ x, T *__restrict__ out,
+                                                                                   int64_t class_rows, int64_t batch, int k, T inv_tau)
+{
+    __shared__ T meet[kGroupSumOnceWaves][16];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int g = blockIdx.y;
+    const int64_t b = (int64_t)blockIdx.x * 16 + (lane & 15);
+    const int64_t b_at = b < batch ? b : batch - 1;                   // lanes past the batch read its last sample and drop it
+    const T *base = x + (int64_t)g * class_rows * batch + b_at;
+    const int64_t first = (int64_t)wave * 4 + (lane >> 4), last = class_rows - 1;
+    T acc = 0;
+    for (int64_t r0 = first; r0 < class_rows; r0 += 16 * 64) {
+        T v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int64_t r = r0 + 64 * u;
+            v[u] = base[(r < last ? r : last) * batch];              // every load unconditional, from a row of the class
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc += r0 + 64 * u < class_rows ? v[u] : T(0);
+    }
+    acc += __shfl_down(acc, 32);                                      // row phases 0 + 2 and 1 + 3 ...
+    acc += __shfl_down(acc, 16);                                      // ... then the two pairs: lanes 0..15 hold the wavefront's sums
+    if (lane < 16) meet[wave][lane] = acc;
+    __syncthreads();
+    if (threadIdx.x < 16 && b < batch) {
+        T part[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)                                   // wavefronts 4q .. 4q + 3, then the four quarters
+            part[q] = (meet[4 * q][threadIdx.x] + meet[4 * q + 1][threadIdx.x]) + (meet[4 * q + 2][threadIdx.x] + meet[4 * q + 3][threadIdx.x]);
+        out[b * k + g] = ((part[0] + part[1]) + (part[2] + part[3])) * inv_tau;
+    }
+}
 // grad_x[f][b] = grad_out[b][class of f] * (1 / tau); a workgroup writes 64 feature rows of one 64-sample column chunk
 template <typename T>
 __global__ __launch_bounds__(256) void group_sum_backward_fm_kernel(const T *__restrict__ grad_out, T *__restrict__ grad_x,
@@ -1254,6 +1293,39 @@ extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch,
                              double tau, void *stream)
 {
     return group_sum_impl(dtype, x, out, scratch, -1, features, batch, k, tau, stream, "clg_group_sum");
+}
+
+extern "C" int clg_group_sum_once_fits(int64_t features, int64_t batch, int64_t k)
+{
+    if (features <= 0 || batch <= 0 || k <= 0 || k > 65535 || features % k != 0) return 0;
+    // enough workgroups to be worth a launch of its own kind, and at most 64 rows per lane
+    return features / k <= kGroupSumOnceMaxRows && features / k >= 64 && clg_ceil_div(batch, (int64_t)16) * k >= 32 &&
+                   clg_ceil_div(batch, (int64_t)16) < (1ll << 31)
+               ? 1
+               : 0;
+}
+
+extern "C" int clg_group_sum_once(int dtype, const void *x, void *out, int64_t features, int64_t batch, int64_t k, double tau,
+                                  void *stream)
+{
+    const char *name = "clg_group_sum_once";
+    CLG_REQUIRE(tau != 0.0, "%s: tau must not be zero", name);
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "%s: dtype must be CLG_F32 or CLG_F64, got %d", name, dtype);
+    CLG_REQUIRE(x && out, "%s: null pointer argument", name);
+    CLG_REQUIRE(features > 0 && batch > 0 && k > 0 && k <= 65535, "%s: features, batch and k must be positive, k <= 65535", name);
+    CLG_REQUIRE(features % k == 0, "in_dim (%lld) has to be divisible by k (%lld) but it is not", (long long)features, (long long)k);
+    CLG_REQUIRE(clg_group_sum_once_fits(features, batch, k), "%s: %lld rows per class x %lld samples is not a size for the one-launch "
+                "kernel (clg_group_sum_once_fits); use clg_group_sum", name, (long long)(features / k), (long long)batch);
+    hipStream_t st = clg_stream(stream);
+    const dim3 grid((unsigned)clg_ceil_div(batch, (int64_t)16), (unsigned)k), block(kGroupSumOnceWaves * kWave);
+    if (dtype == CLG_F32)
+        hipLaunchKernelGGL(group_sum_once_kernel<float>, grid, block, 0, st, (const float *)x, (float *)out, features / k, batch, (int)k,
+                           1.0f / (float)tau);
+    else
+        hipLaunchKernelGGL(group_sum_once_kernel<double>, grid, block, 0, st, (const double *)x, (double *)out, features / k, batch, (int)k,
+                           1.0 / tau);
+    CLG_CHECK_LAUNCH(name);
+    return CLG_OK;
 }
 
 // ---- GroupSum for callers that cannot allocate ---------------------------------------------------

@@ -45,6 +45,8 @@ SIGNATURES = {
     "clg_fc_forward_logits_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
     "clg_group_sum_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _f64, _p]),
+    "clg_group_sum_once_fits": (_i, [_i64, _i64, _i64]),
+    "clg_group_sum_once": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_group_sum_static_max_bytes": (_i64, []),
     "clg_group_sum_static_init": (_i, []),
     "clg_group_sum_static": (_i, [_i, _p, _p, _i64, _i64, _i64, _f64, _p]),

@@ -201,9 +201,12 @@ def group_sum(x_fm, k, tau=1.0):
         raise ValueError(f"in_dim ({features}) has to be divisible by k ({k}) but it is not")
     lib = _lib.load()
     dt = dtype_code(x_fm)
+    out = torch.empty((batch, k), dtype=x_fm.dtype, device=x_fm.device)
+    if lib.clg_group_sum_once_fits(features, batch, k):               # one launch, no partial sums
+        check(lib.clg_group_sum_once(dt, x_fm.data_ptr(), out.data_ptr(), features, batch, k, float(tau), stream_ptr(x_fm)))
+        return out
     nbytes = lib.clg_group_sum_scratch_bytes(dt, features, batch, k)
     scratch = torch.empty((max(int(nbytes), 8),), dtype=torch.uint8, device=x_fm.device)
-    out = torch.empty((batch, k), dtype=x_fm.dtype, device=x_fm.device)
     check(lib.clg_group_sum(dt, x_fm.data_ptr(), out.data_ptr(), scratch.data_ptr(), features, batch, k, float(tau), stream_ptr(x_fm)))
     return out
 

@@ -292,6 +292,38 @@ def test_forward_from_logits_folds_inside(in_dim, out_dim, batch, dtype):
         difflogic_hip.forward_logits(x, *tabs, logits[:, :8].contiguous())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("features,batch,k,once", [(10240, 256, 10, True), (640, 256, 10, True), (3200, 37, 50, True), (40960, 130, 10, True),
+                                                   (40, 7, 4, False), (630, 256, 10, False), (640, 16, 10, False), (81920, 64, 10, False)])
+def test_group_sum_in_one_launch(features, batch, k, once, dtype):
+    # classes of 64 to 4096 rows with enough (class, 16 samples) pairs take the kernel without partial sums: same sums as
+    # the sliced kernels up to rounding, exact on 0/1 activations, ragged batches, reproducible; other sizes are refused
+    from convlogic_amd.hip import _lib
+    lib = _lib.load()
+    assert bool(lib.clg_group_sum_once_fits(features, batch, k)) == once
+    torch.manual_seed(features + batch)
+    x = torch.rand(features, batch, device=DEV, dtype=dtype)
+    dt, st = _lib.dtype_code(x), _lib.stream_ptr(x)
+    out = torch.full((batch, k), float("nan"), device=DEV, dtype=dtype)
+    rc = lib.clg_group_sum_once(dt, x.data_ptr(), out.data_ptr(), features, batch, k, 6.5, st)
+    if not once:
+        assert rc != 0 and b"clg_group_sum_once_fits" in lib.clg_last_error()
+        return
+    assert rc == 0
+    ref = x.double().reshape(k, features // k, batch).sum(1).t() / 6.5
+    assert (out.double() - ref).abs().max().item() <= (1e-5 if dtype == torch.float32 else 1e-13) * ref.abs().max().item()
+    scratch = torch.empty(lib.clg_group_sum_scratch_bytes(dt, features, batch, k), dtype=torch.uint8, device=DEV)
+    sliced = torch.empty_like(out)
+    _lib.check(lib.clg_group_sum(dt, x.data_ptr(), sliced.data_ptr(), scratch.data_ptr(), features, batch, k, 6.5, st))
+    assert torch.allclose(out, sliced, rtol=1e-5 if dtype == torch.float32 else 1e-13, atol=0)
+    again = torch.empty_like(out)
+    _lib.check(lib.clg_group_sum_once(dt, x.data_ptr(), again.data_ptr(), features, batch, k, 6.5, st))
+    assert torch.equal(out, again)
+    bits = (x > 0.5).to(dtype)
+    _lib.check(lib.clg_group_sum_once(dt, bits.data_ptr(), out.data_ptr(), features, batch, k, 1.0, st))
+    assert torch.equal(out.cpu(), bits.cpu().reshape(k, features // k, batch).sum(1).t())
+
+
 @pytest.mark.parametrize("features,batch,k", [(40, 7, 4), (640, 256, 10), (65536, 100, 8), (30, 1, 3), (10240, 256, 10)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_group_sum_on_feature_major_view(features, batch, k, dtype):
