@@ -764,38 +764,40 @@ __global__ __launch_bounds__(256) void group_sum_finish_kernel(const T *__restri
     for (; s < slices; ++s) acc += p[s * step];
     out[b * k + g] = acc * inv_tau;
 }
-// GroupSum in ONE launch for classes of a few thousand rows: a workgroup of 16 wavefronts owns one class and 16
-// samples; a lane keeps sample lane % 16 and takes rows 64 t + 4 wave + lane / 16 (sixteen loads in flight); the four row
-// phases of a wavefront are added through lane shuffles, the 16 wavefronts in LDS, pairwise -- a fixed order.
+// GroupSum in ONE launch for classes of a few thousand rows: a workgroup of 16 wavefronts owns one class and 32
+// samples (a 128-byte line of every row); a lane keeps sample lane % 32 and takes rows 32 t + 2 wave + lane / 32 (sixteen
+// loads in flight); the two row phases of a wavefront are added through a lane shuffle, the 16 wavefronts in LDS,
+// pairwise -- a fixed order.
 constexpr int kGroupSumOnceWaves = 16;
+constexpr int kGroupSumOnceSamples = 32;
 constexpr int64_t kGroupSumOnceMaxRows = 4096;
 template <typename T>
 __global__ __launch_bounds__(kGroupSumOnceWaves * kWave) void group_sum_once_kernel(const T *__restrict__ x, T *__restrict__ out,
                                                                                    int64_t class_rows, int64_t batch, int k, T inv_tau)
 {
-    __shared__ T meet[kGroupSumOnceWaves][16];
+    __shared__ T meet[kGroupSumOnceWaves][kGroupSumOnceSamples];
+    constexpr int kStep = 2 * kGroupSumOnceWaves;                     // rows between two loads of a lane
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int g = blockIdx.y;
-    const int64_t b = (int64_t)blockIdx.x * 16 + (lane & 15);
+    const int64_t b = (int64_t)blockIdx.x * kGroupSumOnceSamples + (lane & 31);
     const int64_t b_at = b < batch ? b : batch - 1;                   // lanes past the batch read its last sample and drop it
     const T *base = x + (int64_t)g * class_rows * batch + b_at;
-    const int64_t first = (int64_t)wave * 4 + (lane >> 4), last = class_rows - 1;
+    const int64_t first = (int64_t)wave * 2 + (lane >> 5), last = class_rows - 1;
     T acc = 0;
-    for (int64_t r0 = first; r0 < class_rows; r0 += 16 * 64) {
+    for (int64_t r0 = first; r0 < class_rows; r0 += 16 * kStep) {
         T v[16];
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
-            const int64_t r = r0 + 64 * u;
+            const int64_t r = r0 + kStep * u;
             v[u] = base[(r < last ? r : last) * batch];              // every load unconditional, from a row of the class
         }
 #pragma unroll
-        for (int u = 0; u < 16; ++u) acc += r0 + 64 * u < class_rows ? v[u] : T(0);
+        for (int u = 0; u < 16; ++u) acc += r0 + kStep * u < class_rows ? v[u] : T(0);
     }
-    acc += __shfl_down(acc, 32);                                      // row phases 0 + 2 and 1 + 3 ...
-    acc += __shfl_down(acc, 16);                                      // ... then the two pairs: lanes 0..15 hold the wavefront's sums
-    if (lane < 16) meet[wave][lane] = acc;
+    acc += __shfl_down(acc, 32);                                      // the two row phases: lanes 0..31 hold the wavefront's sums
+    if (lane < 32) meet[wave][lane] = acc;
     __syncthreads();
-    if (threadIdx.x < 16 && b < batch) {
+    if (threadIdx.x < kGroupSumOnceSamples && b < batch) {
         T part[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q)                                   // wavefronts 4q .. 4q + 3, then the four quarters
@@ -1298,9 +1300,9 @@ extern "C" int clg_group_sum(int dtype, const void *x, void *out, void *scratch,
 extern "C" int clg_group_sum_once_fits(int64_t features, int64_t batch, int64_t k)
 {
     if (features <= 0 || batch <= 0 || k <= 0 || k > 65535 || features % k != 0) return 0;
-    // enough workgroups to be worth a launch of its own kind, and at most 64 rows per lane
-    return features / k <= kGroupSumOnceMaxRows && features / k >= 64 && clg_ceil_div(batch, (int64_t)16) * k >= 32 &&
-                   clg_ceil_div(batch, (int64_t)16) < (1ll << 31)
+    // enough workgroups to be worth a launch of its own kind, and at most 128 rows per lane
+    return features / k <= kGroupSumOnceMaxRows && features / k >= 64 && clg_ceil_div(batch, (int64_t)kGroupSumOnceSamples) * k >= 32 &&
+                   clg_ceil_div(batch, (int64_t)kGroupSumOnceSamples) < (1ll << 31)
                ? 1
                : 0;
 }
@@ -1317,7 +1319,7 @@ extern "C" int clg_group_sum_once(int dtype, const void *x, void *out, int64_t f
     CLG_REQUIRE(clg_group_sum_once_fits(features, batch, k), "%s: %lld rows per class x %lld samples is not a size for the one-launch "
                 "kernel (clg_group_sum_once_fits); use clg_group_sum", name, (long long)(features / k), (long long)batch);
     hipStream_t st = clg_stream(stream);
-    const dim3 grid((unsigned)clg_ceil_div(batch, (int64_t)16), (unsigned)k), block(kGroupSumOnceWaves * kWave);
+    const dim3 grid((unsigned)clg_ceil_div(batch, (int64_t)kGroupSumOnceSamples), (unsigned)k), block(kGroupSumOnceWaves * kWave);
     if (dtype == CLG_F32)
         hipLaunchKernelGGL(group_sum_once_kernel<float>, grid, block, 0, st, (const float *)x, (float *)out, features / k, batch, (int)k,
                            1.0f / (float)tau);

@@ -170,9 +170,9 @@ int clg_fc_forward_logits_ex(int dtype, const void *x, const int64_t *a, const i
 int64_t clg_group_sum_scratch_bytes(int dtype, int64_t features, int64_t batch, int64_t k);
 int clg_group_sum(int dtype, const void *x, void *out /*[batch,k]*/, void *scratch, int64_t features, int64_t batch,
                   int64_t k, double tau, void *stream);
-/* The same sums in ONE launch and without scratch, for classes of 64 to 4096 rows with enough (class, 16 samples) pairs
+/* The same sums in ONE launch and without scratch, for classes of 64 to 4096 rows with enough (class, 32 samples) pairs
  * to fill the GPU (clg_group_sum_once_fits() != 0; the last layer of the reference's CIFAR and MNIST models at training
- * batch sizes): a workgroup owns a class and 16 samples.  Fixed summation order, which is not that of clg_group_sum (the
+ * batch sizes): a workgroup owns a class and 32 samples.  Fixed summation order, which is not that of clg_group_sum (the
  * values agree to rounding, not bit for bit).  Other sizes: CLG_EINVAL. */
 int clg_group_sum_once_fits(int64_t features, int64_t batch, int64_t k);
 int clg_group_sum_once(int dtype, const void *x /*[features,batch]*/, void *out /*[batch,k]*/, int64_t features, int64_t batch,
