@@ -77,7 +77,9 @@ class _FullConvLogicLogitsFunction(Function):
     (same values as softmax + FullConvLogicFunction up to rounding)."""
 
     @staticmethod
-    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False, plan=None):
+    def forward(ctx, x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False, plan=None,
+                prefolded=None):
+        # prefolded: (probs, folded) of these logits, made by the network for all its layers in one launch (fold_many)
         x1, selection, logits = x.contiguous(), selection.contiguous(), logits.contiguous()
         geo = (stride_h, stride_w, pad_h, pad_w)
         ctx.geometry, ctx.kernel = geo, (kernel_h, kernel_w)
@@ -92,7 +94,7 @@ class _FullConvLogicLogitsFunction(Function):
             # needs a gradient and the kernels of this shape read one -- the zero-padded copy of x it staged
             y, argmax, w_prob, folded, *rest = convlogic_hip.full_convlogic_forward_logits(
                 x1, logits.detach(), selection, *geo, kernel_h, kernel_w, feature_major=fm, want_folded=True, validate=False,
-                want_padded=ctx.needs_input_grad[0])
+                want_padded=ctx.needs_input_grad[0], prefolded=prefolded)
             padded = rest[0] if rest else None
             ctx.save_for_backward(x1, w_prob, selection, argmax, folded, *(() if padded is None else (padded,)))
             return y.permute(3, 0, 1, 2) if fm else y
@@ -116,9 +118,9 @@ class _FullConvLogicLogitsFunction(Function):
                                                                                argmax, selection, *ctx.plan, *ctx.geometry, need_grad_x=need_x,
                                                                                validate=not ok, feature_major=use_fm,
                                                                                padded=None if use_fm else padded)
-                return grad_x, grad_l, None, None, None, None, None, None, None, None, None
+                return grad_x, grad_l, None, None, None, None, None, None, None, None, None, None
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y.contiguous(), x1, w_prob, argmax, selection, *ctx.geometry) if need_x else None
-            return grad_x, None, None, None, None, None, None, None, None, None, None
+            return grad_x, None, None, None, None, None, None, None, None, None, None, None
         x1, w_prob, selection, argmax = ctx.saved_tensors
         grad_x = grad_l = None
         grad_fm = grad_y.permute(1, 2, 3, 0)
@@ -126,14 +128,14 @@ class _FullConvLogicLogitsFunction(Function):
                 and convlogic_hip.feature_major_supported(x1, w_prob.shape[0], *ctx.geometry, *ctx.kernel)):
             grad_x, grad_l = convlogic_hip.full_convlogic_backward_fm(grad_fm, x1, w_prob, argmax, selection, *ctx.geometry,
                                                                      need_grad_x=need_x, validate=grad_y.dtype != x1.dtype or grad_y.device != x1.device)
-            return grad_x, grad_l, None, None, None, None, None, None, None, None, None
+            return grad_x, grad_l, None, None, None, None, None, None, None, None, None, None
         grad_y = grad_y.contiguous()
         if need_w:
             grad_x, grad_l = convlogic_hip.full_convlogic_backward_logits(grad_y, x1, w_prob, argmax, selection, *ctx.geometry,
                                                                          need_grad_x=need_x)
         elif need_x:
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y, x1, w_prob, argmax, selection, *ctx.geometry)
-        return grad_x, grad_l, None, None, None, None, None, None, None, None, None
+        return grad_x, grad_l, None, None, None, None, None, None, None, None, None, None
 
 
 class _FullConvLogicBinaryFunction(Function):
@@ -240,6 +242,27 @@ class ConvLogicLayer(nn.Module):
             plan = plans[key] = convlogic_hip.make_backward_plan(x, self.out_channels, sel, *self.stride, *self.padding, *self.kernel)
         return plan
 
+    def prefold_candidate(self):
+        """The logits a network may fold for this layer ahead of its forward call (one launch for all its layers,
+        difflogic_hip.fold_many), or None when the layer's training path does not take the result."""
+        w = self._parameters["weights"]
+        if (self.implementation == "cuda" and self.complete and self.training and not self.return_intermediate
+                and not self.return_indices and not self.__dict__.get("binary_input", False) and w.is_cuda and w.is_contiguous()
+                and w.dtype in (torch.float32, torch.float64)):
+            return w
+        return None
+
+    def set_prefold(self, probs, folded):
+        w = self._parameters["weights"]
+        self.__dict__["_prefold"] = (w._version, w.data_ptr(), probs, folded)
+
+    def _take_prefold(self, weights):
+        """The pair left by set_prefold() if it was made from the weights as they are now (it is used once)."""
+        pf = self.__dict__.pop("_prefold", None)
+        if pf is not None and pf[0] == weights._version and pf[1] == weights.data_ptr() and pf[2].dtype == weights.dtype:
+            return pf[2], pf[3]
+        return None
+
     def _load_from_state_dict(self, *args, **kwargs):
         super()._load_from_state_dict(*args, **kwargs)
         self.invalidate()
@@ -310,8 +333,9 @@ class ConvLogicLayer(nn.Module):
         if (self.complete and self.training and not self.return_intermediate and not self.return_indices and x.is_cuda
                 and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64) and weights.is_contiguous()
                 and weights.device == x.device and sel.device == x.device):
-            return _FullConvLogicLogitsFunction.apply(x, weights, sel, *geo, self.__dict__.get("feature_major_output", False),
-                                                      self._backward_plan(x, sel))
+            plan = self._backward_plan(x, sel)
+            return _FullConvLogicLogitsFunction.apply(x, weights, sel, *geo, self.__dict__.get("feature_major_output", False), plan,
+                                                      self._take_prefold(weights) if plan is not None else None)
         # the kernels read the probabilities in x's element type (the bindings reject any other)
         w_prob = gate_probabilities(self.weights, self.training, x.dtype).to(x.dtype).contiguous()
         if self.complete:

@@ -3,10 +3,42 @@ the logic-layer kernels.  Constructor arguments, layer order and the `network` a
 reference's, so parameters are drawn in the same RNG order and state_dict keys (`network.<i>.weights`,
 `network.<i>.selection`, `network.<i>.indices_0`, ...) match checkpoints written from there (the
 Lightning wrapper of src/convlogic/model.py:111-200 prefixes them with `model.`)."""
+import weakref
+
+import torch
 from torch import nn
 
 from ..difflogic import GroupSum, LogicLayer
 from .convlogic_layer import ConvLogicLayer
+
+
+# per network: (dtype, device), the layers that take a fold made ahead, and the bookkeeping of that launch (kept outside the
+# module so that copies and pickles of a network carry no host pointers)
+_FOLD_PLANS = weakref.WeakKeyDictionary()
+
+
+def _prefold(owner, network, x):
+    """Folds the logits of all layers of a training step in ONE launch and leaves each layer its (probabilities,
+    coefficients): softmax and fold are then no part of the layers' forward launches -- the LogicLayers run their plain
+    streaming kernel, the deep blocks skip their set-up launch.  Same values as the per-layer folds (tested)."""
+    from ..hip import difflogic_hip
+    cache = _FOLD_PLANS.get(owner)
+    if cache is not None and cache[0] == (x.dtype, x.device):
+        _, picked, plan = cache
+        weights = [m._parameters["weights"] for m in picked]
+        if not (plan.matches(weights) and all(m.prefold_candidate() is w for m, w in zip(picked, weights))):
+            cache = None
+    if cache is None:
+        layers = [m for m in network if isinstance(m, (ConvLogicLayer, LogicLayer))]
+        picked = [m for m in layers for w in [m.prefold_candidate()] if w is not None and w.dtype == x.dtype and w.device == x.device]
+        picked = picked[:difflogic_hip.FOLD_MANY_MAX]
+        weights = [m._parameters["weights"] for m in picked]
+        plan = difflogic_hip.FoldPlan([w.detach() for w in weights]) if len(picked) >= 2 else None
+        _FOLD_PLANS[owner] = ((x.dtype, x.device), picked, plan)
+    if plan is None:
+        return
+    for m, (probs, folded) in zip(picked, difflogic_hip.fold_many([w.detach() for w in weights], plan)):
+        m.set_prefold(probs, folded)
 
 
 def _block(c_in, c_out, implementation, **kw):
@@ -43,6 +75,8 @@ class ConvLogicCifarModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
 
     def forward(self, x):
+        if self.training and x.is_cuda and torch.is_grad_enabled() and self.__dict__.get("prefold", True):
+            _prefold(self, self.network, x)
         return self.network(x)
 
 
@@ -61,4 +95,6 @@ class ConvLogicMnistModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head([81 * k, 1280 * k, 640 * k, 320 * k], tau, implementation))
 
     def forward(self, x):
+        if self.training and x.is_cuda and torch.is_grad_enabled() and self.__dict__.get("prefold", True):
+            _prefold(self, self.network, x)
         return self.network(x)

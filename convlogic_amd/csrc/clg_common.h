@@ -91,7 +91,12 @@ __device__ __forceinline__ void softmax16(const T *__restrict__ logits, T (&p)[1
     }
     const T inv = T(1) / sum;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) p[i] *= inv;
+    for (int i = 0; i < 16; ++i) {
+        p[i] *= inv;
+        // the probability as it is stored: a fold of p in the same kernel must not contract this product into its sums, or
+        // its coefficients would differ in the last bit from kernel to kernel and from a fold of the stored values
+        asm volatile("" : "+v"(p[i]));
+    }
 }
 
 template <typename T>

@@ -828,9 +828,14 @@ static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg,
     Geom g;
     if (int e = clg_convblock_check(gg, &g, dtype, name)) return e;
     CLG_REQUIRE(x && w && selection && y && argmax, "%s: null pointer argument", name);
-    CLG_REQUIRE((flags & ~(CLG_FWD_W_LOGITS | CLG_FWD_Y_FEATURE_MAJOR | CLG_FWD_FOLDED_OUT)) == 0, "%s: unknown flags 0x%x", name, flags);
-    const bool logits = (flags & CLG_FWD_W_LOGITS) != 0, fm = (flags & CLG_FWD_Y_FEATURE_MAJOR) != 0;
-    const bool want_folded = (flags & CLG_FWD_FOLDED_OUT) != 0;
+    CLG_REQUIRE((flags & ~(CLG_FWD_W_LOGITS | CLG_FWD_Y_FEATURE_MAJOR | CLG_FWD_FOLDED_OUT | CLG_FWD_FOLDED_IN)) == 0, "%s: unknown flags 0x%x",
+                name, flags);
+    const bool given = (flags & CLG_FWD_FOLDED_IN) != 0;                // probabilities and coefficients are in probs_out already
+    CLG_REQUIRE(!given || ((flags & CLG_FWD_W_LOGITS) && (flags & CLG_FWD_FOLDED_OUT)), "%s: CLG_FWD_FOLDED_IN goes with CLG_FWD_W_LOGITS | "
+                "CLG_FWD_FOLDED_OUT (it says that their outputs are there already)", name);
+    bool logits = (flags & CLG_FWD_W_LOGITS) != 0;
+    const bool fm = (flags & CLG_FWD_Y_FEATURE_MAJOR) != 0;
+    bool want_folded = (flags & CLG_FWD_FOLDED_OUT) != 0;
     CLG_REQUIRE(!logits || probs_out, "%s: CLG_FWD_W_LOGITS needs probs_out [c_out, 7, 16]", name);
     CLG_REQUIRE(!want_folded || probs_out, "%s: CLG_FWD_FOLDED_OUT needs probs_out with room for [c_out, 7, 16] + [c_out, 7, 4]", name);
     CLG_REQUIRE(!fm || (scratch && clg_convblock_fm_supported(dtype, gg)), "%s: CLG_FWD_Y_FEATURE_MAJOR needs scratch and a shape for "
@@ -860,7 +865,9 @@ static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg,
         g.y_fm = fm ? 1 : 0;
         void *fold_to = want_folded ? folded_out : scratch;             // the kernels read them from wherever they are
         const dim3 pgrid((unsigned)clg_ceil_div((int64_t)g.c * 7, 256));
-        if (dtype == CLG_F32)
+        if (given) {
+            // folded by the caller (clg_fold_many): no set-up launch
+        } else if (dtype == CLG_F32)
             hipLaunchKernelGGL((convblock_w_prepare_kernel<float, float>), pgrid, dim3(256), 0, st, (const float *)w, selection,
                                (float *)fold_to, (int32_t *)nullptr, g.c, 0, 0, host_tap_limit(g), no_pad_job<float>(), (int)pgrid.x, logits ? 1 : 0,
                                (float *)probs_out);
@@ -874,6 +881,11 @@ static int forward_ex_impl(const char *name, int dtype, const clg_conv_geom *gg,
             return launch_forward_kpl<double>(g, tp, x, fold_to, selection, y, argmax, padded_out, st, name);
         }
         return clg_convblock_forward_4x4(dtype, g, x, fold_to, selection, y, argmax, st, name);
+    }
+    if (given) {                                                     // the other kernels take the probabilities as their weights
+        w = probs_out;
+        logits = false;
+        want_folded = false;                                         // (the coefficients are there: nothing to fold afterwards)
     }
     if (path == 2) {
         if (dtype == CLG_F32)

@@ -338,21 +338,11 @@ __global__ __launch_bounds__(256) void fc_fold_kernel(const T *__restrict__ w_in
     const int j = blockIdx.x * 256 + threadIdx.x;
     if (j >= out_dim) return;
     T p[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) p[i] = w_in[(int64_t)j * 16 + i];
     if (from_logits) {
-        T m = p[0];
+        softmax16(w_in + (int64_t)j * 16, p);
+    } else {
 #pragma unroll
-        for (int i = 1; i < 16; ++i) m = p[i] > m ? p[i] : m;
-        T sum = 0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            p[i] = exp(p[i] - m);
-            sum += p[i];
-        }
-        const T inv = T(1) / sum;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) p[i] *= inv;
+        for (int i = 0; i < 16; ++i) p[i] = w_in[(int64_t)j * 16 + i];
     }
     if (probs != nullptr) {
 #pragma unroll
@@ -1012,6 +1002,58 @@ extern "C" int clg_fc_fold(int dtype, int from_logits, const void *w_in, void *p
         hipLaunchKernelGGL(fc_fold_kernel<double>, grid, block, 0, st, (const double *)w_in, (double *)probs,
                            (double *)folded, (int)out_dim, from_logits);
     CLG_CHECK_LAUNCH("clg_fc_fold");
+    return CLG_OK;
+}
+
+// softmax + fold of the logits of up to kFoldManyMax tensors [rows_i, 16] in one launch (a network's layers at the
+// start of a training step): the arithmetic of fc_fold_kernel and of the set-up launch of the fused block, row by row.
+constexpr int kFoldManyMax = 16;
+struct FoldMany {
+    const void *logits[kFoldManyMax];
+    void *probs[kFoldManyMax], *folded[kFoldManyMax];
+    int64_t start[kFoldManyMax + 1];                                  // first row of tensor i in the launch's row numbering
+    int n;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void fold_many_kernel(FoldMany m)
+{
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= m.start[m.n]) return;
+    int t = 0;
+    while (q >= m.start[t + 1]) ++t;
+    const int64_t r = q - m.start[t];
+    T p[16];
+    softmax16(reinterpret_cast<const T *>(m.logits[t]) + r * 16, p);
+    T *pr = reinterpret_cast<T *>(m.probs[t]) + r * 16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pr[i] = p[i];
+    const Coef<T> c = fold16(p);
+    T *f = reinterpret_cast<T *>(m.folded[t]) + r * 4;
+    f[0] = c.ab;
+    f[1] = c.a;
+    f[2] = c.b;
+    f[3] = c.one;
+}
+
+extern "C" int clg_fold_many(int dtype, int n, const void *const *logits, void *const *probs, void *const *folded, const int64_t *rows,
+                             void *stream)
+{
+    CLG_REQUIRE(dtype == CLG_F32 || dtype == CLG_F64, "clg_fold_many: dtype must be CLG_F32 or CLG_F64, got %d", dtype);
+    CLG_REQUIRE(n >= 1 && n <= kFoldManyMax, "clg_fold_many: 1 to %d tensors per call, got %d", kFoldManyMax, n);
+    CLG_REQUIRE(logits && probs && folded && rows, "clg_fold_many: null pointer argument");
+    FoldMany m = {};
+    m.n = n;
+    for (int i = 0; i < n; ++i) {
+        CLG_REQUIRE(logits[i] && probs[i] && folded[i] && rows[i] > 0, "clg_fold_many: tensor %d: null pointer or no rows", i);
+        m.logits[i] = logits[i], m.probs[i] = probs[i], m.folded[i] = folded[i];
+        m.start[i + 1] = m.start[i] + rows[i];
+    }
+    CLG_REQUIRE(m.start[n] < (1ll << 31) * 256, "clg_fold_many: too many rows for one launch");
+    const dim3 grid((unsigned)clg_ceil_div(m.start[n], (int64_t)256)), block(256);
+    hipStream_t st = clg_stream(stream);
+    if (dtype == CLG_F32) hipLaunchKernelGGL(fold_many_kernel<float>, grid, block, 0, st, m);
+    else hipLaunchKernelGGL(fold_many_kernel<double>, grid, block, 0, st, m);
+    CLG_CHECK_LAUNCH("clg_fold_many");
     return CLG_OK;
 }
 

@@ -100,10 +100,12 @@ class LogicLayer(torch.nn.Module):
                 and weights.is_contiguous() and weights.device == x.device):
             # a sample-major batch is transposed inside the Function (and its gradient on the way back): one autograd
             # node per layer instead of two
-            inside = _transposes_with_kernel(x)
+            prefolded = self._take_prefold(weights)
+            inside = prefolded is None and _transposes_with_kernel(x)
             return _LogicLayerLogitsFunction.apply(x if inside else _feature_major(x), buffers["indices_0"], buffers["indices_1"],
                                                    weights, buffers["given_x_indices_of_y_start"],
-                                                   buffers["given_x_indices_of_y"], self._sole_consumers(key), inside).transpose(0, 1)
+                                                   buffers["given_x_indices_of_y"], self._sole_consumers(key), inside,
+                                                   prefolded).transpose(0, 1)
         xt = _feature_major(x)
         w = self._gate_weights(xt.dtype)
         args = (xt, self.indices_0, self.indices_1, w, self.given_x_indices_of_y_start, self.given_x_indices_of_y)
@@ -111,6 +113,26 @@ class LogicLayer(torch.nn.Module):
             return LogicLayerCudaFunction.apply(*args).transpose(0, 1)
         with torch.no_grad():
             return LogicLayerCudaFunction.apply(*args).transpose(0, 1)
+
+    def prefold_candidate(self):
+        """The logits a network may fold for this layer ahead of its forward call (one launch for all its layers,
+        difflogic_hip.fold_many), or None when the layer's training path does not take the result."""
+        w = self._parameters["weights"]
+        if (self.implementation == "cuda" and self.training and w.is_cuda and w.is_contiguous()
+                and w.dtype in (torch.float32, torch.float64)):
+            return w
+        return None
+
+    def set_prefold(self, probs, folded):
+        w = self._parameters["weights"]
+        self.__dict__["_prefold"] = (w._version, w.data_ptr(), probs, folded)
+
+    def _take_prefold(self, weights):
+        """The pair left by set_prefold() if it was made from the weights as they are now (it is used once)."""
+        pf = self.__dict__.pop("_prefold", None)
+        if pf is not None and pf[0] == weights._version and pf[1] == weights.data_ptr() and pf[2].dtype == weights.dtype:
+            return pf[2], pf[3]
+        return None
 
     def forward_cuda_eval(self, x: PackBitsTensor):
         """Replaces x.t by the layer output (src/difflogic/difflogic.py:149-164)."""
@@ -318,8 +340,11 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, a, b, logits, given_x_indices_of_y_start, given_x_indices_of_y, sole_consumers=False,
-                sample_major_input=False):
-        if sample_major_input:                                       # x is [B, in]: its gradient goes back in that layout
+                sample_major_input=False, prefolded=None):
+        if prefolded is not None:                                    # (probs, folded) of these logits, made by the network for all
+            w, folded = prefolded                                    # its layers in one launch: the forward is the plain streaming kernel
+            y = difflogic_hip.forward_folded(x, a, b, folded)
+        elif sample_major_input:                                     # x is [B, in]: its gradient goes back in that layout
             y, w, folded, x = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False, sample_major_x=True)
         else:
             y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False)   # the module has checked its buffers
@@ -339,7 +364,7 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
             gy_sm = grad_y.transpose(0, 1)
             grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, gy_sm, start, flat, validate=_needs_check(gy_sm, x),
                                                           sample_major_grad_x=ctx.sample_major_input, sample_major_grad_y=True)
-            return grad_x, None, None, grad_l, None, None, None, None
+            return grad_x, None, None, grad_l, None, None, None, None, None
         grad_y = grad_y if grad_y.is_contiguous() else _contiguous_2d(grad_y)
         grad_x = grad_l = None
         if ctx.sole_consumers and ctx.needs_input_grad[0] and ctx.needs_input_grad[3]:
@@ -348,7 +373,7 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
             # (a sample-major input takes its gradient sample-major straight from the kernel)
             grad_x, grad_l = difflogic_hip.backward_fused(x, a, b, folded, w, grad_y, start, flat, validate=_needs_check(grad_y, x),
                                                           sample_major_grad_x=ctx.sample_major_input)
-            return grad_x, None, None, grad_l, None, None, None, None
+            return grad_x, None, None, grad_l, None, None, None, None, None
         else:
             if ctx.needs_input_grad[0]:
                 grad_x = difflogic_hip.backward_x_folded(x, a, b, folded, grad_y, start, flat, validate=_needs_check(grad_y, x))
@@ -356,7 +381,7 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
                 grad_l = difflogic_hip.backward_logits(x, a, b, w, grad_y, validate=_needs_check(grad_y, x))
         if ctx.sample_major_input and grad_x is not None:
             grad_x = difflogic_hip.transpose(grad_x)
-        return grad_x, None, None, grad_l, None, None, None, None
+        return grad_x, None, None, grad_l, None, None, None, None, None
 
 
 def _needs_check(grad_y, x):

@@ -43,6 +43,7 @@ SIGNATURES = {
     "clg_fc_backward_fused": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_fused_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
     "clg_fc_forward_logits_ex": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i, _p, _p]),
+    "clg_fold_many": (_i, [_i, _i, _p, _p, _p, _p, _p]),
     "clg_group_sum_scratch_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "clg_group_sum": (_i, [_i, _p, _p, _p, _i64, _i64, _i64, _f64, _p]),
     "clg_group_sum_once_fits": (_i, [_i64, _i64, _i64]),

@@ -313,13 +313,15 @@ def full_convlogic_forward_fm(x, weight, selection, stride_h, stride_w, pad_h, p
 
 
 def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w, feature_major=False,
-                                  want_folded=False, validate=True, want_padded=False):
+                                  want_folded=False, validate=True, want_padded=False, prefolded=None):
     """full_convlogic_forward() from the LOGITS [C, 7, 16]: the softmax is taken inside the launch that sets the gate
     parameters up.  -> (y, argmax, probs); with feature_major (where feature_major_supported) y is laid out
     [C, Ho/2, Wo/2, N] as from full_convlogic_forward_fm().  want_folded: -> (y, argmax, probs, folded [C, 7, 4]), the
     folded coefficients of every gate for full_convlogic_backward_planned().  want_padded (with want_folded): a fifth
     result, the zero-padded copy of x that the forward kernels stage anyway and the planned backward pass would otherwise
-    make in a launch of its own -- or None where the pair of kernels at this shape has no use for one."""
+    make in a launch of its own -- or None where the pair of kernels at this shape has no use for one.  prefolded (with
+    want_folded): the (probs, folded) pair that difflogic_hip.fold_many() made from these logits -- the call then launches
+    no softmax or fold of its own and returns that pair."""
     if validate:
         _conv_args(x, logits, selection, 7)
     g = _geom(x, logits.shape[0], stride_h, stride_w, pad_h, pad_w, kernel_h, kernel_w)
@@ -328,14 +330,21 @@ def full_convlogic_forward_logits(x, logits, selection, stride_h, stride_w, pad_
     y = torch.empty((g.c_out, shape[2], shape[3], g.n) if feature_major else shape, dtype=x.dtype, device=x.device)
     argmax = torch.empty(shape, dtype=torch.uint8, device=x.device)
     c = logits.shape[0]
-    if want_folded:                                                  # one buffer: probabilities, then the folded coefficients
+    if prefolded is not None and want_folded:
+        probs, folded = prefolded
+        if validate:
+            check_input(probs, "prefolded probabilities", x.dtype, (c, 7, 16))
+            check_input(folded, "prefolded coefficients", x.dtype, (c, 7, 4))
+        if folded.data_ptr() != probs.data_ptr() + probs.numel() * probs.element_size():
+            raise RuntimeError("prefolded: the folded coefficients must follow the probabilities in one buffer (fold_many)")
+    elif want_folded:                                                # one buffer: probabilities, then the folded coefficients
         both = torch.empty((c * (112 + 28),), dtype=logits.dtype, device=logits.device)
         probs, folded = both[:c * 112].view(c, 7, 16), both[c * 112:].view(c, 7, 4)
     else:
         probs, folded = torch.empty_like(logits), None
     lib = _lib.load()
     scratch = _scratch(lib.clg_convblock_forward_scratch_bytes(dtype_code(x), ctypes.byref(g)), x.device)
-    flags = 1 | (2 if feature_major else 0) | (4 if want_folded else 0)
+    flags = 1 | (2 if feature_major else 0) | (4 if want_folded else 0) | (8 if prefolded is not None and want_folded else 0)
     padded = None
     if want_padded and want_folded and not feature_major:
         elems = lib.clg_convblock_padded_elems(dtype_code(x), ctypes.byref(g), 1 if scratch is not None else 0)

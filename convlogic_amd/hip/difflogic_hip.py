@@ -77,6 +77,58 @@ def fold(w_in, from_logits, want_probs=True):
     return probs, folded
 
 
+FOLD_MANY_MAX = 16
+
+
+class FoldPlan:
+    """What fold_many() needs of a fixed list of logit tensors besides a fresh output buffer: row counts, chunk sizes
+    and shapes, and the host arrays of the call (kept by a network across its training steps)."""
+
+    def __init__(self, logits_list):
+        import ctypes
+        n = len(logits_list)
+        if not 1 <= n <= FOLD_MANY_MAX:
+            raise RuntimeError(f"fold_many takes 1 to {FOLD_MANY_MAX} tensors, got {n}")
+        first = logits_list[0]
+        for t in logits_list:
+            check_input(t, "logits", first.dtype)
+            if t.device != first.device or t.dim() < 2 or t.shape[-1] != 16:
+                raise RuntimeError("fold_many: logits must share a device and have 16 entries per row")
+        self.n, self.dtype, self.device, self.code = n, first.dtype, first.device, dtype_code(first)
+        self.rows = [t.numel() // 16 for t in logits_list]
+        self.sizes = [s for r in self.rows for s in (16 * r, 4 * r)]
+        self.shapes = [s for t in logits_list for s in (tuple(t.shape), (*t.shape[:-1], 4))]
+        self.total = 20 * sum(self.rows)
+        self.ptrs = tuple(t.data_ptr() for t in logits_list)
+        self.logits_arr = (ctypes.c_void_p * n)(*self.ptrs)
+        self.rows_arr = (ctypes.c_int64 * n)(*self.rows)
+        self.out_arr = ctypes.c_void_p * n
+        self.elem = first.element_size()
+
+    def matches(self, logits_list):
+        return len(logits_list) == self.n and all(t.data_ptr() == p and t.dtype == self.dtype for t, p in zip(logits_list, self.ptrs))
+
+
+def fold_many(logits_list, plan=None):
+    """softmax + fold of up to 16 logit tensors [..., 16] of one dtype and device in ONE launch -> a list of
+    (probs, folded) with probs shaped like the logits and folded [..., 4]; each pair lives in one buffer, probabilities
+    first (the layout full_convlogic_forward_logits(prefolded=...) and the block's backward expect).  Row by row the
+    values of fold(from_logits=True).  plan: a FoldPlan made from the same tensors (saves the per-call bookkeeping)."""
+    if plan is None or not plan.matches(logits_list):
+        plan = FoldPlan(logits_list)
+    buf = torch.empty((plan.total,), dtype=plan.dtype, device=plan.device)
+    chunks = buf.split_with_sizes(plan.sizes)
+    views = [c.view(s) for c, s in zip(chunks, plan.shapes)]
+    base, at, pp, fp = buf.data_ptr(), 0, [], []
+    for r in plan.rows:
+        pp.append(base + at * plan.elem)
+        fp.append(base + (at + 16 * r) * plan.elem)
+        at += 20 * r
+    check(_lib.load().clg_fold_many(plan.code, plan.n, plan.logits_arr, plan.out_arr(*pp), plan.out_arr(*fp), plan.rows_arr,
+                                    stream_ptr(buf)))
+    return list(zip(views[0::2], views[1::2]))
+
+
 def forward_folded(x, a, b, folded):
     """forward() with the folded coefficients [out, 4] of fold() in place of w."""
     out_dim = folded.shape[0] if folded.dim() else -1

@@ -106,6 +106,14 @@ int clg_fc_backward_logits(int dtype, const void *x, const int64_t *a, const int
  * backward_x (src/difflogic/cuda/difflogic.cpp:18-19). */
 int clg_fc_fold(int dtype, int from_logits, const void *w_in /*[out_dim,16]*/, void *probs /*[out_dim,16] or NULL*/,
                 void *folded /*[out_dim,4]*/, int64_t out_dim, void *stream);
+/* clg_fc_fold from logits for up to 16 tensors in ONE launch: logits[i] [rows[i], 16] -> probs[i] [rows[i], 16] and
+ * folded[i] [rows[i], 4], row by row the values of clg_fc_fold and of the set-up launch of clg_convblock_forward_ex
+ * (rows = c_out * 7 there, folded = probs + rows * 16).  For a network that folds all its layers at the start of a
+ * training step and hands the results to clg_fc_forward_folded and to clg_convblock_forward_ex (CLG_FWD_FOLDED_IN);
+ * logits, probs, folded, rows: host arrays of n entries.  No counterpart in the reference (torch.softmax per layer,
+ * src/difflogic/difflogic.py:138, src/convlogic/convlogic_layer.py:321). */
+int clg_fold_many(int dtype, int n, const void *const *logits, void *const *probs, void *const *folded, const int64_t *rows,
+                  void *stream);
 int clg_fc_forward_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
                           void *y, int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
 int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
@@ -404,6 +412,8 @@ int clg_convblock_fm_supported(int dtype, const clg_conv_geom *g);
 #define CLG_FWD_FOLDED_OUT 4 /* probs_out holds [c_out, 7, 16] probabilities FOLLOWED BY [c_out, 7, 4] folded coefficients
                               * (ab, a, b, 1 per gate) for clg_convblock_backward_planned; without CLG_FWD_W_LOGITS the
                               * probability part is left untouched (w already holds them) */
+#define CLG_FWD_FOLDED_IN 8  /* with the two flags above: probs_out ALREADY holds the probabilities and the folded coefficients of
+                              * w's logits (clg_fold_many at the start of the step): no softmax or fold launch in this call */
 int clg_convblock_forward_ex(int dtype, const clg_conv_geom *g, const void *x, const void *w, const int32_t *selection, void *y,
                              uint8_t *argmax, void *probs_out, int flags, void *scratch, void *stream);
 /* The same for packed words: y laid out [c_out, ho/2, wo/2, groups], which IS the feature-major [features, words] layout

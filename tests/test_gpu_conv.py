@@ -453,7 +453,8 @@ def test_forward_ex_rejects_bad_options():
         return lib.clg_convblock_forward_ex(0, ctypes.byref(g), x.data_ptr(), layer.weights.data_ptr(), layer.selection.data_ptr(),
                                             y.data_ptr(), am.data_ptr(), probs_ptr, flags, scratch.data_ptr(), None)
 
-    assert call(8, probs.data_ptr()) != 0 and b"unknown flags" in lib.clg_last_error()
+    assert call(16, probs.data_ptr()) != 0 and b"unknown flags" in lib.clg_last_error()
+    assert call(8, probs.data_ptr()) != 0 and b"CLG_FWD_FOLDED_IN goes with" in lib.clg_last_error()
     assert call(1, None) != 0 and b"probs_out" in lib.clg_last_error()
     assert call(2, probs.data_ptr()) != 0 and b"clg_convblock_fm_supported" in lib.clg_last_error()
     assert call(1, probs.data_ptr()) == 0

@@ -70,6 +70,73 @@ def test_config5_training_step_matches_oracle():
     assert_grad_close(xg.grad, xc.grad, rel=1e-6, name="grad_x")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_fold_many_equals_the_folds_of_the_layers(dtype):
+    # one launch for the logits of several layers: row by row what the LogicLayer's fold and the set-up launch of the
+    # fused block give, the pair of a tensor in one buffer (probabilities first)
+    from convlogic_amd.hip import convlogic_hip, difflogic_hip
+    torch.manual_seed(3)
+    tensors = [torch.randn(300, 16, device=DEV, dtype=dtype) * 3, torch.randn(24, 7, 16, device=DEV, dtype=dtype) * 3,
+               torch.randn(1, 16, device=DEV, dtype=dtype), torch.randn(513, 7, 16, device=DEV, dtype=dtype) * 5]
+    pairs = difflogic_hip.fold_many(tensors)
+    for t, (probs, folded) in zip(tensors, pairs):
+        want_p, want_f = difflogic_hip.fold(t.reshape(-1, 16), from_logits=True)
+        assert probs.shape == t.shape and folded.shape == (*t.shape[:-1], 4)
+        assert torch.equal(probs.reshape(-1, 16), want_p) and torch.equal(folded.reshape(-1, 4), want_f)
+        assert torch.equal(folded.reshape(-1, 4), difflogic_hip.fold(probs.reshape(-1, 16), from_logits=False)[1])   # = the fold of the stored values
+        assert folded.data_ptr() == probs.data_ptr() + probs.numel() * probs.element_size()
+    # the block's forward takes such a pair instead of folding itself: same outputs, bit for bit, on every forward path
+    for (n, cin, h, c) in ((40, 16, 4, 24), (6, 8, 8, 24), (3, 4, 16, 24)):
+        layer = C.ConvLogicLayer(cin, c, padding=1, complete=True, implementation="cuda").to(DEV).to(dtype)
+        x = torch.rand(n, cin, h, h, device=DEV, dtype=dtype)
+        lg = layer.weights.detach()
+        pair = difflogic_hip.fold_many([lg, tensors[0]])[0]
+        geo = (*layer.stride, *layer.padding, *layer.kernel)
+        a = convlogic_hip.full_convlogic_forward_logits(x, lg, layer.selection, *geo, want_folded=True)
+        b = convlogic_hip.full_convlogic_forward_logits(x, lg, layer.selection, *geo, want_folded=True, prefolded=pair)
+        for u, v, name in zip(a, b, ("y", "argmax", "probs", "folded")):
+            assert torch.equal(u, v), (name, n, cin, h)
+    with pytest.raises(RuntimeError):
+        difflogic_hip.fold_many([])
+
+
+def test_network_folds_all_layers_in_one_launch():
+    # the CIFAR topology folds its layers' logits once per training step (model.prefold, the default): logits, loss and
+    # every gradient against the same network with the per-layer folds (the blocks bit for bit up to the first
+    # LogicLayer, whose in-kernel softmax sums in another order: 1e-6).  (Against the oracle: the C5 case of
+    # test_gpu_baseline_shapes.py, which runs this model as it is.)
+    torch.manual_seed(5)
+    model = C.ConvLogicCifarModel(k_param=4, input_channels=9, input_size=32, tau=6.5).to(DEV)
+    x = torch.randint(0, 2, (40, 9, 32, 32), device=DEV).float()
+    labels = torch.randint(0, 10, (40,), device=DEV)
+
+    def step(prefold):
+        model.prefold = prefold
+        for p in model.parameters():
+            p.grad = None
+        out = model(x)
+        torch.nn.functional.cross_entropy(out, labels).backward()
+        return out.detach().clone(), [p.grad.clone() for p in model.parameters()]
+
+    out_a, grads_a = step(True)
+    assert all("_prefold" not in m.__dict__ for m in model.network)        # every pair was taken by its layer
+    out_b, grads_b = step(False)
+    assert (out_a - out_b).abs().max().item() <= 1e-5
+    for i, (ga, gb) in enumerate(zip(grads_a, grads_b)):
+        assert_grad_close(ga, gb, rel=1e-4, name=f"parameter {i}")
+    out_c, grads_c = step(True)
+    assert torch.equal(out_a, out_c) and all(torch.equal(u, v) for u, v in zip(grads_a, grads_c))   # reproducible
+    # a stale pair (weights changed in place after it was made) is not used
+    first_fc = next(m for m in model.network if isinstance(m, C.LogicLayer))
+    from convlogic_amd.hip import difflogic_hip
+    first_fc.set_prefold(*difflogic_hip.fold_many([first_fc.weights.detach(), first_fc.weights.detach()])[0])
+    with torch.no_grad():
+        first_fc.weights.add_(1.0)
+    assert first_fc._take_prefold(first_fc.weights) is None
+    with torch.no_grad():
+        first_fc.weights.sub_(1.0)
+
+
 def test_config5_training_step_float32_runs_and_is_deterministic():
     torch.manual_seed(2)
     model = build().to(DEV)
