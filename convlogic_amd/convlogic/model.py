@@ -17,7 +17,10 @@ from .convlogic_layer import ConvLogicLayer
 _FOLD_PLANS = weakref.WeakKeyDictionary()
 
 
-def _prefold(owner, network, x):
+_PREFOLD_MIN_ELEMS = 20 << 19                                     # 512 Ki rows of logits
+
+
+def _prefold(owner, network, x, mode=True):
     """Folds the logits of all layers of a training step in ONE launch and leaves each layer its (probabilities,
     coefficients): softmax and fold are then no part of the layers' forward launches -- the LogicLayers run their plain
     streaming kernel, the deep blocks skip their set-up launch.  Same values as the per-layer folds (tested)."""
@@ -36,6 +39,11 @@ def _prefold(owner, network, x):
         plan = difflogic_hip.FoldPlan([w.detach() for w in weights]) if len(picked) >= 2 else None
         _FOLD_PLANS[owner] = ((x.dtype, x.device), picked, plan)
     if plan is None:
+        return
+    # An eager step of a small network is bound by the host, where the bookkeeping of this launch costs more than the
+    # layers' own allocations save (C5: +15 us per step): by default only networks whose step the GPU bounds fold ahead;
+    # prefold = "always" is for small networks whose step is replayed from a HIP graph (C5: 0.385 -> 0.379 ms).
+    if mode != "always" and plan.total < _PREFOLD_MIN_ELEMS:
         return
     for m, (probs, folded) in zip(picked, difflogic_hip.fold_many([w.detach() for w in weights], plan)):
         m.set_prefold(probs, folded)
@@ -75,8 +83,9 @@ class ConvLogicCifarModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
 
     def forward(self, x):
-        if self.training and x.is_cuda and torch.is_grad_enabled() and self.__dict__.get("prefold", True):
-            _prefold(self, self.network, x)
+        mode = self.__dict__.get("prefold", True)                    # True: where it pays, "always", False
+        if mode and self.training and x.is_cuda and torch.is_grad_enabled():
+            _prefold(self, self.network, x, mode)
         return self.network(x)
 
 
@@ -95,6 +104,7 @@ class ConvLogicMnistModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head([81 * k, 1280 * k, 640 * k, 320 * k], tau, implementation))
 
     def forward(self, x):
-        if self.training and x.is_cuda and torch.is_grad_enabled() and self.__dict__.get("prefold", True):
-            _prefold(self, self.network, x)
+        mode = self.__dict__.get("prefold", True)                    # True: where it pays, "always", False
+        if mode and self.training and x.is_cuda and torch.is_grad_enabled():
+            _prefold(self, self.network, x, mode)
         return self.network(x)

@@ -25,7 +25,7 @@ def _capture(run):
     return graph
 
 
-@pytest.mark.parametrize("kind", ["fc", "block", "block_wide", "mnist_net"])
+@pytest.mark.parametrize("kind", ["fc", "block", "block_wide", "mnist_net", "mnist_net_prefold"])
 def test_training_step_replays_equal_eager(kind):
     torch.manual_seed(3)
     if kind == "fc":
@@ -42,6 +42,8 @@ def test_training_step_replays_equal_eager(kind):
         loss_of = lambda out: (out * out).sum()
     else:
         model = C.ConvLogicMnistModel(k_param=2).to(DEV)
+        if kind == "mnist_net_prefold":
+            model.prefold = "always"                               # the launch that folds all layers' logits is part of the graph
         x = torch.randint(0, 2, (32, 1, 28, 28), device=DEV).float()
         labels = torch.randint(0, 10, (32,), device=DEV)
         loss_of = lambda out: torch.nn.functional.cross_entropy(out, labels)
@@ -68,7 +70,7 @@ def test_training_step_replays_equal_eager(kind):
 
     eager = copy.deepcopy(model)
     for trial in range(3):
-        new_x = torch.rand_like(x) if kind != "mnist_net" else torch.randint(0, 2, x.shape, device=DEV).float()
+        new_x = torch.rand_like(x) if not kind.startswith("mnist_net") else torch.randint(0, 2, x.shape, device=DEV).float()
         with torch.no_grad():
             static_x.copy_(new_x)
         for g in static_grads:

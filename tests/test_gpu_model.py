@@ -101,7 +101,7 @@ def test_fold_many_equals_the_folds_of_the_layers(dtype):
 
 
 def test_network_folds_all_layers_in_one_launch():
-    # the CIFAR topology folds its layers' logits once per training step (model.prefold, the default): logits, loss and
+    # the CIFAR topology folds its layers' logits once per training step (model.prefold): logits, loss and
     # every gradient against the same network with the per-layer folds (the blocks bit for bit up to the first
     # LogicLayer, whose in-kernel softmax sums in another order: 1e-6).  (Against the oracle: the C5 case of
     # test_gpu_baseline_shapes.py, which runs this model as it is.)
@@ -118,13 +118,13 @@ def test_network_folds_all_layers_in_one_launch():
         torch.nn.functional.cross_entropy(out, labels).backward()
         return out.detach().clone(), [p.grad.clone() for p in model.parameters()]
 
-    out_a, grads_a = step(True)
+    out_a, grads_a = step("always")                                      # (True: only where it pays -- big networks, graph capture)
     assert all("_prefold" not in m.__dict__ for m in model.network)        # every pair was taken by its layer
     out_b, grads_b = step(False)
     assert (out_a - out_b).abs().max().item() <= 1e-5
     for i, (ga, gb) in enumerate(zip(grads_a, grads_b)):
         assert_grad_close(ga, gb, rel=1e-4, name=f"parameter {i}")
-    out_c, grads_c = step(True)
+    out_c, grads_c = step("always")
     assert torch.equal(out_a, out_c) and all(torch.equal(u, v) for u, v in zip(grads_a, grads_c))   # reproducible
     # a stale pair (weights changed in place after it was made) is not used
     first_fc = next(m for m in model.network if isinstance(m, C.LogicLayer))
