@@ -9,6 +9,7 @@ import torch
 from torch import nn
 
 from ..difflogic import GroupSum, LogicLayer
+from ..difflogic.difflogic import logic_layer_group_sum
 from .convlogic_layer import ConvLogicLayer
 
 
@@ -49,6 +50,27 @@ def _prefold(owner, network, x, mode=True):
         m.set_prefold(probs, folded)
 
 
+def _forward(owner, x):
+    """The network on x.  In training on the GPU two things happen that a plain nn.Sequential call would not do: the
+    logits of all layers are folded in one launch where that pays (`prefold`), and the last LogicLayer and the GroupSum
+    behind it run as one autograd node (`fused_tail`, default on), whose backward needs no GroupSum launch."""
+    net = owner.network
+    if not (owner.training and isinstance(x, torch.Tensor) and x.is_cuda and torch.is_grad_enabled()):
+        return net(x)
+    mode = owner.__dict__.get("prefold", True)                       # True: where it pays, "always", False
+    if mode:
+        _prefold(owner, net, x, mode)
+    n = len(net)
+    if owner.__dict__.get("fused_tail", True) and n >= 2 and isinstance(net[n - 2], LogicLayer) and isinstance(net[n - 1], GroupSum):
+        h = x
+        for i, m in enumerate(net):
+            if i == n - 2:
+                break
+            h = m(h)
+        return logic_layer_group_sum(net[n - 2], net[n - 1], h)
+    return net(x)
+
+
 def _block(c_in, c_out, implementation, **kw):
     return ConvLogicLayer(in_channels=c_in, out_channels=c_out, residual_init=True, complete=True,
                           implementation=implementation, **kw)
@@ -83,10 +105,7 @@ class ConvLogicCifarModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head(dims, tau, implementation))
 
     def forward(self, x):
-        mode = self.__dict__.get("prefold", True)                    # True: where it pays, "always", False
-        if mode and self.training and x.is_cuda and torch.is_grad_enabled():
-            _prefold(self, self.network, x, mode)
-        return self.network(x)
+        return _forward(self, x)
 
 
 class ConvLogicMnistModel(nn.Module):
@@ -104,7 +123,4 @@ class ConvLogicMnistModel(nn.Module):
         self.network = nn.Sequential(*blocks, *_head([81 * k, 1280 * k, 640 * k, 320 * k], tau, implementation))
 
     def forward(self, x):
-        mode = self.__dict__.get("prefold", True)                    # True: where it pays, "always", False
-        if mode and self.training and x.is_cuda and torch.is_grad_enabled():
-            _prefold(self, self.network, x, mode)
-        return self.network(x)
+        return _forward(self, x)

@@ -208,12 +208,15 @@ __global__ __launch_bounds__(kBlock) void fc_backward_w_kernel(const S *__restri
 // (2 out_dim = in_dim with the reference's random wiring): the input gradient of such a feature is a single
 // product, so the neuron that reads it writes its row and no gather over consumers is needed.  Same arithmetic
 // as fc_backward_w_kernel and fc_backward_x_folded_kernel; 3 row reads and 2 row writes per neuron instead of 7 and 2.
-template <typename T, int VEC, int LPR>
+// CLASSES: the layer feeds a GroupSum and gy is the gradient of ITS output, [batch, k]: the gradient of neuron j's row is
+// gy[b][j / class_rows] * inv_tau, formed here instead of being written out by one kernel and read back by this one.
+template <typename T, int VEC, int LPR, bool CLASSES = false>
 __global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__restrict__ x, const int64_t *__restrict__ a,
                                                                 const int64_t *__restrict__ b, const T *__restrict__ folded,
                                                                 const T *__restrict__ gy, T *__restrict__ gx,
                                                                 T *__restrict__ gw, int out_dim, int64_t batch,
-                                                                const T *__restrict__ probs)
+                                                                const T *__restrict__ probs, int k = 0, int64_t class_rows = 1,
+                                                                T inv_tau = T(1))
 {
     constexpr int ROWS = kWave / LPR;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
@@ -226,11 +229,17 @@ __global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__res
         const Coef<T> c = load_coef(folded + j * 4);
         const T *xa = x + ia * batch;
         const T *xb = x + ib * batch;
-        const T *gj = gy + j * batch;
+        const T *gj = CLASSES ? gy + j / class_rows : gy + j * batch;
         T sab = 0, sa = 0, sb = 0, s1 = 0;
         for (int64_t s = (int64_t)l * VEC; s < batch; s += LPR * VEC) {
-            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s),
-                               vg = load_vec<T, VEC>(gj + s);
+            const Pack<T, VEC> va = load_vec<T, VEC>(xa + s), vb = load_vec<T, VEC>(xb + s);
+            Pack<T, VEC> vg;
+            if constexpr (CLASSES) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) vg.v[i] = gj[(s + i) * k] * inv_tau;   // (the product group_sum_backward writes out)
+            } else {
+                vg = load_vec<T, VEC>(gj + s);
+            }
             Pack<T, VEC> ga, gb;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
@@ -1154,20 +1163,31 @@ extern "C" int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t 
     return CLG_OK;
 }
 
-extern "C" int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
-                                    const void *probs, const void *grad_y, void *grad_x, void *grad_w, int64_t in_dim,
-                                    int64_t out_dim, int64_t batch, void *stream)
+static int backward_sole_impl(const char *name, int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                              const void *probs, const void *grad_y, void *grad_x, void *grad_w, int64_t in_dim, int64_t out_dim,
+                              int64_t batch, int64_t k, double tau, void *stream)
 {
-    if (int e = check_fc(dtype, in_dim, out_dim, batch, "clg_fc_backward_sole")) return e;
-    CLG_REQUIRE(x && a && b && folded && grad_y && grad_x && grad_w, "clg_fc_backward_sole: null pointer argument");
-    CLG_REQUIRE(2 * out_dim == in_dim, "clg_fc_backward_sole: needs 2*out_dim == in_dim (every input read exactly once), got %lld, %lld",
+    if (int e = check_fc(dtype, in_dim, out_dim, batch, name)) return e;
+    CLG_REQUIRE(x && a && b && folded && grad_y && grad_x && grad_w, "%s: null pointer argument", name);
+    CLG_REQUIRE(2 * out_dim == in_dim, "%s: needs 2*out_dim == in_dim (every input read exactly once), got %lld, %lld", name,
                 (long long)out_dim, (long long)in_dim);
+    const bool classes = k > 0;                                      // grad_y is the gradient of a GroupSum's output [batch, k]
+    CLG_REQUIRE(!classes || (k <= 65535 && out_dim % k == 0 && tau != 0.0), "%s: k must divide out_dim (%lld) and tau must not be zero", name,
+                (long long)out_dim);
+    const int64_t class_rows = classes ? out_dim / k : 1;
     const dim3 block(kBlock);
     hipStream_t st = clg_stream(stream);
 #define CLG_LAUNCH_BS(T, VEC, LPR)                                                                                         \
-    hipLaunchKernelGGL((fc_backward_sole_kernel<T, VEC, LPR>), dim3(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave / LPR)))), \
-                       block, 0, st, (const T *)x, a, b, (const T *)folded, (const T *)grad_y, (T *)grad_x, (T *)grad_w,      \
-                       (int)out_dim, batch, (const T *)probs)
+    do {                                                                                                                  \
+        const dim3 grid(grid_for(clg_ceil_div(out_dim, (int64_t)(kWave / LPR))));                                         \
+        if (classes)                                                                                                      \
+            hipLaunchKernelGGL((fc_backward_sole_kernel<T, VEC, LPR, true>), grid, block, 0, st, (const T *)x, a, b, (const T *)folded, \
+                               (const T *)grad_y, (T *)grad_x, (T *)grad_w, (int)out_dim, batch, (const T *)probs, (int)k, class_rows, \
+                               T(1) / (T)tau);                                                                            \
+        else                                                                                                              \
+            hipLaunchKernelGGL((fc_backward_sole_kernel<T, VEC, LPR, false>), grid, block, 0, st, (const T *)x, a, b, (const T *)folded, \
+                               (const T *)grad_y, (T *)grad_x, (T *)grad_w, (int)out_dim, batch, (const T *)probs, 0, (int64_t)1, T(1)); \
+    } while (0)
 #define CLG_LAUNCH_BS_ROWS(T, VEC)                                                                                         \
     do {                                                                                                                  \
         const int lg = lanes_per_row_log2(batch, VEC);                                                                    \
@@ -1184,8 +1204,25 @@ extern "C" int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, 
     }
 #undef CLG_LAUNCH_BS_ROWS
 #undef CLG_LAUNCH_BS
-    CLG_CHECK_LAUNCH("clg_fc_backward_sole");
+    CLG_CHECK_LAUNCH(name);
     return CLG_OK;
+}
+
+extern "C" int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                    const void *probs, const void *grad_y, void *grad_x, void *grad_w, int64_t in_dim,
+                                    int64_t out_dim, int64_t batch, void *stream)
+{
+    return backward_sole_impl("clg_fc_backward_sole", dtype, x, a, b, folded, probs, grad_y, grad_x, grad_w, in_dim, out_dim, batch, 0, 1.0,
+                              stream);
+}
+
+extern "C" int clg_fc_backward_sole_classes(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded,
+                                            const void *probs, const void *grad_out, void *grad_x, void *grad_w, int64_t in_dim,
+                                            int64_t out_dim, int64_t batch, int64_t k, double tau, void *stream)
+{
+    CLG_REQUIRE(k > 0, "clg_fc_backward_sole_classes: k must be positive");
+    return backward_sole_impl("clg_fc_backward_sole_classes", dtype, x, a, b, folded, probs, grad_out, grad_x, grad_w, in_dim, out_dim, batch, k,
+                              tau, stream);
 }
 
 // largest batch one pass of a wavefront row covers: 64 lanes x VEC samples

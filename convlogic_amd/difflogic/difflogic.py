@@ -384,6 +384,50 @@ class _LogicLayerLogitsFunction(torch.autograd.Function):
         return grad_x, None, None, grad_l, None, None, None, None, None
 
 
+class _LogicLayerGroupSumFunction(torch.autograd.Function):
+    """A halving LogicLayer and the GroupSum behind it (the last two modules of the reference's networks,
+    src/convlogic/model.py:55-57) as ONE autograd node: the forward is the two forward launches of the modules; the
+    backward hands the gradient of the GroupSum's output [B, k] to the layer's one-pass kernel, which forms the gradient of
+    its own output from it -- no launch that writes that [features, B] tensor and none that reads it back.  Same values
+    as the two modules, bit for bit."""
+
+    @staticmethod
+    def forward(ctx, x, a, b, logits, k, tau, prefolded=None):
+        if prefolded is not None:
+            w, folded = prefolded
+            y = difflogic_hip.forward_folded(x, a, b, folded)
+        else:
+            y, w, folded = difflogic_hip.forward_logits(x, a, b, logits.detach(), validate=False)
+        ctx.save_for_backward(x, a, b, w, folded)
+        ctx.k, ctx.tau = k, tau
+        return difflogic_hip.group_sum(y, k, tau)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, a, b, w, folded = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad_x, grad_l = difflogic_hip.backward_sole_classes(x, a, b, folded, w, grad_out, ctx.k, ctx.tau,
+                                                            validate=_needs_check(grad_out, x))
+        return grad_x, None, None, grad_l, None, None, None
+
+
+def logic_layer_group_sum(layer, group_sum, x):
+    """group_sum(layer(x)) -- through one autograd node (_LogicLayerGroupSumFunction) when `layer` is a halving
+    LogicLayer in training mode on the GPU, else through the two modules."""
+    weights = layer._parameters["weights"]
+    if (isinstance(layer, LogicLayer) and isinstance(group_sum, GroupSum) and layer.implementation == "cuda" and layer.training
+            and torch.is_grad_enabled() and isinstance(x, torch.Tensor) and x.is_cuda and x.ndim == 2 and x.shape[1] == layer.in_dim
+            and layer.grad_factor == 1.0 and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
+            and weights.is_contiguous() and weights.device == x.device and layer.out_dim % group_sum.k == 0 and x.shape[0] > 0):
+        key = layer._wiring_key()
+        layer._check_wiring(key)
+        if layer._sole_consumers(key):
+            buffers = layer._buffers
+            return _LogicLayerGroupSumFunction.apply(_feature_major(x), buffers["indices_0"], buffers["indices_1"], weights,
+                                                     group_sum.k, group_sum.tau, layer._take_prefold(weights))
+    return group_sum(layer(x))
+
+
 def _needs_check(grad_y, x):
     """The tensors a Function saved were validated on the way in; the incoming gradient is what can still differ
     (autograd hands over the output's shape, but a caller-made gradient may have another dtype or device)."""

@@ -38,6 +38,7 @@ SIGNATURES = {
     "clg_fc_forward_folded": (_i, [_i, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_x_folded": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_sole": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "clg_fc_backward_sole_classes": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f64, _p]),
     "clg_fc_forward_logits": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "clg_fc_backward_fused_fits": (_i, [_i, _i64]),
     "clg_fc_backward_fused": (_i, [_i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),

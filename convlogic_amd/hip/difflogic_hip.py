@@ -210,6 +210,26 @@ def backward_sole(x, a, b, folded, probs, grad_y, validate=True):
     return gx, gw
 
 
+def backward_sole_classes(x, a, b, folded, probs, grad_out, k, tau, validate=True):
+    """backward_sole() for a layer whose output goes straight into a GroupSum: grad_out [B, k] is the gradient of the
+    GroupSum's output; the gradient of the layer's output (grad_out[:, class of the neuron] / tau) is formed inside the
+    kernel.  Same values as group_sum_backward() + backward_sole(), bit for bit."""
+    out_dim = folded.shape[0] if folded.dim() else -1
+    in_dim, batch = x.shape
+    if validate:
+        _wiring(x, a, b, out_dim)
+        check_input(folded, "folded", x.dtype, (out_dim, 4))
+        check_input(grad_out, "grad_out", x.dtype, (batch, k))
+        if probs is not None:
+            check_input(probs, "w", x.dtype, (out_dim, 16))
+    gx = torch.empty_like(x)
+    gw = torch.empty((out_dim, 16), dtype=x.dtype, device=x.device)
+    check(_lib.load().clg_fc_backward_sole_classes(dtype_code(x), x.data_ptr(), a.data_ptr(), b.data_ptr(), folded.data_ptr(),
+                                                   probs.data_ptr() if probs is not None else 0, grad_out.data_ptr(), gx.data_ptr(),
+                                                   gw.data_ptr(), in_dim, out_dim, batch, int(k), float(tau), stream_ptr(x)))
+    return gx, gw
+
+
 def backward_fused_fits(x):
     """True when backward_fused() covers the batch of feature-major x [in, B] in one pass."""
     return bool(_lib.load().clg_fc_backward_fused_fits(dtype_code(x), x.shape[1]))

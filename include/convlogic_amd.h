@@ -130,6 +130,13 @@ int clg_fc_backward_x_folded(int dtype, const void *x, const int64_t *a, const i
 int clg_fc_backward_sole(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
                          const void *probs /*[out_dim,16] or NULL*/, const void *grad_y, void *grad_x, void *grad_w,
                          int64_t in_dim, int64_t out_dim, int64_t batch, void *stream);
+/* The same when the layer's output goes straight into a GroupSum (the last two modules of the reference's models,
+ * src/convlogic/model.py:55-57): grad_out [batch, k] is the gradient of the GroupSum's OUTPUT, and the gradient of neuron
+ * j's row, grad_out[b][j / (out_dim / k)] * (1 / tau), is formed inside the kernel -- the values clg_group_sum_backward
+ * would write and this call read back, bit for bit, without that launch and without the [out_dim, batch] tensor. */
+int clg_fc_backward_sole_classes(int dtype, const void *x, const int64_t *a, const int64_t *b, const void *folded /*[out_dim,4]*/,
+                                 const void *probs /*[out_dim,16] or NULL*/, const void *grad_out /*[batch,k]*/, void *grad_x,
+                                 void *grad_w, int64_t in_dim, int64_t out_dim, int64_t batch, int64_t k, double tau, void *stream);
 
 /* clg_fc_fold (from logits) + clg_fc_forward_folded in one launch: y from the LOGITS [out_dim, 16]; their softmax goes to
  * probs [out_dim, 16] and its 4 folded coefficients per neuron to folded [out_dim, 4] for the backward entry points

@@ -137,6 +137,46 @@ def test_network_folds_all_layers_in_one_launch():
         first_fc.weights.sub_(1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_last_layer_and_group_sum_as_one_autograd_node(dtype):
+    # the networks run their last LogicLayer and the GroupSum behind it as one node whose backward hands the gradient of
+    # the class sums straight to the layer's kernel: outputs and every gradient bit for bit those of the two modules, for
+    # both topologies, ragged batches and a class count that the kernel's lanes do not divide
+    from convlogic_amd.hip import difflogic_hip
+    torch.manual_seed(11)
+    for model, shape in ((C.ConvLogicCifarModel(k_param=2, input_channels=3, input_size=32, tau=6.5), (37, 3, 32, 32)),
+                         (C.ConvLogicMnistModel(k_param=2, tau=3.0), (64, 1, 28, 28))):
+        model = model.to(DEV).to(dtype)
+        x = torch.randint(0, 2, shape, device=DEV).to(dtype)
+        labels = torch.randint(0, 10, (shape[0],), device=DEV)
+
+        def step(fused):
+            model.fused_tail = fused
+            for p in model.parameters():
+                p.grad = None
+            xin = x.clone().requires_grad_(True)
+            out = model(xin)
+            torch.nn.functional.cross_entropy(out, labels).backward()
+            return out.detach().clone(), [xin.grad.clone()] + [p.grad.clone() for p in model.parameters()]
+
+        out_a, grads_a = step(True)
+        out_b, grads_b = step(False)
+        assert torch.equal(out_a, out_b)
+        for i, (u, v) in enumerate(zip(grads_a, grads_b)):
+            assert torch.equal(u, v), (type(model).__name__, i, (u - v).abs().max().item())
+    # the entry point against its two-launch equivalent, k = 7 classes of 9 rows
+    layer = C.LogicLayer(126, 63, implementation="cuda").to(DEV).to(dtype)
+    xf = torch.rand(126, 52, device=DEV, dtype=dtype)
+    go = torch.randn(52, 7, device=DEV, dtype=dtype)
+    probs, folded = difflogic_hip.fold(layer.weights.detach(), from_logits=True)
+    gy = difflogic_hip.group_sum_backward(go, 63, 2.5)
+    want = difflogic_hip.backward_sole(xf, layer.indices_0, layer.indices_1, folded, probs, gy)
+    got = difflogic_hip.backward_sole_classes(xf, layer.indices_0, layer.indices_1, folded, probs, go, 7, 2.5)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    with pytest.raises(RuntimeError):
+        difflogic_hip.backward_sole_classes(xf, layer.indices_0, layer.indices_1, folded, probs, go[:, :5].contiguous(), 5, 2.5)
+
+
 def test_config5_training_step_float32_runs_and_is_deterministic():
     torch.manual_seed(2)
     model = build().to(DEV)
