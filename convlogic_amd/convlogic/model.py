@@ -61,7 +61,8 @@ def _forward(owner, x):
     if mode:
         _prefold(owner, net, x, mode)
     n = len(net)
-    if owner.__dict__.get("fused_tail", True) and n >= 2 and isinstance(net[n - 2], LogicLayer) and isinstance(net[n - 1], GroupSum):
+    if (owner.__dict__.get("fused_tail", True) and n >= 2 and isinstance(net[n - 2], LogicLayer) and isinstance(net[n - 1], GroupSum)
+            and not (net._forward_hooks or net._forward_pre_hooks)):
         h = x
         for i, m in enumerate(net):
             if i == n - 2:

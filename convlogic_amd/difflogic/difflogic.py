@@ -418,7 +418,8 @@ def logic_layer_group_sum(layer, group_sum, x):
     if (isinstance(layer, LogicLayer) and isinstance(group_sum, GroupSum) and layer.implementation == "cuda" and layer.training
             and torch.is_grad_enabled() and isinstance(x, torch.Tensor) and x.is_cuda and x.ndim == 2 and x.shape[1] == layer.in_dim
             and layer.grad_factor == 1.0 and weights.dtype == x.dtype and x.dtype in (torch.float32, torch.float64)
-            and weights.is_contiguous() and weights.device == x.device and layer.out_dim % group_sum.k == 0 and x.shape[0] > 0):
+            and weights.is_contiguous() and weights.device == x.device and layer.out_dim % group_sum.k == 0 and x.shape[0] > 0
+            and group_sum.tau != 0 and not _has_forward_hooks(layer) and not _has_forward_hooks(group_sum)):
         key = layer._wiring_key()
         layer._check_wiring(key)
         if layer._sole_consumers(key):
@@ -426,6 +427,11 @@ def logic_layer_group_sum(layer, group_sum, x):
             return _LogicLayerGroupSumFunction.apply(_feature_major(x), buffers["indices_0"], buffers["indices_1"], weights,
                                                      group_sum.k, group_sum.tau, layer._take_prefold(weights))
     return group_sum(layer(x))
+
+
+def _has_forward_hooks(module):
+    """Hooks that only a call of the module itself would run."""
+    return bool(module._forward_hooks or module._forward_pre_hooks)
 
 
 def _needs_check(grad_y, x):

@@ -164,6 +164,13 @@ def test_last_layer_and_group_sum_as_one_autograd_node(dtype):
         assert torch.equal(out_a, out_b)
         for i, (u, v) in enumerate(zip(grads_a, grads_b)):
             assert torch.equal(u, v), (type(model).__name__, i, (u - v).abs().max().item())
+    # a forward hook on the last layer is a reason to call the module itself: the hook still fires
+    seen = []
+    handle = model.network[-2].register_forward_hook(lambda m, i, o: seen.append(tuple(o.shape)))
+    model.fused_tail = True
+    model(x)
+    handle.remove()
+    assert seen == [(shape[0], model.network[-2].out_dim)]
     # the entry point against its two-launch equivalent, k = 7 classes of 9 rows
     layer = C.LogicLayer(126, 63, implementation="cuda").to(DEV).to(dtype)
     xf = torch.rand(126, 52, device=DEV, dtype=dtype)
