@@ -106,7 +106,8 @@ class FoldPlan:
         self.elem = first.element_size()
 
     def matches(self, logits_list):
-        return len(logits_list) == self.n and all(t.data_ptr() == p and t.dtype == self.dtype for t, p in zip(logits_list, self.ptrs))
+        return len(logits_list) == self.n and all(t.data_ptr() == p and t.dtype == self.dtype and t.numel() == 16 * r and t.is_contiguous()
+                                                  for t, p, r in zip(logits_list, self.ptrs, self.rows))
 
 
 def fold_many(logits_list, plan=None):
