@@ -236,7 +236,10 @@ __global__ __launch_bounds__(kBlock) void fc_backward_sole_kernel(const T *__res
             Pack<T, VEC> vg;
             if constexpr (CLASSES) {
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) vg.v[i] = gj[(s + i) * k] * inv_tau;   // (the product group_sum_backward writes out)
+                for (int i = 0; i < VEC; ++i) {
+                    vg.v[i] = gj[(s + i) * k] * inv_tau;             // (the product group_sum_backward writes out)
+                    asm volatile("" : "+v"(vg.v[i]));                // the rounded product: no contraction into the sums below
+                }
             } else {
                 vg = load_vec<T, VEC>(gj + s);
             }

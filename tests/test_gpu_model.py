@@ -144,7 +144,9 @@ def test_last_layer_and_group_sum_as_one_autograd_node(dtype):
     # both topologies, ragged batches and a class count that the kernel's lanes do not divide
     from convlogic_amd.hip import difflogic_hip
     torch.manual_seed(11)
+    # (batch 200 at 4 samples per lane: the shape on which the compiler once fused the division by tau into the sums)
     for model, shape in ((C.ConvLogicCifarModel(k_param=2, input_channels=3, input_size=32, tau=6.5), (37, 3, 32, 32)),
+                         (C.ConvLogicCifarModel(k_param=1, input_channels=1, input_size=32, tau=6.5), (200, 1, 32, 32)),
                          (C.ConvLogicMnistModel(k_param=2, tau=3.0), (64, 1, 28, 28))):
         model = model.to(DEV).to(dtype)
         x = torch.randint(0, 2, shape, device=DEV).to(dtype)
