@@ -414,6 +414,9 @@ class ConvLogicLayer(nn.Module):
         # the two taps of a gate must not be the same element (same position on different channels is fine)
         for t in range(0, taps, 2):
             same = (ch[:, t] == ch[:, t + 1]) & (rows[:, t] == rows[:, t + 1]) & (cols[:, t] == cols[:, t + 1])
+            if kh * kw == 1 and bool(same.any()):
+                # a window of one element has no other position to draw: the reference's loop (:437-448) would never end
+                raise ValueError("a 1x1 kernel cannot give the two inputs of a gate different taps once both draw the same channel")
             for c in same.nonzero(as_tuple=True)[0].tolist():
                 while True:
                     r = torch.randint(0, kh, (1,), device=dev, dtype=torch.int32)

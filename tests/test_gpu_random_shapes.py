@@ -12,7 +12,8 @@ import pytest
 import torch
 
 import convlogic_amd as C
-from convlogic_amd.difflogic.difflogic import logic_layer_group_sum
+from convlogic_amd.convlogic import binarize
+from convlogic_amd.difflogic.difflogic import LogicLayerCudaFunction, logic_layer_group_sum
 from oracle import convlogic_oracle as O
 from tests.gpu_util import DEV, block_oracle, check_pool_route
 
@@ -237,3 +238,106 @@ def test_random_networks_keep_their_promises():
             y_float = model(xf)
             y_bits = model(C.PackBitsTensor(x.bool(), 64))
         assert y_bits.dtype == torch.int32 and torch.equal(y_bits.float() / tau, y_float), case
+
+
+def _window(rng):
+    """A random (stride, padding, kernel, h, w) with non-square members; windows of one element are left out (the
+    constructor refuses them)."""
+    while True:
+        st = (rng.choice([1, 1, 2, 3]), rng.choice([1, 1, 2]))
+        kn = (rng.choice([1, 2, 3, 3, 4, 5]), rng.choice([2, 3, 3, 5]))
+        pd = (min(rng.choice([0, 1, 2]), kn[0] - 1), min(rng.choice([0, 1, 2]), kn[1] - 1))
+        h, w = rng.choice([1, 2, 3, 5, 8, 9, 12, 17, 28, 33]), rng.choice([1, 2, 4, 7, 10, 16, 31, 40])
+        if h + 2 * pd[0] >= kn[0] and w + 2 * pd[1] >= kn[1]:
+            return st, pd, kn, h, w
+
+
+def test_random_split_layers_tree_levels_packed_blocks_thresholds_and_the_reference_shaped_function():
+    rng = random.Random(15)
+    for _ in range(400):
+        what = rng.choice(["conv4", "tree", "packed", "thresholds", "function"])
+        torch.manual_seed(rng.randrange(1 << 30))
+        dtype = rng.choice([torch.float32, torch.float32, torch.float64])
+        tol, rel = _tolerances(dtype)
+        if what == "conv4":                                          # split layer, any stride / padding / window
+            st, pd, kn, h, w = _window(rng)
+            n, cin, cout = rng.choice([1, 2, 4, 17, 64]), rng.choice([1, 2, 3, 8, 20]), rng.choice([1, 2, 5, 16, 40])
+            case = (what, n, cin, cout, h, w, st, pd, kn, dtype)
+            layer = C.ConvLogicLayer(cin, cout, stride=st, padding=pd, kernel=kn, implementation="cuda").to(DEV).to(dtype)
+            x = torch.randn(n, cin, h, w, device=DEV, dtype=dtype, requires_grad=True)
+            y = layer(x)
+            gy = torch.randn_like(y)
+            y.backward(gy)
+            xl, ll = x.detach().cpu().requires_grad_(True), layer.weights.detach().cpu().requires_grad_(True)
+            want = O.conv4_forward(xl, torch.softmax(ll, -1), layer.selection.cpu(), st, pd, kn)
+            want.backward(gy.cpu())
+            assert y.shape == want.shape, case
+            assert (y.detach().cpu() - want.detach()).abs().max().item() <= tol * max(1.0, want.detach().abs().max().item()), case
+            _grad_close(x.grad, xl.grad, rel, ("grad_x", case))
+            _grad_close(layer.weights.grad, ll.grad, rel, ("grad_logits", case))
+        elif what == "tree":
+            bits = rng.choice([2, 4, 6, 8])
+            n, c, h, w = rng.choice([1, 3, 16, 70]), rng.choice([1, 2, 5, 33]), rng.choice([1, 2, 4, 9, 16]), rng.choice([1, 3, 6, 16])
+            case = (what, n, c, h, w, bits, dtype)
+            layer = C.TreeLogicLayer(c, bits, implementation="cuda").to(DEV).to(dtype)
+            x = torch.rand(n, c, h, w, bits, device=DEV, dtype=dtype, requires_grad=True)
+            y = layer(x)
+            gy = torch.randn_like(y)
+            y.backward(gy)
+            xl, ll = x.detach().cpu().requires_grad_(True), layer.weights.detach().cpu().requires_grad_(True)
+            want = O.tree_forward(xl, torch.softmax(ll, -1))
+            want.backward(gy.cpu())
+            assert (y.detach().cpu() - want.detach()).abs().max().item() <= tol, case
+            _grad_close(x.grad, xl.grad, rel, ("grad_x", case))
+            _grad_close(layer.weights.grad, ll.grad, rel, ("grad_logits", case))
+        elif what == "packed":                                       # packed block: numpy oracle and the float eval path
+            while True:
+                st, pd, kn, h, w = _window(rng)
+                ho, wo = O.conv_out_size(h, w, st, pd, kn)
+                if ho >= 2 and wo >= 2 and ho % 2 == 0 and wo % 2 == 0:
+                    break
+            n, cin, cout = rng.choice([1, 5, 64, 65, 130, 300]), rng.choice([1, 2, 3, 9, 32, 100]), rng.choice([1, 2, 6, 32, 96, 200])
+            case = (what, n, cin, cout, h, w, st, pd, kn)
+            layer = C.ConvLogicLayer(cin, cout, stride=st, padding=pd, kernel=kn, complete=True, implementation="cuda").to(DEV)
+            with torch.no_grad():
+                layer.weights.copy_(torch.randn_like(layer.weights))
+            layer.eval()
+            bits = torch.randint(0, 2, (n, cin, h, w), device=DEV).bool()
+            with torch.no_grad():
+                y_float = layer(bits.float())
+            p = C.PackBitsTensor(bits, 64)
+            words, pad = O.pack_image(bits.cpu().numpy())
+            assert p.pad_len == pad and np.array_equal(p.t.cpu().numpy(), words), case
+            out = layer(p)
+            gates = layer.weights.argmax(-1).to(torch.uint8).cpu().numpy()
+            want = O.conv_block_eval_packed(words, gates, layer.selection.cpu().numpy(), st, pd, kn)
+            assert np.array_equal(out.t.cpu().numpy(), want), case
+            assert np.array_equal(O.unpack_image(out.t.cpu().numpy(), pad), y_float.cpu().numpy() > 0.5), case
+        elif what == "thresholds":
+            n, c0, levels = rng.choice([1, 33, 64, 70, 200]), rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 9])
+            h, w = rng.choice([1, 4, 5, 28, 32]), rng.choice([1, 4, 7, 28, 32])
+            case = (what, n, c0, h, w, levels)
+            x = torch.rand(n, c0, h, w)
+            thr = O.thresholds_uniform(levels)
+            want = O.apply_thresholds(x, thr)
+            assert torch.equal(binarize.apply_thresholds(x.to(DEV), thr).cpu(), want), case
+            p = binarize.pack_thresholds(x.to(DEV), thr)
+            words, pad = O.pack_image(want.numpy() > 0.5)
+            assert p.pad_len == pad and np.array_equal(p.t.cpu().numpy(), words), case
+        else:                                                        # probabilities in, their gradient out (the reference's Function)
+            in_dim = rng.choice([1, 2, 7, 64, 100, 999])
+            out_dim, batch = max((in_dim + 1) // 2, rng.choice([1, 5, 64, 300, 2000])), rng.choice([1, 3, 32, 100, 256, 300])
+            case = (what, in_dim, out_dim, batch, dtype)
+            layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV).to(dtype)
+            x = torch.rand(in_dim, batch, device=DEV, dtype=dtype, requires_grad=True)
+            w = torch.softmax(layer.weights.detach(), -1).requires_grad_(True)
+            y = LogicLayerCudaFunction.apply(x, layer.indices_0, layer.indices_1, w, layer.given_x_indices_of_y_start,
+                                             layer.given_x_indices_of_y)
+            gy = torch.randn_like(y)
+            y.backward(gy)
+            xl, wl = x.detach().cpu().requires_grad_(True), w.detach().cpu().requires_grad_(True)
+            want = O.logic_fc_forward(xl.transpose(0, 1), layer.indices_0.cpu(), layer.indices_1.cpu(), wl).transpose(0, 1)
+            want.backward(gy.cpu())
+            assert (y.detach().cpu() - want.detach()).abs().max().item() <= tol, case
+            _grad_close(x.grad, xl.grad, rel, ("grad_x", case))
+            _grad_close(w.grad, wl.grad, rel, ("grad_w", case))

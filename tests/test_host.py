@@ -198,6 +198,14 @@ def test_constructor_validation():
     assert set(fc.state_dict()) == {"weights", "indices_0", "indices_1"}
 
 
+def test_one_by_one_kernel_raises_instead_of_redrawing_forever():
+    # the reference redraws only (row, column) of the second tap of a pair (src/convlogic/convlogic_layer.py:437-448): with a
+    # window of one element its loop never ends once both taps drew the same channel; this package raises
+    torch.manual_seed(0)
+    with pytest.raises(ValueError):
+        C.ConvLogicLayer(8, 5, kernel=1, padding=0, implementation="python")
+
+
 def test_bad_selection_and_wiring_raise_on_the_host():
     # a tap outside the input channels / receptive field, or a wiring index outside the input features, would be an
     # out-of-range access inside a kernel: both are rejected on the host (ValueError), also after in-place edits
