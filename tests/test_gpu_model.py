@@ -2,6 +2,8 @@
 LogicLayers, GroupSum; src/convlogic/model.py:16-58 with k=32, 9 input channels) built from this
 package's layers, one training step and the packed-bit evaluation of the fully connected tail against
 the CPU oracle at a reduced batch."""
+import copy
+
 import numpy as np
 import pytest
 import torch
@@ -358,3 +360,61 @@ def test_small_network_learns_a_synthetic_task():
             losses.append(loss.item())
         assert all(torch.isfinite(torch.tensor(losses)))
         assert losses[-1] < 0.6 * losses[0], (graphed, losses[0], losses[-1])
+
+
+def test_networks_stepping_on_four_host_threads_equal_their_serial_runs():
+    # calls may come from any host thread and are ordered by the caller's stream only: four networks, each on its own
+    # thread and stream at the same time, give bit for bit what each gives alone (no state shared between calls)
+    import threading
+    torch.manual_seed(0)
+    specs = [("cifar", 2, 3, 40), ("mnist", 2, 1, 64), ("cifar", 4, 9, 17), ("cifar", 1, 1, 200)]
+    nets, data = [], []
+    for kind, k, cin, n in specs:
+        model = (C.ConvLogicCifarModel(k_param=k, input_channels=cin, input_size=32, tau=6.5) if kind == "cifar"
+                 else C.ConvLogicMnistModel(k_param=k, tau=6.5)).to(DEV)
+        size = 32 if kind == "cifar" else 28
+        nets.append(model)
+        data.append([(torch.randint(0, 2, (n, cin, size, size), device=DEV).float(), torch.randint(0, 10, (n,), device=DEV)) for _ in range(5)])
+
+    def run(model, batches, out):
+        for _ in range(4):
+            for x, labels in batches:
+                for p in model.parameters():
+                    p.grad = None
+                logits = model(x)
+                torch.nn.functional.cross_entropy(logits, labels).backward()
+                out.append((logits.detach().clone(), [p.grad.clone() for p in model.parameters()]))
+
+    serial = []
+    for model, batches in zip(nets, data):
+        serial.append([])
+        run(copy.deepcopy(model), batches, serial[-1])
+    torch.cuda.synchronize()
+    results, errors = [[] for _ in nets], []
+    multithreaded = torch.autograd.is_multithreading_enabled()
+    torch.autograd.set_multithreading_enabled(False)              # backward on the thread that calls it
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                run(nets[i], data[i], results[i])
+            stream.synchronize()
+        except Exception as e:                                       # noqa: BLE001 - reported by the assert below
+            errors.append((i, repr(e)))
+
+    try:
+        threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(nets))]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        torch.cuda.synchronize()
+    finally:
+        torch.autograd.set_multithreading_enabled(multithreaded)
+    assert not errors, errors
+    for i, (alone, together) in enumerate(zip(serial, results)):
+        assert len(alone) == len(together) == 20
+        for step, ((oa, ga), (ob, gb)) in enumerate(zip(alone, together)):
+            assert torch.equal(oa, ob), (i, step)
+            assert all(torch.equal(u, v) for u, v in zip(ga, gb)), (i, step)
