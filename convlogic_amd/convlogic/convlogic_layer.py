@@ -117,7 +117,7 @@ class _FullConvLogicLogitsFunction(Function):
                 grad_x, grad_l = convlogic_hip.full_convlogic_backward_planned(grad_fm if use_fm else grad_y.contiguous(), x1, w_prob, folded,
                                                                                argmax, selection, *ctx.plan, *ctx.geometry, need_grad_x=need_x,
                                                                                validate=not ok, feature_major=use_fm,
-                                                                               padded=None if use_fm else padded)
+                                                                               padded=None if use_fm else padded, kernel=ctx.kernel)
                 return grad_x, grad_l, None, None, None, None, None, None, None, None, None, None
             grad_x = convlogic_hip.full_convlogic_backward_x(grad_y.contiguous(), x1, w_prob, argmax, selection, *ctx.geometry) if need_x else None
             return grad_x, None, None, None, None, None, None, None, None, None, None, None

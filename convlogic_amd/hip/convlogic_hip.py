@@ -384,16 +384,22 @@ def make_backward_plan(x, c_out, selection, stride_h, stride_w, pad_h, pad_w, ke
 
 
 def full_convlogic_backward_planned(grad_y, x, weight, folded, argmax, selection, plan, signature, stride_h, stride_w, pad_h, pad_w,
-                                    need_grad_x=True, wrt_logits=True, validate=True, feature_major=False, padded=None):
+                                    need_grad_x=True, wrt_logits=True, validate=True, feature_major=False, padded=None, kernel=None):
     """-> (grad_x or None, grad_w [C,7,16]) with the layer's plan from make_backward_plan(): no list building, no reduce
     launch and -- with folded [C, 7, 4] from full_convlogic_forward_logits(want_folded=True) -- no set-up launch for
     blocks whose images fit LDS.  grad_w is the gradient w.r.t. the logits (weight = their softmax) or, with
     wrt_logits=False, w.r.t. the probabilities; feature_major: grad_y is laid out [C, Ho/2, Wo/2, N] (as for
-    full_convlogic_backward_fm).  Same values as full_convlogic_backward(_logits / _fm)()."""
-    if feature_major:                                                # grad_y laid out [C, Ho/2, Wo/2, N]
-        g = _geom_from_out(x, grad_y.shape[0], 2 * grad_y.shape[1], 2 * grad_y.shape[2], stride_h, stride_w, pad_h, pad_w)
+    full_convlogic_backward_fm).  Same values as full_convlogic_backward(_logits / _fm)().  kernel: (kernel_h, kernel_w) the plan
+    (and the padded copy) were made with; without it the largest window that gives grad_y's size is taken, which is another one
+    where a stride above 1 does not divide the padded image (the plan's signature then refuses the call)."""
+    c_out, ho, wo = ((grad_y.shape[0], 2 * grad_y.shape[1], 2 * grad_y.shape[2]) if feature_major     # [C, Ho/2, Wo/2, N]
+                     else (grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3]))
+    if kernel is None:
+        g = _geom_from_out(x, c_out, ho, wo, stride_h, stride_w, pad_h, pad_w)
     else:
-        g = _geom_from_out(x, grad_y.shape[1], 2 * grad_y.shape[2], 2 * grad_y.shape[3], stride_h, stride_w, pad_h, pad_w)
+        g = _geom(x, c_out, stride_h, stride_w, pad_h, pad_w, *kernel)
+        if _out_size(g) != (ho, wo):
+            raise RuntimeError(f"grad_y is the gradient of a {ho // 2} x {wo // 2} pooled image, the geometry gives {_out_size(g)[0] // 2} x {_out_size(g)[1] // 2}")
     lib = _lib.load()
     dt = dtype_code(x)
     if validate:
