@@ -7,7 +7,10 @@
  *
  * Return value: 0 on success, a negative CLG_E* code on a rejected argument or a
  * failed launch; clg_last_error() then returns a human readable message for the
- * calling thread.  Bad arguments are rejected on the host before any launch.
+ * calling thread.  Bad arguments are rejected on the host before any launch, and so are
+ * sizes beyond what a kernel indexes: more than 65535 logic kernels per fused block in the
+ * gradients and most forward kernels, in_dim / out_dim of 2^31 and above, element counts of
+ * 2^31 and above where an entry point says so in its message.
  *
  * Each declaration cites the function of the reference's native extension modules
  * (`difflogic_cuda`, `convlogic_cuda`; paths relative to the reference checkout) that

@@ -243,6 +243,57 @@ def test_block_config4_full_size_properties():
     assert torch.all((ye == 0) | (ye == 1))
 
 
+@pytest.mark.parametrize("n,cin,cout,h,w,kernel,pad,stride,dtype", [
+    (2, 2, 4, 129, 129, (100, 100), 0, 1, torch.float32), (1, 1, 3, 260, 40, (255, 3), 1, 1, torch.float64),
+    (2, 3, 4, 151, 151, (120, 120), 0, 2, torch.float32), (1, 2, 3, 254, 254, (251, 251), 0, 1, torch.float32)])
+@pytest.mark.parametrize("indices", [True, False])
+def test_block_with_windows_as_large_as_the_image(n, cin, cout, h, w, kernel, pad, stride, dtype, indices):
+    # windows of up to 255 rows: shapes that no tile or padded-copy plan takes end on the any-shape kernels
+    # (per-element gather of the input gradient among them); both the reference-shaped Function (indices) and the
+    # module's training path against the oracle
+    torch.manual_seed(h + w)
+    layer = C.ConvLogicLayer(cin, cout, stride=stride, padding=pad, kernel=kernel, complete=True, implementation="cuda",
+                             return_indices=indices).to(DEV).to(dtype)
+    x = torch.randn(n, cin, h, w, device=DEV, dtype=dtype, requires_grad=True)
+    out = layer(x)
+    y, idx = out if indices else (out, None)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    if idx is None:                                                 # the pooled positions of the same forward, from the Function
+        from convlogic_amd.hip import difflogic_hip
+        probs = difflogic_hip.fold(layer.weights.detach().reshape(-1, 16), from_logits=True)[0].reshape(cout, 7, 16)
+        with torch.no_grad():
+            y_fn, idx = C.FullConvLogicFunction.apply(x.detach(), probs, layer.selection, stride, stride, pad, pad, *kernel, False, True)
+        assert torch.equal(y, y_fn)
+    routed, _, idx_ref, _, _, ll, xl, x4 = block_oracle(x, layer.weights, layer.selection, _pair(stride), _pair(pad), kernel, idx)
+    tol, rel = (1e-5, 1e-4) if dtype == torch.float32 else (1e-12, 1e-10)
+    size = max(1.0, x4.detach().abs().max().item())
+    check_pool_route(idx, idx_ref, x4, tol=tol * size)
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= tol * size
+    routed.backward(gy.cpu())
+    # (most of grad_x is structurally zero here: the per-element bound is taken against a mean that those zeros pull down)
+    assert_grad_close(x.grad, xl.grad, rel=rel, rel_elem=10 * rel, name="grad_x")
+    assert_grad_close(layer.weights.grad, ll.grad, rel=rel, rel_elem=10 * rel, name="grad_logits")
+
+
+def test_block_with_more_kernels_than_a_grid_dimension_is_refused_on_the_host():
+    # 65535 kernels per block is the limit of the gradient kernels and most forward kernels (the kernel index is a grid
+    # dimension): above it a call raises before anything is launched; where a forward kernel without that limit takes the
+    # shape its values are the oracle's
+    torch.manual_seed(1)
+    layer = C.ConvLogicLayer(2, 66000, padding=1, kernel=3, complete=True, implementation="cuda", return_indices=True).to(DEV)
+    x = torch.randn(2, 2, 6, 6, device=DEV, requires_grad=True)
+    y, idx = layer(x)
+    routed, _, idx_ref, _, _, _, _, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (1, 1), (3, 3), idx)
+    check_pool_route(idx, idx_ref, x4, tol=1e-5 * max(1.0, x4.detach().abs().max().item()))
+    assert (y.detach().cpu() - routed.detach()).abs().max().item() <= 1e-5 * max(1.0, x4.detach().abs().max().item())
+    with pytest.raises(RuntimeError, match="65535"):
+        y.backward(torch.randn_like(y))
+    with pytest.raises(RuntimeError, match="65535"):
+        layer(torch.randn(3, 2, 4, 4, device=DEV))
+    torch.cuda.synchronize()
+
+
 def test_block_errors():
     layer = C.ConvLogicLayer(1, 1, kernel=3, padding=0, complete=True).to(DEV)
     with pytest.raises(RuntimeError, match="divisible by 2"):

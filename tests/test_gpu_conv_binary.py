@@ -39,6 +39,8 @@ SHAPES = [
     (3, 2, 8, 6, 5, 1, 3),                                           # rows of 3 pooled cells: written without the ordered write-out
     (2, 93, 32, 32, 48, 1, 3),                                       # the thresholded channels of the large CIFAR topology
     (3, 5, 32, 32, 600, 1, 3),                                       # more kernels than histogram parts, not a multiple of 64
+    (3, 4, 32, 16, 12, 1, 3),                                        # exactly 128 pooled cells: two full blocks of 64 lanes
+    (2, 6, 24, 32, 10, 1, 3),                                        # exactly 192: three
 ]
 
 

@@ -148,9 +148,32 @@ def test_fc_config1_shape_properties():
 
 
 def test_transpose_kernel():
-    for shape, dt in (((7, 130), torch.float32), ((129, 64), torch.float64), ((3, 5), torch.int16), ((65, 66), torch.uint8)):
+    # small matrices take 32 x 32 tiles, from 2048 tiles of 64 x 64 on those: all four element sizes on both
+    for shape, dt in (((7, 130), torch.float32), ((129, 64), torch.float64), ((3, 5), torch.int16), ((65, 66), torch.uint8),
+                      ((3000, 3001), torch.float32), ((2900, 3100), torch.float64), ((3333, 2800), torch.int16), ((2950, 3050), torch.uint8)):
         t = (torch.rand(shape, device=DEV) * 100).to(dt)
         assert torch.equal(difflogic_hip.transpose(t), t.T.contiguous())
+
+
+@pytest.mark.parametrize("batch,dtype", [(21, torch.float32), (30, torch.float32), (19, torch.float64), (31, torch.float64),
+                                         (37, torch.float16), (60, torch.float16), (27, torch.float16)])
+def test_fc_weight_gradient_with_one_sample_per_lane_and_ragged_rows(batch, dtype):
+    # batches that no vector width divides take one sample per lane; 17 to 32 of them are a row of 32 lanes, more a row of 64:
+    # the reference-shaped weight-gradient call against the oracle
+    torch.manual_seed(batch)
+    in_dim, out_dim = 24, 40
+    layer = C.LogicLayer(in_dim, out_dim, implementation="cuda").to(DEV)
+    x = torch.rand(in_dim, batch, device=DEV).to(dtype)
+    gy = torch.randn(out_dim, batch, device=DEV).to(dtype)
+    gw = difflogic_hip.backward_w(x, layer.indices_0, layer.indices_1, gy)
+    assert gw.dtype == dtype and gw.shape == (out_dim, 16)
+    xl = x.float().cpu().double().t().contiguous()
+    wl = torch.full((out_dim, 16), 1 / 16, dtype=torch.float64, requires_grad=True)
+    y = O.logic_fc_forward(xl, layer.indices_0.cpu(), layer.indices_1.cpu(), wl)
+    y.backward(gy.float().cpu().double().t())
+    tol = {torch.float32: 1e-5, torch.float64: 1e-12, torch.float16: 2e-3}[dtype]
+    scale = wl.grad.abs().max().item()
+    assert (gw.double().cpu() - wl.grad).abs().max().item() <= tol * scale + (1e-3 if dtype == torch.float16 else 0.0)
 
 
 def test_fc_rejects_bad_inputs():
