@@ -685,3 +685,63 @@ def test_forward_with_one_kernel_per_lane_equals_the_position_major_kernel(n, ci
     # from the logits, with the folded coefficients and the padded copy left for the backward pass
     res = convlogic_hip.full_convlogic_forward_logits(x, layer.weights.detach(), layer.selection, *geo, want_folded=True, want_padded=True)
     assert (res[0] - y1).abs().max().item() <= (2e-6 if dtype == torch.float32 else 1e-14)
+
+
+def test_kernel_variants_behind_knobs_and_rare_shapes(monkeypatch):
+    # instantiations that only a knob or an unusual shape selects, each against the default path or the split layers
+    torch.manual_seed(12)
+    # 1. the softmax of the logits as a launch of its own instead of inside the staged forward: same step bit for bit
+    layer = C.ConvLogicLayer(4, 24, padding=1, complete=True, implementation="cuda").to(DEV)
+    x = torch.rand(6, 4, 12, 12, device=DEV)
+    gy = None
+    results = []
+    for knob in (None, "0", "1"):
+        set_knobs(monkeypatch, CLG_FWD_SOFTMAX_IN_KERNEL=knob)
+        xin = x.clone().requires_grad_(True)
+        layer.weights.grad = None
+        y = layer(xin)
+        gy = torch.randn_like(y) if gy is None else gy
+        y.backward(gy)
+        results.append((y.detach().clone(), xin.grad.clone(), layer.weights.grad.clone()))
+    set_knobs(monkeypatch, CLG_FWD_SOFTMAX_IN_KERNEL=None)
+    for other in results[1:]:
+        assert all(torch.equal(u, v) for u, v in zip(results[0], other))
+    # 2. narrower histogram shares of the binary-input weight gradient: same sums in another order
+    blayer = C.ConvLogicLayer(3, 10, padding=1, complete=True, implementation="cuda").to(DEV)
+    blayer.binary_input = True
+    xb = torch.randint(0, 2, (9, 3, 16, 16), device=DEV).float()
+    grads = []
+    for hl in (None, "32", "16"):
+        set_knobs(monkeypatch, CLG_BIN_HL=hl)
+        blayer.weights.grad = None
+        yb = blayer(xb)
+        yb.backward(torch.ones_like(yb) * 0.25)
+        grads.append(blayer.weights.grad.clone())
+    set_knobs(monkeypatch, CLG_BIN_HL=None)
+    for g in grads[1:]:
+        assert_grad_close(g, grads[0], rel=1e-5, name="grad_logits by histogram share")
+    # 3. the intermediate tensors in float64 against the split layers
+    full = C.ConvLogicLayer(3, 2, padding=1, kernel=3, implementation="cuda", complete=True, return_indices=True,
+                            return_intermediate=True).double().to(DEV)
+    conv = C.ConvLogicLayer(3, 2, padding=1, kernel=3, implementation="cuda").double().to(DEV)
+    tree1, tree2 = C.TreeLogicLayer(2, 4, implementation="cuda").double().to(DEV), C.TreeLogicLayer(2, 2, implementation="cuda").double().to(DEV)
+    conv.selection = full.selection
+    conv.weights.data.copy_(full.weights[:, 0:4])
+    tree1.weights.data.copy_(full.weights[:, 4:6])
+    tree2.weights.data.copy_(full.weights[:, 6:7])
+    xd = torch.randn(4, 3, 10, 10, device=DEV, dtype=torch.float64)
+    with torch.no_grad():
+        y_full, x1_full, x2_full, idx_full = full(xd)
+        x1 = conv(xd)
+        x2 = tree1(x1)
+        y_split, idx_split = C.PoolLogicLayer(return_indices=True)(tree2(x2))
+    assert torch.equal(idx_split.flatten(start_dim=2).to(torch.int32), idx_full)
+    assert torch.allclose(x1, x1_full, atol=1e-13) and torch.allclose(x2, x2_full, atol=1e-13) and torch.allclose(y_split, y_full, atol=1e-13)
+    # 4. the packed block with a window as large as the image (no staged or padded-copy plan): the float eval path's bits
+    import numpy as np
+    player = C.ConvLogicLayer(2, 5, padding=0, kernel=(120, 120), stride=2, complete=True, implementation="cuda").to(DEV).eval()
+    bits = torch.randint(0, 2, (70, 2, 151, 151), device=DEV).bool()
+    with torch.no_grad():
+        yf = player(bits.float())
+    p = player(C.PackBitsTensor(bits, 64))
+    assert np.array_equal(O.unpack_image(p.t.cpu().numpy(), p.pad_len), yf.cpu().numpy() > 0.5)

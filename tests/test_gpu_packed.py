@@ -274,3 +274,21 @@ def test_eval_packed_config2_full_size_vs_c_oracle():
     for g in range(k):                                               # class g: rows g*per .. (g+1)*per, sample s = bit s%8 of byte s/8
         bits = np.unpackbits(ref[g * per:(g + 1) * per].view(np.uint8), axis=1, bitorder="little")
         assert np.array_equal(counts[:, g], bits.sum(axis=0, dtype=np.int32)), f"class {g}"
+
+
+def test_eval_packed_walk_with_eight_vectors_per_lane(monkeypatch):
+    # the walk-ordered kernel keeps 4 vectors of a row per lane by default; 8 is the variant a knob selects: same words
+    from tests.gpu_util import set_knobs
+    torch.manual_seed(4)
+    layer = C.LogicLayer(120, 200, implementation="cuda").to(DEV).eval()
+    x = torch.randint(0, 2, (70000, 120), device=DEV).bool()         # rows of 1094 words: more than one 8 KiB chunk, ragged
+    outs = []
+    for r in (None, "8", "4"):
+        set_knobs(monkeypatch, CLG_EVAL_WALK_R=r)
+        with torch.no_grad():
+            outs.append(layer(C.PackBitsTensor(x, 64)).t.clone())
+    set_knobs(monkeypatch, CLG_EVAL_WALK_R=None)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    words, pad = O.pack_bits(x.cpu().numpy().T, 64)
+    want = O.eval_packed(words, layer.indices_0.cpu().numpy(), layer.indices_1.cpu().numpy(), layer.weights.argmax(-1).cpu().numpy().astype(np.uint8))
+    assert np.array_equal(outs[1].cpu().numpy(), want)
