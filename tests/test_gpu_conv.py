@@ -745,3 +745,34 @@ def test_kernel_variants_behind_knobs_and_rare_shapes(monkeypatch):
         yf = player(bits.float())
     p = player(C.PackBitsTensor(bits, 64))
     assert np.array_equal(O.unpack_image(p.t.cpu().numpy(), p.pad_len), yf.cpu().numpy() > 0.5)
+
+
+@pytest.mark.parametrize("hw,pad", [(4, 1), (8, 1), (16, 1), (28, 1), (32, 1), (6, 0), (10, 0), (18, 0), (30, 0), (34, 0)])
+def test_staged_forward_at_every_row_pitch_with_all_planes_and_with_a_plane_subset(hw, pad, monkeypatch):
+    # the staged forward is compiled for the row pitches of the common image widths (5, 9, 17, 29, 33 and any other), with all
+    # input planes of a sample in LDS or the two planes a kernel reads, for float and for packed words: every variant gives
+    # the values of the default choice for the shape bit for bit, and the packed block the float eval path's bits
+    import numpy as np
+    torch.manual_seed(hw * 10 + pad)
+    n, cin, cout = 70, 6, 10
+    layer = C.ConvLogicLayer(cin, cout, padding=pad, kernel=3, complete=True, implementation="cuda", return_indices=True).to(DEV)
+    x = torch.randn(n, cin, hw, hw, device=DEV)
+    bits = torch.randint(0, 2, (n, cin, hw, hw), device=DEV).bool()
+    with torch.no_grad():
+        y0, idx0 = layer(x)
+        layer.eval()
+        yb0, _ = layer(bits.float())
+        layer.train()
+    routed, _, idx_ref, _, _, _, _, x4 = block_oracle(x, layer.weights, layer.selection, (1, 1), (pad, pad), (3, 3), idx0)
+    check_pool_route(idx0, idx_ref, x4, tol=1e-5 * max(1.0, x4.abs().max().item()))
+    assert (y0.cpu() - routed).abs().max().item() <= 1e-5 * max(1.0, x4.abs().max().item())
+    for subset in ("0", "1"):
+        set_knobs(monkeypatch, CLG_FWD_DIRECT="0", CLG_FWD_KPL="0", CLG_FWD_4X4="0", CLG_FWD_SUBSET=subset)
+        with torch.no_grad():
+            y, idx = layer(x)
+            assert torch.equal(y, y0) and torch.equal(idx, idx0), (hw, pad, subset)
+            layer.eval()
+            p = layer(C.PackBitsTensor(bits, 64))
+            layer.train()
+        assert np.array_equal(O.unpack_image(p.t.cpu().numpy(), p.pad_len), yb0.cpu().numpy() > 0.5), (hw, pad, subset)
+    set_knobs(monkeypatch, CLG_FWD_DIRECT=None, CLG_FWD_KPL=None, CLG_FWD_4X4=None, CLG_FWD_SUBSET=None)
