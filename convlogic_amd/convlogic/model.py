@@ -30,7 +30,9 @@ def _prefold(owner, network, x, mode=True):
     if cache is not None and cache[0] == (x.dtype, x.device):
         _, picked, plan = cache
         weights = [m._parameters["weights"] for m in picked]
-        if not (plan.matches(weights) and all(m.prefold_candidate() is w for m, w in zip(picked, weights))):
+        if plan is None:                                             # nothing to fold when the cache was made: look again
+            cache = None
+        elif not (plan.matches(weights) and all(m.prefold_candidate() is w for m, w in zip(picked, weights))):
             cache = None
     if cache is None:
         layers = [m for m in network if isinstance(m, (ConvLogicLayer, LogicLayer))]

@@ -418,3 +418,29 @@ def test_networks_stepping_on_four_host_threads_equal_their_serial_runs():
         for step, ((oa, ga), (ob, gb)) in enumerate(zip(alone, together)):
             assert torch.equal(oa, ob), (i, step)
             assert all(torch.equal(u, v) for u, v in zip(ga, gb)), (i, step)
+
+
+def test_python_implementation_of_a_network_trains_on_the_gpu_next_to_the_hip_one():
+    # implementation="python" (torch ops) with device tensors: nothing of the network-level shortcuts applies, and a second
+    # step must find that out as the first did (the fold cache of a network with nothing to fold once broke it);
+    # the HIP network follows the same trajectory
+    torch.manual_seed(6)
+    a = C.ConvLogicMnistModel(k_param=2, tau=6.5, implementation="cuda").to(DEV)
+    b = C.ConvLogicMnistModel(k_param=2, tau=6.5, implementation="python").to(DEV)
+    b.load_state_dict(a.state_dict(), strict=False)
+    opt_a, opt_b = torch.optim.SGD(a.parameters(), lr=0.5), torch.optim.SGD(b.parameters(), lr=0.5)
+    for _ in range(3):
+        x = torch.randint(0, 2, (32, 1, 28, 28), device=DEV).float()
+        labels = torch.randint(0, 10, (32,), device=DEV)
+        loss_a = torch.nn.functional.cross_entropy(a(x), labels)
+        loss_b = torch.nn.functional.cross_entropy(b(x), labels)
+        opt_a.zero_grad()
+        opt_b.zero_grad()
+        loss_a.backward()
+        loss_b.backward()
+        # (the losses, not the gradients: on 0/1 inputs the pooling windows are full of ties and near ties, which the two
+        # implementations may route to different positions -- both valid, but not the same gradient element by element)
+        assert abs(loss_a.item() - loss_b.item()) <= 1e-4 * max(1.0, abs(loss_b.item()))
+        assert all(torch.isfinite(q.grad).all() for q in b.parameters())
+        opt_a.step()
+        opt_b.step()
