@@ -32,6 +32,19 @@ def _grad_close(got, ref, rel, what):
     assert (got - ref).norm().item() <= rel * (ref.norm().item() + 1e-30), (what, "L2")
 
 
+def _grad_close_or_as_good_as_float32(got, ref32, ref64, rel, what):
+    """_grad_close against the oracle in the tensors' own precision; where cancellation (the softmax backward of a peaked
+    distribution, sums of terms of both signs) makes that oracle itself lose more than the bound, the kernel has to be within
+    four times the float32 oracle's distance from the float64 oracle."""
+    try:
+        _grad_close(got, ref32, rel, what)
+    except AssertionError:
+        r64 = ref64().detach().double().cpu()
+        lost = (ref32.detach().double().cpu() - r64).abs().max().item()
+        mine = (got.detach().double().cpu() - r64).abs().max().item()
+        assert got.dtype == torch.float32 and mine <= 4 * lost + 1e-12, (what, mine, lost)
+
+
 def _block_cases(seed, count):
     rng = random.Random(seed)
     while count:
@@ -125,7 +138,13 @@ def test_random_blocks_on_the_training_path_of_the_module():
         routed.backward(gy.cpu())
         if need_gx:
             _grad_close(x.grad, xl.grad, rel, ("grad_x", case))
-        _grad_close(layer.weights.grad, ll.grad, rel, ("grad_logits", case))
+
+        def in_float64():
+            r64, _, _, _, _, l64, _, _ = block_oracle(x.detach().double(), layer.weights.detach().double(), layer.selection, *pairs, idx)
+            r64.backward(gy.cpu().double())
+            return l64.grad
+
+        _grad_close_or_as_good_as_float32(layer.weights.grad, ll.grad, in_float64, rel, ("grad_logits", case))
         layer.check_binary_input()
 
 
@@ -185,7 +204,16 @@ def test_random_logic_layers_and_group_sums_against_the_oracle():
         tol, rel = _tolerances(dtype)
         assert (y.detach().cpu() - y_ref.detach()).abs().max().item() <= tol * max(1.0, y_ref.detach().abs().max().item()), case
         _grad_close(x.grad, xl.grad * gf, rel, ("grad_x", case))
-        _grad_close(layer.weights.grad, ll.grad, rel, ("grad_logits", case))
+
+        def in_float64():
+            x64, l64 = x.detach().cpu().double(), layer.weights.detach().cpu().double().requires_grad_(True)
+            y64 = O.logic_fc_forward(x64.transpose(0, 1) if case["feature_major_view"] else x64, idx0, idx1, torch.softmax(l64, -1))
+            if case["tail"] != "none":
+                y64 = O.group_sum(y64, case["k"], case["tau"])
+            y64.backward(gy.cpu().double())
+            return l64.grad
+
+        _grad_close_or_as_good_as_float32(layer.weights.grad, ll.grad, in_float64, rel, ("grad_logits", case))
         layer.eval()
         with torch.no_grad():
             ye = layer(xin.detach())
